@@ -1,0 +1,199 @@
+"""Benchmark of the MXFP4 block-scaled GEMM on one MI355X.
+
+One "step" is one GEMM of the headline workload (M = N = K = 8192, bf16 out,
+seed 1, inputs resident in HBM).  Prints ONE JSON line: whole-job TFLOP/s, the
+MFMA roofline of the tile kernel, the HBM roofline of the M = 16 decode shape
+and the reference's CPU path (torch dequantise + f32 matmul) timed on a bounded
+sample on this box's host cores.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3_m16|...]
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_MXFP4_TFLOPS = 10100.0   # MI355X dense FP4 MFMA
+PEAK_HBM_GBPS = 8000.0        # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (m, n, k, out dtype, seed, scale range)
+    "cfg1": (1024, 1024, 1024, "f32", 0, (124, 130)),
+    "cfg2": (8192, 8192, 8192, "bf16", 1, (124, 130)),
+    "cfg3_m1": (1, 28672, 8192, "bf16", 2, (120, 134)),
+    "cfg3_m16": (16, 28672, 8192, "bf16", 2, (120, 134)),
+    "cfg3_m32": (32, 28672, 8192, "bf16", 2, (120, 134)),
+    "cfg5": (4093, 6144, 7168, "f32", 4, (100, 154)),
+}
+
+
+def gemm_flops(m, n, k):
+    return 2 * m * n * k
+
+
+def gemm_bytes(m, n, k, out_bytes):
+    return m * k // 2 + m * k // 32 + n * k // 2 + n * k // 32 + m * n * out_bytes
+
+
+def make_gpu_inputs(torch, m, n, k, seed, scale_range, device, copies=1):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    lo, hi = scale_range
+    sets = []
+    for _ in range(copies):
+        x = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+        w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+        xs = torch.randint(lo, hi + 1, (m, k // 32), dtype=torch.uint8, generator=g)
+        ws = torch.randint(lo, hi + 1, (n, k // 32), dtype=torch.uint8, generator=g)
+        sets.append(tuple(t.to(device) for t in (x, xs, w, ws)))
+    return sets
+
+
+def time_gemm(torch, wave_amd, sets, out, steps, warmup, **kw):
+    """K launches back to back on the current stream; returns (wall seconds for
+    all K, average seconds per launch from HIP events on that stream)."""
+    for i in range(warmup):
+        x, xs, w, ws = sets[i % len(sets)]
+        wave_amd.mxfp4_gemm(x, xs, w, ws, out, **kw)
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(steps):
+        x, xs, w, ws = sets[i % len(sets)]
+        wave_amd.mxfp4_gemm(x, xs, w, ws, out, **kw)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, ev0.elapsed_time(ev1) * 1e-3 / steps
+
+
+def cpu_baseline(torch, m, n, k, seed, scale_range, sample_rows):
+    """The reference's CPU path (torch dequantise + f32 mm) on `sample_rows`
+    rows of A against all of B, on this box's host cores."""
+    from oracle.torch_oracle import torch_scaled_gemm_mxfp4
+
+    cores = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    threads = min(cores, int(env)) if env and env.isdigit() else cores
+    torch.set_num_threads(threads)
+    rows = min(sample_rows, m)
+    (x, xs, w, ws), = make_gpu_inputs(torch, rows, n, k, seed, scale_range, "cpu")
+    timings = {}
+    torch_scaled_gemm_mxfp4(x[:8], w[:64], xs[:8], ws[:64])  # warm the thread pool
+    t0 = time.perf_counter()
+    torch_scaled_gemm_mxfp4(x, w, xs, ws, timings=timings)
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(gemm_flops(rows, n, k) / dt / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"rows 0..{rows - 1} of A against all of B ({rows}x{n}x{k}), one run after a warm-up",
+        "seconds": round(dt, 3),
+        "dequant_s": round(timings["dequant_s"], 3),
+        "matmul_s": round(timings["matmul_s"], 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode-shape leg")
+    ap.add_argument("--cpu-rows", type=int, default=2048)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this operator runs on one GPU; --gpus N with N > 1 is not supported "
+              "(the path shards by N or M with no exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import wave_amd
+    from wave_amd import _lib
+
+    _lib.load()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    m, n, k, od, seed, srange = WORKLOADS[args.workload]
+    out_dtype = torch.bfloat16 if od == "bf16" else torch.float32
+    out_bytes = 2 if od == "bf16" else 4
+    memory_bound = m <= 64
+    # memory-bound shapes rotate distinct operand sets so B is not cache resident
+    copies = 4 if memory_bound else 1
+    sets = make_gpu_inputs(torch, m, n, k, seed, srange, dev, copies=copies)
+    out = torch.empty(m, n, dtype=out_dtype, device=dev)
+    wall, per_launch = time_gemm(torch, wave_amd, sets, out, args.steps, args.warmup, variant=args.variant)
+
+    flops, nbytes = gemm_flops(m, n, k), gemm_bytes(m, n, k, out_bytes)
+    ms_per_step = wall / args.steps * 1e3
+    tflops = flops / (wall / args.steps) / 1e12
+    if memory_bound:
+        achieved = nbytes / per_launch / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": None,
+                    "kernel": "skinny_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
+    else:
+        achieved = flops / per_launch / 1e12
+        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_MXFP4_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_MXFP4_TFLOPS, 4), "traffic": None,
+                    "kernel": "tile_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
+
+    result = {
+        "metric": "MXFP4 GEMM TFLOPS + % of FP4 MFMA peak (8192^3); GB/s % HBM at M=16",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, " + od + " out",
+        "data": "synthetic (seeded uniform nibbles and scales), random weights",
+        "config": {"workload": f"{args.workload}: M={m} N={n} K={k} {od} out seed {seed}",
+                   "variant": args.variant, "operand_sets_rotated": copies},
+        "frac_of_mxfp4_peak": round(tflops / PEAK_MXFP4_TFLOPS, 4),
+        "gbps": round(nbytes / (wall / args.steps) / 1e9, 1),
+        "roofline": roofline,
+    }
+
+    if not args.no_decode and args.workload == "cfg2":
+        dm, dn, dk, _, dseed, drange = WORKLOADS["cfg3_m16"]
+        dsets = make_gpu_inputs(torch, dm, dn, dk, dseed, drange, dev, copies=4)
+        dout = torch.empty(dm, dn, dtype=torch.bfloat16, device=dev)
+        dwall, dper = time_gemm(torch, wave_amd, dsets, dout, max(args.steps, 20) * 4, args.warmup)
+        dbytes = gemm_bytes(dm, dn, dk, 2)
+        result["decode_m16"] = {
+            "workload": f"cfg3_m16: M={dm} N={dn} K={dk} bf16 out seed {dseed}, 4 operand sets rotated (HBM-cold B)",
+            "launch_us": round(dper * 1e6, 2),
+            "gbps": round(dbytes / dper / 1e9, 1),
+            "frac_of_hbm_peak": round(dbytes / dper / 1e9 / PEAK_HBM_GBPS, 4),
+            "bytes": dbytes,
+        }
+        del dsets, dout
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, m, n, k, seed, srange, args.cpu_rows)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,148 @@
+/*
+ * wave_mxfp4.h - C ABI of the MI355X (gfx950) MXFP4 block-scaled GEMM library.
+ *
+ * The library replaces the GPU kernels the reference generates from its
+ * scaled-GEMM templates together with the launch call that runs them.  Every
+ * entry point takes plain device pointers, sizes and a HIP stream, validates
+ * its arguments before touching HIP, never synchronises and never throws;
+ * it returns 0 or a negative wave_mxfp4_status.  Work is enqueued on the given
+ * stream (NULL = the default stream), like the reference's launch
+ * (wave_lang/kernel/wave/runtime/runtime.cpp:123-203 called from
+ * wave_lang/kernel/wave/utils/run_utils.py:62-134).
+ *
+ * Data formats (inputs of the drop-in API):
+ *   A        [M, K/2]  uint8, two e2m1 codes per byte, low nibble first
+ *   B        [N, K/2]  uint8, N-major, so C = A . B^T
+ *   A_scale  [M, K/32] uint8 e8m0, one per 32 elements along K
+ *   B_scale  [N, K/32] uint8 e8m0
+ *   C        [M, N]    float or bf16, row-major, written in place
+ * (wave_lang/kernel/wave/templates/tagged_mxfp4_gemm.py:93-122,
+ *  wave_lang/kernel/wave/utils/mxfp_utils.py:20-57).
+ */
+#ifndef WAVE_MXFP4_H_
+#define WAVE_MXFP4_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  WAVE_MXFP4_OK = 0,
+  WAVE_MXFP4_ERR_NULL_POINTER = -1,
+  WAVE_MXFP4_ERR_BAD_SHAPE = -2,     /* negative dims, K % 32 != 0, layout divisibility */
+  WAVE_MXFP4_ERR_BAD_ENUM = -3,      /* dtype / layout / variant out of range */
+  WAVE_MXFP4_ERR_MISALIGNED = -4,    /* a pointer is not aligned as documented */
+  WAVE_MXFP4_ERR_WORKSPACE = -5,     /* split-K workspace missing or too small */
+  WAVE_MXFP4_ERR_BAD_SPLIT = -6,     /* K per split < 256 or not a multiple of 256 */
+  WAVE_MXFP4_ERR_HIP = -7,           /* a HIP call failed; see wave_mxfp4_last_hip_error */
+  WAVE_MXFP4_ERR_UNSUPPORTED = -8
+} wave_mxfp4_status;
+
+/* Output element type, fixed per kernel build in the reference
+ * (tagged_mxfp4_gemm.py:62-65,120-122); bf16 is round-to-nearest-even of the
+ * f32 accumulator. */
+typedef enum { WAVE_MXFP4_OUT_F32 = 0, WAVE_MXFP4_OUT_BF16 = 1 } wave_mxfp4_out_dtype;
+
+/* Scale storage.  ROW_MAJOR is [R, K/32].  E8M0_SHUFFLE is the tile order of
+ * e8m0_shuffle (mxfp_utils.py:113-128, tagged_mxfp4_gemm.py:485-536) over a
+ * buffer padded to ceil(R/32)*32 rows and ceil(K/32/8)*8 columns; the buffer
+ * must hold every byte of that padded shape (the reference's final slice back
+ * to [R, K/32] loses bytes unless R % 32 == 0 and K % 256 == 0). */
+typedef enum { WAVE_MXFP4_SCALE_ROW_MAJOR = 0, WAVE_MXFP4_SCALE_E8M0_SHUFFLE = 1 } wave_mxfp4_scale_layout;
+
+/* B storage.  PRESHUFFLE is b_preshuffle (mxfp_utils.py:98-110,
+ * tagged_mxfp4_gemm.py:465-483); needs N % 16 == 0 and K % 64 == 0. */
+typedef enum { WAVE_MXFP4_B_ROW_MAJOR = 0, WAVE_MXFP4_B_PRESHUFFLE = 1 } wave_mxfp4_b_layout;
+
+/* Kernel selection.  AUTO picks by shape.  The others force one kernel and
+ * mirror the reference's (block_shape, wave_shape) template arguments
+ * (tagged_mxfp4_gemm.py:38-48). */
+typedef enum {
+  WAVE_MXFP4_VARIANT_AUTO = 0,
+  WAVE_MXFP4_VARIANT_T256x256_W2x2 = 1, /* 256x256x256 tile, 4 waves */
+  WAVE_MXFP4_VARIANT_T256x256_W4x2 = 2, /* 256x256x256 tile, 8 waves */
+  WAVE_MXFP4_VARIANT_T128x128_W2x2 = 3, /* 128x128x256 tile, 4 waves */
+  WAVE_MXFP4_VARIANT_T256x128_W2x2 = 4, /* 256x128x256 tile, 4 waves */
+  WAVE_MXFP4_VARIANT_T128x256_W2x2 = 5, /* 128x256x256 tile, 4 waves */
+  WAVE_MXFP4_VARIANT_SKINNY = 6,        /* M <= 64 streaming kernel */
+  WAVE_MXFP4_VARIANT_NAIVE = 7,         /* one thread per C element, for cross-checks */
+  WAVE_MXFP4_VARIANT_COUNT_
+} wave_mxfp4_variant;
+
+/*
+ * C[M,N] = dequant(A) . dequant(B)^T.
+ * Replaces the compiled kernel call gemm(x, x_scales, w_t, w_scales, out)
+ * (tests/kernel/wave_gemm_mxfp_test.py:194-201; kernels of
+ * tagged_mxfp4_gemm.py:38-145,334-403,950-991 and the split-K family
+ * :611-947) and its launch (runtime.cpp:123-203).
+ *   split_k   0 = automatic, 1 = off, n > 1 = n splits along K; each split
+ *             must own a multiple of 256 elements (tagged_mxfp4_gemm.py:636-645).
+ *             Partial sums are kept in f32 in `workspace` and reduced in a
+ *             fixed order, so C is overwritten, never accumulated into.
+ *   workspace device scratch of at least wave_mxfp4_workspace_bytes(...) bytes,
+ *             256-byte aligned; may be NULL when that size is 0.
+ * A, B must be 16-byte aligned; scales 8-byte aligned; C 16-byte aligned.
+ */
+int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
+                    int64_t m, int64_t n, int64_t k, int out_dtype, int a_scale_layout,
+                    int b_scale_layout, int b_layout, int split_k, void *workspace,
+                    size_t workspace_bytes, int variant, void *hip_stream);
+
+/* Scratch bytes wave_mxfp4_gemm needs for (m, n, k, split_k, variant); 0 when no
+ * split is taken.  With split_k == 0 it returns the size for the split the
+ * library would pick by itself. */
+size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant);
+
+/*
+ * Grouped (MoE) GEMM: rows offsets[e] .. offsets[e+1]-1 of A (sorted by expert)
+ * are multiplied by expert e's B[e] [N, K/2] with B_scale[e]; C is
+ * [total_rows, N].  `offsets` is a DEVICE array of num_groups+1 int32,
+ * non-decreasing, offsets[0] = 0, offsets[num_groups] <= total_rows; empty
+ * groups are allowed.  B is [E, N, K/2]; B_scale is [E, N, K/32] row-major, or
+ * E shuffled buffers of ceil(N/32)*32 x ceil(K/256)*8 bytes each.
+ * The reference has no grouped MXFP4 kernel: this replaces its per-expert
+ * Python loop over single GEMMs (tests/kernel/moe_test.py:175-246).
+ */
+int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,
+                            void *c, const int32_t *offsets, int num_groups, int64_t total_rows,
+                            int64_t n, int64_t k, int out_dtype, int a_scale_layout,
+                            int b_scale_layout, int b_layout, int variant, void *hip_stream);
+
+/* Packed e2m1 [rows, kp] -> f32 [rows, 2*kp] through the 16-entry table, code 8
+ * gives -0.0 (mxfp_utils.py:60-83).  Bit-exact. */
+int wave_mxfp4_to_f32(const void *q, float *out, int64_t rows, int64_t kp, void *hip_stream);
+
+/* e8m0 bytes -> f32 2^(s-127), 255 -> NaN, 0 -> 2^-127 (mxfp_utils.py:86-95).
+ * Bit-exact. */
+int wave_mxfp4_e8m0_to_f32(const void *s, float *out, int64_t count, void *hip_stream);
+
+/* out[r, e] = value(q[r, e]) * scale(r, e / 32), f32, the operand the reference
+ * feeds to its matmul (mxfp_utils.py:135-143).  Bit-exact. */
+int wave_mxfp4_dequant(const void *q, const void *scale, float *out, int64_t rows, int64_t k,
+                       int scale_layout, void *hip_stream);
+
+/* Device-side e8m0_shuffle (mxfp_utils.py:113-128) into the padded buffer of
+ * ceil(rows/32)*32 x ceil(ks/8)*8 bytes (padding bytes written as 0). */
+int wave_mxfp4_e8m0_shuffle(const void *scale, void *out, int64_t rows, int64_t ks, void *hip_stream);
+size_t wave_mxfp4_e8m0_shuffle_bytes(int64_t rows, int64_t ks);
+
+/* Device-side b_preshuffle (mxfp_utils.py:98-110); rows % 16 == 0, kp % 32 == 0. */
+int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, void *hip_stream);
+
+/* Text for a status code; never NULL (the reference reports errors as
+ * exceptions carrying hipGetErrorName/String, runtime.cpp:96-109). */
+const char *wave_mxfp4_status_string(int status);
+
+/* Name and text of the last HIP error this thread hit inside the library. */
+const char *wave_mxfp4_last_hip_error(void);
+
+/* Library ABI version (bumped on any signature change). */
+int wave_mxfp4_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WAVE_MXFP4_H_ */

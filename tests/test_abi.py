@@ -1,0 +1,135 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol the header
+declares, and rejects bad arguments with a status code before touching HIP."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from wave_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "wave_mxfp4.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(wave_mxfp4_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 12
+    for name in names:
+        assert hasattr(lib, name), name
+    assert sorted(_lib.EXPORTS) == names
+
+
+def test_abi_version_and_status_strings():
+    lib = _lib.load()
+    assert lib.wave_mxfp4_abi_version() == _lib.ABI_VERSION
+    seen = set()
+    for code in range(0, -9, -1):
+        s = lib.wave_mxfp4_status_string(code).decode()
+        assert s and s != "unknown status"
+        seen.add(s)
+    assert len(seen) == 9
+    assert lib.wave_mxfp4_status_string(-99).decode() == "unknown status"
+
+
+# A 16-byte aligned fake address: validation must reject the call before any
+# pointer is dereferenced or any HIP call is made (there is no GPU here).
+P = 0x1000
+
+
+def gemm(lib, a=P, as_=P, b=P, bs=P, c=P, m=64, n=64, k=256, od=0, asl=0, bsl=0, bl=0, split=1, ws=None,
+         wsb=0, variant=0):
+    return lib.wave_mxfp4_gemm(a, as_, b, bs, c, m, n, k, od, asl, bsl, bl, split, ws, wsb, variant, None)
+
+
+def test_gemm_argument_validation():
+    lib = _lib.load()
+    assert gemm(lib, a=None) == _lib.ERR_NULL_POINTER
+    assert gemm(lib, as_=None) == _lib.ERR_NULL_POINTER
+    assert gemm(lib, b=None) == _lib.ERR_NULL_POINTER
+    assert gemm(lib, bs=None) == _lib.ERR_NULL_POINTER
+    assert gemm(lib, c=None) == _lib.ERR_NULL_POINTER
+    assert gemm(lib, m=-1) == _lib.ERR_BAD_SHAPE
+    assert gemm(lib, n=-5) == _lib.ERR_BAD_SHAPE
+    assert gemm(lib, k=-32) == _lib.ERR_BAD_SHAPE
+    assert gemm(lib, k=48) == _lib.ERR_BAD_SHAPE          # K % 32 != 0
+    assert gemm(lib, od=2) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, asl=2) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, bsl=-1) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, bl=7) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, variant=99) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, bl=1, n=24) == _lib.ERR_BAD_SHAPE    # preshuffle needs N % 16 == 0
+    assert gemm(lib, bl=1, k=96) == _lib.ERR_BAD_SHAPE    # and K % 64 == 0
+    assert gemm(lib, a=P + 4) == _lib.ERR_MISALIGNED
+    assert gemm(lib, b=P + 8) == _lib.ERR_MISALIGNED
+    assert gemm(lib, as_=P + 2) == _lib.ERR_MISALIGNED
+    assert gemm(lib, c=P + 8) == _lib.ERR_MISALIGNED
+    assert gemm(lib, split=-1) == _lib.ERR_BAD_SPLIT
+    assert gemm(lib, k=512, split=4) == _lib.ERR_BAD_SPLIT             # 128 per split < 256
+    assert gemm(lib, k=768, split=2) == _lib.ERR_BAD_SPLIT             # 384 not a multiple of 256
+    assert gemm(lib, m=128, k=1024, split=2, variant=3) == _lib.ERR_WORKSPACE  # no workspace given
+    assert gemm(lib, m=128, k=1024, split=2, variant=3, ws=P, wsb=16) == _lib.ERR_WORKSPACE
+    assert gemm(lib, m=128, variant=_lib.VARIANT_SKINNY) == _lib.ERR_UNSUPPORTED
+    # empty problems are fine and touch nothing
+    assert gemm(lib, m=0, a=None, as_=None, c=None) == _lib.OK
+    assert gemm(lib, n=0, b=None, bs=None, c=None) == _lib.OK
+
+
+def test_grouped_argument_validation():
+    lib = _lib.load()
+
+    def grouped(a=P, as_=P, b=P, bs=P, c=P, off=P, e=4, rows=256, n=64, k=256, od=1, asl=0, bsl=0, bl=0,
+                variant=0):
+        return lib.wave_mxfp4_gemm_grouped(a, as_, b, bs, c, off, e, rows, n, k, od, asl, bsl, bl, variant,
+                                           None)
+
+    assert grouped(off=None) == _lib.ERR_NULL_POINTER
+    assert grouped(a=None) == _lib.ERR_NULL_POINTER
+    assert grouped(e=-1) == _lib.ERR_BAD_SHAPE
+    assert grouped(k=40) == _lib.ERR_BAD_SHAPE
+    assert grouped(od=5) == _lib.ERR_BAD_ENUM
+    assert grouped(off=P + 2) == _lib.ERR_MISALIGNED
+    assert grouped(variant=_lib.VARIANT_SKINNY) == _lib.ERR_UNSUPPORTED
+    assert grouped(e=0) == _lib.OK
+    assert grouped(rows=0, a=None, as_=None, c=None) == _lib.OK
+
+
+def test_aux_argument_validation():
+    lib = _lib.load()
+    assert lib.wave_mxfp4_to_f32(None, P, 4, 4, None) == _lib.ERR_NULL_POINTER
+    assert lib.wave_mxfp4_to_f32(P, P, -1, 4, None) == _lib.ERR_BAD_SHAPE
+    assert lib.wave_mxfp4_to_f32(P, P, 0, 4, None) == _lib.OK
+    assert lib.wave_mxfp4_e8m0_to_f32(P, None, 4, None) == _lib.ERR_NULL_POINTER
+    assert lib.wave_mxfp4_e8m0_to_f32(P, P, -4, None) == _lib.ERR_BAD_SHAPE
+    assert lib.wave_mxfp4_dequant(P, P, P, 4, 48, 0, None) == _lib.ERR_BAD_SHAPE
+    assert lib.wave_mxfp4_dequant(P, P, P, 4, 64, 3, None) == _lib.ERR_BAD_ENUM
+    assert lib.wave_mxfp4_dequant(P, None, P, 4, 64, 0, None) == _lib.ERR_NULL_POINTER
+    assert lib.wave_mxfp4_e8m0_shuffle(None, P, 4, 4, None) == _lib.ERR_NULL_POINTER
+    assert lib.wave_mxfp4_b_preshuffle(P, P, 24, 32, None) == _lib.ERR_BAD_SHAPE
+    assert lib.wave_mxfp4_b_preshuffle(P, P, 32, 48, None) == _lib.ERR_BAD_SHAPE
+    assert lib.wave_mxfp4_b_preshuffle(P + 1, P, 32, 64, None) == _lib.ERR_MISALIGNED
+    assert lib.wave_mxfp4_e8m0_shuffle_bytes(4093, 224) == 4096 * 224
+    assert lib.wave_mxfp4_e8m0_shuffle_bytes(33, 9) == 64 * 16
+
+
+def test_workspace_bytes():
+    lib = _lib.load()
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, 0) == 0
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 4, 3) == 4 * 512 * 512 * 4
+    assert lib.wave_mxfp4_workspace_bytes(-1, 512, 1024, 4, 3) == 0
+
+
+def test_check_maps_status_to_exceptions():
+    with pytest.raises(ValueError, match="K not a multiple of 32"):
+        _lib.check(_lib.ERR_BAD_SHAPE, "x")
+    with pytest.raises(RuntimeError, match="HIP call failed"):
+        _lib.check(_lib.ERR_HIP, "x")
+    _lib.check(_lib.OK, "x")

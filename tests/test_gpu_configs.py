@@ -1,0 +1,203 @@
+"""GPU parity at the five benchmark configurations, full size.
+
+Where the whole exact oracle is too slow on host cores, rows are sampled
+(tile corners, tile interiors, the last row) against the exact oracle, every
+element is compared with the independent one-thread-per-element device kernel
+(itself pinned against the oracle on the sampled rows), and size-independent
+identities (checksum of checksums) close the gap."""
+
+import numpy as np
+import pytest
+import torch
+
+import wave_amd
+from oracle import c_oracle
+from oracle import mxfp4_oracle as orc
+from wave_amd import _lib
+
+from gpu_util import (BF16_ABS, BF16_REL, DEV, TILE_VARIANTS, assert_bf16_close, assert_close,
+                      assert_f32_close, run_gemm, to_gpu)
+
+pytestmark = pytest.mark.gpu
+
+
+def sample_rows(m, count, seed, tile=256):
+    rng = np.random.default_rng(seed)
+    fixed = [0, 1, 31, 32, tile - 1, tile, m // 2, m - tile, m - 2, m - 1]
+    rows = {r for r in fixed if 0 <= r < m}
+    while len(rows) < min(count, m):
+        rows.add(int(rng.integers(0, m)))
+    return np.array(sorted(rows), dtype=np.int64)
+
+
+def checksum_identities(c, x, xs, w_t, ws, rel_per_elem):
+    """C . 1 == deq(A) . (deq(B)^T . 1) and 1^T . C == (1^T . deq(A)) . deq(B)^T,
+    each within the sum of the per-element rounding allowances."""
+    c = c.astype(np.float64)
+    a = orc.dequant_f32(x, xs).astype(np.float64)
+    b = orc.dequant_f32(w_t, ws).astype(np.float64)
+    row_sum = a @ b.sum(axis=0)
+    col_sum = a.sum(axis=0) @ b.T
+    allow_r = rel_per_elem * np.abs(c).sum(axis=1) + 1e-6 * np.abs(row_sum).max()
+    allow_c = rel_per_elem * np.abs(c).sum(axis=0) + 1e-6 * np.abs(col_sum).max()
+    assert np.all(np.abs(c.sum(axis=1) - row_sum) <= allow_r)
+    assert np.all(np.abs(c.sum(axis=0) - col_sum) <= allow_c)
+
+
+def test_config1_1024_cubed_f32_seed0():
+    m = n = k = 1024
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=0, scale_lo=124, scale_hi=130)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    for vname, v in dict(TILE_VARIANTS, auto=_lib.VARIANT_AUTO, naive=_lib.VARIANT_NAIVE).items():
+        assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, variant=v), ref, vname)
+    # the reference's own f32 path agrees with the exact oracle at this size
+    assert_f32_close(orc.scaled_gemm_f32(x, w_t, xs, ws), ref, "f32 oracle")
+
+
+def test_config2_8192_cubed_bf16_seed1():
+    m = n = k = 8192
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=1, scale_lo=124, scale_hi=130)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    rows = sample_rows(m, 48, seed=1)
+    ref_rows = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+
+    naive = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, naive, variant=_lib.VARIANT_NAIVE)
+    naive = naive.cpu().numpy()
+    assert_f32_close(naive[rows], ref_rows, "naive kernel vs oracle rows")
+
+    for vname in ("auto", "t256x256_w2x2", "t256x256_w4x2"):
+        v = dict(TILE_VARIANTS, auto=_lib.VARIANT_AUTO)[vname]
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out, variant=v)
+        c = out.float().cpu().numpy()
+        assert_bf16_close(c[rows], ref_rows, f"{vname} vs oracle rows")
+        assert_bf16_close(c, naive, f"{vname} vs naive kernel, all elements")
+    checksum_identities(c, x, xs, w_t, ws, rel_per_elem=BF16_REL / 2 + BF16_ABS)
+
+
+@pytest.mark.parametrize("m", [1, 16, 32])
+def test_config3_decode_shapes_bf16_seed2(m):
+    n, k = 28672, 8192
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=2, scale_lo=120, scale_hi=134)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+
+    def run(**kw):
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out, **kw)
+        return out.float().cpu().numpy()
+
+    assert_bf16_close(run(), ref, "auto (skinny)")
+    for splits in (2, 4, 8):
+        assert_bf16_close(run(split_k=splits), ref, f"skinny split {splits}")
+        assert_bf16_close(run(split_k=splits, variant=_lib.VARIANT_T128x128_W2x2), ref, f"tile split {splits}")
+    # preshuffled weights and shuffled weight scales (static, prepared once)
+    gwp = wave_amd.b_preshuffle(gw)
+    gwss = wave_amd.e8m0_shuffle(gws)
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    wave_amd.mxfp4_gemm(gx, gxs, gwp, gwss, out, b_layout=_lib.B_PRESHUFFLE,
+                        b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
+    assert_bf16_close(out.float().cpu().numpy(), ref, "preshuffled B + shuffled B scales")
+
+
+def grouped_inputs(e, n, k, rows, seed, force_empty=()):
+    off = orc.make_group_offsets(e, rows, seed, force_empty=force_empty)
+    x, xs, _, _ = orc.make_inputs(rows, 1, k, seed, scale_lo=124, scale_hi=130)
+    rng = np.random.default_rng(seed + 100)
+    w = rng.integers(0, 256, size=(e, n, k // 2), dtype=np.uint8)
+    ws = rng.integers(124, 131, size=(e, n, k // 32), dtype=np.uint8)
+    return x, xs, w, ws, off
+
+
+def run_grouped(x, xs, w, ws, off, out_dtype, **kw):
+    gx, gxs, gw, gws, goff = to_gpu(x, xs, w, ws, off)
+    out = torch.full((x.shape[0], w.shape[1]), float("nan"), dtype=out_dtype, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out, **kw)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+def test_config4_grouped_moe_bf16_seed3():
+    e, n, k, rows = 8, 14336, 4096, 8192
+    x, xs, w, ws, off = grouped_inputs(e, n, k, rows, seed=3)
+    assert off[-1] == rows and len(set(np.diff(off))) > 1          # ragged
+    # sampled rows of every expert against the exact per-expert oracle
+    picks = []
+    for g in range(e):
+        lo, hi = int(off[g]), int(off[g + 1])
+        picks += [r for r in (lo, lo + 1, (lo + hi) // 2, hi - 1) if lo <= r < hi]
+    picks = np.array(sorted(set(picks)))
+    ref = np.empty((len(picks), n))
+    for i, r in enumerate(picks):
+        g = int(np.searchsorted(off, r, side="right") - 1)
+        ref[i] = c_oracle.scaled_gemm_exact(x[r:r + 1], w[g], xs[r:r + 1], ws[g])[0]
+    naive = run_grouped(x, xs, w, ws, off, torch.float32, variant=_lib.VARIANT_NAIVE)
+    assert_f32_close(naive[picks], ref, "naive grouped vs oracle rows")
+    for vname in ("auto", "t256x256_w2x2", "t128x128_w2x2"):
+        v = dict(TILE_VARIANTS, auto=_lib.VARIANT_AUTO)[vname]
+        c = run_grouped(x, xs, w, ws, off, torch.bfloat16, variant=v)
+        assert_bf16_close(c[picks], ref, f"{vname} vs oracle rows")
+        assert_bf16_close(c, naive, f"{vname} vs naive kernel, all elements")
+
+
+@pytest.mark.parametrize("force_empty", [(0,), (3, 4), (7,), (0, 1, 2, 3, 4, 5, 6)])
+def test_grouped_empty_groups_and_small(force_empty):
+    e, n, k, rows = 8, 160, 512, 700
+    x, xs, w, ws, off = grouped_inputs(e, n, k, rows, seed=21, force_empty=force_empty)
+    for g in force_empty:
+        assert off[g] == off[g + 1]
+    ref = orc.scaled_gemm_grouped_exact(x, xs, w, ws, off)
+    for v in (_lib.VARIANT_AUTO, _lib.VARIANT_T256x256_W4x2, _lib.VARIANT_NAIVE):
+        assert_f32_close(run_grouped(x, xs, w, ws, off, torch.float32, variant=v), ref, str(v))
+
+
+def test_grouped_rows_past_last_offset_untouched_and_layouts():
+    e, n, k, rows = 4, 96, 256, 300
+    x, xs, w, ws, off = grouped_inputs(e, n, k, 260, seed=22)
+    x = np.concatenate([x, np.zeros((40, k // 2), np.uint8)])
+    xs = np.concatenate([xs, np.full((40, k // 32), 127, np.uint8)])
+    ref = orc.scaled_gemm_grouped_exact(x, xs, w, ws, off)
+    c = run_grouped(x, xs, w, ws, off, torch.float32)
+    assert_f32_close(c[:260], ref[:260])
+    assert np.isnan(c[260:]).all()                                  # never written
+    # preshuffled expert weights and shuffled expert scales
+    wp = np.stack([orc.b_preshuffle(w[g]) for g in range(e)])
+    wss = np.stack([orc.e8m0_shuffle_padded(ws[g])[:96] for g in range(e)])
+    c2 = run_grouped(x, xs, wp, wss, off, torch.float32, b_layout=_lib.B_PRESHUFFLE,
+                     b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
+    assert np.array_equal(c2[:260], c[:260])
+
+
+def test_config5_edge_shape_shuffled_scales_f32_seed4():
+    m, n, k = 4093, 6144, 7168
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=4, scale_lo=100, scale_hi=154)
+    rows = sample_rows(m, 40, seed=4)
+    ref_rows = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+
+    def run(a_s, b_s, **kw):
+        out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+        wave_amd.mxfp4_gemm(gx, a_s, gw, b_s, out, **kw)
+        return out.cpu().numpy()
+
+    plain = run(gxs, gws)
+    assert_f32_close(plain[rows], ref_rows, "row-major scales vs oracle rows")
+    naive = run(gxs, gws, variant=_lib.VARIANT_NAIVE)
+    assert_f32_close(naive[rows], ref_rows, "naive kernel vs oracle rows")
+    assert_f32_close(plain, naive, "row-major scales vs naive kernel, all elements")
+
+    # scales in the preshuffled tile order: B clean (6144 % 32 == 0), A padded to 4096 rows
+    xs_sh = wave_amd.e8m0_shuffle(gxs)
+    ws_sh = wave_amd.e8m0_shuffle(gws)
+    assert xs_sh.shape == (4096, 224) and ws_sh.shape == (6144, 224)
+    assert np.array_equal(xs_sh.cpu().numpy(), orc.e8m0_shuffle_padded(xs)[:4096])
+    shuffled = run(xs_sh, ws_sh, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
+    assert np.array_equal(shuffled, plain)                          # same arithmetic, same bits
+    # and with preshuffled B on top
+    gwp = wave_amd.b_preshuffle(gw)
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm(gx, xs_sh, gwp, ws_sh, out, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
+                        b_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_layout=_lib.B_PRESHUFFLE)
+    assert np.array_equal(out.cpu().numpy(), plain)
+    checksum_identities(plain, x, xs, w_t, ws, rel_per_elem=2e-6)

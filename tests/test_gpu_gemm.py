@@ -1,0 +1,224 @@
+"""GPU parity of the MXFP4 GEMM through the C ABI: golden fixtures and small
+seeded cases against the exact oracle on every kernel variant and layout, the
+edge cases the reference's tests touch (M = 1, K tails, ragged N, NaN scales),
+and properties that hold at any size."""
+
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import wave_amd
+from oracle import c_oracle
+from oracle import mxfp4_oracle as orc
+from wave_amd import _lib
+
+from gpu_util import DEV, TILE_VARIANTS, assert_bf16_close, assert_close, assert_f32_close, run_gemm, to_gpu
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+ALL_VARIANTS = dict(TILE_VARIANTS, skinny=_lib.VARIANT_SKINNY, naive=_lib.VARIANT_NAIVE, auto=_lib.VARIANT_AUTO)
+
+
+@pytest.mark.parametrize("vname", sorted(ALL_VARIANTS))
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(HERE, "golden", "g_*x*.npz"))),
+                         ids=lambda p: os.path.basename(p)[:-4])
+def test_golden_fixtures_every_variant(path, vname):
+    g = np.load(path)
+    x, xs, w_t, ws, ref = g["x"], g["x_scales"], g["w_t"], g["w_scales"], g["c_exact"]
+    if vname == "skinny" and x.shape[0] > 64:
+        pytest.skip("skinny kernel serves M <= 64")
+    v = ALL_VARIANTS[vname]
+    assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, variant=v), ref, "f32")
+    assert_bf16_close(run_gemm(x, xs, w_t, ws, torch.bfloat16, variant=v), ref, "bf16")
+    # shuffled scales (padded buffers) give the same numbers
+    got = run_gemm(x, g["x_scales_shuffled"], w_t, g["w_scales_shuffled"], torch.float32, variant=v,
+                   a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
+    assert_f32_close(got, ref, "shuffled scales")
+    if g["w_t_preshuffled"].size:
+        got = run_gemm(x, xs, g["w_t_preshuffled"], ws, torch.float32, variant=v, b_layout=_lib.B_PRESHUFFLE)
+        assert_f32_close(got, ref, "preshuffled B")
+
+
+SMALL_SHAPES = [
+    (256, 256, 256), (512, 384, 1024), (300, 200, 512), (129, 257, 768), (1, 1, 32), (2, 3, 64),
+    (64, 64, 2048), (17, 1000, 1024), (1000, 17, 256), (255, 255, 8192), (4, 6, 224), (96, 130, 1664),
+]
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("m,n,k", SMALL_SHAPES)
+def test_auto_dispatch_small_shapes(m, n, k, out_dtype):
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + n + k, scale_lo=120, scale_hi=134)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    assert_close(run_gemm(x, xs, w_t, ws, out_dtype), ref, out_dtype, f"{m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("vname", sorted(TILE_VARIANTS))
+@pytest.mark.parametrize("m,n,k", [(512, 512, 512), (300, 520, 1280), (1, 40, 256), (257, 33, 2304)])
+def test_tile_variants_ragged_shapes(m, n, k, vname):
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=7 * m + n, scale_lo=110, scale_hi=140)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, variant=TILE_VARIANTS[vname]), ref, vname)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 32, 48, 64])
+@pytest.mark.parametrize("n,k", [(128, 1024), (1000, 4096), (48, 256), (30, 160)])
+def test_skinny_kernel(m, n, k):
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m * 31 + n, scale_lo=120, scale_hi=134)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    assert_bf16_close(run_gemm(x, xs, w_t, ws, torch.bfloat16, variant=_lib.VARIANT_SKINNY), ref)
+    assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, variant=_lib.VARIANT_SKINNY), ref)
+
+
+@pytest.mark.parametrize("vname", ["t128x128_w2x2", "t256x256_w2x2", "skinny"])
+@pytest.mark.parametrize("splits", [2, 4])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_split_k_equals_unsplit(vname, splits, out_dtype):
+    m = 48 if vname == "skinny" else 384
+    n, k = 640, 2048
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=splits, scale_lo=120, scale_hi=134)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    v = ALL_VARIANTS[vname]
+    got = run_gemm(x, xs, w_t, ws, out_dtype, variant=v, split_k=splits)
+    # f32 partials + one final rounding: the bf16 result stays within one ulp
+    assert_close(got, ref, out_dtype, f"{vname} split {splits}")
+    # C is overwritten, not accumulated into: a second call gives the same bits
+    again = run_gemm(x, xs, w_t, ws, out_dtype, variant=v, split_k=splits)
+    assert np.array_equal(got, again)
+
+
+def test_split_k_auto_and_caller_workspace():
+    m, n, k = 256, 256, 8192
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=3)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    need = wave_amd.workspace_bytes(m, n, k, split_k=0)
+    assert need > 0                      # a 1-tile grid with long K: the library wants to split
+    work = torch.empty(need, dtype=torch.uint8, device=DEV)
+    assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, split_k=0, workspace=work), ref)
+    with pytest.raises(ValueError, match="K per split"):
+        run_gemm(x, xs, w_t, ws, torch.float32, split_k=3)
+
+
+def test_exact_when_sums_fit_24_bits():
+    """Scales 124..127: every product is a multiple of 2^-8 and the sums stay
+    below 2^16, so the f32 result must equal the exact one bit for bit, on
+    every kernel (any summation order)."""
+    x, xs, w_t, ws = orc.make_inputs(320, 288, 1024, seed=9, scale_lo=124, scale_hi=127)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws).astype(np.float32)
+    for vname, v in ALL_VARIANTS.items():
+        if vname == "skinny":
+            continue
+        assert np.array_equal(run_gemm(x, xs, w_t, ws, torch.float32, variant=v), ref), vname
+    assert np.array_equal(run_gemm(x[:64], xs[:64], w_t, ws, torch.float32, variant=_lib.VARIANT_SKINNY), ref[:64])
+
+
+def test_one_hot_rows_read_back_dequantised_b_exactly():
+    """A row with a single 1.0 at element e and scale 2^0 makes C[m, :] the
+    dequantised column e of B: every value is representable, so it must match
+    the bit-exact dequantiser exactly (nibble order, scale group, layout)."""
+    n, k = 96, 512
+    rng = np.random.default_rng(4)
+    w_t = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    ws = rng.integers(100, 155, size=(n, k // 32), dtype=np.uint8)
+    picks = [0, 1, 31, 32, 33, 255, 256, 257, 511]
+    x = np.zeros((len(picks), k // 2), dtype=np.uint8)
+    for r, e in enumerate(picks):
+        x[r, e // 2] = 2 << (4 * (e & 1))          # code 2 = 1.0
+    xs = np.full((len(picks), k // 32), 127, dtype=np.uint8)
+    deq = orc.dequant_f32(w_t, ws)
+    want = deq[:, picks].T.astype(np.float32)
+    for v in (_lib.VARIANT_SKINNY, _lib.VARIANT_T128x128_W2x2, _lib.VARIANT_T256x256_W2x2):
+        got = run_gemm(x, xs, w_t, ws, torch.float32, variant=v)
+        assert np.array_equal(got, want), v
+
+
+def test_nan_scale_poisons_its_row_and_column():
+    x, xs, w_t, ws = orc.make_inputs(70, 90, 512, seed=5)
+    xs[3, 2] = 255
+    ws[40, 15] = 255
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    for v in (_lib.VARIANT_T128x128_W2x2, _lib.VARIANT_T256x256_W4x2, _lib.VARIANT_NAIVE):
+        assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, variant=v), ref, str(v))
+    assert_f32_close(run_gemm(x[:8], xs[:8], w_t, ws, torch.float32, variant=_lib.VARIANT_SKINNY), ref[:8])
+
+
+def test_extreme_scales_zero_byte():
+    """Scale byte 0 is 2^-127; paired with a large scale the product is an
+    ordinary number and must not be flushed."""
+    m, n, k = 32, 32, 256
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=6)
+    xs[:] = 0
+    ws[:] = 250
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    assert np.abs(ref).max() > 1.0
+    for v in (_lib.VARIANT_T128x128_W2x2, _lib.VARIANT_SKINNY):
+        assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, variant=v), ref, str(v))
+
+
+def test_row_and_column_permutation_equivariance():
+    """Permuting rows of A (with their scales) permutes rows of C bit for bit;
+    same for rows of B and columns of C."""
+    m, n, k = 512, 512, 1024
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=8, scale_lo=110, scale_hi=140)
+    base = run_gemm(x, xs, w_t, ws, torch.float32)
+    rng = np.random.default_rng(0)
+    pm, pn = rng.permutation(m), rng.permutation(n)
+    assert np.array_equal(run_gemm(x[pm], xs[pm], w_t, ws, torch.float32), base[pm])
+    assert np.array_equal(run_gemm(x, xs, w_t[pn], ws[pn], torch.float32), base[:, pn])
+
+
+def test_scale_shift_is_exact_power_of_two():
+    """Adding 1 to every A scale byte doubles C exactly."""
+    x, xs, w_t, ws = orc.make_inputs(200, 136, 768, seed=10, scale_lo=120, scale_hi=130)
+    a = run_gemm(x, xs, w_t, ws, torch.float32)
+    b = run_gemm(x, xs + 1, w_t, ws, torch.float32)
+    assert np.array_equal(b, 2.0 * a)
+
+
+def test_repeatable_and_poisoned_output():
+    """Same inputs, same bits, on every call; the kernel overwrites whatever C held."""
+    x, xs, w_t, ws = orc.make_inputs(700, 520, 2048, seed=11)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    outs = []
+    for fill in (0.0, float("nan"), 1e30):
+        out = torch.full((700, 520), fill, dtype=torch.float32, device=DEV)
+        wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out)
+        outs.append(out.cpu().numpy())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+def test_non_contiguous_inputs_and_side_stream():
+    """Non-contiguous operands are copied, not rejected; work goes to the
+    current stream without a sync (reference launch semantics)."""
+    m, n, k = 128, 192, 512
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=12)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    w_view = gw.T.contiguous().T           # [N, K/2] values, column-major storage
+    assert not w_view.is_contiguous()
+    out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert wave_amd.mxfp4_gemm(gx, gxs, w_view, gws, out) is None
+    side.synchronize()
+    assert_f32_close(out.cpu().numpy(), ref)
+
+
+def test_bad_arguments_raise():
+    x, xs, w_t, ws = to_gpu(*orc.make_inputs(64, 64, 256, seed=13))
+    out = torch.empty(64, 64, dtype=torch.float32, device=DEV)
+    with pytest.raises(ValueError):
+        wave_amd.mxfp4_gemm(x, xs, w_t[:, :64], ws, out)            # K mismatch
+    with pytest.raises(ValueError):
+        wave_amd.mxfp4_gemm(x, xs[:, :4], w_t, ws, out)             # scale shape
+    with pytest.raises(ValueError):
+        wave_amd.mxfp4_gemm(x, xs, w_t, ws, out.to(torch.float16))  # out dtype
+    with pytest.raises(ValueError):
+        wave_amd.mxfp4_gemm(x, xs, w_t, ws, out[:32])               # out shape
+    with pytest.raises(ValueError):
+        wave_amd.mxfp4_gemm(x.float(), xs, w_t, ws, out)            # operand dtype

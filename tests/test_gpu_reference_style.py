@@ -1,0 +1,151 @@
+"""The reference's own end-to-end tests of this path, re-expressed against the
+mirrored interface (wave_lang -> wave_amd): same template getters, schedules,
+``wave_compile``, input generator, call shape and tolerances
+(tests/kernel/wave_gemm_mxfp_test.py:637-775,778-1085,
+tests/kernel/wave_gemm_test.py:3641-3690).  The torch oracle is this
+repository's port of the reference's ``torchScaledGemmMXFP4``."""
+
+import pytest
+import torch
+
+import wave_amd.kernel.lang as tkl
+from oracle.torch_oracle import torch_scaled_gemm_mxfp4
+from wave_amd.kernel.lang import TORCH_DTYPE_TO_WAVE
+from wave_amd.kernel.wave.compile import wave_compile
+from wave_amd.kernel.wave.constraints import ScaledMMAType
+from wave_amd.kernel.wave.schedules import (
+    get_mxfp4_asymmetric_schedule,
+    get_mxfp4_dbuf_pingpong_schedule,
+    get_mxfp4_dbuf_pingpong_schedule_Bshuffled,
+    get_mxfp4_dbuf_schedule,
+)
+from wave_amd.kernel.wave.templates import (
+    get_tagged_mxfp4_gemm,
+    get_tagged_mxfp4_gemm_preshuffle_b,
+    get_tagged_mxfp4_gemm_preshuffle_b_wide_store,
+    get_tagged_mxfp4_gemm_preshuffle_scales,
+    get_tagged_mxfp4_gemm_preshuffle_scales_and_B,
+    get_tagged_splitk_mxfp4_gemm,
+)
+from wave_amd.kernel.wave.utils.mxfp_utils import (
+    b_preshuffle,
+    e8m0_shuffle,
+    generate_gemm_afp4wfp4_inputs,
+)
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def torchScaledGemmMXFP4(x, w, x_scales, w_scales):
+    """Reference signature: ``w`` is the transposed view [K/2, N]."""
+    return torch_scaled_gemm_mxfp4(x.cpu(), w.T.contiguous().cpu(), x_scales.cpu(), w_scales.cpu())
+
+
+@pytest.mark.parametrize("shape", [(1024, 1024, 8192)])
+@pytest.mark.parametrize("block_shape", [(256, 256, 256)])
+@pytest.mark.parametrize("wave_shape,use_stagger", [((2, 2), False), ((4, 2), True)])
+def testScaledGemmMXFP4ManualDoubleBuf(shape, block_shape, wave_shape, use_stagger):
+    gemm, options = get_tagged_mxfp4_gemm(shape, block_shape, wave_shape=wave_shape,
+                                          mfma_variant=ScaledMMAType.F32_16x16x128_F8F6F4)
+    gemm = wave_compile(options, gemm, get_mxfp4_dbuf_schedule(use_stagger=use_stagger))
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.float32, device=DEV)
+    w_t = w.T.contiguous()
+    gemm(x, x_scales, w_t, w_scales, out)
+    torch_out = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+@pytest.mark.parametrize("shape", [(1024, 1024, 8192), (1024, 3072, 8192)])
+def testScaledGemmMXFP4Bf16Output(shape):
+    gemm, options = get_tagged_mxfp4_gemm(shape, (256, 256, 256), wave_shape=(2, 2), output_dtype=tkl.bf16)
+    gemm = wave_compile(options, gemm, get_mxfp4_dbuf_schedule(use_stagger=False))
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.bfloat16, device=DEV)
+    gemm(x, x_scales, w.T.contiguous(), w_scales, out)
+    torch_out = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+@pytest.mark.parametrize("shape", [(1024, 1024, 8192), (256, 1024, 2048)])
+def testScaledGemmMXFP4PreshuffleScales(shape):
+    gemm, options = get_tagged_mxfp4_gemm_preshuffle_scales(shape, (256, 256, 256), wave_shape=(4, 2))
+    gemm = wave_compile(options, gemm, get_mxfp4_dbuf_pingpong_schedule(use_stagger=True, shape=shape))
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.float32, device=DEV)
+    gemm(x, e8m0_shuffle(x_scales), w.T.contiguous(), e8m0_shuffle(w_scales), out)
+    torch_out = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+@pytest.mark.parametrize("shape", [(1024, 1024, 8192)])
+@pytest.mark.parametrize("output_dtype", [tkl.f32, tkl.bf16])
+def testScaledGemmMXFP4PreshuffleScalesAndB(shape, output_dtype):
+    gemm, options = get_tagged_mxfp4_gemm_preshuffle_scales_and_B(shape, (256, 256, 256), wave_shape=(4, 2),
+                                                                  output_dtype=output_dtype)
+    gemm = wave_compile(options, gemm, get_mxfp4_dbuf_pingpong_schedule_Bshuffled(use_stagger=True, shape=shape))
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=output_dtype.torch_dtype, device=DEV)
+    gemm(x, e8m0_shuffle(x_scales), b_preshuffle(w.T.contiguous()), e8m0_shuffle(w_scales), out)
+    torch_out = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+@pytest.mark.parametrize("shape,block_shape", [((1024, 1024, 8192), (256, 256, 256)),
+                                               ((512, 768, 4096), (128, 256, 256)),
+                                               ((1024, 3072, 8192), (256, 192, 256))])
+@pytest.mark.parametrize("a_scale_preshuffle", [True, False])
+def testScaledGemmMXFP4PreshuffleB(shape, block_shape, a_scale_preshuffle):
+    gemm, options = get_tagged_mxfp4_gemm_preshuffle_b(shape, block_shape, wave_shape=(2, 2),
+                                                       a_scale_preshuffle=a_scale_preshuffle)
+    gemm = wave_compile(options, gemm, get_mxfp4_asymmetric_schedule())
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.float32, device=DEV)
+    xs_in = e8m0_shuffle(x_scales) if a_scale_preshuffle else x_scales
+    gemm(x, xs_in, b_preshuffle(w.T.contiguous()), e8m0_shuffle(w_scales), out)
+    torch_out = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+def testScaledGemmMXFP4PreshuffleBWideStore():
+    shape = (1024, 3072, 8192)
+    gemm, options = get_tagged_mxfp4_gemm_preshuffle_b_wide_store(shape, (256, 192, 256), wave_shape=(2, 2))
+    gemm = wave_compile(options, gemm, get_mxfp4_asymmetric_schedule())
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.bfloat16, device=DEV)
+    gemm(x, e8m0_shuffle(x_scales), b_preshuffle(w.T.contiguous()), e8m0_shuffle(w_scales), out)
+    torch_out = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+@pytest.mark.parametrize("shape, num_splits", [((256, 256, 256), 2), ((256, 256, 512), 4),
+                                               ((256, 256, 1024), 4), ((512, 512, 1024), 4)])
+@pytest.mark.parametrize("output_type", [torch.float32, torch.bfloat16])
+def testSplitKMxfp4Gemm(shape, num_splits, output_type):
+    splitk_gemm, options = get_tagged_splitk_mxfp4_gemm(shape, num_splits=num_splits,
+                                                        block_shape=(128, 128, 128),
+                                                        mfma_variant=ScaledMMAType.F32_16x16x128_F8F6F4,
+                                                        output_type=TORCH_DTYPE_TO_WAVE[output_type])
+    splitk_gemm = wave_compile(options, splitk_gemm, get_mxfp4_dbuf_schedule(use_stagger=True, k_partitions=1))
+    m, n, k = shape
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=torch.device("cpu"))
+    torch_ref = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    c_gpu = torch.zeros(m, n, dtype=output_type, device=DEV)
+    splitk_gemm(x.cuda(), x_scales.cuda(), w.T.contiguous().cuda(), w_scales.cuda(), c_gpu)
+    if output_type == torch.float32:
+        torch.testing.assert_close(c_gpu.cpu(), torch_ref, rtol=1e-3, atol=1e-2)
+    else:
+        torch.testing.assert_close(c_gpu.cpu().to(torch.float32), torch_ref, rtol=1e-1, atol=4.0)
+
+
+def testScaledGemmMXFP4BatchedStyleM1():
+    """The reference runs M = 1, K = 1664 through its generic kernel
+    (tests/kernel/wave_gemm_mxfp_test.py:296); K is not a multiple of 256."""
+    shape = (1, 1024, 1664)
+    gemm, options = get_tagged_mxfp4_gemm(shape, (256, 256, 256), wave_shape=(2, 2))
+    gemm = wave_compile(options, gemm)
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(1, 1024, dtype=torch.float32, device=DEV)
+    gemm(x, x_scales, w.T.contiguous(), w_scales, out)
+    torch.testing.assert_close(torchScaledGemmMXFP4(x, w, x_scales, w_scales), out.cpu(), check_dtype=False)

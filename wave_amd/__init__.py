@@ -1,0 +1,26 @@
+"""wave_amd: MI355X-native MXFP4 block-scaled GEMM behind the calling
+convention of the reference's scaled-GEMM kernels
+(``gemm(x, x_scales, w_t, w_scales, out)``)."""
+
+from . import _lib
+from .mxfp4 import (
+    b_preshuffle,
+    dequant,
+    e8m0_shuffle,
+    e8m0_to_f32,
+    mxfp4_gemm,
+    mxfp4_gemm_grouped,
+    mxfp4_to_f32,
+    workspace_bytes,
+)
+
+__all__ = [
+    "b_preshuffle",
+    "dequant",
+    "e8m0_shuffle",
+    "e8m0_to_f32",
+    "mxfp4_gemm",
+    "mxfp4_gemm_grouped",
+    "mxfp4_to_f32",
+    "workspace_bytes",
+]

@@ -1,0 +1,289 @@
+// C ABI of the library: argument validation (before any HIP call), kernel
+// selection and launch.  Declarations and the reference interfaces they
+// replace are in include/wave_mxfp4.h.
+#include <stdio.h>
+#include <string.h>
+
+#include "mxfp4_common.h"
+
+using namespace wave_mxfp4;
+
+namespace {
+
+thread_local char g_hip_error[256] = "";
+
+int record_hip(hipError_t e) {
+  if (e == hipSuccess) return WAVE_MXFP4_OK;
+  snprintf(g_hip_error, sizeof(g_hip_error), "%s: %s", hipGetErrorName(e), hipGetErrorString(e));
+  return WAVE_MXFP4_ERR_HIP;
+}
+
+inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
+
+constexpr int kAbiVersion = 1;
+constexpr int64_t kMaxDim = (int64_t)1 << 30;
+
+// Shape checks shared by the dense and grouped entry points.
+int check_common(const void *a, const void *as, const void *b, const void *bs, const void *c, int64_t m,
+                 int64_t n, int64_t k, int out_dtype, int asl, int bsl, int bl, int variant) {
+  if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (k % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (bad_enum(out_dtype, 2) || bad_enum(asl, 2) || bad_enum(bsl, 2) || bad_enum(bl, 2) ||
+      bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
+    return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (bl == WAVE_MXFP4_B_PRESHUFFLE && (n % 16 != 0 || k % 64 != 0)) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (m == 0 || n == 0) return WAVE_MXFP4_OK;  // nothing to read or write
+  if (!c) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (k > 0 && (!a || !as || !b || !bs)) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(a, 16) || !aligned(b, 16) || !aligned(as, 8) || !aligned(bs, 8) || !aligned(c, 16))
+    return WAVE_MXFP4_ERR_MISALIGNED;
+  // 32-bit offsets inside a tile: 256 rows of kp bytes must fit in 31 bits.
+  if ((k / 2) * 256 >= ((int64_t)1 << 31)) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  return 1;  // proceed
+}
+
+void fill_params(GemmParams &p, const void *a, const void *as, const void *b, const void *bs, void *c,
+                 int64_t m, int64_t n, int64_t k, int out_dtype, int asl, int bsl, int bl) {
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t *)a;
+  p.a_scale = (const uint8_t *)as;
+  p.b = (const uint8_t *)b;
+  p.b_scale = (const uint8_t *)bs;
+  p.c = c;
+  p.m = (int)m;
+  p.n = (int)n;
+  p.k = (int)k;
+  p.kp = (int)(k / 2);
+  p.ks = (int)(k / 32);
+  p.ksp = (p.ks + 7) / 8 * 8;
+  p.k_tiles = (int)((k + kTileK - 1) / kTileK);
+  p.tiles_per_split = p.k_tiles;
+  p.splits = 1;
+  p.out_bf16 = out_dtype == WAVE_MXFP4_OUT_BF16;
+  p.a_scale_shuffled = asl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
+  p.b_scale_shuffled = bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
+  p.b_preshuffled = bl == WAVE_MXFP4_B_PRESHUFFLE;
+}
+
+int pick_tile_variant(int64_t m, int64_t n) {
+  const int64_t t256 = ((m + 255) / 256) * ((n + 255) / 256);
+  if (t256 >= 128) return WAVE_MXFP4_VARIANT_T256x256_W2x2;
+  return WAVE_MXFP4_VARIANT_T128x128_W2x2;
+}
+
+bool is_tile_variant(int v) {
+  int bm, bn;
+  tile_variant_shape(v, &bm, &bn);
+  return bm != 0;
+}
+
+// K % 256 != 0 is only built for the 128x128 tile kernel.
+int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
+  int v = variant;
+  if (v == WAVE_MXFP4_VARIANT_AUTO)
+    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
+  if (is_tile_variant(v) && k % kTileK != 0) v = WAVE_MXFP4_VARIANT_T128x128_W2x2;
+  return v;
+}
+
+// Split the library takes by itself for a tile kernel: only when the tile
+// grid leaves most of the 256 CUs idle and K is long.
+int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
+  int bm, bn;
+  tile_variant_shape(variant, &bm, &bn);
+  if (bm == 0 || k % kTileK != 0) return 1;
+  const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+  const int64_t k_tiles = k / kTileK;
+  if (tiles >= 128 || k_tiles < 8) return 1;
+  int s = (int)(256 / tiles);
+  if (s > 8) s = 8;
+  while (s > 1 && (k_tiles % s != 0 || k_tiles / s < 2)) --s;
+  return s < 1 ? 1 : s;
+}
+
+// Reference rule for an explicit split (tagged_mxfp4_gemm.py:636-645) with
+// BLOCK_K = 256: K per split = ceil(K / splits) must be >= 256 and a multiple
+// of 256.
+bool split_ok(int64_t k, int splits, int *tiles_per_split) {
+  const int64_t per = (k + splits - 1) / splits;
+  if (per < kTileK || per % kTileK != 0) return false;
+  *tiles_per_split = (int)(per / kTileK);
+  return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wave_mxfp4_abi_version(void) { return kAbiVersion; }
+
+const char *wave_mxfp4_status_string(int status) {
+  switch (status) {
+    case WAVE_MXFP4_OK: return "ok";
+    case WAVE_MXFP4_ERR_NULL_POINTER: return "null pointer argument";
+    case WAVE_MXFP4_ERR_BAD_SHAPE: return "bad shape (negative dims, K not a multiple of 32, or layout divisibility)";
+    case WAVE_MXFP4_ERR_BAD_ENUM: return "dtype, layout or variant out of range";
+    case WAVE_MXFP4_ERR_MISALIGNED: return "pointer not aligned as documented";
+    case WAVE_MXFP4_ERR_WORKSPACE: return "split-K workspace missing or too small";
+    case WAVE_MXFP4_ERR_BAD_SPLIT: return "K per split is below 256 or not a multiple of 256";
+    case WAVE_MXFP4_ERR_HIP: return "HIP call failed";
+    case WAVE_MXFP4_ERR_UNSUPPORTED: return "unsupported argument combination";
+    default: return "unknown status";
+  }
+}
+
+const char *wave_mxfp4_last_hip_error(void) { return g_hip_error; }
+
+size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant) {
+  if (m <= 0 || n <= 0 || k <= 0 || split_k < 0 || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_)) return 0;
+  const int v = pick_variant(m, n, k, variant);
+  int splits = split_k;
+  if (splits == 0) splits = auto_split(m, n, k, v);
+  if (splits <= 1 || v == WAVE_MXFP4_VARIANT_NAIVE) return 0;
+  return (size_t)splits * (size_t)m * (size_t)n * sizeof(float);
+}
+
+int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
+                    int64_t m, int64_t n, int64_t k, int out_dtype, int a_scale_layout,
+                    int b_scale_layout, int b_layout, int split_k, void *workspace,
+                    size_t workspace_bytes, int variant, void *hip_stream) {
+  int rc = check_common(a, a_scale, b, b_scale, c, m, n, k, out_dtype, a_scale_layout, b_scale_layout,
+                        b_layout, variant);
+  if (rc <= 0) return rc;
+  if (split_k < 0) return WAVE_MXFP4_ERR_BAD_SPLIT;
+  hipStream_t stream = (hipStream_t)hip_stream;
+
+  GemmParams p;
+  fill_params(p, a, a_scale, b, b_scale, c, m, n, k, out_dtype, a_scale_layout, b_scale_layout, b_layout);
+  const int v = pick_variant(m, n, k, variant);
+  if (v == WAVE_MXFP4_VARIANT_SKINNY && m > skinny_max_m()) return WAVE_MXFP4_ERR_UNSUPPORTED;
+
+  if (k == 0) return record_hip(launch_naive_gemm(p, stream));  // empty reduction: C = 0
+
+  int splits = 1;
+  if (v != WAVE_MXFP4_VARIANT_NAIVE) {
+    if (split_k > 1) {
+      int tps;
+      if (!split_ok(k, split_k, &tps)) return WAVE_MXFP4_ERR_BAD_SPLIT;
+      splits = split_k;
+      p.tiles_per_split = tps;
+    } else if (split_k == 0) {
+      splits = auto_split(m, n, k, v);
+      const size_t need = (size_t)splits * m * n * sizeof(float);
+      if (splits > 1 && (!workspace || workspace_bytes < need)) splits = 1;  // no scratch: no split
+      if (splits > 1) p.tiles_per_split = p.k_tiles / splits;
+    }
+  }
+  if (splits > 1) {
+    const size_t need = (size_t)splits * m * n * sizeof(float);
+    if (!workspace || workspace_bytes < need) return WAVE_MXFP4_ERR_WORKSPACE;
+    if (!aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
+    p.splits = splits;
+    p.partial = (float *)workspace;
+  }
+
+  hipError_t e;
+  if (v == WAVE_MXFP4_VARIANT_NAIVE) {
+    e = launch_naive_gemm(p, stream);
+  } else if (v == WAVE_MXFP4_VARIANT_SKINNY) {
+    e = launch_skinny_gemm(p, stream);
+  } else {
+    int bm, bn;
+    tile_variant_shape(v, &bm, &bn);
+    p.tiles_m = (int)((m + bm - 1) / bm);
+    p.tiles_n = (int)((n + bn - 1) / bn);
+    e = launch_tile_gemm(p, v, stream);
+  }
+  if (e != hipSuccess) return record_hip(e);
+  if (splits > 1) e = launch_splitk_reduce(p.partial, c, m * n, splits, p.out_bf16, stream);
+  return record_hip(e);
+}
+
+int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,
+                            void *c, const int32_t *offsets, int num_groups, int64_t total_rows,
+                            int64_t n, int64_t k, int out_dtype, int a_scale_layout,
+                            int b_scale_layout, int b_layout, int variant, void *hip_stream) {
+  if (num_groups < 0 || num_groups > 65536) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  int rc = check_common(a, a_scale, b, b_scale, c, total_rows, n, k, out_dtype, a_scale_layout,
+                        b_scale_layout, b_layout, variant);
+  if (rc <= 0) return rc;
+  if (num_groups == 0) return WAVE_MXFP4_OK;
+  if (!offsets) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(offsets, 4)) return WAVE_MXFP4_ERR_MISALIGNED;
+  if (k == 0) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  hipStream_t stream = (hipStream_t)hip_stream;
+
+  GemmParams p;
+  fill_params(p, a, a_scale, b, b_scale, c, total_rows, n, k, out_dtype, a_scale_layout, b_scale_layout,
+              b_layout);
+  p.offsets = offsets;
+  p.num_groups = num_groups;
+  p.b_group_stride = n * (k / 2);
+  p.b_scale_group_stride =
+      p.b_scale_shuffled ? ((n + 31) / 32 * 32) * (int64_t)p.ksp : n * (int64_t)p.ks;
+  // every expert's B and B_scale must keep the base alignment
+  if (p.b_group_stride % 16 != 0 || p.b_scale_group_stride % 8 != 0) return WAVE_MXFP4_ERR_MISALIGNED;
+
+  if (variant == WAVE_MXFP4_VARIANT_SKINNY) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_variant(total_rows > 64 ? total_rows : 65, n, k, variant)
+                                                   : pick_variant(total_rows, n, k, variant);
+  if (v == WAVE_MXFP4_VARIANT_NAIVE) return record_hip(launch_naive_gemm(p, stream));
+  int bm, bn;
+  tile_variant_shape(v, &bm, &bn);
+  // sum over groups of ceil(rows_e / bm) <= total_rows / bm + num_groups
+  p.tiles_m = (int)(total_rows / bm + num_groups);
+  p.tiles_n = (int)((n + bn - 1) / bn);
+  return record_hip(launch_tile_gemm(p, v, stream));
+}
+
+int wave_mxfp4_to_f32(const void *q, float *out, int64_t rows, int64_t kp, void *hip_stream) {
+  if (rows < 0 || kp < 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (rows == 0 || kp == 0) return WAVE_MXFP4_OK;
+  if (!q || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(out, 8)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_to_f32((const uint8_t *)q, out, rows, kp, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_e8m0_to_f32(const void *s, float *out, int64_t count, void *hip_stream) {
+  if (count < 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (count == 0) return WAVE_MXFP4_OK;
+  if (!s || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(out, 4)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_e8m0_to_f32((const uint8_t *)s, out, count, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_dequant(const void *q, const void *scale, float *out, int64_t rows, int64_t k,
+                       int scale_layout, void *hip_stream) {
+  if (rows < 0 || k < 0 || k % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (bad_enum(scale_layout, 2)) return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (rows == 0 || k == 0) return WAVE_MXFP4_OK;
+  if (!q || !scale || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(out, 8)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_dequant((const uint8_t *)q, (const uint8_t *)scale, out, rows, k,
+                                   scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE, (hipStream_t)hip_stream));
+}
+
+size_t wave_mxfp4_e8m0_shuffle_bytes(int64_t rows, int64_t ks) {
+  if (rows <= 0 || ks <= 0) return 0;
+  return (size_t)((rows + 31) / 32 * 32) * (size_t)((ks + 7) / 8 * 8);
+}
+
+int wave_mxfp4_e8m0_shuffle(const void *scale, void *out, int64_t rows, int64_t ks, void *hip_stream) {
+  if (rows < 0 || ks < 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (rows == 0 || ks == 0) return WAVE_MXFP4_OK;
+  if (!scale || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
+  return record_hip(
+      launch_e8m0_shuffle((const uint8_t *)scale, (uint8_t *)out, rows, ks, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, void *hip_stream) {
+  if (rows < 0 || kp < 0 || rows % 16 != 0 || kp % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (rows == 0 || kp == 0) return WAVE_MXFP4_OK;
+  if (!b || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(b, 16) || !aligned(out, 16)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(
+      launch_b_preshuffle((const uint8_t *)b, (uint8_t *)out, rows, kp, (hipStream_t)hip_stream));
+}
+
+}  // extern "C"

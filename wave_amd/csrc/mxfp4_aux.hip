@@ -1,0 +1,195 @@
+// Small kernels around the GEMM: element decode (bit-exact restatements of the
+// reference's mxfp4_to_f32 / e8m0_to_f32, wave_lang/kernel/wave/utils/
+// mxfp_utils.py:60-95), dequantisation, the two layout shuffles
+// (mxfp_utils.py:98-128), the split-K reduction and a one-thread-per-element
+// GEMM used to cross-check the MFMA kernels on the device.
+#include "mxfp4_common.h"
+
+namespace wave_mxfp4 {
+
+constexpr int kThreads = 256;
+
+static inline unsigned blocks_for(int64_t work, int per_block) {
+  int64_t b = (work + per_block - 1) / per_block;
+  if (b < 1) b = 1;
+  if (b > 1048576) b = 1048576;
+  return (unsigned)b;
+}
+
+// ---- packed e2m1 -> f32, one thread per packed byte (grid-stride) ----
+__global__ void to_f32_kernel(const uint8_t *__restrict__ q, float *__restrict__ out, int64_t nbytes) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nbytes;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const uint32_t b = q[i];
+    v2f v = {e2m1_to_f32(b & 0xFu), e2m1_to_f32(b >> 4)};
+    *(v2f *)(out + 2 * i) = v;
+  }
+}
+
+__global__ void e8m0_kernel(const uint8_t *__restrict__ s, float *__restrict__ out, int64_t count) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < count;
+       i += (int64_t)gridDim.x * blockDim.x)
+    out[i] = e8m0_to_f32(s[i]);
+}
+
+// out[r, e] = value * scale(r, e/32); one thread per packed byte.
+__global__ void dequant_kernel(const uint8_t *__restrict__ q, const uint8_t *__restrict__ scale,
+                               float *__restrict__ out, int64_t rows, int64_t kp, int64_t ks, int64_t ksp,
+                               int shuffled) {
+  const int64_t nbytes = rows * kp;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nbytes;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / kp, kb = i - r * kp, g = kb >> 4;
+    const uint32_t sbyte = shuffled ? scale[e8m0_shuffle_offset(r, g, ksp)] : scale[r * ks + g];
+    const float sc = e8m0_to_f32(sbyte);
+    const uint32_t b = q[i];
+    v2f v = {e2m1_to_f32(b & 0xFu) * sc, e2m1_to_f32(b >> 4) * sc};
+    *(v2f *)(out + 2 * i) = v;
+  }
+}
+
+// One thread per byte of the padded, tile-ordered output.
+__global__ void e8m0_shuffle_kernel(const uint8_t *__restrict__ scale, uint8_t *__restrict__ out,
+                                    int64_t rows, int64_t ks, int64_t rows_p, int64_t ksp) {
+  const int64_t total = rows_p * ksp;
+  for (int64_t o = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; o < total;
+       o += (int64_t)gridDim.x * blockDim.x) {
+    // invert the offset formula: o = rt*(ksp/8*256) + kt*256 + g4*64 + r16*4 + kh*2 + rh
+    const int64_t tile_row_bytes = (ksp >> 3) * 256;
+    const int64_t rt = o / tile_row_bytes;
+    const int64_t w = o - rt * tile_row_bytes;
+    const int64_t kt = w >> 8, in = w & 255;
+    const int64_t g4 = in >> 6, r16 = (in >> 2) & 15, kh = (in >> 1) & 1, rh = in & 1;
+    const int64_t r = rt * 32 + rh * 16 + r16;
+    const int64_t g = kt * 8 + kh * 4 + g4;
+    out[o] = (r < rows && g < ks) ? scale[r * ks + g] : (uint8_t)0;
+  }
+}
+
+// One thread per 16-byte chunk.
+__global__ void b_preshuffle_kernel(const uint8_t *__restrict__ b, uint8_t *__restrict__ out, int64_t rows,
+                                    int64_t kp) {
+  const int64_t chunks_per_row = kp >> 4;
+  const int64_t total = rows * chunks_per_row;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t n = i / chunks_per_row, c = i - n * chunks_per_row;
+    const v4i v = *(const v4i *)(b + n * kp + c * 16);
+    *(v4i *)(out + b_preshuffle_offset(n, c * 16, kp)) = v;
+  }
+}
+
+// C = sum over splits of partial[s], converted to the output type.  Fixed
+// summation order, so the result does not depend on scheduling.
+__global__ void splitk_reduce_kernel(const float *__restrict__ partial, void *__restrict__ c, int64_t mn,
+                                     int splits, int out_bf16) {
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < mn;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    float acc = partial[i];
+    for (int s = 1; s < splits; ++s) acc += partial[(int64_t)s * mn + i];
+    if (out_bf16)
+      ((__bf16 *)c)[i] = (__bf16)acc;
+    else
+      ((float *)c)[i] = acc;
+  }
+}
+
+// One thread per C element: table decode, f32 multiply-add in K order.  Slow;
+// exists so the MFMA kernels can be checked on the device at any shape.
+__global__ void naive_gemm_kernel(const GemmParams p) {
+  const int64_t total = (int64_t)p.m * p.n;
+  for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int m = (int)(idx / p.n), n = (int)(idx - (int64_t)m * p.n);
+    const uint8_t *bp = p.b;
+    const uint8_t *bsp = p.b_scale;
+    if (p.num_groups > 0) {
+      int e = 0;
+      while (e < p.num_groups && !(m >= p.offsets[e] && m < p.offsets[e + 1])) ++e;
+      if (e == p.num_groups) continue;  // row belongs to no group: left untouched
+      bp += (int64_t)e * p.b_group_stride;
+      bsp += (int64_t)e * p.b_scale_group_stride;
+    }
+    float acc = 0.f;
+    for (int g = 0; g < p.ks; ++g) {
+      const uint32_t sa = p.a_scale_shuffled ? p.a_scale[e8m0_shuffle_offset(m, g, p.ksp)]
+                                             : p.a_scale[(int64_t)m * p.ks + g];
+      const uint32_t sb = p.b_scale_shuffled ? bsp[e8m0_shuffle_offset(n, g, p.ksp)]
+                                             : bsp[(int64_t)n * p.ks + g];
+      const float fa = e8m0_to_f32(sa), fb = e8m0_to_f32(sb);
+      // one scale group = 16 packed bytes, contiguous in both B layouts
+      const v4i av = *(const v4i *)(p.a + (int64_t)m * p.kp + g * 16);
+      const v4i bv = *(const v4i *)(p.b_preshuffled ? bp + b_preshuffle_offset(n, g * 16, p.kp)
+                                                    : bp + (int64_t)n * p.kp + g * 16);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t aw = (uint32_t)av[w], bw = (uint32_t)bv[w];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t ac = (aw >> (4 * j)) & 0xFu, bc = (bw >> (4 * j)) & 0xFu;
+          acc += (e2m1_to_f32(ac) * fa) * (e2m1_to_f32(bc) * fb);
+        }
+      }
+    }
+    if (p.out_bf16)
+      ((__bf16 *)p.c)[idx] = (__bf16)acc;
+    else
+      ((float *)p.c)[idx] = acc;
+  }
+}
+
+hipError_t launch_to_f32(const uint8_t *q, float *out, int64_t rows, int64_t kp, hipStream_t stream) {
+  const int64_t n = rows * kp;
+  if (n == 0) return hipSuccess;
+  to_f32_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(q, out, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_e8m0_to_f32(const uint8_t *s, float *out, int64_t count, hipStream_t stream) {
+  if (count == 0) return hipSuccess;
+  e8m0_kernel<<<blocks_for(count, kThreads), kThreads, 0, stream>>>(s, out, count);
+  return hipGetLastError();
+}
+
+hipError_t launch_dequant(const uint8_t *q, const uint8_t *scale, float *out, int64_t rows, int64_t k,
+                          int shuffled, hipStream_t stream) {
+  const int64_t n = rows * (k / 2);
+  if (n == 0) return hipSuccess;
+  const int64_t ks = k / 32, ksp = (ks + 7) / 8 * 8;
+  dequant_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(q, scale, out, rows, k / 2, ks, ksp,
+                                                                  shuffled);
+  return hipGetLastError();
+}
+
+hipError_t launch_e8m0_shuffle(const uint8_t *scale, uint8_t *out, int64_t rows, int64_t ks,
+                               hipStream_t stream) {
+  const int64_t rows_p = (rows + 31) / 32 * 32, ksp = (ks + 7) / 8 * 8;
+  const int64_t n = rows_p * ksp;
+  if (n == 0) return hipSuccess;
+  e8m0_shuffle_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(scale, out, rows, ks, rows_p, ksp);
+  return hipGetLastError();
+}
+
+hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t kp,
+                               hipStream_t stream) {
+  const int64_t n = rows * (kp / 16);
+  if (n == 0) return hipSuccess;
+  b_preshuffle_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(b, out, rows, kp);
+  return hipGetLastError();
+}
+
+hipError_t launch_splitk_reduce(const float *partial, void *c, int64_t mn, int splits, int out_bf16,
+                                hipStream_t stream) {
+  if (mn == 0) return hipSuccess;
+  splitk_reduce_kernel<<<blocks_for(mn, kThreads), kThreads, 0, stream>>>(partial, c, mn, splits, out_bf16);
+  return hipGetLastError();
+}
+
+hipError_t launch_naive_gemm(const GemmParams &p, hipStream_t stream) {
+  const int64_t n = (int64_t)p.m * p.n;
+  if (n == 0) return hipSuccess;
+  naive_gemm_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(p);
+  return hipGetLastError();
+}
+
+}  // namespace wave_mxfp4

@@ -1,0 +1,108 @@
+// Shared declarations of the gfx950 MXFP4 GEMM library (device helpers, the
+// kernel parameter block, launcher prototypes).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/wave_mxfp4.h"
+
+namespace wave_mxfp4 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef unsigned short v4us __attribute__((ext_vector_type(4)));
+
+#define WAVE_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+#define WAVE_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+
+// One K tile is 256 elements = 128 packed bytes = 8 chunks of 16 bytes (one
+// chunk is the 32 elements a lane feeds to one scaled MFMA) = 8 scale groups.
+constexpr int kTileK = 256;
+constexpr int kTileKBytes = 128;
+
+// Parameter block of the tile, skinny and naive GEMM kernels.
+struct GemmParams {
+  const uint8_t *a;        // [M, kp]
+  const uint8_t *a_scale;  // row-major [M, ks] or shuffled
+  const uint8_t *b;        // [E, N, kp] (E = 1 unless grouped)
+  const uint8_t *b_scale;  // [E, N, ks] or E shuffled buffers
+  void *c;                 // [M, N] f32 / bf16
+  float *partial;          // split-K slices [splits, M, N] f32, or null
+  const int32_t *offsets;  // grouped: device [E+1]; else null
+  int m, n, k;
+  int kp;              // K / 2
+  int ks;              // K / 32
+  int ksp;             // padded scale row length of the shuffled layout: ceil(ks/8)*8
+  int k_tiles;         // ceil(K / 256)
+  int tiles_per_split; // K tiles owned by one split
+  int splits;
+  int out_bf16;
+  int a_scale_shuffled, b_scale_shuffled, b_preshuffled;
+  int num_groups;      // 0 = dense
+  int tiles_m, tiles_n;
+  int64_t b_group_stride;        // bytes between experts in b
+  int64_t b_scale_group_stride;  // bytes between experts in b_scale
+};
+
+// e2m1 code -> f32.  Bit 3 is the sign; codes 0..7 are 0, .5, 1, 1.5, 2, 3, 4, 6.
+__device__ __forceinline__ float e2m1_to_f32(uint32_t code) {
+  const uint32_t mag = code & 7u;
+  // magnitudes as f32 bit patterns: exponent/mantissa follow the e2m1 fields
+  // (e = mag >> 1, m = mag & 1): e == 0 -> m * 0.5, else 2^(e-1) * (1 + m/2)
+  const uint32_t e = mag >> 1, mnt = mag & 1u;
+  uint32_t bits = e == 0 ? (mnt ? 0x3F000000u : 0u) : (((126u + e) << 23) | (mnt << 22));
+  bits |= (code & 8u) << 28;
+  return __uint_as_float(bits);
+}
+
+// e8m0 byte -> f32: 2^(s-127); 0 -> 2^-127 (subnormal); 255 -> NaN.
+__device__ __forceinline__ float e8m0_to_f32(uint32_t s) {
+  const uint32_t bits = s == 255u ? 0x7FC00000u : (s == 0u ? 0x00400000u : (s << 23));
+  return __uint_as_float(bits);
+}
+
+// f32 -> bf16 bits, round to nearest even, NaN kept quiet.
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// Byte offset of scale (row r, group g) in the e8m0_shuffle tile order with
+// padded row length ksp.
+__device__ __host__ __forceinline__ int64_t e8m0_shuffle_offset(int64_t r, int64_t g, int64_t ksp) {
+  return (r >> 5) * ((ksp >> 3) * 256) + (g >> 3) * 256 + (g & 3) * 64 + (r & 15) * 4 +
+         ((g & 7) >> 2) * 2 + ((r & 31) >> 4);
+}
+
+// Byte offset of packed byte (row n, byte kb) in the b_preshuffle order.
+__device__ __host__ __forceinline__ int64_t b_preshuffle_offset(int64_t n, int64_t kb, int64_t kp) {
+  return (n >> 4) * 16 * kp + (kb >> 5) * 512 + ((kb >> 4) & 1) * 256 + (n & 15) * 16 + (kb & 15);
+}
+
+// ---- launchers (defined in the .hip files, called from the C ABI) ----
+hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream);
+hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);
+hipError_t launch_naive_gemm(const GemmParams &p, hipStream_t stream);
+hipError_t launch_splitk_reduce(const float *partial, void *c, int64_t mn, int splits, int out_bf16,
+                                hipStream_t stream);
+hipError_t launch_to_f32(const uint8_t *q, float *out, int64_t rows, int64_t kp, hipStream_t stream);
+hipError_t launch_e8m0_to_f32(const uint8_t *s, float *out, int64_t count, hipStream_t stream);
+hipError_t launch_dequant(const uint8_t *q, const uint8_t *scale, float *out, int64_t rows, int64_t k,
+                          int shuffled, hipStream_t stream);
+hipError_t launch_e8m0_shuffle(const uint8_t *scale, uint8_t *out, int64_t rows, int64_t ks,
+                               hipStream_t stream);
+hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t kp,
+                               hipStream_t stream);
+
+// Tile geometry of a variant (0 if the variant is not a tile kernel).
+void tile_variant_shape(int variant, int *bm, int *bn);
+int skinny_max_m();
+
+}  // namespace wave_mxfp4

@@ -1,0 +1,21 @@
+from .tagged_mxfp4_gemm import (
+    get_tagged_mxfp4_gemm,
+    get_tagged_mxfp4_gemm_preshuffle_b,
+    get_tagged_mxfp4_gemm_preshuffle_b_wide_store,
+    get_tagged_mxfp4_gemm_preshuffle_scales,
+    get_tagged_mxfp4_gemm_preshuffle_scales_and_B,
+    get_tagged_splitk_mxfp4_gemm,
+    get_tagged_splitk_mxfp4_gemm_preshuffle_b,
+    get_tagged_splitk_mxfp4_gemm_preshuffle_scales,
+)
+
+__all__ = [
+    "get_tagged_mxfp4_gemm",
+    "get_tagged_mxfp4_gemm_preshuffle_b",
+    "get_tagged_mxfp4_gemm_preshuffle_b_wide_store",
+    "get_tagged_mxfp4_gemm_preshuffle_scales",
+    "get_tagged_mxfp4_gemm_preshuffle_scales_and_B",
+    "get_tagged_splitk_mxfp4_gemm",
+    "get_tagged_splitk_mxfp4_gemm_preshuffle_b",
+    "get_tagged_splitk_mxfp4_gemm_preshuffle_scales",
+]

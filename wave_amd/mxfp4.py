@@ -1,0 +1,211 @@
+"""Torch-facing operators over the C ABI.  Torch supplies device memory and
+the current stream; all arithmetic happens in the HIP library.
+
+Calling convention kept from the reference launch path
+(wave_lang/kernel/wave/compile.py:225-339, utils/run_utils.py:62-134):
+tensors are passed positionally, non-contiguous inputs are silently made
+contiguous, the output is pre-allocated by the caller and mutated in place,
+the work is enqueued on the current stream without synchronising, and the
+call returns None."""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_OUT_DTYPES = {torch.float32: _lib.OUT_F32, torch.bfloat16: _lib.OUT_BF16}
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _as_u8(t: torch.Tensor, name: str) -> torch.Tensor:
+    # the reference annotates these buffers i8 and its tests pass uint8
+    if t.dtype not in (torch.uint8, torch.int8):
+        raise ValueError(f"{name}: expected uint8/int8, got {t.dtype}")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: expected a GPU tensor (there is no CPU path)")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _check_out(out: torch.Tensor, shape) -> int:
+    if out.dtype not in _OUT_DTYPES:
+        raise ValueError(f"out: expected float32 or bfloat16, got {out.dtype}")
+    if not out.is_cuda or not out.is_contiguous():
+        raise ValueError("out: expected a contiguous GPU tensor")
+    if tuple(out.shape) != tuple(shape):
+        raise ValueError(f"out: expected shape {tuple(shape)}, got {tuple(out.shape)}")
+    return _OUT_DTYPES[out.dtype]
+
+
+def _scale_rows_ok(scale: torch.Tensor, rows: int, ks: int, layout: int, name: str) -> None:
+    if layout == _lib.SCALE_ROW_MAJOR:
+        if tuple(scale.shape) != (rows, ks):
+            raise ValueError(f"{name}: expected shape {(rows, ks)}, got {tuple(scale.shape)}")
+    else:
+        need = ((rows + 31) // 32 * 32) * ((ks + 7) // 8 * 8)
+        if scale.numel() < need:
+            raise ValueError(
+                f"{name}: shuffled scales need {need} bytes (rows padded to 32, groups to 8), got {scale.numel()}")
+
+
+def workspace_bytes(m: int, n: int, k: int, split_k: int = 0, variant: int = _lib.VARIANT_AUTO) -> int:
+    return int(_lib.load().wave_mxfp4_workspace_bytes(m, n, k, split_k, variant))
+
+
+def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,
+               b_scale_layout=_lib.SCALE_ROW_MAJOR, b_layout=_lib.B_ROW_MAJOR, split_k=1,
+               variant=_lib.VARIANT_AUTO, workspace=None) -> None:
+    """``out[M, N] = dequant(x[M, K/2]) @ dequant(w_t[N, K/2]).T`` in place.
+    Same arguments, in the same order, as the reference's compiled kernel
+    (tests/kernel/wave_gemm_mxfp_test.py:194-201)."""
+    lib = _lib.load()
+    x = _as_u8(x, "x")
+    w_t = _as_u8(w_t, "w_t")
+    x_scales = _as_u8(x_scales, "x_scales")
+    w_scales = _as_u8(w_scales, "w_scales")
+    if x.dim() != 2 or w_t.dim() != 2:
+        raise ValueError("x and w_t must be 2-D")
+    m, kp = x.shape
+    n = w_t.shape[0]
+    if w_t.shape[1] != kp:
+        raise ValueError(f"x and w_t disagree on K/2: {kp} vs {w_t.shape[1]}")
+    k = kp * 2
+    if k % 32 != 0:
+        raise ValueError(f"K = {k} must be a multiple of 32")
+    ks = k // 32
+    _scale_rows_ok(x_scales, m, ks, a_scale_layout, "x_scales")
+    _scale_rows_ok(w_scales, n, ks, b_scale_layout, "w_scales")
+    od = _check_out(out, (m, n))
+    ws_ptr, ws_bytes = None, 0
+    if split_k != 1:
+        need = workspace_bytes(m, n, k, split_k, variant)
+        if need:
+            if workspace is None:
+                workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+            ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    with torch.cuda.device(x.device):
+        st = lib.wave_mxfp4_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
+                                 out.data_ptr(), m, n, k, od, a_scale_layout, b_scale_layout, b_layout,
+                                 split_k, ws_ptr, ws_bytes, variant, _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp4_gemm")
+
+
+def mxfp4_gemm_grouped(x, x_scales, w_t, w_scales, offsets, out, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,
+                       b_scale_layout=_lib.SCALE_ROW_MAJOR, b_layout=_lib.B_ROW_MAJOR,
+                       variant=_lib.VARIANT_AUTO) -> None:
+    """Grouped (MoE) GEMM: rows ``offsets[e]:offsets[e+1]`` of ``x`` times
+    expert ``e``'s ``w_t[e]`` ``[N, K/2]``; ``offsets`` is an int32 GPU tensor
+    of E+1 entries.  ``out`` is ``[rows, N]``; rows past ``offsets[-1]`` are
+    left untouched."""
+    lib = _lib.load()
+    x = _as_u8(x, "x")
+    w_t = _as_u8(w_t, "w_t")
+    x_scales = _as_u8(x_scales, "x_scales")
+    w_scales = _as_u8(w_scales, "w_scales")
+    if x.dim() != 2 or w_t.dim() != 3:
+        raise ValueError("x must be [rows, K/2] and w_t [E, N, K/2]")
+    if offsets.dtype != torch.int32 or not offsets.is_cuda or not offsets.is_contiguous():
+        raise ValueError("offsets: expected a contiguous int32 GPU tensor")
+    rows, kp = x.shape
+    e, n, kp2 = w_t.shape
+    if kp2 != kp:
+        raise ValueError(f"x and w_t disagree on K/2: {kp} vs {kp2}")
+    if offsets.numel() != e + 1:
+        raise ValueError(f"offsets: expected {e + 1} entries, got {offsets.numel()}")
+    k = kp * 2
+    if k % 32 != 0:
+        raise ValueError(f"K = {k} must be a multiple of 32")
+    ks = k // 32
+    _scale_rows_ok(x_scales, rows, ks, a_scale_layout, "x_scales")
+    if b_scale_layout == _lib.SCALE_ROW_MAJOR:
+        if tuple(w_scales.shape) != (e, n, ks):
+            raise ValueError(f"w_scales: expected {(e, n, ks)}, got {tuple(w_scales.shape)}")
+    else:
+        need = e * ((n + 31) // 32 * 32) * ((ks + 7) // 8 * 8)
+        if w_scales.numel() < need:
+            raise ValueError(f"w_scales: shuffled scales need {need} bytes, got {w_scales.numel()}")
+    od = _check_out(out, (rows, n))
+    with torch.cuda.device(x.device):
+        st = lib.wave_mxfp4_gemm_grouped(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(),
+                                         w_scales.data_ptr(), out.data_ptr(), offsets.data_ptr(), e, rows,
+                                         n, k, od, a_scale_layout, b_scale_layout, b_layout, variant,
+                                         _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp4_gemm_grouped")
+
+
+def mxfp4_to_f32(x: torch.Tensor) -> torch.Tensor:
+    """Packed e2m1 ``[R, K/2]`` -> f32 ``[R, K]``
+    (wave_lang/kernel/wave/utils/mxfp_utils.py:60-83)."""
+    lib = _lib.load()
+    x = _as_u8(x, "x")
+    rows, kp = x.shape
+    out = torch.empty(rows, kp * 2, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.wave_mxfp4_to_f32(x.data_ptr(), out.data_ptr(), rows, kp, _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp4_to_f32")
+    return out
+
+
+def e8m0_to_f32(s: torch.Tensor) -> torch.Tensor:
+    """e8m0 bytes -> f32 ``2^(s-127)``, 255 -> NaN
+    (wave_lang/kernel/wave/utils/mxfp_utils.py:86-95)."""
+    lib = _lib.load()
+    s = _as_u8(s, "s")
+    out = torch.empty(s.shape, dtype=torch.float32, device=s.device)
+    with torch.cuda.device(s.device):
+        st = lib.wave_mxfp4_e8m0_to_f32(s.data_ptr(), out.data_ptr(), s.numel(), _stream_ptr(s.device))
+    _lib.check(st, "wave_mxfp4_e8m0_to_f32")
+    return out
+
+
+def dequant(x: torch.Tensor, scales: torch.Tensor, scale_layout=_lib.SCALE_ROW_MAJOR) -> torch.Tensor:
+    """``[R, K/2]`` codes and their scales -> f32 ``[R, K]`` (value times the
+    scale of its 32-group), the operand the reference feeds to ``torch.mm``
+    (wave_lang/kernel/wave/utils/mxfp_utils.py:135-143)."""
+    lib = _lib.load()
+    x = _as_u8(x, "x")
+    scales = _as_u8(scales, "scales")
+    rows, kp = x.shape
+    k = kp * 2
+    _scale_rows_ok(scales, rows, k // 32, scale_layout, "scales")
+    out = torch.empty(rows, k, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.wave_mxfp4_dequant(x.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, k, scale_layout,
+                                    _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp4_dequant")
+    return out
+
+
+def e8m0_shuffle(scale: torch.Tensor) -> torch.Tensor:
+    """Scale matrix ``[R, K/32]`` -> the tile order the kernels read with one
+    dword per lane (wave_lang/kernel/wave/utils/mxfp_utils.py:113-128).
+
+    Returns the PADDED buffer ``[ceil(R/32)*32, ceil(K/32/8)*8]``; when R is a
+    multiple of 32 and K of 256 that is exactly the reference's result.  (The
+    reference slices back to ``[R, K/32]``, which drops bytes of valid rows
+    otherwise.)"""
+    lib = _lib.load()
+    scale = _as_u8(scale, "scale")
+    rows, ks = scale.shape
+    out = torch.empty((rows + 31) // 32 * 32, (ks + 7) // 8 * 8, dtype=torch.uint8, device=scale.device)
+    with torch.cuda.device(scale.device):
+        st = lib.wave_mxfp4_e8m0_shuffle(scale.data_ptr(), out.data_ptr(), rows, ks, _stream_ptr(scale.device))
+    _lib.check(st, "wave_mxfp4_e8m0_shuffle")
+    return out
+
+
+def b_preshuffle(b: torch.Tensor) -> torch.Tensor:
+    """``[N, K/2]`` packed weights -> same shape in the order a lane reads with
+    one 16-byte load per MFMA operand
+    (wave_lang/kernel/wave/utils/mxfp_utils.py:98-110)."""
+    lib = _lib.load()
+    b = _as_u8(b, "b")
+    rows, kp = b.shape
+    out = torch.empty_like(b)
+    with torch.cuda.device(b.device):
+        st = lib.wave_mxfp4_b_preshuffle(b.data_ptr(), out.data_ptr(), rows, kp, _stream_ptr(b.device))
+    _lib.check(st, "wave_mxfp4_b_preshuffle")
+    return out

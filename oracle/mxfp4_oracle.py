@@ -86,7 +86,8 @@ def dequant_f32(packed: np.ndarray, scales: np.ndarray) -> np.ndarray:
     v = mxfp4_to_f32(packed)
     s = e8m0_to_f32(np.repeat(np.asarray(scales, dtype=np.uint8),
                               SCALE_GROUP_SIZE, axis=-1))
-    return v * s
+    with np.errstate(over="ignore", invalid="ignore"):
+        return v * s
 
 
 # --------------------------------------------------------------------------

@@ -51,7 +51,17 @@ typedef enum { WAVE_MXFP4_OUT_F32 = 0, WAVE_MXFP4_OUT_BF16 = 1 } wave_mxfp4_out_
  * buffer padded to ceil(R/32)*32 rows and ceil(K/32/8)*8 columns; the buffer
  * must hold every byte of that padded shape (the reference's final slice back
  * to [R, K/32] loses bytes unless R % 32 == 0 and K % 256 == 0). */
-typedef enum { WAVE_MXFP4_SCALE_ROW_MAJOR = 0, WAVE_MXFP4_SCALE_E8M0_SHUFFLE = 1 } wave_mxfp4_scale_layout;
+typedef enum {
+  WAVE_MXFP4_SCALE_ROW_MAJOR = 0,
+  WAVE_MXFP4_SCALE_E8M0_SHUFFLE = 1,
+  /* The layout the 32x32x64 scaled MFMA kernels read with one dword per lane:
+   * per 32-row tile and 256-element K tile a 256-byte block; lane
+   * (g%2)*32 + r%32 holds, in byte (g%8)/2, the scale of row r, group g.  Same
+   * byte count as the padded E8M0_SHUFFLE buffer.  Produced by
+   * wave_mxfp4_scale_convert (no counterpart in the reference, whose
+   * e8m0_shuffle is matched to the 16x16x128 instruction). */
+  WAVE_MXFP4_SCALE_MFMA32 = 2
+} wave_mxfp4_scale_layout;
 
 /* B storage.  PRESHUFFLE is b_preshuffle (mxfp_utils.py:98-110,
  * tagged_mxfp4_gemm.py:465-483); needs N % 16 == 0 and K % 64 == 0. */
@@ -65,10 +75,8 @@ typedef enum {
   WAVE_MXFP4_VARIANT_T256x256_W2x2 = 1, /* 256x256x256 tile, 4 waves */
   WAVE_MXFP4_VARIANT_T256x256_W4x2 = 2, /* 256x256x256 tile, 8 waves */
   WAVE_MXFP4_VARIANT_T128x128_W2x2 = 3, /* 128x128x256 tile, 4 waves */
-  WAVE_MXFP4_VARIANT_T256x128_W2x2 = 4, /* 256x128x256 tile, 4 waves */
-  WAVE_MXFP4_VARIANT_T128x256_W2x2 = 5, /* 128x256x256 tile, 4 waves */
-  WAVE_MXFP4_VARIANT_SKINNY = 6,        /* M <= 64 streaming kernel */
-  WAVE_MXFP4_VARIANT_NAIVE = 7,         /* one thread per C element, for cross-checks */
+  WAVE_MXFP4_VARIANT_SKINNY = 4,        /* M <= 64 streaming kernel */
+  WAVE_MXFP4_VARIANT_NAIVE = 5,         /* one thread per C element, for cross-checks */
   WAVE_MXFP4_VARIANT_COUNT_
 } wave_mxfp4_variant;
 
@@ -82,8 +90,11 @@ typedef enum {
  *             must own a multiple of 256 elements (tagged_mxfp4_gemm.py:636-645).
  *             Partial sums are kept in f32 in `workspace` and reduced in a
  *             fixed order, so C is overwritten, never accumulated into.
- *   workspace device scratch of at least wave_mxfp4_workspace_bytes(...) bytes,
- *             256-byte aligned; may be NULL when that size is 0.
+ *   workspace device scratch, 256-byte aligned, of wave_mxfp4_workspace_bytes(...)
+ *             bytes: the split-K partial sums (required for a split) plus room
+ *             to re-lay ROW_MAJOR / E8M0_SHUFFLE scales out as MFMA32 before the
+ *             tile kernels run (optional: without it the kernels read the given
+ *             layout directly, which costs vector-L1 time).  May be NULL.
  * A, B must be 16-byte aligned; scales 8-byte aligned; C 16-byte aligned.
  */
 int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
@@ -91,9 +102,9 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
                     int b_scale_layout, int b_layout, int split_k, void *workspace,
                     size_t workspace_bytes, int variant, void *hip_stream);
 
-/* Scratch bytes wave_mxfp4_gemm needs for (m, n, k, split_k, variant); 0 when no
- * split is taken.  With split_k == 0 it returns the size for the split the
- * library would pick by itself. */
+/* Scratch bytes wave_mxfp4_gemm can use for (m, n, k, split_k, variant): the
+ * split-K partials (for split_k == 0, of the split the library would pick by
+ * itself) plus the re-laid-out scales of both operands. */
 size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant);
 
 /*
@@ -128,6 +139,13 @@ int wave_mxfp4_dequant(const void *q, const void *scale, float *out, int64_t row
  * ceil(rows/32)*32 x ceil(ks/8)*8 bytes (padding bytes written as 0). */
 int wave_mxfp4_e8m0_shuffle(const void *scale, void *out, int64_t rows, int64_t ks, void *hip_stream);
 size_t wave_mxfp4_e8m0_shuffle_bytes(int64_t rows, int64_t ks);
+
+/* Re-lays a scale tensor out from one wave_mxfp4_scale_layout to another
+ * (device side; generalises e8m0_shuffle, mxfp_utils.py:113-128).  Non row-major
+ * buffers hold wave_mxfp4_e8m0_shuffle_bytes(rows, ks) bytes; padding is
+ * written as 0. */
+int wave_mxfp4_scale_convert(const void *src, int src_layout, void *dst, int dst_layout, int64_t rows,
+                             int64_t ks, void *hip_stream);
 
 /* Device-side b_preshuffle (mxfp_utils.py:98-110); rows % 16 == 0, kp % 32 == 0. */
 int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, void *hip_stream);

@@ -201,6 +201,28 @@ def e8m0_unshuffle(shuffled: np.ndarray, m: int, n: int) -> np.ndarray:
     return flat[e8m0_shuffle_flat_index(r, k, sn)]
 
 
+def mfma32_scale_flat_index(r, g, k_tiles):
+    """Flat byte offset of scale (row r, group g) in the library's own MFMA32
+    order (no counterpart in the reference): per 32-row tile and K tile of 8
+    groups a 256-byte block; the lane (g%2)*32 + r%32 of the 32x32x64 scaled MFMA
+    holds, in byte (g%8)//2, the scale of (r, g)."""
+    r = np.asarray(r, dtype=np.int64)
+    g = np.asarray(g, dtype=np.int64)
+    return ((r // 32) * k_tiles + g // 8) * 256 + ((g % 2) * 32 + r % 32) * 4 + (g % 8) // 2
+
+
+def mfma32_scale_layout(scale: np.ndarray) -> np.ndarray:
+    """Scale matrix [m, n] -> MFMA32-ordered buffer of ceil(m/32)*32 x
+    ceil(n/8)*8 bytes, padding 0."""
+    scale = np.asarray(scale, dtype=np.uint8)
+    m, n = scale.shape
+    sm, sn = (m + 31) // 32 * 32, (n + 7) // 8 * 8
+    out = np.zeros(sm * sn, dtype=np.uint8)
+    r, g = np.meshgrid(np.arange(m), np.arange(n), indexing="ij")
+    out[mfma32_scale_flat_index(r, g, sn // 8)] = scale
+    return out.reshape(sm, sn)
+
+
 def b_preshuffle(b: np.ndarray) -> np.ndarray:
     """[N, K/2] packed weights -> same shape, each 16-row x 32-byte tile
     reordered from [n, k_sub, k_elem] to [k_sub, n, k_elem]:

@@ -62,7 +62,7 @@ def test_gemm_argument_validation():
     assert gemm(lib, k=-32) == _lib.ERR_BAD_SHAPE
     assert gemm(lib, k=48) == _lib.ERR_BAD_SHAPE          # K % 32 != 0
     assert gemm(lib, od=2) == _lib.ERR_BAD_ENUM
-    assert gemm(lib, asl=2) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, asl=3) == _lib.ERR_BAD_ENUM
     assert gemm(lib, bsl=-1) == _lib.ERR_BAD_ENUM
     assert gemm(lib, bl=7) == _lib.ERR_BAD_ENUM
     assert gemm(lib, variant=99) == _lib.ERR_BAD_ENUM
@@ -111,6 +111,11 @@ def test_aux_argument_validation():
     assert lib.wave_mxfp4_e8m0_to_f32(P, P, -4, None) == _lib.ERR_BAD_SHAPE
     assert lib.wave_mxfp4_dequant(P, P, P, 4, 48, 0, None) == _lib.ERR_BAD_SHAPE
     assert lib.wave_mxfp4_dequant(P, P, P, 4, 64, 3, None) == _lib.ERR_BAD_ENUM
+    assert lib.wave_mxfp4_scale_convert(P, 0, P + 256, 3, 4, 4, None) == _lib.ERR_BAD_ENUM
+    assert lib.wave_mxfp4_scale_convert(P, 0, None, 2, 4, 4, None) == _lib.ERR_NULL_POINTER
+    assert lib.wave_mxfp4_scale_convert(P, 0, P, 2, 4, 4, None) == _lib.ERR_UNSUPPORTED
+    assert lib.wave_mxfp4_scale_convert(P, 0, P + 258, 2, 4, 4, None) == _lib.ERR_MISALIGNED
+    assert lib.wave_mxfp4_scale_convert(P, 0, P + 256, 2, -1, 4, None) == _lib.ERR_BAD_SHAPE
     assert lib.wave_mxfp4_dequant(P, None, P, 4, 64, 0, None) == _lib.ERR_NULL_POINTER
     assert lib.wave_mxfp4_e8m0_shuffle(None, P, 4, 4, None) == _lib.ERR_NULL_POINTER
     assert lib.wave_mxfp4_b_preshuffle(P, P, 24, 32, None) == _lib.ERR_BAD_SHAPE
@@ -122,8 +127,11 @@ def test_aux_argument_validation():
 
 def test_workspace_bytes():
     lib = _lib.load()
-    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, 0) == 0
-    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 4, 3) == 4 * 512 * 512 * 4
+    scales = 2 * 512 * 32                     # both operands re-laid out as MFMA32
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, 0) == scales
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 4, 3) == 4 * 512 * 512 * 4 + scales
+    assert lib.wave_mxfp4_workspace_bytes(16, 512, 1024, 1, 0) == 0      # skinny kernel: nothing to stage
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, _lib.VARIANT_NAIVE) == 0
     assert lib.wave_mxfp4_workspace_bytes(-1, 512, 1024, 4, 3) == 0
 
 

@@ -194,6 +194,10 @@ def test_config5_edge_shape_shuffled_scales_f32_seed4():
     assert np.array_equal(xs_sh.cpu().numpy(), orc.e8m0_shuffle_padded(xs)[:4096])
     shuffled = run(xs_sh, ws_sh, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
     assert np.array_equal(shuffled, plain)                          # same arithmetic, same bits
+    direct = run(xs_sh, ws_sh, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
+                 workspace=False)
+    assert np.array_equal(direct, plain)                            # read in place, no pre-pass
+    assert np.array_equal(run(gxs, gws, workspace=False), plain)
     # and with preshuffled B on top
     gwp = wave_amd.b_preshuffle(gw)
     out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)

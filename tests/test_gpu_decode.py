@@ -72,6 +72,29 @@ def test_e8m0_shuffle_matches_oracle(rows, ks):
     assert np.array_equal(got, orc.e8m0_shuffle_padded(s)[:rp])
 
 
+@pytest.mark.parametrize("rows,ks", [(256, 64), (4093, 224), (33, 9), (1, 1)])
+def test_scale_convert_every_layout_pair(rows, ks):
+    rng = np.random.default_rng(rows * 7 + ks)
+    s = rng.integers(0, 256, size=(rows, ks), dtype=np.uint8)
+    rp = (rows + 31) // 32 * 32
+    forms = {
+        _lib.SCALE_ROW_MAJOR: s,
+        _lib.SCALE_E8M0_SHUFFLE: orc.e8m0_shuffle_padded(s)[:rp],
+        _lib.SCALE_MFMA32: orc.mfma32_scale_layout(s),
+    }
+    for src, src_arr in forms.items():
+        (g,) = to_gpu(src_arr)
+        for dst, want in forms.items():
+            got = wave_amd.scale_convert(g, rows, ks, src, dst).cpu().numpy()
+            assert np.array_equal(got, want), (src, dst)
+    # dequantisation reads the MFMA32 order too
+    q = rng.integers(0, 256, size=(rows, ks * 16), dtype=np.uint8)
+    s2 = np.clip(s, 1, 254)
+    gq, gs = to_gpu(q, orc.mfma32_scale_layout(s2))
+    got = wave_amd.dequant(gq, gs, scale_layout=_lib.SCALE_MFMA32).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), orc.dequant_f32(q, s2).view(np.uint32))
+
+
 @pytest.mark.parametrize("n,kp", [(16, 32), (6144, 3584), (48, 96)])
 def test_b_preshuffle_matches_oracle(n, kp):
     rng = np.random.default_rng(n + kp)

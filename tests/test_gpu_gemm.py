@@ -41,6 +41,18 @@ def test_golden_fixtures_every_variant(path, vname):
     if g["w_t_preshuffled"].size:
         got = run_gemm(x, xs, g["w_t_preshuffled"], ws, torch.float32, variant=v, b_layout=_lib.B_PRESHUFFLE)
         assert_f32_close(got, ref, "preshuffled B")
+    # without scratch the kernels read each layout directly; with MFMA32 scales
+    # given by the caller they need no pre-pass
+    assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32, variant=v, workspace=False), ref, "direct row-major")
+    got = run_gemm(x, g["x_scales_shuffled"], w_t, g["w_scales_shuffled"], torch.float32, variant=v,
+                   a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE, workspace=False)
+    assert_f32_close(got, ref, "direct shuffled")
+    got = run_gemm(x, orc.mfma32_scale_layout(xs), w_t, orc.mfma32_scale_layout(ws), torch.float32, variant=v,
+                   a_scale_layout=_lib.SCALE_MFMA32, b_scale_layout=_lib.SCALE_MFMA32, workspace=False)
+    assert_f32_close(got, ref, "MFMA32 scales")
+    got = run_gemm(x, orc.mfma32_scale_layout(xs), w_t, ws, torch.bfloat16, variant=v,
+                   a_scale_layout=_lib.SCALE_MFMA32, workspace=False)
+    assert_bf16_close(got, ref, "mixed scale layouts")
 
 
 SMALL_SHAPES = [

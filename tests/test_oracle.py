@@ -120,6 +120,28 @@ def test_e8m0_shuffle_reference_slice_is_lossless_when_aligned():
     assert np.array_equal(np.sort(orc.e8m0_shuffle(scale).reshape(-1)), np.sort(scale.reshape(-1)))
 
 
+def test_mfma32_scale_layout_is_a_bijection_with_the_lane_property():
+    """Own layout: per (row tile, K tile) block, lane (g%2)*32 + r%32 reads one
+    dword whose byte t is the scale of group 2t + g%2."""
+    rng = np.random.default_rng(11)
+    m, ks = 70, 19
+    scale = rng.integers(1, 256, size=(m, ks), dtype=np.uint8)
+    buf = orc.mfma32_scale_layout(scale)
+    sm, sn = 96, 24
+    assert buf.shape == (sm, sn)
+    rr, gg = np.meshgrid(np.arange(sm), np.arange(sn), indexing="ij")
+    allflat = orc.mfma32_scale_flat_index(rr, gg, sn // 8).reshape(-1)
+    assert np.array_equal(np.sort(allflat), np.arange(sm * sn))
+    flat = buf.reshape(-1)
+    for rt in range(3):
+        for kt in range(3):
+            for lane in range(64):
+                for t in range(4):
+                    r, g = rt * 32 + lane % 32, kt * 8 + 2 * t + lane // 32
+                    want = scale[r, g] if r < m and g < ks else 0
+                    assert flat[(rt * 3 + kt) * 256 + lane * 4 + t] == want
+
+
 @pytest.mark.parametrize("n,kp", [(16, 32), (64, 128), (48, 96)])
 def test_b_preshuffle_statements_agree(n, kp):
     rng = np.random.default_rng(n + kp)

@@ -11,6 +11,7 @@ from .mxfp4 import (
     mxfp4_gemm,
     mxfp4_gemm_grouped,
     mxfp4_to_f32,
+    scale_convert,
     workspace_bytes,
 )
 
@@ -22,5 +23,6 @@ __all__ = [
     "mxfp4_gemm",
     "mxfp4_gemm_grouped",
     "mxfp4_to_f32",
+    "scale_convert",
     "workspace_bytes",
 ]

@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # status codes of include/wave_mxfp4.h
 OK = 0
@@ -24,17 +24,15 @@ ERR_HIP = -7
 ERR_UNSUPPORTED = -8
 
 OUT_F32, OUT_BF16 = 0, 1
-SCALE_ROW_MAJOR, SCALE_E8M0_SHUFFLE = 0, 1
+SCALE_ROW_MAJOR, SCALE_E8M0_SHUFFLE, SCALE_MFMA32 = 0, 1, 2
 B_ROW_MAJOR, B_PRESHUFFLE = 0, 1
 
 VARIANT_AUTO = 0
 VARIANT_T256x256_W2x2 = 1
 VARIANT_T256x256_W4x2 = 2
 VARIANT_T128x128_W2x2 = 3
-VARIANT_T256x128_W2x2 = 4
-VARIANT_T128x256_W2x2 = 5
-VARIANT_SKINNY = 6
-VARIANT_NAIVE = 7
+VARIANT_SKINNY = 4
+VARIANT_NAIVE = 5
 
 # every symbol include/wave_mxfp4.h declares
 EXPORTS = (
@@ -46,6 +44,7 @@ EXPORTS = (
     "wave_mxfp4_dequant",
     "wave_mxfp4_e8m0_shuffle",
     "wave_mxfp4_e8m0_shuffle_bytes",
+    "wave_mxfp4_scale_convert",
     "wave_mxfp4_b_preshuffle",
     "wave_mxfp4_status_string",
     "wave_mxfp4_last_hip_error",
@@ -82,6 +81,8 @@ def load():
     lib.wave_mxfp4_e8m0_shuffle.restype = i32
     lib.wave_mxfp4_e8m0_shuffle_bytes.argtypes = [i64, i64]
     lib.wave_mxfp4_e8m0_shuffle_bytes.restype = sz
+    lib.wave_mxfp4_scale_convert.argtypes = [p, i32, p, i32, i64, i64, p]
+    lib.wave_mxfp4_scale_convert.restype = i32
     lib.wave_mxfp4_b_preshuffle.argtypes = [p, p, i64, i64, p]
     lib.wave_mxfp4_b_preshuffle.restype = i32
     lib.wave_mxfp4_status_string.argtypes = [i32]

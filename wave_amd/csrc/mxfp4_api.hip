@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 1;
+constexpr int kAbiVersion = 2;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -29,7 +29,7 @@ int check_common(const void *a, const void *as, const void *b, const void *bs, c
                  int64_t n, int64_t k, int out_dtype, int asl, int bsl, int bl, int variant) {
   if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim) return WAVE_MXFP4_ERR_BAD_SHAPE;
   if (k % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
-  if (bad_enum(out_dtype, 2) || bad_enum(asl, 2) || bad_enum(bsl, 2) || bad_enum(bl, 2) ||
+  if (bad_enum(out_dtype, 2) || bad_enum(asl, 3) || bad_enum(bsl, 3) || bad_enum(bl, 2) ||
       bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
     return WAVE_MXFP4_ERR_BAD_ENUM;
   if (bl == WAVE_MXFP4_B_PRESHUFFLE && (n % 16 != 0 || k % 64 != 0)) return WAVE_MXFP4_ERR_BAD_SHAPE;
@@ -61,8 +61,8 @@ void fill_params(GemmParams &p, const void *a, const void *as, const void *b, co
   p.tiles_per_split = p.k_tiles;
   p.splits = 1;
   p.out_bf16 = out_dtype == WAVE_MXFP4_OUT_BF16;
-  p.a_scale_shuffled = asl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
-  p.b_scale_shuffled = bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
+  p.a_scale_layout = asl;
+  p.b_scale_layout = bsl;
   p.b_preshuffled = bl == WAVE_MXFP4_B_PRESHUFFLE;
 }
 
@@ -135,13 +135,24 @@ const char *wave_mxfp4_status_string(int status) {
 
 const char *wave_mxfp4_last_hip_error(void) { return g_hip_error; }
 
+// Bytes of one operand's scales in the padded non row-major layouts.
+static size_t scale_buffer_bytes(int64_t rows, int64_t k) {
+  const int64_t ks = k / 32;
+  return (size_t)((rows + 31) / 32 * 32) * (size_t)((ks + 7) / 8 * 8);
+}
+static size_t round_up_256(size_t v) { return (v + 255) / 256 * 256; }
+
 size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant) {
   if (m <= 0 || n <= 0 || k <= 0 || split_k < 0 || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_)) return 0;
   const int v = pick_variant(m, n, k, variant);
+  if (v == WAVE_MXFP4_VARIANT_NAIVE) return 0;
   int splits = split_k;
   if (splits == 0) splits = auto_split(m, n, k, v);
-  if (splits <= 1 || v == WAVE_MXFP4_VARIANT_NAIVE) return 0;
-  return (size_t)splits * (size_t)m * (size_t)n * sizeof(float);
+  size_t bytes = 0;
+  if (splits > 1) bytes += round_up_256((size_t)splits * (size_t)m * (size_t)n * sizeof(float));
+  if (is_tile_variant(v) && k % kTileK == 0)
+    bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
+  return bytes;
 }
 
 int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
@@ -175,15 +186,43 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
       if (splits > 1) p.tiles_per_split = p.k_tiles / splits;
     }
   }
+  size_t ws_used = 0;
+  if (workspace && !aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
   if (splits > 1) {
     const size_t need = (size_t)splits * m * n * sizeof(float);
     if (!workspace || workspace_bytes < need) return WAVE_MXFP4_ERR_WORKSPACE;
-    if (!aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
     p.splits = splits;
     p.partial = (float *)workspace;
+    ws_used = round_up_256(need);
   }
 
   hipError_t e;
+  // The tile kernels read MFMA32-ordered scales with one dword per lane and one
+  // cache line per wave instruction; row-major scales cost 32 lines per
+  // instruction.  With scratch available, re-lay both operands out first
+  // (a few MB, microseconds) and run the native-scale kernel.
+  if (is_tile_variant(v) && k % kTileK == 0 && workspace) {
+    const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
+    const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? a_bytes : 0;
+    const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? b_bytes : 0;
+    if (ws_used + a_need + b_need <= workspace_bytes) {
+      uint8_t *ws = (uint8_t *)workspace + ws_used;
+      if (a_need) {
+        e = launch_scale_convert(p.a_scale, p.a_scale_layout, ws, WAVE_MXFP4_SCALE_MFMA32, m, p.ks, stream);
+        if (e != hipSuccess) return record_hip(e);
+        p.a_scale = ws;
+        p.a_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+        ws += a_need;
+      }
+      if (b_need) {
+        e = launch_scale_convert(p.b_scale, p.b_scale_layout, ws, WAVE_MXFP4_SCALE_MFMA32, n, p.ks, stream);
+        if (e != hipSuccess) return record_hip(e);
+        p.b_scale = ws;
+        p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+      }
+    }
+  }
+
   if (v == WAVE_MXFP4_VARIANT_NAIVE) {
     e = launch_naive_gemm(p, stream);
   } else if (v == WAVE_MXFP4_VARIANT_SKINNY) {
@@ -220,8 +259,9 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   p.offsets = offsets;
   p.num_groups = num_groups;
   p.b_group_stride = n * (k / 2);
-  p.b_scale_group_stride =
-      p.b_scale_shuffled ? ((n + 31) / 32 * 32) * (int64_t)p.ksp : n * (int64_t)p.ks;
+  p.b_scale_group_stride = p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR
+                               ? ((n + 31) / 32 * 32) * (int64_t)p.ksp
+                               : n * (int64_t)p.ks;
   // every expert's B and B_scale must keep the base alignment
   if (p.b_group_stride % 16 != 0 || p.b_scale_group_stride % 8 != 0) return WAVE_MXFP4_ERR_MISALIGNED;
 
@@ -256,12 +296,12 @@ int wave_mxfp4_e8m0_to_f32(const void *s, float *out, int64_t count, void *hip_s
 int wave_mxfp4_dequant(const void *q, const void *scale, float *out, int64_t rows, int64_t k,
                        int scale_layout, void *hip_stream) {
   if (rows < 0 || k < 0 || k % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
-  if (bad_enum(scale_layout, 2)) return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (bad_enum(scale_layout, 3)) return WAVE_MXFP4_ERR_BAD_ENUM;
   if (rows == 0 || k == 0) return WAVE_MXFP4_OK;
   if (!q || !scale || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
   if (!aligned(out, 8)) return WAVE_MXFP4_ERR_MISALIGNED;
-  return record_hip(launch_dequant((const uint8_t *)q, (const uint8_t *)scale, out, rows, k,
-                                   scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE, (hipStream_t)hip_stream));
+  return record_hip(launch_dequant((const uint8_t *)q, (const uint8_t *)scale, out, rows, k, scale_layout,
+                                   (hipStream_t)hip_stream));
 }
 
 size_t wave_mxfp4_e8m0_shuffle_bytes(int64_t rows, int64_t ks) {
@@ -275,6 +315,18 @@ int wave_mxfp4_e8m0_shuffle(const void *scale, void *out, int64_t rows, int64_t 
   if (!scale || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
   return record_hip(
       launch_e8m0_shuffle((const uint8_t *)scale, (uint8_t *)out, rows, ks, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_scale_convert(const void *src, int src_layout, void *dst, int dst_layout, int64_t rows,
+                             int64_t ks, void *hip_stream) {
+  if (rows < 0 || ks < 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (bad_enum(src_layout, 3) || bad_enum(dst_layout, 3)) return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (rows == 0 || ks == 0) return WAVE_MXFP4_OK;
+  if (!src || !dst) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (src == dst) return WAVE_MXFP4_ERR_UNSUPPORTED;  // not in place
+  if (dst_layout == WAVE_MXFP4_SCALE_MFMA32 && !aligned(dst, 4)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_scale_convert((const uint8_t *)src, src_layout, (uint8_t *)dst, dst_layout, rows, ks,
+                                         (hipStream_t)hip_stream));
 }
 
 int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, void *hip_stream) {

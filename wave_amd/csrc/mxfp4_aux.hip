@@ -35,12 +35,12 @@ __global__ void e8m0_kernel(const uint8_t *__restrict__ s, float *__restrict__ o
 // out[r, e] = value * scale(r, e/32); one thread per packed byte.
 __global__ void dequant_kernel(const uint8_t *__restrict__ q, const uint8_t *__restrict__ scale,
                                float *__restrict__ out, int64_t rows, int64_t kp, int64_t ks, int64_t ksp,
-                               int shuffled) {
+                               int layout) {
   const int64_t nbytes = rows * kp;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nbytes;
        i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t r = i / kp, kb = i - r * kp, g = kb >> 4;
-    const uint32_t sbyte = shuffled ? scale[e8m0_shuffle_offset(r, g, ksp)] : scale[r * ks + g];
+    const uint32_t sbyte = scale[scale_offset(layout, r, g, ks, ksp)];
     const float sc = e8m0_to_f32(sbyte);
     const uint32_t b = q[i];
     v2f v = {e2m1_to_f32(b & 0xFu) * sc, e2m1_to_f32(b >> 4) * sc};
@@ -63,6 +63,43 @@ __global__ void e8m0_shuffle_kernel(const uint8_t *__restrict__ scale, uint8_t *
     const int64_t r = rt * 32 + rh * 16 + r16;
     const int64_t g = kt * 8 + kh * 4 + g4;
     out[o] = (r < rows && g < ks) ? scale[r * ks + g] : (uint8_t)0;
+  }
+}
+
+// Any scale layout -> any scale layout, one thread per dword of the padded
+// (32 rows x 8 groups) index space; every destination byte, padding included, is
+// written exactly once.
+__global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_layout, uint8_t *__restrict__ dst,
+                                     int dst_layout, int64_t rows, int64_t ks, int64_t rows_p, int64_t ksp) {
+  const int64_t total = rows_p * (ksp >> 2);
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    // consecutive threads walk the MFMA32 order: block (row tile, K tile), lane, so
+    // that the writes of the common conversion (to MFMA32) are whole dwords
+    const int64_t blk = i >> 6, lane = i & 63;
+    const int64_t k_tiles = ksp >> 3;
+    const int64_t rt = blk / k_tiles, kt = blk - rt * k_tiles;
+    const int64_t r = rt * 32 + (lane & 31), fg = lane >> 5;
+    uint32_t word = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int64_t g = kt * 8 + 2 * t + fg;
+      const uint32_t b = (r < rows && g < ks) ? src[scale_offset(src_layout, r, g, ks, ksp)] : 0u;
+      word |= b << (8 * t);
+    }
+    if (dst_layout == WAVE_MXFP4_SCALE_MFMA32) {
+      *(uint32_t *)(dst + i * 4) = word;
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int64_t g = kt * 8 + 2 * t + fg;
+        if (dst_layout == WAVE_MXFP4_SCALE_ROW_MAJOR) {
+          if (r < rows && g < ks) dst[r * ks + g] = (uint8_t)(word >> (8 * t));
+        } else {
+          dst[scale_offset(dst_layout, r, g, ks, ksp)] = (uint8_t)(word >> (8 * t));
+        }
+      }
+    }
   }
 }
 
@@ -112,10 +149,8 @@ __global__ void naive_gemm_kernel(const GemmParams p) {
     }
     float acc = 0.f;
     for (int g = 0; g < p.ks; ++g) {
-      const uint32_t sa = p.a_scale_shuffled ? p.a_scale[e8m0_shuffle_offset(m, g, p.ksp)]
-                                             : p.a_scale[(int64_t)m * p.ks + g];
-      const uint32_t sb = p.b_scale_shuffled ? bsp[e8m0_shuffle_offset(n, g, p.ksp)]
-                                             : bsp[(int64_t)n * p.ks + g];
+      const uint32_t sa = p.a_scale[scale_offset(p.a_scale_layout, m, g, p.ks, p.ksp)];
+      const uint32_t sb = bsp[scale_offset(p.b_scale_layout, n, g, p.ks, p.ksp)];
       const float fa = e8m0_to_f32(sa), fb = e8m0_to_f32(sb);
       // one scale group = 16 packed bytes, contiguous in both B layouts
       const v4i av = *(const v4i *)(p.a + (int64_t)m * p.kp + g * 16);
@@ -152,12 +187,12 @@ hipError_t launch_e8m0_to_f32(const uint8_t *s, float *out, int64_t count, hipSt
 }
 
 hipError_t launch_dequant(const uint8_t *q, const uint8_t *scale, float *out, int64_t rows, int64_t k,
-                          int shuffled, hipStream_t stream) {
+                          int layout, hipStream_t stream) {
   const int64_t n = rows * (k / 2);
   if (n == 0) return hipSuccess;
   const int64_t ks = k / 32, ksp = (ks + 7) / 8 * 8;
   dequant_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(q, scale, out, rows, k / 2, ks, ksp,
-                                                                  shuffled);
+                                                                  layout);
   return hipGetLastError();
 }
 
@@ -167,6 +202,16 @@ hipError_t launch_e8m0_shuffle(const uint8_t *scale, uint8_t *out, int64_t rows,
   const int64_t n = rows_p * ksp;
   if (n == 0) return hipSuccess;
   e8m0_shuffle_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(scale, out, rows, ks, rows_p, ksp);
+  return hipGetLastError();
+}
+
+hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst, int dst_layout, int64_t rows,
+                                int64_t ks, hipStream_t stream) {
+  const int64_t rows_p = (rows + 31) / 32 * 32, ksp = (ks + 7) / 8 * 8;
+  const int64_t n = rows_p * (ksp / 4);
+  if (n == 0) return hipSuccess;
+  scale_convert_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(src, src_layout, dst, dst_layout, rows,
+                                                                        ks, rows_p, ksp);
   return hipGetLastError();
 }
 

@@ -42,7 +42,8 @@ struct GemmParams {
   int tiles_per_split; // K tiles owned by one split
   int splits;
   int out_bf16;
-  int a_scale_shuffled, b_scale_shuffled, b_preshuffled;
+  int a_scale_layout, b_scale_layout;  // wave_mxfp4_scale_layout
+  int b_preshuffled;
   int num_groups;      // 0 = dense
   int tiles_m, tiles_n;
   int64_t b_group_stride;        // bytes between experts in b
@@ -81,6 +82,22 @@ __device__ __host__ __forceinline__ int64_t e8m0_shuffle_offset(int64_t r, int64
          ((g & 7) >> 2) * 2 + ((r & 31) >> 4);
 }
 
+// Byte offset of scale (row r, group g) in the library's MFMA32 order: per 32-row
+// tile and K tile (8 groups) one 256-byte block holding, for the lane
+// (g%2)*32 + r%32 of the 32x32x64 scaled MFMA, the four bytes of its K steps
+// t = (g%8)/2 = 0..3.
+__device__ __host__ __forceinline__ int64_t mfma32_scale_offset(int64_t r, int64_t g, int64_t k_tiles) {
+  return ((r >> 5) * k_tiles + (g >> 3)) * 256 + (((g & 1) << 5) | (r & 31)) * 4 + ((g & 7) >> 1);
+}
+
+// Byte offset of scale (r, g) for any wave_mxfp4_scale_layout.
+__device__ __host__ __forceinline__ int64_t scale_offset(int layout, int64_t r, int64_t g, int64_t ks,
+                                                         int64_t ksp) {
+  if (layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) return e8m0_shuffle_offset(r, g, ksp);
+  if (layout == WAVE_MXFP4_SCALE_MFMA32) return mfma32_scale_offset(r, g, ksp >> 3);
+  return r * ks + g;
+}
+
 // Byte offset of packed byte (row n, byte kb) in the b_preshuffle order.
 __device__ __host__ __forceinline__ int64_t b_preshuffle_offset(int64_t n, int64_t kb, int64_t kp) {
   return (n >> 4) * 16 * kp + (kb >> 5) * 512 + ((kb >> 4) & 1) * 256 + (n & 15) * 16 + (kb & 15);
@@ -95,7 +112,9 @@ hipError_t launch_splitk_reduce(const float *partial, void *c, int64_t mn, int s
 hipError_t launch_to_f32(const uint8_t *q, float *out, int64_t rows, int64_t kp, hipStream_t stream);
 hipError_t launch_e8m0_to_f32(const uint8_t *s, float *out, int64_t count, hipStream_t stream);
 hipError_t launch_dequant(const uint8_t *q, const uint8_t *scale, float *out, int64_t rows, int64_t k,
-                          int shuffled, hipStream_t stream);
+                          int scale_layout, hipStream_t stream);
+hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst, int dst_layout, int64_t rows,
+                                int64_t ks, hipStream_t stream);
 hipError_t launch_e8m0_shuffle(const uint8_t *scale, uint8_t *out, int64_t rows, int64_t ks,
                                hipStream_t stream);
 hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t kp,

@@ -67,8 +67,11 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) skinny_gemm_kernel(const Ge
   const bool scale_bytes = (p.ks & 7) != 0;
   const int tail_chunks = (p.k & (kTileK - 1)) >> 5;
 
-  auto load_scale_raw = [&](const uint8_t *base, bool shuffled, int row, int kt, uint32_t(&raw)[2]) {
-    if (shuffled) {
+  auto load_scale_raw = [&](const uint8_t *base, int layout, int row, int kt, uint32_t(&raw)[2]) {
+    if (layout == WAVE_MXFP4_SCALE_MFMA32) {
+      raw[0] = base[mfma32_scale_offset(row, kt * 8 + fg, p.ksp >> 3)];
+      raw[1] = base[mfma32_scale_offset(row, kt * 8 + 4 + fg, p.ksp >> 3)];
+    } else if (layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {
       const int64_t off = (int64_t)(row >> 5) * ((p.ksp >> 3) * 256) + (int64_t)kt * 256 + fg * 64 +
                           (row & 15) * 4;
       raw[0] = *(const uint32_t *)(base + off);
@@ -84,8 +87,10 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) skinny_gemm_kernel(const Ge
       raw[1] = g1 < p.ks ? rp[g1] : 127u;
     }
   };
-  auto canon_scale = [&](bool shuffled, int row, const uint32_t(&raw)[2]) -> uint32_t {
-    if (shuffled) {
+  auto canon_scale = [&](int layout, int row, const uint32_t(&raw)[2]) -> uint32_t {
+    if (layout == WAVE_MXFP4_SCALE_MFMA32) {
+      return (raw[0] & 0xFFu) | ((raw[1] & 0xFFu) << 8);
+    } else if (layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {
       const int sh = ((row >> 4) & 1) * 8;
       return ((raw[0] >> sh) & 0xFFu) | (((raw[0] >> (16 + sh)) & 0xFFu) << 8);
     } else if (!scale_bytes) {
@@ -105,9 +110,9 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) skinny_gemm_kernel(const Ge
       for (int i = 0; i < MT_M; ++i)
         st.a[i][s] = valid ? *(const v4i *)(a_lane[i] + (int64_t)kt * kTileKBytes + s * 64) : zero;
     }
-    load_scale_raw(p.b_scale, p.b_scale_shuffled, brow, kt, st.sb);
+    load_scale_raw(p.b_scale, p.b_scale_layout, brow, kt, st.sb);
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) load_scale_raw(p.a_scale, p.a_scale_shuffled, arow[i], kt, st.sa[i]);
+    for (int i = 0; i < MT_M; ++i) load_scale_raw(p.a_scale, p.a_scale_layout, arow[i], kt, st.sa[i]);
   };
 
   v4f acc[MT_M];
@@ -115,12 +120,12 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) skinny_gemm_kernel(const Ge
   for (int i = 0; i < MT_M; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
 
   auto compute_stage = [&](const SkinnyStage<MT_M> &st) {
-    const int scb = (int)canon_scale(p.b_scale_shuffled, brow, st.sb);
+    const int scb = (int)canon_scale(p.b_scale_layout, brow, st.sb);
     const v8i vb0 = {st.b[0].x, st.b[0].y, st.b[0].z, st.b[0].w, 0, 0, 0, 0};
     const v8i vb1 = {st.b[1].x, st.b[1].y, st.b[1].z, st.b[1].w, 0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
-      const int sca = (int)canon_scale(p.a_scale_shuffled, arow[i], st.sa[i]);
+      const int sca = (int)canon_scale(p.a_scale_layout, arow[i], st.sa[i]);
       const v8i va0 = {st.a[i][0].x, st.a[i][0].y, st.a[i][0].z, st.a[i][0].w, 0, 0, 0, 0};
       const v8i va1 = {st.a[i][1].x, st.a[i][1].y, st.a[i][1].z, st.a[i][1].w, 0, 0, 0, 0};
       // first port = B rows (N index), second port = A rows (M index): the

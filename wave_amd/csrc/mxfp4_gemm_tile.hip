@@ -7,13 +7,31 @@
 // :334-403 (preshuffled scales / B) and :611-816 (split-K).
 //
 // Data flow per K tile of 256 elements (128 packed bytes per row):
-//   global --(global_load_lds_dwordx4, 16 B per lane)--> LDS stage (2 stages)
+//   global --(global_load_lds_dwordx4, 16 B per lane)--> LDS ring slot
 //   LDS --(ds_read_b128)--> one 16 B MFMA operand fragment per lane
-//   scales: global -> VGPR (one iteration ahead), one byte per lane per MFMA
+//   scales: global -> VGPR one K tile ahead, one byte per lane per MFMA
+//
+// What bounds the design (measured on MI355X):
+// * A wave's DMA instruction moves 8 rows x 128 B = 8 full cache lines; the
+//   vector L1 retires about one line per 2 clocks whatever part of the line is
+//   used, so rows are always fetched as whole 128-byte lines (K tile = 256).
+// * At full MFMA rate a 256x256 tile needs 32 B/clk/CU of the ~55 B/clk/CU the
+//   DMA path sustains.  A burst of DMA instructions blocks the issuing wave
+//   (and the MFMAs queued behind it), so the DMA instructions are spread
+//   evenly: one half operand tile per 64-wide K step.
+// * That needs more than two buffers in flight.  LDS (160 KB) is used as a
+//   ring of five operand-tile slots A(j) B(j) A(j+1) B(j+1) A(j+2): slot of
+//   operand tile h = 2*j + (0 for A, 1 for B) is h % 5.
+// * Scale bytes are read as dwords.  In the e8m0_shuffle tile order a wave's
+//   load touches one cache line; in row-major order it touches 32, which costs
+//   more L1 time than the operand data, so row-major scales are reshuffled by a
+//   pre-pass (see the C ABI) and only fall back to direct reads without scratch.
+//
 // LDS rows are 128 B; 16-byte chunk c of row r is stored at chunk position
 // c ^ ((r / 2) % 8), which keeps the 16 lanes ds_read_b128 serves together on
-// 16 different 16-byte bank groups.  The DMA writes LDS linearly, so the XOR is applied to the
-// global source address, and undone by the fragment reader.
+// 16 different 16-byte bank groups (no conflicts measured).  The DMA writes
+// LDS linearly, so the XOR is applied to the global source address and undone
+// by the fragment reader.
 //
 // MFMA operand order is swapped (B rows feed the "A" port) so that a lane's
 // accumulator holds runs of four consecutive N columns of one M row, each
@@ -32,11 +50,13 @@ struct TileCfg {
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // per-wave tile
   static constexpr int MT_M = WM / 32, MT_N = WN / 32;        // 32x32 MFMA tiles per wave
   static constexpr int A_BYTES = BM * kTileKBytes, B_BYTES = BN * kTileKBytes;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int RING_SLOTS = 5;
+  static constexpr int SLOT_BYTES = A_BYTES > B_BYTES ? A_BYTES : B_BYTES;
+  static constexpr int LDS_BYTES = RING_SLOTS * SLOT_BYTES;
   // One DMA instruction of a wave fills 8 LDS rows (64 lanes x 16 B).
   static constexpr int A_LD = BM / 8 / NWAVES, B_LD = BN / 8 / NWAVES;
-  static_assert(BM % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0, "tile rows must split over waves");
+  static_assert(BM % (16 * NWAVES) == 0 && BN % (16 * NWAVES) == 0, "half operand tiles must split over waves");
+  static_assert(LDS_BYTES <= 160 * 1024, "ring does not fit LDS");
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be MFMA aligned");
 };
 
@@ -70,35 +90,77 @@ __device__ __forceinline__ uint32_t perm_bytes(uint32_t hi, uint32_t lo, uint32_
   return __builtin_amdgcn_perm(hi, lo, sel);
 }
 
-// How one operand's scales are addressed by the kernel, whatever their layout:
-// per 32-row tile a lane reads two dwords at `off + kt*kt_stride` and that plus
-// `delta`, then picks its four bytes (K steps 0..3) with v_perm and `sel`.
-//   row-major : off = row*ks, kt_stride = 8, delta = 4; the row's bytes 0..7 are
-//               groups 0..7, the lane needs 2t + fg            -> sel 0x06040200 / 0x07050301
-//   shuffled  : group g of row r sits at tile(r/32, kt)*256 + (g%4)*64 + (r%16)*4 +
-//               (g/4)*2 + (r/16)%2.  off = tile row + fg*64 + (r%16)*4, kt_stride = 256,
-//               delta = 128; dword0 = groups {fg, 4+fg}, dword1 = groups {2+fg, 6+fg},
-//               each for both 16-row halves                    -> sel 0x06020400 / 0x07030501
+// How one operand's scales are addressed by the kernel.  Per 32-row tile and K
+// tile a lane needs four bytes: the scales of (row, group 2t + fg), t = 0..3.
+//   MFMA32    : they are one dword, at block(r/32, kt)*256 + lane*4 (one load,
+//               one cache line per wave instruction, no byte shuffling).
+//   otherwise : two dwords at `off + kt*kt_stride` and that plus `delta`, then
+//               v_perm with `sel`:
+//     row-major : off = row*ks, kt_stride = 8, delta = 4; the row's bytes 0..7 are
+//                 groups 0..7                                  -> sel 0x06040200 / 0x07050301
+//     shuffled  : group g of row r sits at tile(r/32, kt)*256 + (g%4)*64 + (r%16)*4 +
+//                 (g/4)*2 + (r/16)%2.  off = tile row + fg*64 + (r%16)*4, kt_stride = 256,
+//                 delta = 128; dword0 = groups {fg, 4+fg}, dword1 = groups {2+fg, 6+fg},
+//                 each for both 16-row halves                  -> sel 0x06020400 / 0x07030501
 struct ScaleAddr {
   int kt_stride;
   int delta;
 };
 
-__device__ __forceinline__ void scale_lane_setup(bool shuffled, int row, int fg, int ks, int ksp,
+__device__ __forceinline__ ScaleAddr scale_addr(int layout) {
+  if (layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) return ScaleAddr{256, 128};
+  if (layout == WAVE_MXFP4_SCALE_MFMA32) return ScaleAddr{256, 0};
+  return ScaleAddr{8, 4};
+}
+
+// `row` is the absolute row, `row0` the first row of the workgroup's tile; the
+// offset is relative to scale_tile_base(row0).
+__device__ __forceinline__ void scale_lane_setup(int layout, int row, int row0, int fg, int ks, int ksp,
                                                  uint32_t &off, uint32_t &sel) {
-  if (shuffled) {
-    off = (uint32_t)((row >> 5) * ((ksp >> 3) * 256) + fg * 64 + (row & 15) * 4);
+  if (layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {
+    off = (uint32_t)(((row >> 5) - (row0 >> 5)) * ((ksp >> 3) * 256) + fg * 64 + (row & 15) * 4);
     sel = ((row >> 4) & 1) ? 0x07030501u : 0x06020400u;
+  } else if (layout == WAVE_MXFP4_SCALE_MFMA32) {
+    off = (uint32_t)(((row >> 5) - (row0 >> 5)) * ((ksp >> 3) * 256) + (fg * 32 + (row & 31)) * 4);
+    sel = 0x03020100u;  // identity on the low dword
   } else {
-    off = (uint32_t)(row * ks);
+    off = (uint32_t)((row - row0) * ks);
     sel = fg ? 0x07050301u : 0x06040200u;
   }
 }
 
-template <class Cfg, bool GENERIC_K>
-__global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams p) {
+__device__ __forceinline__ const uint8_t *scale_tile_base(const uint8_t *base, int layout, int row0, int ks,
+                                                          int ksp) {
+  return layout == WAVE_MXFP4_SCALE_ROW_MAJOR ? base + (int64_t)row0 * ks
+                                              : base + (int64_t)(row0 >> 5) * ((ksp >> 3) * 256);
+}
+
+// Raw (stride 0) buffer descriptor over [base, base + 2 GiB): loads take a
+// 32-bit per-lane offset plus a scalar offset, so no 64-bit address math is
+// issued between the MFMAs.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7FFFFFFF, 0x00020000);
+}
+
+// s_waitcnt immediate that waits for vmcnt <= n and lgkmcnt == 0 (gfx9
+// encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14).
+__host__ __device__ constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | (7 << 4) | ((n >> 4) << 14); }
+
+// The kernel body lives in a __device__ function so that only the device pass
+// sees the gfx950 buffer-resource types and builtins.
+// MODE: kDirect reads the scales in whatever layout they come in (two dwords
+// and a v_perm per 32-row tile); kNative requires both scale tensors in MFMA32
+// order (one dword); kGenericK is kDirect plus a partial last K tile and scale
+// rows that are not 8-byte multiples (K % 256 != 0).
+enum TileMode { kDirect = 0, kNative = 1, kGenericK = 2 };
+
+template <class Cfg, int MODE>
+__device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
+  constexpr bool GENERIC_K = MODE == kGenericK;
+  constexpr bool NATIVE = MODE == kNative;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
+  constexpr int SLOT = Cfg::SLOT_BYTES, RING = Cfg::RING_SLOTS;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   const int lane = threadIdx.x & 63;
@@ -144,58 +206,53 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
   if (nkt <= 0) return;
 
   // ---------------- global -> LDS addressing ----------------
-  // DMA instruction d of this wave fills LDS rows (d*NWAVES + wave)*8 .. +7;
-  // lane t lands at row t/8, chunk position t%8, which must hold logical
-  // chunk (t%8) ^ swz(row), swz(row) = (row/2) % 8.  Consecutive d are 8*NWAVES
-  // rows apart (a multiple of 16), so the chunk does not depend on d.
+  // DMA instruction d of this wave fills LDS rows (d*NWAVES + wave)*8 .. +7 of
+  // an operand tile; lane t lands at row t/8, chunk position t%8, which must
+  // hold logical chunk (t%8) ^ swz(row), swz(row) = (row/2) % 8.  Consecutive d
+  // are 8*NWAVES rows apart (a multiple of 16), so the chunk does not depend on d.
   const int kp = p.kp;
-  const uint8_t *a_tile = p.a + (int64_t)m0 * kp;
-  const uint8_t *b_tile = b_ptr + (int64_t)n0 * kp;  // preshuffle keeps 16-row blocks contiguous
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(p.a + (int64_t)m0 * kp);
+  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_ptr + (int64_t)n0 * kp);  // preshuffle keeps 16-row blocks contiguous
   const int ld_row0 = wave * 8 + (lane >> 3);
   const int ld_chunk = (lane & 7) ^ ((ld_row0 >> 1) & 7);
   const int a_row_lim = p.m - 1 - m0, b_row_lim = p.n - 1 - n0;  // clamp to allocated rows
-  // B offset of (row r, chunk c) inside the tile, K tile 0:
+  // Per-lane byte offsets inside the operand tile at K tile 0, one per DMA
+  // instruction; K tile kt adds a scalar kt*128 (kt*2048 for preshuffled B).
   //   row-major  : r*kp + c*16
   //   preshuffle : (r/16)*16*kp + (c/2)*512 + (c%2)*256 + (r%16)*16
-  const int b_row_shift = p.b_preshuffled ? 4 : 0;
-  const int b_row_mask = p.b_preshuffled ? 15 : 0;
-  const int b_blk_stride = p.b_preshuffled ? 16 * kp : kp;
-  const int b_chunk_off = p.b_preshuffled ? (ld_chunk >> 1) * 512 + (ld_chunk & 1) * 256 : ld_chunk * 16;
+  int a_goff[A_LD], b_goff[B_LD];
+#pragma unroll
+  for (int d = 0; d < A_LD; ++d) a_goff[d] = min(ld_row0 + d * NWAVES * 8, a_row_lim) * kp + ld_chunk * 16;
+#pragma unroll
+  for (int d = 0; d < B_LD; ++d) {
+    const int r = min(ld_row0 + d * NWAVES * 8, b_row_lim);
+    b_goff[d] = p.b_preshuffled
+                    ? (r >> 4) * 16 * kp + (r & 15) * 16 + (ld_chunk >> 1) * 512 + (ld_chunk & 1) * 256
+                    : r * kp + ld_chunk * 16;
+  }
   const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
   const int tail_chunks = GENERIC_K ? ((p.k & (kTileK - 1)) >> 5) : 0;  // valid chunks of a partial last tile
 
-  auto issue_g2l = [&](int kt, int stage) {
-    uint8_t *sa = smem + stage * Cfg::STAGE_BYTES;
-    uint8_t *sb = sa + Cfg::A_BYTES;
-    const uint8_t *ga = a_tile + (int64_t)kt * kTileKBytes;
-    const uint8_t *gb = b_tile + (int64_t)kt * b_kt_stride;
-    // The row offsets are recomputed per K tile (a handful of VALU ops hidden
-    // under the MFMAs) rather than kept in 2*(A_LD+B_LD) registers.
-    int lr = ld_row0;
-    asm volatile("" : "+v"(lr));
+  // DMA instructions [d0, d1) of operand tile `op` (0 = A, 1 = B) of K tile
+  // `kt` into ring slot `slot`.
+  auto issue_g2l = [&](int op, int kt, int slot, int d0, int d1) {
+    uint8_t *dst_tile = smem + slot * SLOT;
     // Partial last K tile: chunks at or past the end of K are written as zeros
     // (fp4 +0.0), so they add nothing whatever their scale.
     const bool tail = GENERIC_K && tail_chunks != 0 && kt == p.k_tiles - 1;
     const v4i zero = {0, 0, 0, 0};
+    const int soff = op == 0 ? kt * kTileKBytes : kt * b_kt_stride;
 #pragma unroll
-    for (int d = 0; d < A_LD; ++d) {
-      const int r = min(lr + d * NWAVES * 8, a_row_lim);
-      const uint32_t off = (uint32_t)(r * kp + ld_chunk * 16);
-      uint8_t *dst = sa + (d * NWAVES + wave) * 1024;
-      if (!tail || ld_chunk < tail_chunks)
-        __builtin_amdgcn_global_load_lds(WAVE_GLOBAL_PTR(ga + off), WAVE_LDS_PTR(dst), 16, 0, 0);
-      else
+    for (int d = d0; d < d1; ++d) {
+      uint8_t *dst = dst_tile + (d * NWAVES + wave) * 1024;
+      if (!tail || ld_chunk < tail_chunks) {
+        if (op == 0)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, WAVE_LDS_PTR(dst), 16, a_goff[d], soff, 0, 0);
+        else
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst), 16, b_goff[d], soff, 0, 0);
+      } else {
         *(v4i *)(dst + lane * 16) = zero;
-    }
-#pragma unroll
-    for (int d = 0; d < B_LD; ++d) {
-      const int r = min(lr + d * NWAVES * 8, b_row_lim);
-      const uint32_t off = (uint32_t)((r >> b_row_shift) * b_blk_stride + (r & b_row_mask) * 16 + b_chunk_off);
-      uint8_t *dst = sb + (d * NWAVES + wave) * 1024;
-      if (!tail || ld_chunk < tail_chunks)
-        __builtin_amdgcn_global_load_lds(WAVE_GLOBAL_PTR(gb + off), WAVE_LDS_PTR(dst), 16, 0, 0);
-      else
-        *(v4i *)(dst + lane * 16) = zero;
+      }
     }
   };
 
@@ -209,14 +266,15 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
 #pragma unroll
   for (int t = 0; t < 4; ++t) foff[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
   const uint32_t a_fbase = (uint32_t)(wave_m * Cfg::WM * kTileKBytes);
-  const uint32_t b_fbase = (uint32_t)(Cfg::A_BYTES + wave_n * Cfg::WN * kTileKBytes);
+  const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
 
-  auto read_frags = [&](int stage, int t, v4i(&fa)[MT_M], v4i(&fb)[MT_N]) {
-    const uint8_t *base = smem + stage * Cfg::STAGE_BYTES + foff[t];
+  auto read_frags = [&](int slot_a, int slot_b, int t, v4i(&fa)[MT_M], v4i(&fb)[MT_N]) {
+    const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
+    const uint8_t *bb = smem + slot_b * SLOT + b_fbase + foff[t];
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(base + a_fbase + i * 32 * kTileKBytes);
+    for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(ba + i * 32 * kTileKBytes);
 #pragma unroll
-    for (int j = 0; j < MT_N; ++j) fb[j] = *(const v4i *)(base + b_fbase + j * 32 * kTileKBytes);
+    for (int j = 0; j < MT_N; ++j) fb[j] = *(const v4i *)(bb + j * 32 * kTileKBytes);
   };
 
   // ---------------- scales ----------------
@@ -226,14 +284,18 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
   uint32_t a_soff[MT_M], a_ssel[MT_M], b_soff[MT_N], b_ssel[MT_N];
 #pragma unroll
   for (int i = 0; i < MT_M; ++i)
-    scale_lane_setup(p.a_scale_shuffled, min(m0 + wave_m * Cfg::WM + i * 32 + fr, p.m - 1), fg, p.ks, p.ksp,
+    scale_lane_setup(p.a_scale_layout, min(m0 + wave_m * Cfg::WM + i * 32 + fr, p.m - 1), m0, fg, p.ks, p.ksp,
                      a_soff[i], a_ssel[i]);
 #pragma unroll
   for (int j = 0; j < MT_N; ++j)
-    scale_lane_setup(p.b_scale_shuffled, min(n0 + wave_n * Cfg::WN + j * 32 + fr, p.n - 1), fg, p.ks, p.ksp,
+    scale_lane_setup(p.b_scale_layout, min(n0 + wave_n * Cfg::WN + j * 32 + fr, p.n - 1), n0, fg, p.ks, p.ksp,
                      b_soff[j], b_ssel[j]);
-  const ScaleAddr a_sa = {p.a_scale_shuffled ? 256 : 8, p.a_scale_shuffled ? 128 : 4};
-  const ScaleAddr b_sa = {p.b_scale_shuffled ? 256 : 8, p.b_scale_shuffled ? 128 : 4};
+  const ScaleAddr a_sa = scale_addr(p.a_scale_layout);
+  const ScaleAddr b_sa = scale_addr(p.b_scale_layout);
+  const uint8_t *as_base = scale_tile_base(p.a_scale, p.a_scale_layout, m0, p.ks, p.ksp);
+  const uint8_t *bs_base = scale_tile_base(bs_ptr, p.b_scale_layout, n0, p.ks, p.ksp);
+  const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc(as_base);
+  const __amdgpu_buffer_rsrc_t bs_rsrc = make_rsrc(bs_base);
 
   uint32_t raw_a[MT_M][2], raw_b[MT_N][2];
   uint32_t sc_a[MT_M], sc_b[MT_N];
@@ -245,8 +307,8 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
 #pragma unroll
       for (int i = 0; i < MT_M + MT_N; ++i) {
         const bool is_a = i < MT_M;
-        const bool shuffled = is_a ? p.a_scale_shuffled : p.b_scale_shuffled;
-        const uint8_t *base = is_a ? p.a_scale : bs_ptr;
+        const bool shuffled = (is_a ? p.a_scale_layout : p.b_scale_layout) != WAVE_MXFP4_SCALE_ROW_MAJOR;
+        const uint8_t *base = is_a ? as_base : bs_base;
         const uint32_t off = is_a ? a_soff[i] : b_soff[i - MT_M];
         const ScaleAddr sa = is_a ? a_sa : b_sa;
         uint32_t(&raw)[2] = is_a ? raw_a[i] : raw_b[i - MT_M];
@@ -266,28 +328,29 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
       }
       return;
     }
-    const uint8_t *ab = p.a_scale + (int64_t)kt * a_sa.kt_stride;
-    const uint8_t *bb = bs_ptr + (int64_t)kt * b_sa.kt_stride;
+    const int ao = kt * a_sa.kt_stride, bo = kt * b_sa.kt_stride;
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
-      raw_a[i][0] = *(const uint32_t *)(ab + a_soff[i]);
-      raw_a[i][1] = *(const uint32_t *)(ab + a_sa.delta + a_soff[i]);
+      raw_a[i][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, (int)a_soff[i], ao, 0);
+      if (!NATIVE)
+        raw_a[i][1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, (int)a_soff[i], ao + a_sa.delta, 0);
     }
 #pragma unroll
     for (int j = 0; j < MT_N; ++j) {
-      raw_b[j][0] = *(const uint32_t *)(bb + b_soff[j]);
-      raw_b[j][1] = *(const uint32_t *)(bb + b_sa.delta + b_soff[j]);
+      raw_b[j][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(bs_rsrc, (int)b_soff[j], bo, 0);
+      if (!NATIVE)
+        raw_b[j][1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(bs_rsrc, (int)b_soff[j], bo + b_sa.delta, 0);
     }
   };
   auto canon_scales = [&]() {
-    const bool a_bytes = GENERIC_K && (p.ks & 7) != 0 && !p.a_scale_shuffled;
-    const bool b_bytes = GENERIC_K && (p.ks & 7) != 0 && !p.b_scale_shuffled;
+    const bool a_bytes = GENERIC_K && (p.ks & 7) != 0 && p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
+    const bool b_bytes = GENERIC_K && (p.ks & 7) != 0 && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
 #pragma unroll
     for (int i = 0; i < MT_M; ++i)
-      sc_a[i] = a_bytes ? raw_a[i][0] : perm_bytes(raw_a[i][1], raw_a[i][0], a_ssel[i]);
+      sc_a[i] = (NATIVE || a_bytes) ? raw_a[i][0] : perm_bytes(raw_a[i][1], raw_a[i][0], a_ssel[i]);
 #pragma unroll
     for (int j = 0; j < MT_N; ++j)
-      sc_b[j] = b_bytes ? raw_b[j][0] : perm_bytes(raw_b[j][1], raw_b[j][0], b_ssel[j]);
+      sc_b[j] = (NATIVE || b_bytes) ? raw_b[j][0] : perm_bytes(raw_b[j][1], raw_b[j][0], b_ssel[j]);
   };
 
   // ---------------- accumulators ----------------
@@ -318,131 +381,226 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
   typedef std::integral_constant<int, 2> T2;
   typedef std::integral_constant<int, 3> T3;
 
-  // ---------------- main loop ----------------
-  // Two LDS stages; the DMA of K tile it+2 is issued as soon as every wave has
-  // finished reading tile it (3/4 through iteration it) and is waited for at
-  // the same point of iteration it+1.  Fragments are double-buffered in
-  // registers across the four 64-wide K steps of a tile.
-  v4i fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  // Issue order inside a phase (16 MFMAs of a 4-wave 256x256 tile): the LDS
+  // reads of the next K step go out behind the first MFMAs, the DMA
+  // instructions are spread one per group.  Masks: 0x008 MFMA, 0x100 LDS read,
+  // 0x020 VMEM read.
+  constexpr int HALF_LD = (A_LD < B_LD ? A_LD : B_LD) / 2;  // DMA instructions per phase
+  constexpr int NGROUP = HALF_LD < 1 ? 1 : HALF_LD;
+  auto order_phase = [&]() {
+    constexpr int R = MT_M + MT_N, Q = MT_M * MT_N;
+    constexpr int RG = (R + NGROUP - 1) / NGROUP, QG = Q / NGROUP;
+#pragma unroll
+    for (int g = 0; g < NGROUP; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, RG, 0);
+      if (QG > 1) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (QG > 2) __builtin_amdgcn_sched_group_barrier(0x008, QG - 2, 0);
+    }
+  };
 
-  issue_g2l(kt_begin, 0);
+  // ---------------- main loop ----------------
+  // Ring slots: operand tile h = 2*j + op lives in slot h % 5.  While K tile j
+  // is multiplied (phases P0..P3 = its four 64-wide K steps):
+  //   P0: second half of B(j+1)      P1: first half of A(j+2)
+  //   P2: second half of A(j+2)      P3: barrier, then first half of B(j+2)
+  // The barrier at P3 needs this wave's part of A(j+1), B(j+1) landed: every DMA
+  // issued after B(j+1) is the A_LD instructions of A(j+2), hence vmcnt(A_LD).
+  // After it all waves have finished reading tile j, which frees the slots of
+  // A(j) (-> B(j+2), issued from P3 on) and B(j) (-> A(j+3)).
+  // Fragments are double-buffered in registers across the K steps.
+  v4i fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  constexpr int kWaitSteady = GENERIC_K ? 0 : A_LD;
+  constexpr int kWaitPrologue = GENERIC_K ? 0 : A_LD + B_LD / 2;
+
+  issue_g2l(0, kt_begin, 0, 0, A_LD);
+  issue_g2l(1, kt_begin, 1, 0, B_LD);
   load_scales(kt_begin);
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  if (nkt > 1) issue_g2l(kt_begin + 1, 1);
+  if (nkt > 1) {
+    issue_g2l(0, kt_begin + 1, 2, 0, A_LD);
+    issue_g2l(1, kt_begin + 1, 3, 0, B_LD / 2);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kWaitPrologue));
+  } else {
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  }
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
   canon_scales();
   if (nkt > 1) load_scales(kt_begin + 1);
-  read_frags(0, 0, fa0, fb0);
+  read_frags(0, 1, 0, fa0, fb0);
   __builtin_amdgcn_sched_barrier(0);
 
-  // One K tile.  The sched_barriers pin the phase order (the scheduler may
-  // interleave inside a phase, i.e. the LDS reads of step t+1 with the MFMAs of
-  // step t, but not merge phases, which would need every step's fragments
-  // live at once).  HAS1: tile it+1 exists; HAS2: tile it+2 exists.
-  // Issue order inside a phase: the LDS reads of the next K step go out first,
-  // two behind each of the first MFMAs, so their latency is covered by the
-  // remaining MFMAs of the phase.  Masks: 0x008 MFMA, 0x100 LDS read, 0x020 VMEM read.
-  auto order_reads_then_mfma = [&]() {
-#pragma unroll
-    for (int r = 0; r < (MT_M + MT_N) / 2; ++r) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, MT_M * MT_N - (MT_M + MT_N) / 2, 0);
-  };
-  auto k_tile = [&](int it, auto has1_tag, auto has2_tag) {
+  // One K tile.  sa/sb: ring slots of A(j), B(j).  HAS1: tile j+1 exists;
+  // HAS2: tile j+2 exists.  The sched_barriers pin the phase order.
+  auto k_tile = [&](int j, int sa, int sb, auto has1_tag, auto has2_tag) {
     constexpr bool HAS1 = decltype(has1_tag)::value, HAS2 = decltype(has2_tag)::value;
-    const int cur = it & 1;
-    read_frags(cur, 1, fa1, fb1);
+    const int kt = kt_begin + j;
+    // slots: A(j+1) = sa+2, B(j+1) = sa+3, A(j+2) = sa+4, B(j+2) = sa (mod 5)
+    const int sa1 = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
+    const int sb1 = sa + 3 >= RING ? sa + 3 - RING : sa + 3;
+    const int sa2 = sa + 4 >= RING ? sa + 4 - RING : sa + 4;
+    read_frags(sa, sb, 1, fa1, fb1);
     mfma_block(fa0, fb0, T0{});
-    order_reads_then_mfma();
+    if (HAS1) issue_g2l(1, kt + 1, sb1, B_LD / 2, B_LD);
+    order_phase();
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(cur, 2, fa0, fb0);
+    read_frags(sa, sb, 2, fa0, fb0);
     mfma_block(fa1, fb1, T1{});
-    order_reads_then_mfma();
+    if (HAS2) issue_g2l(0, kt + 2, sa2, 0, A_LD / 2);
+    order_phase();
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(cur, 3, fa1, fb1);
+    read_frags(sa, sb, 3, fa1, fb1);
     mfma_block(fa0, fb0, T2{});
-    order_reads_then_mfma();
+    if (HAS2) issue_g2l(0, kt + 2, sa2, A_LD / 2, A_LD);
+    order_phase();
     __builtin_amdgcn_sched_barrier(0);
-    // Own DMA of tile it+1 and all fragment reads of stage `cur` are complete
-    // before the barrier; after it every wave's are.
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    __builtin_amdgcn_sched_barrier(0);
-    if (HAS2) issue_g2l(kt_begin + it + 2, cur);
-    if (HAS1) read_frags(cur ^ 1, 0, fa0, fb0);
-    mfma_block(fa1, fb1, T3{});
-    if (HAS2) {
-      // DMA first (longest latency), LDS reads next, all within the first MFMAs
-      constexpr int G = A_LD + B_LD, R = MT_M + MT_N, Q = MT_M * MT_N;
-      constexpr int SLOTS = Q / 2;
-#pragma unroll
-      for (int r = 0; r < SLOTS; ++r) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x020, (G + SLOTS - 1) / SLOTS, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, (R + SLOTS - 1) / SLOTS, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, Q - SLOTS, 0);
-    } else if (HAS1) {
-      order_reads_then_mfma();
+    if (HAS1) {
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(HAS2 ? kWaitSteady : 0));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(sa1, sb1, 0, fa0, fb0);
     }
+    mfma_block(fa1, fb1, T3{});
+    if (HAS2) issue_g2l(1, kt + 2, sa, 0, B_LD / 2);
+    order_phase();
     __builtin_amdgcn_sched_barrier(0);
     if (HAS1) canon_scales();
-    if (HAS2) load_scales(kt_begin + it + 2);
+    if (HAS2) load_scales(kt + 2);
     __builtin_amdgcn_sched_barrier(0);
   };
-  int it = 0;
-  for (; it < nkt - 2; ++it) k_tile(it, std::true_type{}, std::true_type{});
-  if (it < nkt - 1) {
-    k_tile(it, std::true_type{}, std::false_type{});
-    ++it;
+  int j = 0, sa = 0;
+  for (; j < nkt - 2; ++j) {
+    const int sb = sa + 1 >= RING ? 0 : sa + 1;
+    k_tile(j, sa, sb, std::true_type{}, std::true_type{});
+    sa = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
   }
-  k_tile(it, std::false_type{}, std::false_type{});
+  if (j < nkt - 1) {
+    const int sb = sa + 1 >= RING ? 0 : sa + 1;
+    k_tile(j, sa, sb, std::true_type{}, std::false_type{});
+    sa = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
+    ++j;
+  }
+  {
+    const int sb = sa + 1 >= RING ? 0 : sa + 1;
+    k_tile(j, sa, sb, std::false_type{}, std::false_type{});
+  }
 
   // ---------------- epilogue ----------------
-  // acc[i][j][4q + e]: M row = lane%32, N column = 8q + 4*(lane/32) + e.
+  // acc[i][jn][4q + e]: M row = lane%32, N column = 8q + 4*(lane/32) + e of the
+  // 32x32 tile (i, jn).  Storing that directly would touch 32 cache lines per
+  // store instruction with 8-16 bytes each; instead every wave transposes its
+  // sub-tile through its own share of LDS (the ring is no longer needed) and
+  // writes whole rows: 16 bytes per lane, full 128-byte lines.
   const int64_t ldc = p.n;
-  const bool vec_ok = (p.n & 3) == 0;
+  const bool to_partial = p.partial != nullptr;
+  const bool out_bf16 = !to_partial && p.out_bf16;
+  const int wm0 = m0 + wave_m * Cfg::WM, wn0 = n0 + wave_n * Cfg::WN;
+  const int align_elems = out_bf16 ? 8 : 4;
+  if ((p.n % align_elems) == 0) {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+    __builtin_amdgcn_s_barrier();  // every wave is done reading the ring
+    asm volatile("" ::: "memory");
+    uint8_t *stage = smem + wave * (Cfg::LDS_BYTES / NWAVES);
+    if (out_bf16) {
+      // [WM rows][WN bf16] with rows padded by 8 bytes (bank spread of the b64 writes)
+      constexpr int ROWB = Cfg::WN * 2 + 8;
+      static_assert(Cfg::WM * ROWB <= Cfg::LDS_BYTES / NWAVES, "bf16 staging does not fit");
+      typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i)
+#pragma unroll
+        for (int jn = 0; jn < MT_N; ++jn)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const bf4 h = {(__bf16)acc[i][jn][4 * q], (__bf16)acc[i][jn][4 * q + 1], (__bf16)acc[i][jn][4 * q + 2],
+                           (__bf16)acc[i][jn][4 * q + 3]};
+            *(bf4 *)(stage + (i * 32 + fr) * ROWB + (jn * 32 + q * 8 + fg * 4) * 2) = h;
+          }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));
+      constexpr int LPR = Cfg::WN * 2 / 16;  // lanes per row
+      constexpr int RPI = 64 / LPR;          // rows per store instruction
+      const int lr = lane / LPR, lc = lane % LPR;
+      __bf16 *cbase = (__bf16 *)p.c;
+#pragma unroll
+      for (int r0 = 0; r0 < Cfg::WM; r0 += RPI) {
+        const int r = r0 + lr, m = wm0 + r, n = wn0 + lc * 8;
+        const v4i v = *(const v4i *)(stage + r * ROWB + lc * 16);
+        if (m < row_end && n < p.n) *(v4i *)(cbase + (int64_t)m * ldc + n) = v;
+      }
+    } else {
+      // f32: two passes of WM/2 rows, [WM/2 rows][WN f32] padded by 16 bytes
+      constexpr int ROWB = Cfg::WN * 4 + 16;
+      constexpr int HALF_M = MT_M > 1 ? MT_M / 2 : 1;
+      constexpr int PASSES = MT_M / HALF_M;
+      static_assert(HALF_M * 32 * ROWB <= Cfg::LDS_BYTES / NWAVES, "f32 staging does not fit");
+      float *cbase = to_partial ? p.partial + (int64_t)split * p.m * ldc : (float *)p.c;
+      constexpr int LPR = Cfg::WN * 4 / 16;
+      constexpr int RPI = 64 / LPR;
+      const int lr = lane / LPR, lc = lane % LPR;
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) {
+        if (ps > 0) {
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));  // previous pass's LDS reads are done
+        }
+#pragma unroll
+        for (int ih = 0; ih < HALF_M; ++ih)
+#pragma unroll
+          for (int jn = 0; jn < MT_N; ++jn)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int i = ps * HALF_M + ih;
+              const v4f v = {acc[i][jn][4 * q], acc[i][jn][4 * q + 1], acc[i][jn][4 * q + 2], acc[i][jn][4 * q + 3]};
+              *(v4f *)(stage + (ih * 32 + fr) * ROWB + (jn * 32 + q * 8 + fg * 4) * 4) = v;
+            }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));
+#pragma unroll
+        for (int r0 = 0; r0 < HALF_M * 32; r0 += RPI) {
+          const int r = r0 + lr, m = wm0 + ps * HALF_M * 32 + r, n = wn0 + lc * 4;
+          const v4f v = *(const v4f *)(stage + r * ROWB + lc * 16);
+          if (m < row_end && n < p.n) *(v4f *)(cbase + (int64_t)m * ldc + n) = v;
+        }
+      }
+    }
+    return;
+  }
+  // N not a multiple of the vector width: element-wise stores straight from
+  // the accumulators.
 #pragma unroll
   for (int i = 0; i < MT_M; ++i) {
-    const int m = m0 + wave_m * Cfg::WM + i * 32 + fr;
+    const int m = wm0 + i * 32 + fr;
     if (m >= row_end) continue;
 #pragma unroll
-    for (int j = 0; j < MT_N; ++j) {
+    for (int jn = 0; jn < MT_N; ++jn) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wave_n * Cfg::WN + j * 32 + q * 8 + fg * 4;
+        const int n = wn0 + jn * 32 + q * 8 + fg * 4;
         if (n >= p.n) continue;
-        const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
         const int64_t idx = (int64_t)m * ldc + n;
-        if (p.partial != nullptr) {
-          float *dst = p.partial + (int64_t)split * p.m * ldc + idx;
-          if (vec_ok) {
-            *(v4f *)dst = v;
-          } else {
-            for (int r = 0; r < 4 && n + r < p.n; ++r) dst[r] = v[r];
-          }
-        } else if (p.out_bf16) {
-          __bf16 *dst = (__bf16 *)p.c + idx;
-          if (vec_ok) {
-            typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
-            const bf4 h = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-            *(bf4 *)dst = h;
-          } else {
-            for (int r = 0; r < 4 && n + r < p.n; ++r) dst[r] = (__bf16)v[r];
-          }
-        } else {
-          float *dst = (float *)p.c + idx;
-          if (vec_ok) {
-            *(v4f *)dst = v;
-          } else {
-            for (int r = 0; r < 4 && n + r < p.n; ++r) dst[r] = v[r];
-          }
+        for (int r = 0; r < 4 && n + r < p.n; ++r) {
+          const float v = acc[i][jn][4 * q + r];
+          if (to_partial)
+            p.partial[(int64_t)split * p.m * ldc + idx + r] = v;
+          else if (out_bf16)
+            ((__bf16 *)p.c)[idx + r] = (__bf16)v;
+          else
+            ((float *)p.c)[idx + r] = v;
         }
       }
     }
   }
+}
+
+template <class Cfg, int MODE>
+__global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams p) {
+  tile_gemm_body<Cfg, MODE>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -451,25 +609,21 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
 typedef TileCfg<256, 256, 2, 2> Cfg256x256w4;
 typedef TileCfg<256, 256, 4, 2> Cfg256x256w8;
 typedef TileCfg<128, 128, 2, 2> Cfg128x128w4;
-typedef TileCfg<256, 128, 2, 2> Cfg256x128w4;
-typedef TileCfg<128, 256, 2, 2> Cfg128x256w4;
 
 void tile_variant_shape(int variant, int *bm, int *bn) {
   switch (variant) {
     case WAVE_MXFP4_VARIANT_T256x256_W2x2:
     case WAVE_MXFP4_VARIANT_T256x256_W4x2: *bm = 256; *bn = 256; break;
     case WAVE_MXFP4_VARIANT_T128x128_W2x2: *bm = 128; *bn = 128; break;
-    case WAVE_MXFP4_VARIANT_T256x128_W2x2: *bm = 256; *bn = 128; break;
-    case WAVE_MXFP4_VARIANT_T128x256_W2x2: *bm = 128; *bn = 256; break;
     default: *bm = 0; *bn = 0; break;
   }
 }
 
-template <class Cfg, bool GENERIC_K>
+template <class Cfg, int MODE>
 static hipError_t launch_cfg(const GemmParams &p, hipStream_t stream) {
   static bool attr_done = false;  // benign race: the attribute is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)tile_gemm_kernel<Cfg, GENERIC_K>,
+    hipError_t e = hipFuncSetAttribute((const void *)tile_gemm_kernel<Cfg, MODE>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
@@ -477,21 +631,26 @@ static hipError_t launch_cfg(const GemmParams &p, hipStream_t stream) {
   const int total = p.tiles_m * p.tiles_n;
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
   dim3 grid(per_xcd * kNumXcd, p.splits, 1);
-  tile_gemm_kernel<Cfg, GENERIC_K><<<grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  tile_gemm_kernel<Cfg, MODE><<<grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
   return hipGetLastError();
+}
+
+template <class Cfg>
+static hipError_t launch_by_scales(const GemmParams &p, hipStream_t stream) {
+  const bool native =
+      p.a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+  return native ? launch_cfg<Cfg, kNative>(p, stream) : launch_cfg<Cfg, kDirect>(p, stream);
 }
 
 // K % 256 != 0 (partial last K tile, scale rows that are not 8-byte multiples)
 // is served by one extra instantiation of the 128x128 kernel; the caller maps
-// every tile variant onto it for such K (see tile_variant_shape_for_k).
+// every tile variant onto it for such K.
 hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream) {
-  if ((p.k & (kTileK - 1)) != 0) return launch_cfg<Cfg128x128w4, true>(p, stream);
+  if ((p.k & (kTileK - 1)) != 0) return launch_cfg<Cfg128x128w4, kGenericK>(p, stream);
   switch (variant) {
-    case WAVE_MXFP4_VARIANT_T256x256_W2x2: return launch_cfg<Cfg256x256w4, false>(p, stream);
-    case WAVE_MXFP4_VARIANT_T256x256_W4x2: return launch_cfg<Cfg256x256w8, false>(p, stream);
-    case WAVE_MXFP4_VARIANT_T128x128_W2x2: return launch_cfg<Cfg128x128w4, false>(p, stream);
-    case WAVE_MXFP4_VARIANT_T256x128_W2x2: return launch_cfg<Cfg256x128w4, false>(p, stream);
-    case WAVE_MXFP4_VARIANT_T128x256_W2x2: return launch_cfg<Cfg128x256w4, false>(p, stream);
+    case WAVE_MXFP4_VARIANT_T256x256_W2x2: return launch_by_scales<Cfg256x256w4>(p, stream);
+    case WAVE_MXFP4_VARIANT_T256x256_W4x2: return launch_by_scales<Cfg256x256w8>(p, stream);
+    case WAVE_MXFP4_VARIANT_T128x128_W2x2: return launch_by_scales<Cfg128x128w4>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }

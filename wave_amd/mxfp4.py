@@ -55,12 +55,31 @@ def workspace_bytes(m: int, n: int, k: int, split_k: int = 0, variant: int = _li
     return int(_lib.load().wave_mxfp4_workspace_bytes(m, n, k, split_k, variant))
 
 
+# One scratch buffer per (device, stream), grown on demand: the split-K partial
+# sums and the re-laid-out scales of a call live there.  Calls on one stream are
+# ordered, so they can share it; different streams get different buffers.
+_scratch: dict = {}
+
+
+def _workspace(device, nbytes: int):
+    if nbytes == 0:
+        return None
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    buf = _scratch.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _scratch[key] = buf
+    return buf
+
+
 def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,
                b_scale_layout=_lib.SCALE_ROW_MAJOR, b_layout=_lib.B_ROW_MAJOR, split_k=1,
                variant=_lib.VARIANT_AUTO, workspace=None) -> None:
     """``out[M, N] = dequant(x[M, K/2]) @ dequant(w_t[N, K/2]).T`` in place.
     Same arguments, in the same order, as the reference's compiled kernel
-    (tests/kernel/wave_gemm_mxfp_test.py:194-201)."""
+    (tests/kernel/wave_gemm_mxfp_test.py:194-201).  ``workspace`` is an optional
+    uint8 GPU tensor of ``workspace_bytes(...)`` bytes; by default a buffer cached
+    per device and stream is used, ``False`` runs without scratch."""
     lib = _lib.load()
     x = _as_u8(x, "x")
     w_t = _as_u8(w_t, "w_t")
@@ -80,12 +99,12 @@ def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW
     _scale_rows_ok(w_scales, n, ks, b_scale_layout, "w_scales")
     od = _check_out(out, (m, n))
     ws_ptr, ws_bytes = None, 0
-    if split_k != 1:
-        need = workspace_bytes(m, n, k, split_k, variant)
-        if need:
-            if workspace is None:
-                workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
-            ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    if workspace is None:
+        workspace = _workspace(x.device, workspace_bytes(m, n, k, split_k, variant))
+    elif workspace is False:  # run without scratch: scales are read in the layout given
+        workspace = None
+    if workspace is not None:
+        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     with torch.cuda.device(x.device):
         st = lib.wave_mxfp4_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
                                  out.data_ptr(), m, n, k, od, a_scale_layout, b_scale_layout, b_layout,
@@ -176,6 +195,24 @@ def dequant(x: torch.Tensor, scales: torch.Tensor, scale_layout=_lib.SCALE_ROW_M
         st = lib.wave_mxfp4_dequant(x.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, k, scale_layout,
                                     _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp4_dequant")
+    return out
+
+
+def scale_convert(scale: torch.Tensor, rows: int, ks: int, src_layout: int, dst_layout: int) -> torch.Tensor:
+    """Re-lays a scale tensor of the logical shape ``[rows, ks]`` out from one
+    layout to another on the GPU.  Row-major results are ``[rows, ks]``; the
+    others the padded ``[ceil(rows/32)*32, ceil(ks/8)*8]`` buffer."""
+    lib = _lib.load()
+    scale = _as_u8(scale, "scale")
+    _scale_rows_ok(scale, rows, ks, src_layout, "scale")
+    if dst_layout == _lib.SCALE_ROW_MAJOR:
+        out = torch.empty(rows, ks, dtype=torch.uint8, device=scale.device)
+    else:
+        out = torch.empty((rows + 31) // 32 * 32, (ks + 7) // 8 * 8, dtype=torch.uint8, device=scale.device)
+    with torch.cuda.device(scale.device):
+        st = lib.wave_mxfp4_scale_convert(scale.data_ptr(), src_layout, out.data_ptr(), dst_layout, rows, ks,
+                                          _stream_ptr(scale.device))
+    _lib.check(st, "wave_mxfp4_scale_convert")
     return out
 
 

@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
+# WAVE_MXFP4_LIB points at another build of the same ABI (e.g. an experiment)
+LIB_PATH = os.environ.get("WAVE_MXFP4_LIB") or os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
 ABI_VERSION = 2
 

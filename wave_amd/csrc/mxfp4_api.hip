@@ -72,6 +72,19 @@ int pick_tile_variant(int64_t m, int64_t n) {
   return WAVE_MXFP4_VARIANT_T128x128_W2x2;
 }
 
+// CUs of the current device (cached per device ordinal).
+int device_cus() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    cached[dev] = cus;
+  }
+  return cached[dev];
+}
+
 bool is_tile_variant(int v) {
   int bm, bn;
   tile_variant_shape(v, &bm, &bn);
@@ -90,6 +103,14 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
 // Split the library takes by itself for a tile kernel: only when the tile
 // grid leaves most of the 256 CUs idle and K is long.
 int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
+  if (variant == WAVE_MXFP4_VARIANT_SKINNY) {
+    // split K so that each workgroup's range fits the streaming kernel's resident A
+    const int64_t k_tiles = (k + kTileK - 1) / kTileK, cap = stream_max_k_tiles();
+    if (k_tiles <= cap || k % kTileK != 0) return 1;
+    int s = (int)((k_tiles + cap - 1) / cap);
+    while (s <= 16 && k_tiles % s != 0) ++s;
+    return s <= 16 ? s : 1;
+  }
   int bm, bn;
   tile_variant_shape(variant, &bm, &bn);
   if (bm == 0 || k % kTileK != 0) return 1;
@@ -226,7 +247,11 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (v == WAVE_MXFP4_VARIANT_NAIVE) {
     e = launch_naive_gemm(p, stream);
   } else if (v == WAVE_MXFP4_VARIANT_SKINNY) {
-    e = launch_skinny_gemm(p, stream);
+    // The streaming kernel keeps A in registers and serves up to 32 K tiles per
+    // workgroup; a longer K range without a split goes to the direct kernel.
+    e = p.tiles_per_split <= stream_max_k_tiles() ? launch_stream_gemm(p, device_cus(), stream)
+                                                  : hipErrorInvalidValue;
+    if (e == hipErrorInvalidValue) e = launch_skinny_gemm(p, stream);
   } else {
     int bm, bn;
     tile_variant_shape(v, &bm, &bn);

@@ -106,6 +106,8 @@ __device__ __host__ __forceinline__ int64_t b_preshuffle_offset(int64_t n, int64
 // ---- launchers (defined in the .hip files, called from the C ABI) ----
 hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream);
 hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);
+hipError_t launch_stream_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
+int stream_max_k_tiles();
 hipError_t launch_naive_gemm(const GemmParams &p, hipStream_t stream);
 hipError_t launch_splitk_reduce(const float *partial, void *c, int64_t mn, int splits, int out_bf16,
                                 hipStream_t stream);

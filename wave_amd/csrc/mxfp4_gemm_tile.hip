@@ -345,12 +345,23 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   auto canon_scales = [&]() {
     const bool a_bytes = GENERIC_K && (p.ks & 7) != 0 && p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
     const bool b_bytes = GENERIC_K && (p.ks & 7) != 0 && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
+    if (NATIVE) {
+      // A real register move, pinned here: if the copy were left to the
+      // compiler it would be folded into the loop's phi, the next scale load
+      // (issued right after) could then not reuse this register, and the copy
+      // it needs instead would wait for that load at the top of every iteration.
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_a[i]) : "v"(raw_a[i][0]));
+#pragma unroll
+      for (int j = 0; j < MT_N; ++j) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_b[j]) : "v"(raw_b[j][0]));
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < MT_M; ++i)
-      sc_a[i] = (NATIVE || a_bytes) ? raw_a[i][0] : perm_bytes(raw_a[i][1], raw_a[i][0], a_ssel[i]);
+      sc_a[i] = a_bytes ? raw_a[i][0] : perm_bytes(raw_a[i][1], raw_a[i][0], a_ssel[i]);
 #pragma unroll
     for (int j = 0; j < MT_N; ++j)
-      sc_b[j] = (NATIVE || b_bytes) ? raw_b[j][0] : perm_bytes(raw_b[j][1], raw_b[j][0], b_ssel[j]);
+      sc_b[j] = b_bytes ? raw_b[j][0] : perm_bytes(raw_b[j][1], raw_b[j][0], b_ssel[j]);
   };
 
   // ---------------- accumulators ----------------

@@ -4,21 +4,26 @@
 // N*K/2 bytes), so the kernel is organised around the memory system:
 //
 // * B goes global -> LDS with 16-byte-per-lane DMA (buffer_load ... lds), one
-//   instruction = 8 rows x 128 bytes = 8 whole cache lines.  (Loading MFMA
-//   fragments straight from global touches 16 half lines per instruction and
-//   the vector L1 retires lines, not bytes: that path tops out near 2.5 TB/s.)
-//   DMA costs no VGPRs, so every wave keeps a private ring of 8 K tiles
-//   (16 rows x 256 elements = 2 KB each) in flight: 64 KB per CU.
+//   instruction = 1 KB contiguous of one B row = 8 whole cache lines.  (Loading
+//   MFMA fragments straight from global touches 16 half lines per instruction
+//   and the vector L1 retires lines, not bytes: that path tops out near
+//   2.5 TB/s.)  DMA costs no VGPRs.
 // * A (the few activation rows) is loaded ONCE per workgroup into registers in
 //   MFMA fragment layout: each of the 4 waves owns a quarter of the workgroup's
 //   K range (at most 8 K tiles = 64 VGPRs per 16 rows of A) and streams only
-//   that quarter of every B row.  The waves never wait for each other inside
-//   the stream; their four partial 16x16 tiles are added through LDS once per
-//   16 rows of B.
+//   that quarter of every B row.
+// * Every wave runs a private three-deep pipeline over 16-row B tiles: two
+//   tiles live in its LDS buffers and, as soon as a tile has landed, all of its
+//   fragments are pulled into registers, which frees the buffer for the DMA of
+//   the tile after next BEFORE the MFMAs run.  Two tiles (32 KB per wave,
+//   128 KB per CU) are therefore always in flight; waiting is by counted
+//   vmcnt, never for an empty queue.  The waves meet only to add their four
+//   partial 16x16 tiles through LDS, once per 16 rows of B.
 // * A workgroup walks a contiguous range of 16-row B tiles, so the grid is one
 //   workgroup per CU and all CUs pull from HBM for the whole kernel.
 // * B's scales for a 16-row tile and the wave's K quarter travel by the same
-//   DMA (2 KB per tile, any layout) and are picked out of LDS per lane.
+//   DMA (1 KB per tile, 2 KB for the e8m0_shuffle layout whose 32-row blocks
+//   interleave both halves) and are picked out of LDS per lane with v_perm.
 //
 // v_mfma_scale_f32_16x16x128_f8f6f4 is used (16 rows of B per tile balances
 // N = 28672 over 256 CUs; MFMA rate is irrelevant here).  Operand order is
@@ -38,18 +43,29 @@ constexpr int kStreamMaxKTiles = kStreamWaves * kStreamKtPerWave;  // per workgr
 constexpr int kStreamRowBytes = kStreamKtPerWave * kTileKBytes;    // 1 KB of one B row per DMA instruction
 constexpr int kStreamRowPitch = kStreamRowBytes + 16;              // LDS pitch: 16 rows spread over all banks
 constexpr int kStreamTileBytes = 16 * kStreamRowPitch;             // one 16-row B tile, one wave's K range
-constexpr int kStreamScaleBytes = 2048;                            // its scale image
+constexpr int kStreamScaleBytes = 2048;                            // its scale image (1 KB used by two layouts)
 
 int stream_max_k_tiles() { return kStreamMaxKTiles; }
 
 struct StreamLds {
-  uint8_t tile[kStreamWaves][2][kStreamTileBytes];     // double-buffered per wave
+  uint8_t tile[kStreamWaves][2][kStreamTileBytes];  // two tiles per wave
   uint8_t scales[kStreamWaves][2][kStreamScaleBytes];
-  float red[kStreamWaves - 1][4][64][4];               // partial 16x16 tiles of waves 1..3
+  float red[kStreamWaves - 1][4][64][4];            // partial 16x16 tiles of waves 1..3
 };
 static_assert(sizeof(StreamLds) <= 160 * 1024, "stream kernel LDS");
 
-template <int MT_M>
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vm[3:0], exp[6:4], lgkm[11:8], vm[15:14])
+template <int N>
+__device__ __forceinline__ void stream_wait_vm() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// FULL: every wave owns exactly 8 whole K tiles and the scale rows are whole
+// 16-byte pieces, so every B tile costs the same number of DMA instructions,
+// nothing is predicated and waits can be counted.  Otherwise (K tails, fewer
+// K tiles) the same pipeline runs with predicated loads and full waits.
+template <int MT_M, bool FULL>
 __device__ __forceinline__ void stream_body(const GemmParams &p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
   StreamLds &lds = *reinterpret_cast<StreamLds *>(smem_raw);
@@ -66,14 +82,57 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const int split = blockIdx.y;
   const int kt_begin = split * p.tiles_per_split;
   const int nkt = min(p.k_tiles, kt_begin + p.tiles_per_split) - kt_begin;
-  const int ktw = (nkt + kStreamWaves - 1) / kStreamWaves;  // <= kStreamKtPerWave
+  const int ktw = FULL ? kStreamKtPerWave : (nkt + kStreamWaves - 1) / kStreamWaves;  // <= kStreamKtPerWave
   const int kt0 = kt_begin + wave * ktw;
-  const int my_nkt = max(0, min(ktw, kt_begin + nkt - kt0));
+  const int my_nkt = FULL ? kStreamKtPerWave : max(0, min(ktw, kt_begin + nkt - kt0));
 
   const int kp = p.kp;
   const v4i zero = {0, 0, 0, 0};
-  const int tail_chunks = (p.k & (kTileK - 1)) >> 5;  // valid chunks of a partial last K tile
-  auto chunk_ok = [&](int kt, int chunk) { return tail_chunks == 0 || kt != p.k_tiles - 1 || chunk < tail_chunks; };
+  const int tail_chunks = FULL ? 0 : (p.k & (kTileK - 1)) >> 5;  // valid chunks of a partial last K tile
+  auto chunk_ok = [&](int kt, int chunk) {
+    return FULL || tail_chunks == 0 || kt != p.k_tiles - 1 || chunk < tail_chunks;
+  };
+
+  // ---- A: resident fragments and scales; issued first, they land under the first B tiles ----
+  v4i a_frag[MT_M][kStreamKtPerWave][2];
+  // Scale bytes stay in the registers they were loaded into (byte 0, op_sel 0):
+  // combining them would be a use of loaded data in front of the stream, and
+  // with DMA and ordinary loads both pending the compiler waits for vmcnt(0)
+  // at such a use.
+  // All vector memory traffic of the kernel is buffer instructions: with a
+  // global_load ... lds pending the compiler treats the queue as unordered.
+  uint32_t a_sc[MT_M][kStreamKtPerWave][2];
+  const __amdgpu_buffer_rsrc_t a_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a), 0, 0x7FFFFFFF, 0x00020000);
+  const __amdgpu_buffer_rsrc_t as_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a_scale), 0, 0x7FFFFFFF, 0x00020000);
+  auto load_b128 = [&](__amdgpu_buffer_rsrc_t r, int voff, int soff) -> v4i {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const u4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+    return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+  };
+#pragma unroll
+  for (int i = 0; i < MT_M; ++i) {
+    const int row = min(i * 16 + fr, p.m - 1);
+    const int ao = row * kp + fg * 16;
+    // scale (row, group kt*8 + s*4 + fg): every layout is linear in kt
+    const int so0 = (int)scale_offset(p.a_scale_layout, row, fg, p.ks, p.ksp);
+    const int so1 = (int)scale_offset(p.a_scale_layout, row, 4 + fg, p.ks, p.ksp);
+    const int so_kt = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR ? 8 : 256;
+#pragma unroll
+    for (int j = 0; j < kStreamKtPerWave; ++j) {
+      a_frag[i][j][0] = a_frag[i][j][1] = zero;
+      a_sc[i][j][0] = a_sc[i][j][1] = 127u;
+      if (j < my_nkt) {
+        const int kt = kt0 + j;
+        if (chunk_ok(kt, fg)) a_frag[i][j][0] = load_b128(a_rsrc, ao, kt * kTileKBytes);
+        if (chunk_ok(kt, 4 + fg)) a_frag[i][j][1] = load_b128(a_rsrc, ao, kt * kTileKBytes + 64);
+        if (FULL || kt * 8 + fg < p.ks) a_sc[i][j][0] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so0, kt * so_kt, 0);
+        if (FULL || kt * 8 + 4 + fg < p.ks)
+          a_sc[i][j][1] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so1, kt * so_kt, 0);
+      }
+    }
+  }
 
   // ---- B data DMA: one instruction = up to 1 KB contiguous ----
   //   row-major   : row r of the tile, K tiles kt0 .. kt0+7 (lane t: K tile t/8, chunk t%8),
@@ -85,13 +144,22 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const bool bpre = p.b_preshuffled != 0;
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t *>(p.b + (int64_t)nt_begin * 16 * kp), 0, 0x7FFFFFFF, 0x00020000);
-  auto issue_rows = [&](int nt, int buf, int i0, int i1) {
+  auto issue_rows = [&](int nt, int buf) {
     uint8_t *dst = lds.tile[wave][buf];
     const int tile_off = (nt - nt_begin) * 16 * kp;
     const int row_lim = p.n - 1 - nt * 16;
+    if (FULL) {
+      // one instruction per i, no control flow: the two layouts differ in scalars only
+      const int pitch = bpre ? 1024 : kStreamRowPitch;
 #pragma unroll
-    for (int i = i0; i < i1; ++i) {
-      if (bpre) {
+      for (int i = 0; i < 16; ++i) {
+        const int soff = bpre ? tile_off + ((kt0 + (i >> 1)) * 4 + (i & 1) * 2) * 512
+                              : tile_off + min(i, row_lim) * kp + kt0 * kTileKBytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * pitch), 16, lane * 16, soff, 0, 0);
+      }
+    } else if (bpre) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
         const int j = i >> 1, s = i & 1;
         if (j < my_nkt) {
           if (chunk_ok(kt0 + j, s * 4 + fg))
@@ -100,10 +168,12 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
           else
             *(v4i *)(dst + i * 1024 + lane * 16) = zero;
         }
-      } else {
-        const int j = lane >> 3;
-        if (j < my_nkt) {
-          if (chunk_ok(kt0 + j, lane & 7))
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if ((lane >> 3) < my_nkt) {
+          if (chunk_ok(kt0 + (lane >> 3), lane & 7))
             __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * kStreamRowPitch), 16, lane * 16,
                                                      tile_off + min(i, row_lim) * kp + kt0 * kTileKBytes, 0, 0);
           else
@@ -116,83 +186,110 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const uint32_t frag_j = bpre ? 2048u : (uint32_t)kTileKBytes;  // per K tile
   const uint32_t frag_s = bpre ? 1024u : 64u;                    // per K step
 
-  // ---- B scales: a 2 KB image of the source bytes per B tile ----
-  //   row-major : 16 rows x 128 bytes starting at group kt0*8 (lane t -> row t/8, piece t%8)
-  //   shuffled / MFMA32 : the 8 consecutive 256-byte blocks (32-row tile, kt0 .. kt0+7)
-  // and, per lane, where its two bytes of K tile j sit in that image.
+  // ---- B scales: an image of the source bytes per B tile and wave ----
+  //   row-major : 16 rows x 64 bytes starting at group kt0*8 (lane t -> row t/4, piece t%4);
+  //               K tile j, step s of row fr is byte fg of the dword at fr*64 + j*8 + s*4.
+  //   MFMA32    : of each of the 8 consecutive 256-byte blocks (32 rows x one K tile) the two
+  //               64-byte runs that hold this tile's 16 rows (lane t -> block t/8, piece t%8);
+  //               K tile j of row r is the dword at j*128 + (fg&1)*64 + (r%16)*4, whose bytes
+  //               are (step 0, fg/2 = 0), (0, 1), (1, 0), (1, 1).
+  //   shuffled  : the 8 whole blocks (both 16-row halves share every dword): K tile j of row r
+  //               is the dword at j*256 + fg*64 + (r%16)*4, bytes (step 0, half 0), (0, 1),
+  //               (1, 0), (1, 1) with half = (r/16)%2.
+  // One v_perm per K tile then forms the MFMA scale operand (step 0 in byte 0, step 1 in byte 1).
   const int bsl = p.b_scale_layout;
-  const int64_t sc_block_row_bytes = (int64_t)(p.ksp >> 3) * 256;  // one 32-row tile, all K tiles
-  auto scale_byte_off = [&](int n_row, int s) -> int {              // offset for K tile 0 of the image
-    if (bsl == WAVE_MXFP4_SCALE_ROW_MAJOR) return fr * 128 + s * 4 + fg;
-    if (bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) return fg * 64 + (n_row & 15) * 4 + s * 2 + ((n_row >> 4) & 1);
-    return (((fg & 1) << 5) | (n_row & 31)) * 4 + s * 2 + (fg >> 1);
-  };
-  const int sc_kt_stride = bsl == WAVE_MXFP4_SCALE_ROW_MAJOR ? 8 : 256;
-
+  const int sc_block_row_bytes = (p.ksp >> 3) * 256;  // one 32-row tile, all K tiles
+  const bool sc_pieces = (p.ks & 15) == 0;
+  const __amdgpu_buffer_rsrc_t bs_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.b_scale), 0, 0x7FFFFFFF, 0x00020000);
   auto issue_scales = [&](int nt, int buf) {
     uint8_t *dst = lds.scales[wave][buf];
     const int n0 = nt * 16;
-    if (bsl == WAVE_MXFP4_SCALE_ROW_MAJOR) {
-#pragma unroll
-      for (int d = 0; d < 2; ++d) {
-        const int row = min(n0 + d * 8 + (lane >> 3), p.n - 1);
-        const int64_t off = (int64_t)row * p.ks + (int64_t)kt0 * 8 + (lane & 7) * 16;
-        // 16-byte pieces past the end of the scale matrix are not read (their groups are past K)
-        if ((p.ks & 15) == 0 && off + 16 <= (int64_t)p.n * p.ks) {
-          __builtin_amdgcn_global_load_lds(WAVE_GLOBAL_PTR(p.b_scale + off), WAVE_LDS_PTR(dst + d * 1024), 16, 0, 0);
-        } else {
-          // rows that are not 16-byte multiples: byte copies of the groups that exist
-          uint8_t *d8 = dst + d * 1024 + lane * 16;
-          for (int e = 0; e < 16; ++e) {
-            const int g = kt0 * 8 + (lane & 7) * 16 + e;
-            d8[e] = g < p.ks ? p.b_scale[(int64_t)row * p.ks + g] : (uint8_t)127;
-          }
+    const int blocked_off = (n0 >> 5) * sc_block_row_bytes + kt0 * 256;
+    if (FULL) {
+      // one instruction whatever the layout, a second one for the shuffled blocks
+      const int row = min(n0 + (lane >> 2), p.n - 1);
+      const int off_rm = row * p.ks + kt0 * 8 + (lane & 3) * 16;
+      const int off_native = blocked_off + (lane >> 3) * 256 + ((lane & 7) >> 2) * 128 + ((n0 >> 4) & 1) * 64 +
+                             (lane & 3) * 16;
+      const int off_shuf = blocked_off + lane * 16;
+      const int off = bsl == WAVE_MXFP4_SCALE_ROW_MAJOR ? off_rm : bsl == WAVE_MXFP4_SCALE_MFMA32 ? off_native : off_shuf;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, off, 0, 0, 0);
+      if (bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst + 1024), 16, off, 1024, 0, 0);
+    } else if (bsl == WAVE_MXFP4_SCALE_ROW_MAJOR) {
+      const int row = min(n0 + (lane >> 2), p.n - 1);
+      const int64_t off = (int64_t)row * p.ks + (int64_t)kt0 * 8 + (lane & 3) * 16;
+      if (sc_pieces && off + 16 <= (int64_t)p.n * p.ks) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, (int)off, 0, 0, 0);
+      } else {
+        // rows that are not 16-byte multiples: byte copies of the groups that exist
+        uint8_t *d8 = dst + lane * 16;
+        for (int e = 0; e < 16; ++e) {
+          const int g = kt0 * 8 + (lane & 3) * 16 + e;
+          d8[e] = g < p.ks ? p.b_scale[(int64_t)row * p.ks + g] : (uint8_t)127;
         }
       }
+    } else if (bsl == WAVE_MXFP4_SCALE_MFMA32) {
+      const int blk = lane >> 3, piece = lane & 7;
+      const int off = blocked_off + blk * 256 + (piece >> 2) * 128 + ((n0 >> 4) & 1) * 64 + (piece & 3) * 16;
+      if (kt0 + blk < p.k_tiles) __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, off, 0, 0, 0);
     } else {
-      // blocks (n0/32, kt0 + t/16), 16-byte piece t%16; blocks past the last K tile are not read
-      const uint8_t *src = p.b_scale + (int64_t)(n0 >> 5) * sc_block_row_bytes + (int64_t)kt0 * 256;
+      const int off = blocked_off + lane * 16;
 #pragma unroll
       for (int d = 0; d < 2; ++d) {
         const int blk = d * 4 + (lane >> 4);
         if (kt0 + blk < p.k_tiles)
-          __builtin_amdgcn_global_load_lds(WAVE_GLOBAL_PTR(src + d * 1024 + lane * 16), WAVE_LDS_PTR(dst + d * 1024),
-                                           16, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst + d * 1024), 16, off, d * 1024, 0, 0);
       }
     }
   };
+  // per-lane position in the image and byte selector for v_perm (0x0c = constant zero byte)
+  const bool sc_rowmajor = bsl == WAVE_MXFP4_SCALE_ROW_MAJOR;
 
-  // first B tile in flight before anything else
-  if (my_nkt > 0) {
-    issue_scales(nt_begin, 0);
-    issue_rows(nt_begin, 0, 0, 16);
-  }
+  auto issue_tile = [&](int nt, int buf) {
+    if (FULL || my_nkt > 0) {
+      issue_scales(nt, buf);
+      issue_rows(nt, buf);
+    }
+  };
 
-  // ---- A: resident fragments and scales (loaded while the first B tile is in flight) ----
-  v4i a_frag[MT_M][kStreamKtPerWave][2];
-  uint32_t a_sc[MT_M][kStreamKtPerWave];
+  // two B tiles in flight from the start (FULL mode is only launched with at
+  // least two tiles per workgroup, which keeps this prologue branch-free)
+  issue_tile(nt_begin, 0);
+  if (FULL || nt_begin + 1 < nt_end) issue_tile(nt_begin + 1, 1);
+
+  // Wait until tile nt has landed; tile nt+1 stays in flight.  In FULL mode a
+  // tile is 17 DMA instructions (18 with e8m0_shuffle scales, whose first then
+  // falls under the wait as well), and the youngest in the queue are those of
+  // tile nt+1.
+  auto wait_tile = [&](int nt) {
+    if (FULL && nt + 1 < nt_end) {
+      stream_wait_vm<17>();
+    } else {
+      __builtin_amdgcn_s_waitcnt(0);
+    }
+    asm volatile("" ::: "memory");
+  };
+  // A is older than both tiles, so it has landed with the first of them.  Its
+  // registers are pinned behind this wait, so that no use of them can be
+  // hoisted in front of it (where the compiler would add its own wait).
+  if (FULL) {
+    stream_wait_vm<17>();
+    asm volatile("" ::: "memory");
 #pragma unroll
-  for (int i = 0; i < MT_M; ++i) {
-    const int row = min(i * 16 + fr, p.m - 1);
-    const uint8_t *ap = p.a + (int64_t)row * kp + fg * 16;
+    for (int i = 0; i < MT_M; ++i) {
 #pragma unroll
-    for (int j = 0; j < kStreamKtPerWave; ++j) {
-      a_frag[i][j][0] = a_frag[i][j][1] = zero;
-      a_sc[i][j] = 0x7F7Fu;
-      if (j < my_nkt) {
-        const int kt = kt0 + j;
-        if (chunk_ok(kt, fg)) a_frag[i][j][0] = *(const v4i *)(ap + (int64_t)kt * kTileKBytes);
-        if (chunk_ok(kt, 4 + fg)) a_frag[i][j][1] = *(const v4i *)(ap + (int64_t)kt * kTileKBytes + 64);
-        const int g0 = kt * 8 + fg, g1 = g0 + 4;
-        const uint32_t b0 = g0 < p.ks ? p.a_scale[scale_offset(p.a_scale_layout, row, g0, p.ks, p.ksp)] : 127u;
-        const uint32_t b1 = g1 < p.ks ? p.a_scale[scale_offset(p.a_scale_layout, row, g1, p.ks, p.ksp)] : 127u;
-        a_sc[i][j] = b0 | (b1 << 8);
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        asm volatile("" : "+v"(a_frag[i][j][0]), "+v"(a_frag[i][j][1]), "+v"(a_sc[i][j][0]), "+v"(a_sc[i][j][1]));
       }
     }
+  } else {
+    wait_tile(nt_begin);
   }
 
-  // Workgroup barrier that orders LDS traffic only: the DMA of the next tile
-  // stays in flight across it (a __syncthreads() would wait for vmcnt(0)).
+  // Workgroup barrier that orders LDS traffic only: DMA stays in flight across
+  // it (a __syncthreads() would wait for vmcnt(0)).
   auto lds_barrier = [&]() {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_waitcnt((7 << 4) | (3 << 14) | 15);  // lgkmcnt(0) only
@@ -232,93 +329,135 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     }
   };
 
-  // ---- the stream: B tile nt is multiplied while tile nt+1 is in flight ----
-  // Per tile: wait for this wave's DMA (everything it has in flight), start the
-  // DMA of the next tile, finish the previous tile (wave 0 adds the partials of
-  // waves 1..3 and stores, so its stores never sit in front of a DMA wait),
-  // multiply, hand the partial tile over.
+  // ---- the stream ----
+  // Per tile nt: wait until it has landed (tile nt+1 stays in flight), pull its
+  // fragments and scales into registers, let wave 0 store the finished tile
+  // nt-1 (so the stores are older than the next DMA and counted waits stay
+  // exact), start the DMA of tile nt+2 into the buffer just emptied, multiply,
+  // add the four partial tiles through LDS.
   v4f prev[MT_M];
-  for (int nt = nt_begin; nt <= nt_end; ++nt) {
+  for (int nt = nt_begin; nt < nt_end; ++nt) {
     const int buf = (nt - nt_begin) & 1;
-    const bool have = nt < nt_end;
-    if (have) {
-      __builtin_amdgcn_s_waitcnt(0);  // DMA of tile nt (and the scale image) has landed
-      asm volatile("" ::: "memory");
-      if (nt + 1 < nt_end && my_nkt > 0) {
-        issue_scales(nt + 1, buf ^ 1);
-        issue_rows(nt + 1, buf ^ 1, 0, 16);
-      }
-    }
-    if (nt > nt_begin) {
-      // finish tile nt-1: partials of waves 1..3 are in LDS (barrier below, previous iteration)
-      if (wave == 0) {
-#pragma unroll
-        for (int i = 0; i < MT_M; ++i) {
-          v4f v = prev[i];
-#pragma unroll
-          for (int w = 0; w < kStreamWaves - 1; ++w) v += *(const v4f *)lds.red[w][i][lane];
-          store_tile(nt - 1, i, lane, v);
-        }
-      }
-      lds_barrier();  // red is free again
-    }
-    if (!have) break;
+    if (nt > nt_begin) wait_tile(nt);
 
     const int n_row = min(nt * 16 + fr, p.n - 1);
     const uint8_t *sc_img = lds.scales[wave][buf];
     const uint8_t *tile = lds.tile[wave][buf] + frag_base;
-    const int sc0 = scale_byte_off(n_row, 0), sc1 = scale_byte_off(n_row, 1);
+    v4i bfrag[kStreamKtPerWave][2];
+    uint32_t scb[kStreamKtPerWave];
+#pragma unroll
+    for (int j = 0; j < kStreamKtPerWave; ++j) {
+      if (FULL || j < my_nkt) {
+        bfrag[j][0] = *(const v4i *)(tile + j * frag_j);
+        bfrag[j][1] = *(const v4i *)(tile + j * frag_j + frag_s);
+      } else {
+        bfrag[j][0] = bfrag[j][1] = zero;
+      }
+    }
+    if (sc_rowmajor) {
+      const uint32_t sel = 0x0c0c0000u | (uint32_t)fg | ((uint32_t)(4 + fg) << 8);
+      const v4i *img = (const v4i *)(sc_img + fr * 64);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4i d = img[q];
+        scb[2 * q] = __builtin_amdgcn_perm((uint32_t)d.y, (uint32_t)d.x, sel);
+        scb[2 * q + 1] = __builtin_amdgcn_perm((uint32_t)d.w, (uint32_t)d.z, sel);
+      }
+    } else {
+      const bool native = bsl == WAVE_MXFP4_SCALE_MFMA32;
+      const uint32_t h = native ? (uint32_t)(fg >> 1) : (uint32_t)((n_row >> 4) & 1);
+      const uint32_t sel = 0x0c0c0000u | h | ((2 + h) << 8);
+      const uint32_t *img = (const uint32_t *)(sc_img + (native ? (fg & 1) * 64 : fg * 64) + (n_row & 15) * 4);
+      const int stride = native ? 32 : 64;  // dwords per K tile
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        const uint32_t d = img[j * stride];
+        scb[j] = __builtin_amdgcn_perm(d, d, sel);
+      }
+    }
+
+    if (wave == 0 && nt > nt_begin) {
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) store_tile(nt - 1, i, lane, prev[i]);
+    }
+
+    // the buffer is free once the reads above have returned
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt((7 << 4) | (3 << 14) | 15);  // lgkmcnt(0)
+    asm volatile("" ::: "memory");
+    if (nt + 2 < nt_end) issue_tile(nt + 2, buf);
+
     v4f acc[MT_M];
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < kStreamKtPerWave; ++j) {
-      if (j < my_nkt) {
-        const v4i b0 = *(const v4i *)(tile + j * frag_j);
-        const v4i b1 = *(const v4i *)(tile + j * frag_j + frag_s);
-        const uint32_t scb = (uint32_t)sc_img[sc0 + j * sc_kt_stride] | ((uint32_t)sc_img[sc1 + j * sc_kt_stride] << 8);
-        const v8i vb0 = {b0.x, b0.y, b0.z, b0.w, 0, 0, 0, 0};
-        const v8i vb1 = {b1.x, b1.y, b1.z, b1.w, 0, 0, 0, 0};
+      if (FULL || j < my_nkt) {
+        const v8i vb0 = {bfrag[j][0].x, bfrag[j][0].y, bfrag[j][0].z, bfrag[j][0].w, 0, 0, 0, 0};
+        const v8i vb1 = {bfrag[j][1].x, bfrag[j][1].y, bfrag[j][1].z, bfrag[j][1].w, 0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < MT_M; ++i) {
           const v8i va0 = {a_frag[i][j][0].x, a_frag[i][j][0].y, a_frag[i][j][0].z, a_frag[i][j][0].w, 0, 0, 0, 0};
           const v8i va1 = {a_frag[i][j][1].x, a_frag[i][j][1].y, a_frag[i][j][1].z, a_frag[i][j][1].w, 0, 0, 0, 0};
-          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb0, va0, acc[i], 4, 4, 0, (int)scb, 0,
-                                                                     (int)a_sc[i][j]);
-          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb1, va1, acc[i], 4, 4, 1, (int)scb, 1,
-                                                                     (int)a_sc[i][j]);
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb0, va0, acc[i], 4, 4, 0, (int)scb[j], 0,
+                                                                     (int)a_sc[i][j][0]);
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb1, va1, acc[i], 4, 4, 1, (int)scb[j], 0,
+                                                                     (int)a_sc[i][j][1]);
         }
       }
     }
-    // hand over: wave 0 keeps its tile in registers, the others go through LDS
+
+    // add the partial tiles: waves 1..3 hand theirs to wave 0 through LDS
+    if (wave != 0) {
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) {
-      if (wave == 0)
-        prev[i] = acc[i];
-      else
-        *(v4f *)lds.red[wave - 1][i][lane] = acc[i];
+      for (int i = 0; i < MT_M; ++i) *(v4f *)lds.red[wave - 1][i][lane] = acc[i];
     }
     lds_barrier();  // partials visible
+    if (wave == 0) {
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) {
+        v4f v = acc[i];
+#pragma unroll
+        for (int w = 0; w < kStreamWaves - 1; ++w) v += *(const v4f *)lds.red[w][i][lane];
+        prev[i] = v;
+      }
+    }
+    lds_barrier();  // red is free again
+  }
+  if (wave == 0) {
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) store_tile(nt_end - 1, i, lane, prev[i]);
   }
 }
 
-template <int MT_M>
+template <int MT_M, bool FULL>
 __global__ void __launch_bounds__(kStreamWaves * 64, 1) stream_gemm_kernel(const GemmParams p) {
-  stream_body<MT_M>(p);
+  stream_body<MT_M, FULL>(p);
 }
 
-template <int MT_M>
+template <int MT_M, bool FULL>
 static hipError_t launch_stream_mt(const GemmParams &p, int grid_x, hipStream_t stream) {
   static bool attr_done = false;
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)stream_gemm_kernel<MT_M>,
+    hipError_t e = hipFuncSetAttribute((const void *)stream_gemm_kernel<MT_M, FULL>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(StreamLds));
     if (e != hipSuccess) return e;
     attr_done = true;
   }
   dim3 grid(grid_x, p.splits, 1);
-  stream_gemm_kernel<MT_M><<<grid, dim3(kStreamWaves * 64), sizeof(StreamLds), stream>>>(p);
+  stream_gemm_kernel<MT_M, FULL><<<grid, dim3(kStreamWaves * 64), sizeof(StreamLds), stream>>>(p);
   return hipGetLastError();
+}
+
+template <bool FULL>
+static hipError_t launch_stream_full(const GemmParams &p, int grid_x, hipStream_t stream) {
+  switch ((p.m + 15) / 16) {
+    case 1: return launch_stream_mt<1, FULL>(p, grid_x, stream);
+    case 2: return launch_stream_mt<2, FULL>(p, grid_x, stream);
+    case 3: return launch_stream_mt<3, FULL>(p, grid_x, stream);
+    case 4: return launch_stream_mt<4, FULL>(p, grid_x, stream);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 // One workgroup per CU (or per 16-row tile of B if there are fewer tiles).
@@ -331,14 +470,14 @@ hipError_t launch_stream_gemm(const GemmParams &p, int num_cus, hipStream_t stre
   if (grid_x < 1) grid_x = 1;
   // 32-bit DMA offsets inside a workgroup's range of B rows
   if (((int64_t)(nt_total + grid_x - 1) / grid_x + 1) * 16 * p.kp >= ((int64_t)1 << 31)) return hipErrorInvalidValue;
-  const int mt = (p.m + 15) / 16;
-  switch (mt) {
-    case 1: return launch_stream_mt<1>(p, grid_x, stream);
-    case 2: return launch_stream_mt<2>(p, grid_x, stream);
-    case 3: return launch_stream_mt<3>(p, grid_x, stream);
-    case 4: return launch_stream_mt<4>(p, grid_x, stream);
-    default: return hipErrorInvalidValue;
-  }
+  // ... and into A and both scale matrices (padded to 32-row blocks)
+  if ((int64_t)p.m * p.kp >= ((int64_t)1 << 31) || ((int64_t)p.n + 32) * (p.ksp + 8) >= ((int64_t)1 << 31))
+    return hipErrorInvalidValue;
+  // every wave of every split owns 8 whole K tiles
+  // ... and every workgroup at least two tiles of B
+  const bool full = p.tiles_per_split == kStreamMaxKTiles && p.k_tiles % kStreamMaxKTiles == 0 &&
+                    (p.k & (kTileK - 1)) == 0 && nt_total >= 2 * grid_x;
+  return full ? launch_stream_full<true>(p, grid_x, stream) : launch_stream_full<false>(p, grid_x, stream);
 }
 
 }  // namespace wave_mxfp4

@@ -94,14 +94,23 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   };
 
   // ---- A: resident fragments and scales; issued first, they land under the first B tiles ----
-  v4i a_frag[MT_M][kStreamKtPerWave][2];
-  // Scale bytes stay in the registers they were loaded into (byte 0, op_sel 0):
-  // combining them would be a use of loaded data in front of the stream, and
-  // with DMA and ordinary loads both pending the compiler waits for vmcnt(0)
-  // at such a use.
   // All vector memory traffic of the kernel is buffer instructions: with a
-  // global_load ... lds pending the compiler treats the queue as unordered.
+  // global_load ... lds pending the compiler treats the queue as unordered and
+  // turns every counted wait into a wait for an empty queue.
+  //
+  // FULL mode loads A in whole cache lines (lane t: row t/8, chunk t%8 of one
+  // K tile, two instructions per 16 rows and K tile) and turns the registers
+  // into MFMA fragments (lane l: row l%16, chunk l/16) through a small LDS
+  // stage after the B stream has been started: fragment-shaped loads touch 16
+  // half lines per instruction and cost the vector L1 four times the cycles,
+  // in front of the stream.  Scales: one 16-byte piece per lane and row quarter
+  // redistributed by ds_bpermute (row-major), or the lane's own dword of each
+  // 256-byte block (blocked layouts).  a_sc[..][0] then holds the scales of
+  // both K steps in bytes 0 and 1.
+  // The generic mode loads fragment-shaped, one scale byte per register.
+  v4i a_frag[MT_M][kStreamKtPerWave][2];
   uint32_t a_sc[MT_M][kStreamKtPerWave][2];
+  constexpr int kOpselA1 = FULL ? 1 : 0;  // op_sel of the A scale for the second K step
   const __amdgpu_buffer_rsrc_t a_rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a), 0, 0x7FFFFFFF, 0x00020000);
   const __amdgpu_buffer_rsrc_t as_rsrc =
@@ -111,25 +120,52 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     const u4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
     return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
   };
+  const int asl = p.a_scale_layout;
+  v4i a_sq[MT_M];  // row-major scale pieces
+  if (FULL) {
 #pragma unroll
-  for (int i = 0; i < MT_M; ++i) {
-    const int row = min(i * 16 + fr, p.m - 1);
-    const int ao = row * kp + fg * 16;
-    // scale (row, group kt*8 + s*4 + fg): every layout is linear in kt
-    const int so0 = (int)scale_offset(p.a_scale_layout, row, fg, p.ks, p.ksp);
-    const int so1 = (int)scale_offset(p.a_scale_layout, row, 4 + fg, p.ks, p.ksp);
-    const int so_kt = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR ? 8 : 256;
+    for (int i = 0; i < MT_M; ++i) {
+      const int ao0 = min(i * 16 + (lane >> 3), p.m - 1) * kp + (lane & 7) * 16;
+      const int ao1 = min(i * 16 + 8 + (lane >> 3), p.m - 1) * kp + (lane & 7) * 16;
 #pragma unroll
-    for (int j = 0; j < kStreamKtPerWave; ++j) {
-      a_frag[i][j][0] = a_frag[i][j][1] = zero;
-      a_sc[i][j][0] = a_sc[i][j][1] = 127u;
-      if (j < my_nkt) {
-        const int kt = kt0 + j;
-        if (chunk_ok(kt, fg)) a_frag[i][j][0] = load_b128(a_rsrc, ao, kt * kTileKBytes);
-        if (chunk_ok(kt, 4 + fg)) a_frag[i][j][1] = load_b128(a_rsrc, ao, kt * kTileKBytes + 64);
-        if (FULL || kt * 8 + fg < p.ks) a_sc[i][j][0] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so0, kt * so_kt, 0);
-        if (FULL || kt * 8 + 4 + fg < p.ks)
-          a_sc[i][j][1] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so1, kt * so_kt, 0);
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        a_frag[i][j][0] = load_b128(a_rsrc, ao0, (kt0 + j) * kTileKBytes);
+        a_frag[i][j][1] = load_b128(a_rsrc, ao1, (kt0 + j) * kTileKBytes);
+      }
+      // Both scale shapes are loaded, the one that does not apply from offset
+      // 0: separate code paths per layout would make the compiler guard the
+      // registers of the other path with waits in front of the stream.
+      const bool rm = asl == WAVE_MXFP4_SCALE_ROW_MAJOR;
+      // row-major: lane t holds row t/4, bytes 16*(t%4) .. +15 of the wave's 64 = K tiles 2*(t%4), 2*(t%4)+1
+      a_sq[i] = load_b128(as_rsrc, rm ? min(i * 16 + (lane >> 2), p.m - 1) * p.ks + (lane & 3) * 16 : 0, rm ? kt0 * 8 : 0);
+      // blocked: the dword of block (row/32, K tile) that holds this lane's two scale bytes
+      const int row = i * 16 + fr;  // rows up to the next multiple of 32 exist in blocked layouts
+      const int in_blk = asl == WAVE_MXFP4_SCALE_MFMA32 ? (((fg & 1) << 5) | (row & 31)) * 4 : fg * 64 + (row & 15) * 4;
+      const int so = rm ? 0 : (row >> 5) * (p.ksp >> 3) * 256 + in_blk;
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j)
+        a_sc[i][j][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, so, rm ? 0 : (kt0 + j) * 256, 0);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+      const int row = min(i * 16 + fr, p.m - 1);
+      const int ao = row * kp + fg * 16;
+      // scale (row, group kt*8 + s*4 + fg): every layout is linear in kt
+      const int so0 = (int)scale_offset(asl, row, fg, p.ks, p.ksp);
+      const int so1 = (int)scale_offset(asl, row, 4 + fg, p.ks, p.ksp);
+      const int so_kt = asl == WAVE_MXFP4_SCALE_ROW_MAJOR ? 8 : 256;
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        a_frag[i][j][0] = a_frag[i][j][1] = zero;
+        a_sc[i][j][0] = a_sc[i][j][1] = 127u;
+        if (j < my_nkt) {
+          const int kt = kt0 + j;
+          if (chunk_ok(kt, fg)) a_frag[i][j][0] = load_b128(a_rsrc, ao, kt * kTileKBytes);
+          if (chunk_ok(kt, 4 + fg)) a_frag[i][j][1] = load_b128(a_rsrc, ao, kt * kTileKBytes + 64);
+          if (kt * 8 + fg < p.ks) a_sc[i][j][0] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so0, kt * so_kt, 0);
+          if (kt * 8 + 4 + fg < p.ks) a_sc[i][j][1] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so1, kt * so_kt, 0);
+        }
       }
     }
   }
@@ -271,23 +307,6 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     }
     asm volatile("" ::: "memory");
   };
-  // A is older than both tiles, so it has landed with the first of them.  Its
-  // registers are pinned behind this wait, so that no use of them can be
-  // hoisted in front of it (where the compiler would add its own wait).
-  if (FULL) {
-    stream_wait_vm<17>();
-    asm volatile("" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < MT_M; ++i) {
-#pragma unroll
-      for (int j = 0; j < kStreamKtPerWave; ++j) {
-        asm volatile("" : "+v"(a_frag[i][j][0]), "+v"(a_frag[i][j][1]), "+v"(a_sc[i][j][0]), "+v"(a_sc[i][j][1]));
-      }
-    }
-  } else {
-    wait_tile(nt_begin);
-  }
-
   // Workgroup barrier that orders LDS traffic only: DMA stays in flight across
   // it (a __syncthreads() would wait for vmcnt(0)).
   auto lds_barrier = [&]() {
@@ -296,6 +315,58 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
+
+  if (FULL) {
+    // A into fragment shape.  The stage is the wave's share of the partial-tile
+    // area, 16 rows of 128 + 16 bytes (fragment reads then spread over all
+    // banks); LDS executes a wave's accesses in order, so one K tile after the
+    // other can pass through the same 2.25 KB.
+    // (uses of the loaded registers stay behind the DMA issue above)
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) asm volatile("" : "+v"(a_sc[i][j][0]));
+      asm volatile("" : "+v"(a_sq[i]));
+    }
+    uint8_t *stage = reinterpret_cast<uint8_t *>(lds.red) + wave * (16 * 144);
+    static_assert(kStreamWaves * 16 * 144 <= (int)sizeof(lds.red), "A stage fits the partial-tile area");
+    const uint32_t wr = (uint32_t)((lane >> 3) * 144 + (lane & 7) * 16), rd = (uint32_t)(fr * 144 + fg * 16);
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        *(v4i *)(stage + wr) = a_frag[i][j][0];
+        *(v4i *)(stage + 8 * 144 + wr) = a_frag[i][j][1];
+        asm volatile("" ::: "memory");
+        a_frag[i][j][0] = *(const v4i *)(stage + rd);
+        a_frag[i][j][1] = *(const v4i *)(stage + rd + 64);
+        asm volatile("" ::: "memory");
+      }
+      {
+        // row-major: K tile j, step s of row fr is byte fg of dword (j%2)*2 + s held by lane fr*4 + j/2;
+        // blocked: bytes (step 0, h), (step 1, h) of the lane's dword, h = fg/2 (MFMA32) or the
+        // 16-row half (shuffled)
+        const bool rm = asl == WAVE_MXFP4_SCALE_ROW_MAJOR;
+        const uint32_t h = asl == WAVE_MXFP4_SCALE_MFMA32 ? (uint32_t)(fg >> 1) : (uint32_t)(i & 1);
+        const uint32_t sel = rm ? (0x0c0c0000u | (uint32_t)fg | ((uint32_t)(4 + fg) << 8)) : (0x0c0c0000u | h | ((2 + h) << 8));
+        const int q[4] = {a_sq[i].x, a_sq[i].y, a_sq[i].z, a_sq[i].w};
+#pragma unroll
+        for (int j = 0; j < kStreamKtPerWave; ++j) {
+          const int src = (fr * 4 + (j >> 1)) * 4;
+          const uint32_t d0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, q[(j & 1) * 2]);
+          const uint32_t d1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, q[(j & 1) * 2 + 1]);
+          a_sc[i][j][0] = __builtin_amdgcn_perm(rm ? d1 : a_sc[i][j][0], rm ? d0 : a_sc[i][j][0], sel);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) a_sc[i][j][1] = a_sc[i][j][0];
+    }
+    lds_barrier();  // the stage becomes the partial-tile area
+    stream_wait_vm<17>();  // tile nt_begin has landed
+    asm volatile("" ::: "memory");
+  } else {
+    wait_tile(nt_begin);
+  }
 
   auto store_tile = [&](int nt, int i, int l, const v4f &v) {
     const int m = i * 16 + (l & 15);
@@ -401,7 +472,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
           const v8i va1 = {a_frag[i][j][1].x, a_frag[i][j][1].y, a_frag[i][j][1].z, a_frag[i][j][1].w, 0, 0, 0, 0};
           acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb0, va0, acc[i], 4, 4, 0, (int)scb[j], 0,
                                                                      (int)a_sc[i][j][0]);
-          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb1, va1, acc[i], 4, 4, 1, (int)scb[j], 0,
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vb1, va1, acc[i], 4, 4, 1, (int)scb[j], kOpselA1,
                                                                      (int)a_sc[i][j][1]);
         }
       }

@@ -148,7 +148,7 @@ def main():
         achieved = nbytes / per_launch / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                     "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": None,
-                    "kernel": "skinny_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
+                    "kernel": "stream_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
     else:
         achieved = flops / per_launch / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_MXFP4_TFLOPS,

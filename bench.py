@@ -113,6 +113,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode-shape leg")
     ap.add_argument("--cpu-rows", type=int, default=2048)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="instead of a GEMM, run device-to-device copies of 256 MiB (the known-size kernel "
+                         "that hardware byte counters are scaled by) and print their size")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this operator runs on one GPU; --gpus N with N > 1 is not supported "
@@ -130,6 +133,17 @@ def main():
         sys.exit(3)
     dev = "cuda:0"
     torch.cuda.set_device(0)
+
+    if args.copy_calibration:
+        nbytes = 256 << 20
+        src = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.warmup + args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": True, "bytes_read_per_launch": nbytes,
+                          "bytes_written_per_launch": nbytes, "launches": args.warmup + args.steps}))
+        return
 
     m, n, k, od, seed, srange = WORKLOADS[args.workload]
     out_dtype = torch.bfloat16 if od == "bf16" else torch.float32

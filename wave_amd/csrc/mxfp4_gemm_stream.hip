@@ -76,8 +76,9 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
 
   // ---- work split: N tiles over workgroups, K tiles over splits and waves ----
   const int nt_total = (p.n + 15) >> 4;
-  const int nt_begin = (int)(((int64_t)blockIdx.x * nt_total) / gridDim.x);
-  const int nt_end = (int)(((int64_t)(blockIdx.x + 1) * nt_total) / gridDim.x);
+  const uint32_t nt_q = (uint32_t)nt_total / gridDim.x, nt_r = (uint32_t)nt_total - nt_q * gridDim.x;
+  const int nt_begin = (int)(blockIdx.x * nt_q + min(blockIdx.x, nt_r));  // the first nt_r workgroups take one more
+  const int nt_end = nt_begin + (int)nt_q + (blockIdx.x < nt_r ? 1 : 0);
   if (nt_begin >= nt_end) return;
   const int split = blockIdx.y;
   const int kt_begin = split * p.tiles_per_split;
@@ -401,12 +402,19 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   };
 
   // ---- the stream ----
-  // Per tile nt: wait until it has landed (tile nt+1 stays in flight), pull its
-  // fragments and scales into registers, let wave 0 store the finished tile
-  // nt-1 (so the stores are older than the next DMA and counted waits stay
-  // exact), start the DMA of tile nt+2 into the buffer just emptied, multiply,
-  // add the four partial tiles through LDS.
-  v4f prev[MT_M];
+  // Per tile t: wait until it has landed (tile t+1 stays in flight), pull its
+  // fragments and scales into registers, start the DMA of tile t+2 into the
+  // buffer just emptied, multiply, add the four partial tiles through LDS.
+  // The sum of tile t is formed by wave t%4 and stays in its registers
+  // (kHold tiles per wave): C is written at the end of the kernel, by all four
+  // waves at once, so that in the common case no write traffic (16 partial
+  // lines per tile) is mixed into the read stream.  With more than 4*kHold
+  // tiles per workgroup the oldest held tile is stored just before the DMA
+  // issue of the iteration that replaces it: the stores are then older than
+  // that DMA and the counted waits stay exact.
+  constexpr int kHold = FULL ? 2 : 1;
+  v4f hold[kHold][MT_M];
+  const int ntiles = nt_end - nt_begin;
   for (int nt = nt_begin; nt < nt_end; ++nt) {
     const int buf = (nt - nt_begin) & 1;
     if (nt > nt_begin) wait_tile(nt);
@@ -447,9 +455,16 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       }
     }
 
-    if (wave == 0 && nt > nt_begin) {
+    const int t = nt - nt_begin;
+    const int slot = (t >> 2) & (kHold - 1);
+    if (t >= 4 * kHold && wave == (t & 3)) {
 #pragma unroll
-      for (int i = 0; i < MT_M; ++i) store_tile(nt - 1, i, lane, prev[i]);
+      for (int h = 0; h < kHold; ++h) {
+        if (h == slot) {
+#pragma unroll
+          for (int i = 0; i < MT_M; ++i) store_tile(nt - 4 * kHold, i, lane, hold[h][i]);
+        }
+      }
     }
 
     // the buffer is free once the reads above have returned
@@ -478,26 +493,38 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       }
     }
 
-    // add the partial tiles: waves 1..3 hand theirs to wave 0 through LDS
-    if (wave != 0) {
+    // add the partial tiles: the other three waves hand theirs to wave t%4 through LDS
+    const int reducer = t & 3;
+    if (wave != reducer) {
 #pragma unroll
-      for (int i = 0; i < MT_M; ++i) *(v4f *)lds.red[wave - 1][i][lane] = acc[i];
+      for (int i = 0; i < MT_M; ++i) *(v4f *)lds.red[(wave - reducer - 1) & 3][i][lane] = acc[i];
     }
     lds_barrier();  // partials visible
-    if (wave == 0) {
+    if (wave == reducer) {
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) {
         v4f v = acc[i];
 #pragma unroll
         for (int w = 0; w < kStreamWaves - 1; ++w) v += *(const v4f *)lds.red[w][i][lane];
-        prev[i] = v;
+#pragma unroll
+        for (int h = 0; h < kHold; ++h) {
+          if (h == slot) hold[h][i] = v;
+        }
       }
     }
     lds_barrier();  // red is free again
   }
-  if (wave == 0) {
+  // the tiles still held: the last 4*kHold (or fewer) of the workgroup
+  for (int t = max(0, ntiles - 4 * kHold); t < ntiles; ++t) {
+    if (wave == (t & 3)) {
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) store_tile(nt_end - 1, i, lane, prev[i]);
+      for (int h = 0; h < kHold; ++h) {
+        if (h == ((t >> 2) & (kHold - 1))) {
+#pragma unroll
+          for (int i = 0; i < MT_M; ++i) store_tile(nt_begin + t, i, lane, hold[h][i]);
+        }
+      }
+    }
   }
 }
 

@@ -94,83 +94,6 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     return FULL || tail_chunks == 0 || kt != p.k_tiles - 1 || chunk < tail_chunks;
   };
 
-  // ---- A: resident fragments and scales; issued first, they land under the first B tiles ----
-  // All vector memory traffic of the kernel is buffer instructions: with a
-  // global_load ... lds pending the compiler treats the queue as unordered and
-  // turns every counted wait into a wait for an empty queue.
-  //
-  // FULL mode loads A in whole cache lines (lane t: row t/8, chunk t%8 of one
-  // K tile, two instructions per 16 rows and K tile) and turns the registers
-  // into MFMA fragments (lane l: row l%16, chunk l/16) through a small LDS
-  // stage after the B stream has been started: fragment-shaped loads touch 16
-  // half lines per instruction and cost the vector L1 four times the cycles,
-  // in front of the stream.  Scales: one 16-byte piece per lane and row quarter
-  // redistributed by ds_bpermute (row-major), or the lane's own dword of each
-  // 256-byte block (blocked layouts).  a_sc[..][0] then holds the scales of
-  // both K steps in bytes 0 and 1.
-  // The generic mode loads fragment-shaped, one scale byte per register.
-  v4i a_frag[MT_M][kStreamKtPerWave][2];
-  uint32_t a_sc[MT_M][kStreamKtPerWave][2];
-  constexpr int kOpselA1 = FULL ? 1 : 0;  // op_sel of the A scale for the second K step
-  const __amdgpu_buffer_rsrc_t a_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a), 0, 0x7FFFFFFF, 0x00020000);
-  const __amdgpu_buffer_rsrc_t as_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a_scale), 0, 0x7FFFFFFF, 0x00020000);
-  auto load_b128 = [&](__amdgpu_buffer_rsrc_t r, int voff, int soff) -> v4i {
-    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
-    const u4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
-    return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-  };
-  const int asl = p.a_scale_layout;
-  v4i a_sq[MT_M];  // row-major scale pieces
-  if (FULL) {
-#pragma unroll
-    for (int i = 0; i < MT_M; ++i) {
-      const int ao0 = min(i * 16 + (lane >> 3), p.m - 1) * kp + (lane & 7) * 16;
-      const int ao1 = min(i * 16 + 8 + (lane >> 3), p.m - 1) * kp + (lane & 7) * 16;
-#pragma unroll
-      for (int j = 0; j < kStreamKtPerWave; ++j) {
-        a_frag[i][j][0] = load_b128(a_rsrc, ao0, (kt0 + j) * kTileKBytes);
-        a_frag[i][j][1] = load_b128(a_rsrc, ao1, (kt0 + j) * kTileKBytes);
-      }
-      // Both scale shapes are loaded, the one that does not apply from offset
-      // 0: separate code paths per layout would make the compiler guard the
-      // registers of the other path with waits in front of the stream.
-      const bool rm = asl == WAVE_MXFP4_SCALE_ROW_MAJOR;
-      // row-major: lane t holds row t/4, bytes 16*(t%4) .. +15 of the wave's 64 = K tiles 2*(t%4), 2*(t%4)+1
-      a_sq[i] = load_b128(as_rsrc, rm ? min(i * 16 + (lane >> 2), p.m - 1) * p.ks + (lane & 3) * 16 : 0, rm ? kt0 * 8 : 0);
-      // blocked: the dword of block (row/32, K tile) that holds this lane's two scale bytes
-      const int row = i * 16 + fr;  // rows up to the next multiple of 32 exist in blocked layouts
-      const int in_blk = asl == WAVE_MXFP4_SCALE_MFMA32 ? (((fg & 1) << 5) | (row & 31)) * 4 : fg * 64 + (row & 15) * 4;
-      const int so = rm ? 0 : (row >> 5) * (p.ksp >> 3) * 256 + in_blk;
-#pragma unroll
-      for (int j = 0; j < kStreamKtPerWave; ++j)
-        a_sc[i][j][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, so, rm ? 0 : (kt0 + j) * 256, 0);
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < MT_M; ++i) {
-      const int row = min(i * 16 + fr, p.m - 1);
-      const int ao = row * kp + fg * 16;
-      // scale (row, group kt*8 + s*4 + fg): every layout is linear in kt
-      const int so0 = (int)scale_offset(asl, row, fg, p.ks, p.ksp);
-      const int so1 = (int)scale_offset(asl, row, 4 + fg, p.ks, p.ksp);
-      const int so_kt = asl == WAVE_MXFP4_SCALE_ROW_MAJOR ? 8 : 256;
-#pragma unroll
-      for (int j = 0; j < kStreamKtPerWave; ++j) {
-        a_frag[i][j][0] = a_frag[i][j][1] = zero;
-        a_sc[i][j][0] = a_sc[i][j][1] = 127u;
-        if (j < my_nkt) {
-          const int kt = kt0 + j;
-          if (chunk_ok(kt, fg)) a_frag[i][j][0] = load_b128(a_rsrc, ao, kt * kTileKBytes);
-          if (chunk_ok(kt, 4 + fg)) a_frag[i][j][1] = load_b128(a_rsrc, ao, kt * kTileKBytes + 64);
-          if (kt * 8 + fg < p.ks) a_sc[i][j][0] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so0, kt * so_kt, 0);
-          if (kt * 8 + 4 + fg < p.ks) a_sc[i][j][1] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so1, kt * so_kt, 0);
-        }
-      }
-    }
-  }
-
   // ---- B data DMA: one instruction = up to 1 KB contiguous ----
   //   row-major   : row r of the tile, K tiles kt0 .. kt0+7 (lane t: K tile t/8, chunk t%8),
   //                 landing at r*pitch + t*16; a fragment (row fr, K tile j, chunk c) is read
@@ -294,6 +217,85 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   // two B tiles in flight from the start (FULL mode is only launched with at
   // least two tiles per workgroup, which keeps this prologue branch-free)
   issue_tile(nt_begin, 0);
+
+  // ---- A: resident fragments and scales; issued between the first two B tiles ----
+  // All vector memory traffic of the kernel is buffer instructions: with a
+  // global_load ... lds pending the compiler treats the queue as unordered and
+  // turns every counted wait into a wait for an empty queue.
+  //
+  // FULL mode loads A in whole cache lines (lane t: row t/8, chunk t%8 of one
+  // K tile, two instructions per 16 rows and K tile) and turns the registers
+  // into MFMA fragments (lane l: row l%16, chunk l/16) through a small LDS
+  // stage after the B stream has been started: fragment-shaped loads touch 16
+  // half lines per instruction and cost the vector L1 four times the cycles,
+  // in front of the stream.  Scales: one 16-byte piece per lane and row quarter
+  // redistributed by ds_bpermute (row-major), or the lane's own dword of each
+  // 256-byte block (blocked layouts).  a_sc[..][0] then holds the scales of
+  // both K steps in bytes 0 and 1.
+  // The generic mode loads fragment-shaped, one scale byte per register.
+  v4i a_frag[MT_M][kStreamKtPerWave][2];
+  uint32_t a_sc[MT_M][kStreamKtPerWave][2];
+  constexpr int kOpselA1 = FULL ? 1 : 0;  // op_sel of the A scale for the second K step
+  const __amdgpu_buffer_rsrc_t a_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a), 0, 0x7FFFFFFF, 0x00020000);
+  const __amdgpu_buffer_rsrc_t as_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a_scale), 0, 0x7FFFFFFF, 0x00020000);
+  auto load_b128 = [&](__amdgpu_buffer_rsrc_t r, int voff, int soff) -> v4i {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const u4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+    return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+  };
+  const int asl = p.a_scale_layout;
+  v4i a_sq[MT_M];  // row-major scale pieces
+  if (FULL) {
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+      const int ao0 = min(i * 16 + (lane >> 3), p.m - 1) * kp + (lane & 7) * 16;
+      const int ao1 = min(i * 16 + 8 + (lane >> 3), p.m - 1) * kp + (lane & 7) * 16;
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        a_frag[i][j][0] = load_b128(a_rsrc, ao0, (kt0 + j) * kTileKBytes);
+        a_frag[i][j][1] = load_b128(a_rsrc, ao1, (kt0 + j) * kTileKBytes);
+      }
+      // Both scale shapes are loaded, the one that does not apply from offset
+      // 0: separate code paths per layout would make the compiler guard the
+      // registers of the other path with waits in front of the stream.
+      const bool rm = asl == WAVE_MXFP4_SCALE_ROW_MAJOR;
+      // row-major: lane t holds row t/4, bytes 16*(t%4) .. +15 of the wave's 64 = K tiles 2*(t%4), 2*(t%4)+1
+      a_sq[i] = load_b128(as_rsrc, rm ? min(i * 16 + (lane >> 2), p.m - 1) * p.ks + (lane & 3) * 16 : 0, rm ? kt0 * 8 : 0);
+      // blocked: the dword of block (row/32, K tile) that holds this lane's two scale bytes
+      const int row = i * 16 + fr;  // rows up to the next multiple of 32 exist in blocked layouts
+      const int in_blk = asl == WAVE_MXFP4_SCALE_MFMA32 ? (((fg & 1) << 5) | (row & 31)) * 4 : fg * 64 + (row & 15) * 4;
+      const int so = rm ? 0 : (row >> 5) * (p.ksp >> 3) * 256 + in_blk;
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j)
+        a_sc[i][j][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, so, rm ? 0 : (kt0 + j) * 256, 0);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+      const int row = min(i * 16 + fr, p.m - 1);
+      const int ao = row * kp + fg * 16;
+      // scale (row, group kt*8 + s*4 + fg): every layout is linear in kt
+      const int so0 = (int)scale_offset(asl, row, fg, p.ks, p.ksp);
+      const int so1 = (int)scale_offset(asl, row, 4 + fg, p.ks, p.ksp);
+      const int so_kt = asl == WAVE_MXFP4_SCALE_ROW_MAJOR ? 8 : 256;
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        a_frag[i][j][0] = a_frag[i][j][1] = zero;
+        a_sc[i][j][0] = a_sc[i][j][1] = 127u;
+        if (j < my_nkt) {
+          const int kt = kt0 + j;
+          if (chunk_ok(kt, fg)) a_frag[i][j][0] = load_b128(a_rsrc, ao, kt * kTileKBytes);
+          if (chunk_ok(kt, 4 + fg)) a_frag[i][j][1] = load_b128(a_rsrc, ao, kt * kTileKBytes + 64);
+          if (kt * 8 + fg < p.ks) a_sc[i][j][0] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so0, kt * so_kt, 0);
+          if (kt * 8 + 4 + fg < p.ks) a_sc[i][j][1] = __builtin_amdgcn_raw_buffer_load_b8(as_rsrc, so1, kt * so_kt, 0);
+        }
+      }
+    }
+  }
+
+
   if (FULL || nt_begin + 1 < nt_end) issue_tile(nt_begin + 1, 1);
 
   // Wait until tile nt has landed; tile nt+1 stays in flight.  In FULL mode a

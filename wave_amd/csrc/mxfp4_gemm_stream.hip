@@ -41,7 +41,7 @@ constexpr int kStreamWaves = 4;
 constexpr int kStreamKtPerWave = 8;                                // K tiles per wave: resident A, 1 KB of a B row
 constexpr int kStreamMaxKTiles = kStreamWaves * kStreamKtPerWave;  // per workgroup (K <= 8192)
 constexpr int kStreamRowBytes = kStreamKtPerWave * kTileKBytes;    // 1 KB of one B row per DMA instruction
-constexpr int kStreamRowPitch = kStreamRowBytes + 16;              // LDS pitch: 16 rows spread over all banks
+constexpr int kStreamRowPitch = kStreamRowBytes + 32;              // LDS pitch (measured: fragment reads are conflict-free at 32 mod 64)
 constexpr int kStreamTileBytes = 16 * kStreamRowPitch;             // one 16-row B tile, one wave's K range
 constexpr int kStreamScaleBytes = 2048;                            // its scale image (1 KB used by two layouts)
 
@@ -97,7 +97,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   // ---- B data DMA: one instruction = up to 1 KB contiguous ----
   //   row-major   : row r of the tile, K tiles kt0 .. kt0+7 (lane t: K tile t/8, chunk t%8),
   //                 landing at r*pitch + t*16; a fragment (row fr, K tile j, chunk c) is read
-  //                 at fr*pitch + j*128 + c*16 (the pitch is 1 KB + 16 B, so the 16 rows of a
+  //                 at fr*pitch + j*128 + c*16 (the pitch is 1 KB + 32 B, with which the 16 rows of a
   //                 fragment read fall on different banks).
   //   preshuffled : K step i = 2*j + s of the 16-row block (already in MFMA order: lane l's
   //                 16 bytes at l*16), landing at i*1024 + l*16 and read back from there.
@@ -147,8 +147,10 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const uint32_t frag_s = bpre ? 1024u : 64u;                    // per K step
 
   // ---- B scales: an image of the source bytes per B tile and wave ----
-  //   row-major : 16 rows x 64 bytes starting at group kt0*8 (lane t -> row t/4, piece t%4);
-  //               K tile j, step s of row fr is byte fg of the dword at fr*64 + j*8 + s*4.
+  //   row-major : 16 rows x 64 bytes starting at group kt0*8, stored piece-major (lane t -> row
+  //               t%16, 16-byte piece t/16, so the 16 rows of a piece are 256 contiguous bytes and
+  //               the reads below are conflict-free); K tiles 2q, 2q+1 of row fr are the 16 bytes
+  //               at q*256 + fr*16, step s of K tile j byte fg of dword (j%2)*2 + s.
   //   MFMA32    : of each of the 8 consecutive 256-byte blocks (32 rows x one K tile) the two
   //               64-byte runs that hold this tile's 16 rows (lane t -> block t/8, piece t%8);
   //               K tile j of row r is the dword at j*128 + (fg&1)*64 + (r%16)*4, whose bytes
@@ -168,8 +170,8 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     const int blocked_off = (n0 >> 5) * sc_block_row_bytes + kt0 * 256;
     if (FULL) {
       // one instruction whatever the layout, a second one for the shuffled blocks
-      const int row = min(n0 + (lane >> 2), p.n - 1);
-      const int off_rm = row * p.ks + kt0 * 8 + (lane & 3) * 16;
+      const int row = min(n0 + (lane & 15), p.n - 1);
+      const int off_rm = row * p.ks + kt0 * 8 + (lane >> 4) * 16;
       const int off_native = blocked_off + (lane >> 3) * 256 + ((lane & 7) >> 2) * 128 + ((n0 >> 4) & 1) * 64 +
                              (lane & 3) * 16;
       const int off_shuf = blocked_off + lane * 16;
@@ -178,15 +180,15 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       if (bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst + 1024), 16, off, 1024, 0, 0);
     } else if (bsl == WAVE_MXFP4_SCALE_ROW_MAJOR) {
-      const int row = min(n0 + (lane >> 2), p.n - 1);
-      const int64_t off = (int64_t)row * p.ks + (int64_t)kt0 * 8 + (lane & 3) * 16;
+      const int row = min(n0 + (lane & 15), p.n - 1);
+      const int64_t off = (int64_t)row * p.ks + (int64_t)kt0 * 8 + (lane >> 4) * 16;
       if (sc_pieces && off + 16 <= (int64_t)p.n * p.ks) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, (int)off, 0, 0, 0);
       } else {
         // rows that are not 16-byte multiples: byte copies of the groups that exist
         uint8_t *d8 = dst + lane * 16;
         for (int e = 0; e < 16; ++e) {
-          const int g = kt0 * 8 + (lane & 3) * 16 + e;
+          const int g = kt0 * 8 + (lane >> 4) * 16 + e;
           d8[e] = g < p.ks ? p.b_scale[(int64_t)row * p.ks + g] : (uint8_t)127;
         }
       }
@@ -321,9 +323,9 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
 
   if (FULL) {
     // A into fragment shape.  The stage is the wave's share of the partial-tile
-    // area, 16 rows of 128 + 16 bytes (fragment reads then spread over all
+    // area, 16 rows of 128 + 32 bytes (fragment reads then spread over all
     // banks); LDS executes a wave's accesses in order, so one K tile after the
-    // other can pass through the same 2.25 KB.
+    // other can pass through the same 2.5 KB.
     // (uses of the loaded registers stay behind the DMA issue above)
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
@@ -331,15 +333,15 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       for (int j = 0; j < kStreamKtPerWave; ++j) asm volatile("" : "+v"(a_sc[i][j][0]));
       asm volatile("" : "+v"(a_sq[i]));
     }
-    uint8_t *stage = reinterpret_cast<uint8_t *>(lds.red) + wave * (16 * 144);
-    static_assert(kStreamWaves * 16 * 144 <= (int)sizeof(lds.red), "A stage fits the partial-tile area");
-    const uint32_t wr = (uint32_t)((lane >> 3) * 144 + (lane & 7) * 16), rd = (uint32_t)(fr * 144 + fg * 16);
+    uint8_t *stage = reinterpret_cast<uint8_t *>(lds.red) + wave * (16 * 160);
+    static_assert(kStreamWaves * 16 * 160 <= (int)sizeof(lds.red), "A stage fits the partial-tile area");
+    const uint32_t wr = (uint32_t)((lane >> 3) * 160 + (lane & 7) * 16), rd = (uint32_t)(fr * 160 + fg * 16);
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
 #pragma unroll
       for (int j = 0; j < kStreamKtPerWave; ++j) {
         *(v4i *)(stage + wr) = a_frag[i][j][0];
-        *(v4i *)(stage + 8 * 144 + wr) = a_frag[i][j][1];
+        *(v4i *)(stage + 8 * 160 + wr) = a_frag[i][j][1];
         asm volatile("" ::: "memory");
         a_frag[i][j][0] = *(const v4i *)(stage + rd);
         a_frag[i][j][1] = *(const v4i *)(stage + rd + 64);
@@ -437,10 +439,9 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     }
     if (sc_rowmajor) {
       const uint32_t sel = 0x0c0c0000u | (uint32_t)fg | ((uint32_t)(4 + fg) << 8);
-      const v4i *img = (const v4i *)(sc_img + fr * 64);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const v4i d = img[q];
+        const v4i d = *(const v4i *)(sc_img + q * 256 + fr * 16);
         scb[2 * q] = __builtin_amdgcn_perm((uint32_t)d.y, (uint32_t)d.x, sel);
         scb[2 * q + 1] = __builtin_amdgcn_perm((uint32_t)d.w, (uint32_t)d.z, sel);
       }

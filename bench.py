@@ -155,18 +155,22 @@ def main():
     out = torch.empty(m, n, dtype=out_dtype, device=dev)
     wall, per_launch = time_gemm(torch, wave_amd, sets, out, args.steps, args.warmup, variant=args.variant)
 
+    # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this
+    # command, scaled by a device copy of known size (profiles/pmc_*.txt); not measurable from here
+    measured_traffic = {"cfg2": 440e6 + 172e6, "cfg3_m16": 125.5e6 + 0.92e6}.get(args.workload) \
+        if args.variant == 0 else None
     flops, nbytes = gemm_flops(m, n, k), gemm_bytes(m, n, k, out_bytes)
     ms_per_step = wall / args.steps * 1e3
     tflops = flops / (wall / args.steps) / 1e12
     if memory_bound:
         achieved = nbytes / per_launch / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                    "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": None,
+                    "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": measured_traffic,
                     "kernel": "stream_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
     else:
         achieved = flops / per_launch / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_MXFP4_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_MXFP4_TFLOPS, 4), "traffic": None,
+                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_MXFP4_TFLOPS, 4), "traffic": measured_traffic,
                     "kernel": "tile_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
 
     result = {

@@ -72,7 +72,7 @@ def test_e8m0_shuffle_matches_oracle(rows, ks):
     assert np.array_equal(got, orc.e8m0_shuffle_padded(s)[:rp])
 
 
-@pytest.mark.parametrize("rows,ks", [(256, 64), (4093, 224), (33, 9), (1, 1)])
+@pytest.mark.parametrize("rows,ks", [(256, 64), (4093, 224), (70, 264), (33, 9), (1, 1)])
 def test_scale_convert_every_layout_pair(rows, ks):
     rng = np.random.default_rng(rows * 7 + ks)
     s = rng.integers(0, 256, size=(rows, ks), dtype=np.uint8)

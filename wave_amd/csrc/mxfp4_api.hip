@@ -68,7 +68,7 @@ void fill_params(GemmParams &p, const void *a, const void *as, const void *b, co
 
 int pick_tile_variant(int64_t m, int64_t n) {
   const int64_t t256 = ((m + 255) / 256) * ((n + 255) / 256);
-  if (t256 >= 128) return WAVE_MXFP4_VARIANT_T256x256_W2x2;
+  if (t256 >= 128) return WAVE_MXFP4_VARIANT_T256x256_W4x2;  // 8 waves: measured 4-5 % ahead of 4 at 8192^3
   return WAVE_MXFP4_VARIANT_T128x128_W2x2;
 }
 

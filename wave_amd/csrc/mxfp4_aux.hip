@@ -103,6 +103,36 @@ __global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_la
   }
 }
 
+// Row-major -> MFMA32 for ks % 8 == 0, the conversion in front of every tile
+// GEMM with row-major scales.  A workgroup takes 32 rows x 32 K tiles: 8-byte
+// reads that walk each row contiguously, the even and odd groups of a K tile
+// split with v_perm into the two dwords of its block (lanes r%32 and 32 + r%32),
+// a pass through LDS (block stride 65 dwords: conflict-free both ways), and
+// dword writes that walk the destination contiguously.
+__global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__restrict__ src,
+                                                              uint8_t *__restrict__ dst, int rows, int ks) {
+  __shared__ uint32_t stage[32 * 65];
+  const int k_tiles = ks >> 3;
+  const int rt = blockIdx.y, kt0 = blockIdx.x * 32;
+  const int t = threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int unit = t + 256 * u, r = unit >> 5, ktl = unit & 31;
+    const int row = rt * 32 + r, kt = kt0 + ktl;
+    uint2 v = make_uint2(0u, 0u);
+    if (row < rows && kt < k_tiles) v = *(const uint2 *)(src + (int64_t)row * ks + (int64_t)kt * 8);
+    stage[ktl * 65 + r] = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u);       // groups 0, 2, 4, 6
+    stage[ktl * 65 + 32 + r] = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);  // groups 1, 3, 5, 7
+  }
+  __syncthreads();
+  uint32_t *out = (uint32_t *)dst + ((int64_t)rt * k_tiles + kt0) * 64;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int d = t + 256 * u, blk = d >> 6, lane = d & 63;
+    if (kt0 + blk < k_tiles) out[d] = stage[blk * 65 + lane];
+  }
+}
+
 // One thread per 16-byte chunk.
 __global__ void b_preshuffle_kernel(const uint8_t *__restrict__ b, uint8_t *__restrict__ out, int64_t rows,
                                     int64_t kp) {
@@ -210,6 +240,12 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
   const int64_t rows_p = (rows + 31) / 32 * 32, ksp = (ks + 7) / 8 * 8;
   const int64_t n = rows_p * (ksp / 4);
   if (n == 0) return hipSuccess;
+  if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 7) == 0 &&
+      ((uintptr_t)src & 7) == 0 && rows < ((int64_t)1 << 31) && ks < ((int64_t)1 << 31) && rows_p / 32 <= 65535) {
+    dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)(rows_p / 32), 1);
+    scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, (int)ks);
+    return hipGetLastError();
+  }
   scale_convert_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(src, src_layout, dst, dst_layout, rows,
                                                                         ks, rows_p, ksp);
   return hipGetLastError();

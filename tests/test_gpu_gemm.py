@@ -234,3 +234,34 @@ def test_bad_arguments_raise():
         wave_amd.mxfp4_gemm(x, xs, w_t, ws, out[:32])               # out shape
     with pytest.raises(ValueError):
         wave_amd.mxfp4_gemm(x.float(), xs, w_t, ws, out)            # operand dtype
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("vname", ["t256x256_w2x2", "t256x256_w4x2"])
+@pytest.mark.parametrize("shape", [(4352, 4352, 768), (4608, 4352, 1024)], ids=lambda s: "x".join(map(str, s)))
+def test_persistent_path_more_tiles_than_cus(shape, vname, out_dtype):
+    """More 256x256 tiles than workgroups: some workgroups compute two or three
+    tiles in a row, with the operand stream running across the tile boundary
+    and the C stores of one tile in flight under the next (scales reach the
+    kernel in MFMA32 order through the scratch pre-pass)."""
+    m, n, k = shape
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + k, scale_lo=118, scale_hi=136)
+    rng = np.random.default_rng(7)
+    rows = np.unique(np.concatenate([rng.integers(0, m, size=40), [0, 255, 256, m - 257, m - 256, m - 1]]))
+    ref_rows = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    naive = run_gemm(x, xs, w_t, ws, torch.float32, variant=_lib.VARIANT_NAIVE)
+    assert_f32_close(naive[rows], ref_rows, "naive vs oracle rows")
+    v = TILE_VARIANTS[vname]
+    got = run_gemm(x, xs, w_t, ws, out_dtype, variant=v)
+    assert_close(got[rows], ref_rows, out_dtype, "persistent vs oracle rows")
+    assert_close(got, naive, out_dtype, "persistent vs naive, all elements")
+    # preshuffled B and caller-provided MFMA32 scales take the same path
+    gx, gw = to_gpu(x, w_t)
+    gwp = wave_amd.b_preshuffle(gw).cpu().numpy()
+    got = run_gemm(x, orc.mfma32_scale_layout(xs), gwp, orc.mfma32_scale_layout(ws), out_dtype, variant=v,
+                   a_scale_layout=_lib.SCALE_MFMA32, b_scale_layout=_lib.SCALE_MFMA32, b_layout=_lib.B_PRESHUFFLE,
+                   workspace=False)
+    assert_close(got, naive, out_dtype, "persistent, preshuffled B, MFMA32 scales")
+    # and twice in a row into the same output (stale stores must not land late)
+    got2 = run_gemm(x, xs, w_t, ws, out_dtype, variant=v)
+    assert np.array_equal(got2, run_gemm(x, xs, w_t, ws, out_dtype, variant=v))

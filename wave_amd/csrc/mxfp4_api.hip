@@ -257,7 +257,8 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     tile_variant_shape(v, &bm, &bn);
     p.tiles_m = (int)((m + bm - 1) / bm);
     p.tiles_n = (int)((n + bn - 1) / bn);
-    e = launch_tile_gemm(p, v, stream);
+    e = persist_gemm_applies(p, v, device_cus()) ? launch_persist_gemm(p, v, device_cus(), stream)
+                                                 : launch_tile_gemm(p, v, stream);
   }
   if (e != hipSuccess) return record_hip(e);
   if (splits > 1) e = launch_splitk_reduce(p.partial, c, m * n, splits, p.out_bf16, stream);

@@ -1,0 +1,426 @@
+// Persistent tiled MXFP4 GEMM for gfx950 (MI355X): the large-shape fast path.
+//
+// Same tile machinery as the one-tile-per-workgroup kernel (256x256x256 tile,
+// v_mfma_scale_f32_32x32x64_f8f6f4, five-slot LDS ring filled by 16-byte DMA,
+// scales in the MFMA-native order), but one workgroup per CU walks a sequence
+// of output tiles, and the operand stream does not stop at a tile boundary:
+// while the last two K tiles of a tile are multiplied, the first two K tiles
+// of the NEXT tile are already being fetched, so a new tile starts without the
+// 3-4 us it otherwise takes to launch a workgroup and fill the ring.  The C
+// tile is written from a single free ring slot (32 KB for the workgroup,
+// passes of 32 rows through LDS so that every store instruction writes whole
+// lines), and those stores are left in flight under the MFMAs of the next
+// tile.  Vector memory operations retire in issue order (loads and stores
+// share vmcnt), so the first wait of the new tile allows for the stores
+// behind the loads it needs; from the second K tile on the stores must have
+// drained, which by then they have had a whole K tile of time to do.
+//
+// Taken for M % 256 == 0, N % 256 == 0, K % 256 == 0, K >= 768, MFMA-native
+// scales for both operands, no grouping, no split.  Everything else runs the
+// one-tile-per-workgroup kernel.  The reference writes one tile per workgroup
+// (wave_lang/kernel/wave/templates/tagged_mxfp4_gemm.py:38-145); the result
+// contract is the same.
+#include <type_traits>
+
+#include "mxfp4_tile_common.h"
+
+namespace wave_mxfp4 {
+
+enum KtKind {
+  kSteady = 0,  // K tiles j+1, j+2 belong to this output tile
+  kFirst = 1,   // first K tile of an output tile (B(1) was fetched whole ahead of it)
+  kBound1 = 2,  // K tile j+2 is K tile 0 of the next output tile
+  kBound2 = 3   // K tiles j+1, j+2 are K tiles 0, 1 of the next output tile
+};
+
+// OUT_BF16 is a template parameter so that the C stores are straight-line code:
+// behind a run-time branch the compiler's wait insertion has to assume the
+// store-free path and waits for the stores long before it must.
+template <class Cfg, bool OUT_BF16>
+__device__ __forceinline__ void persist_body(const GemmParams &p) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
+  constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
+  constexpr int SLOT = Cfg::SLOT_BYTES, RING = Cfg::RING_SLOTS;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
+  const int kp = p.kp, nkt = p.k_tiles;
+  const int total = p.tiles_m * p.tiles_n;
+  const int padded = (total + kNumXcd - 1) / kNumXcd * kNumXcd;
+  const int k_tiles_blocks = (p.ksp >> 3) * 256;  // bytes of one 32-row scale tile row
+
+  // ---------------- the tile sequence of this workgroup ----------------
+  // Workgroup w takes ids w, w + grid, w + 2*grid, ...: the grid is a multiple
+  // of the XCD count, so all of them map to the same XCD's run of tiles.
+  const uint8_t *a_base[2], *b_base[2], *as_base[2], *bs_base[2];
+  int m0[2], n0[2];
+  auto set_tile = [&](int which, int pid) -> bool {
+    int tm, tn;
+    if (pid >= padded || !map_tile(pid, p.tiles_m, p.tiles_n, tm, tn)) return false;
+    m0[which] = tm * BM;
+    n0[which] = tn * BN;
+    a_base[which] = p.a + (int64_t)m0[which] * kp;
+    b_base[which] = p.b + (int64_t)n0[which] * kp;
+    as_base[which] = p.a_scale + (int64_t)(m0[which] >> 5) * k_tiles_blocks;
+    bs_base[which] = p.b_scale + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
+    return true;
+  };
+  int pid = blockIdx.x;
+  if (!set_tile(0, pid)) return;
+
+  // ---------------- global -> LDS addressing (see the one-tile kernel) ----------------
+  const int ld_row0 = wave * 8 + (lane >> 3);
+  const int ld_chunk = (lane & 7) ^ ((ld_row0 >> 1) & 7);
+  // DMA instruction d of a wave fills rows 8*NWAVES*d further down: one per-lane
+  // offset per operand, the rest is scalar (registers are what this kernel is short of).
+  const int a_goff = ld_row0 * kp + ld_chunk * 16;
+  const int b_goff = p.b_preshuffled ? (ld_row0 >> 4) * 16 * kp + (ld_row0 & 15) * 16 + (ld_chunk >> 1) * 512 +
+                                           (ld_chunk & 1) * 256
+                                     : ld_row0 * kp + ld_chunk * 16;
+  const int ld_step = NWAVES * 8 * kp;  // bytes between consecutive d, either layout (8*NWAVES is a multiple of 16)
+  const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
+
+  // DMA instructions [d0, d1) of operand `op` (0 = A, 1 = B), K tile `kt` of
+  // output tile `which` (0 = current, 1 = next), into ring slot `slot`.
+  auto issue_g2l = [&](int which, int op, int kt, int slot, int d0, int d1) {
+    uint8_t *dst_tile = smem + slot * SLOT;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(op == 0 ? a_base[which] : b_base[which]);
+    const int soff = op == 0 ? kt * kTileKBytes : kt * b_kt_stride;
+#pragma unroll
+    for (int d = d0; d < d1; ++d) {
+      uint8_t *dst = dst_tile + (d * NWAVES + wave) * 1024;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, WAVE_LDS_PTR(dst), 16, op == 0 ? a_goff : b_goff,
+                                               soff + d * ld_step, 0, 0);
+    }
+  };
+
+  // ---------------- fragments ----------------
+  const int fr = lane & 31, fg = lane >> 5;
+  uint32_t foff[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) foff[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
+  const uint32_t a_fbase = (uint32_t)(wave_m * Cfg::WM * kTileKBytes);
+  const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
+  auto read_frags = [&](int slot_a, int slot_b, int t, v4i(&fa)[MT_M], v4i(&fb)[MT_N]) {
+    const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
+    const uint8_t *bb = smem + slot_b * SLOT + b_fbase + foff[t];
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(ba + i * 32 * kTileKBytes);
+#pragma unroll
+    for (int j = 0; j < MT_N; ++j) fb[j] = *(const v4i *)(bb + j * 32 * kTileKBytes);
+  };
+
+  // ---------------- scales (MFMA-native order: one dword per lane, 32 rows and K tile) ----------------
+  const int a_srow = ((wave_m * Cfg::WM) >> 5) * k_tiles_blocks, b_srow = ((wave_n * Cfg::WN) >> 5) * k_tiles_blocks;
+  const int s_lane = lane * 4;
+  uint32_t raw_a[MT_M], raw_b[MT_N], sc_a[MT_M], sc_b[MT_N];
+  auto load_scales = [&](int which, int kt) {
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(as_base[which]), rb = make_rsrc(bs_base[which]);
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i)
+      raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, s_lane, a_srow + i * k_tiles_blocks + kt * 256, 0);
+#pragma unroll
+    for (int j = 0; j < MT_N; ++j)
+      raw_b[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + kt * 256, 0);
+  };
+  // Real register moves, pinned here (a compiler copy would be folded into the
+  // loop's phi and wait for the next scale load at the top of every iteration).
+  auto canon_scales = [&]() {
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_a[i]) : "v"(raw_a[i]));
+#pragma unroll
+    for (int j = 0; j < MT_N; ++j) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_b[j]) : "v"(raw_b[j]));
+  };
+
+  // ---------------- accumulators and MFMA ----------------
+  v16f acc[MT_M][MT_N];  // started from 0 by the first K step of every tile
+
+  // ZERO: start the tile's sums from 0 (the first K step of a new output tile).
+  auto mfma_block = [&](const v4i(&fa)[MT_M], const v4i(&fb)[MT_N], auto t_tag, auto zero_tag) {
+    constexpr int T = decltype(t_tag)::value;
+    constexpr bool ZERO = decltype(zero_tag)::value;
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+      const v8i va = {fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < MT_N; ++j) {
+        const v8i vb = {fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
+        v16f c = acc[i][j];
+        if (ZERO) {
+#pragma unroll
+          for (int g = 0; g < 16; ++g) c[g] = 0.f;
+        }
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, c, 4, 4, T, (int)sc_b[j], T, (int)sc_a[i]);
+      }
+    }
+  };
+  typedef std::integral_constant<int, 0> T0;
+  typedef std::integral_constant<int, 1> T1;
+  typedef std::integral_constant<int, 2> T2;
+  typedef std::integral_constant<int, 3> T3;
+
+  constexpr int HALF_LD = (A_LD < B_LD ? A_LD : B_LD) / 2;
+  constexpr int NGROUP = HALF_LD < 1 ? 1 : HALF_LD;
+  auto order_phase = [&]() {
+    constexpr int R = MT_M + MT_N, Q = MT_M * MT_N;
+    constexpr int RG = (R + NGROUP - 1) / NGROUP, QG = Q / NGROUP;
+#pragma unroll
+    for (int g = 0; g < NGROUP; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, RG, 0);
+      if (QG > 1) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      if (QG > 2) __builtin_amdgcn_sched_group_barrier(0x008, QG - 2, 0);
+    }
+  };
+
+  // C store instructions per wave and tile (1 KB each)
+  constexpr int NS_BF16 = Cfg::WM * Cfg::WN * 2 / 1024, NS_F32 = Cfg::WM * Cfg::WN * 4 / 1024;
+  constexpr int kWaitFirstBf16 = NS_BF16 + A_LD > 63 ? 63 : NS_BF16 + A_LD;
+  constexpr int kWaitFirstF32 = NS_F32 + A_LD > 63 ? 63 : NS_F32 + A_LD;
+  constexpr bool out_bf16 = OUT_BF16;
+
+  // ---------------- one K tile (phases as in the one-tile kernel) ----------------
+  //   P0: second half of B(j+1)      P1, P2: A(j+2)      P3: barrier, first half of B(j+2)
+  // with (j+1), (j+2) running on into the next output tile at a boundary.
+  v4i fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  // PENDING: the C stores of the previous output tile are in the queue (every tile but the first).
+  auto k_tile = [&](int j, int sa, int sb, auto kind_tag, auto pending_tag) {
+    constexpr int KIND = decltype(kind_tag)::value;
+    constexpr bool PENDING = decltype(pending_tag)::value;
+    constexpr int W1 = KIND == kBound2 ? 1 : 0;                      // output tile of K tile j+1
+    constexpr int W2 = (KIND == kBound1 || KIND == kBound2) ? 1 : 0;  // ... of K tile j+2
+    const int kt1 = KIND == kBound2 ? 0 : j + 1;
+    const int kt2 = KIND == kBound1 ? 0 : KIND == kBound2 ? 1 : j + 2;
+    typedef std::integral_constant<bool, KIND == kFirst> Zero;
+    typedef std::false_type Keep;
+    const int sa1 = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
+    const int sb1 = sa + 3 >= RING ? sa + 3 - RING : sa + 3;
+    const int sa2 = sa + 4 >= RING ? sa + 4 - RING : sa + 4;
+    read_frags(sa, sb, 1, fa1, fb1);
+    mfma_block(fa0, fb0, T0{}, Zero{});
+    if (KIND != kFirst) issue_g2l(W1, 1, kt1, sb1, B_LD / 2, B_LD);
+    order_phase();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(sa, sb, 2, fa0, fb0);
+    mfma_block(fa1, fb1, T1{}, Keep{});
+    issue_g2l(W2, 0, kt2, sa2, 0, A_LD / 2);
+    order_phase();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(sa, sb, 3, fa1, fb1);
+    mfma_block(fa0, fb0, T2{}, Keep{});
+    issue_g2l(W2, 0, kt2, sa2, A_LD / 2, A_LD);
+    order_phase();
+    __builtin_amdgcn_sched_barrier(0);
+    // Everything this wave issued up to B(j+1) has landed.  Younger than that:
+    // the A_LD instructions of A(j+2) and, in the first K tile after a
+    // boundary, the C stores of the previous output tile.
+    if (KIND == kFirst && PENDING) {
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(OUT_BF16 ? kWaitFirstBf16 : kWaitFirstF32));
+    } else {
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(A_LD));
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(sa1, sb1, 0, fa0, fb0);
+    mfma_block(fa1, fb1, T3{}, Keep{});
+    issue_g2l(W2, 1, kt2, sa, 0, B_LD / 2);
+    order_phase();
+    __builtin_amdgcn_sched_barrier(0);
+    canon_scales();
+    load_scales(W2, kt2);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // ---------------- C tile: accumulators -> one ring slot -> global ----------------
+  // acc[i][jn][4q + e] is row lane%32, column 8q + 4*(lane/32) + e of the 32x32
+  // tile (i, jn).  Each wave owns 1/NWAVES of the slot: 32 rows whose 16-byte
+  // chunk c sits at position c ^ (row % chunks per row) (conflict-free 16-byte
+  // reads, two-way on the 8-byte writes), written pass by pass and read back as
+  // whole rows, 16 bytes per lane.
+  auto store_tile = [&](int slot, int tm0, int tn0) {
+    constexpr int SW = SLOT / NWAVES;  // staging bytes of a wave
+    constexpr int RP = SW / 32;        // row pitch
+    constexpr int NCH = RP / 16;       // chunks per row
+    constexpr int LPR = NCH, RPI = 64 / LPR;
+    uint8_t *stage = smem + slot * SLOT + wave * SW;
+    const int wm0 = tm0 + wave_m * Cfg::WM, wn0 = tn0 + wave_n * Cfg::WN;
+    // Staging addresses are recomputed from the lane id at every tile: hoisted
+    // out of the tile loop they would sit in registers through the main loop,
+    // which has none to spare (a spill there costs a wait for the whole queue).
+    int lane_v = lane;
+    asm volatile("" : "+v"(lane_v));
+    const int fr = lane_v & 31, fg = lane_v >> 5;
+    const int lr = lane_v / LPR, lc = lane_v % LPR;
+    const int64_t ldc = p.n;
+    if (out_bf16) {
+      constexpr int CP = RP / 2, JP = CP / 32;  // columns, 32-column tiles per pass
+      typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+      __bf16 *cbase = (__bf16 *)p.c;
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) {
+#pragma unroll
+        for (int jg = 0; jg < MT_N / JP; ++jg) {
+#pragma unroll
+          for (int jj = 0; jj < JP; ++jj) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const v16f &a = acc[i][jg * JP + jj];
+              const bf4 h = {(__bf16)a[4 * q], (__bf16)a[4 * q + 1], (__bf16)a[4 * q + 2], (__bf16)a[4 * q + 3]};
+              const int chunk = jj * 4 + q;
+              *(bf4 *)(stage + fr * RP + ((chunk ^ (fr & (NCH - 1))) << 4) + fg * 8) = h;
+            }
+          }
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int r0 = 0; r0 < 32; r0 += RPI) {
+            const int r = r0 + lr;
+            const v4i v = *(const v4i *)(stage + r * RP + ((lc ^ (r & (NCH - 1))) << 4));
+            *(v4i *)(cbase + (int64_t)(wm0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 8) = v;
+          }
+          asm volatile("" ::: "memory");
+        }
+      }
+    } else {
+      constexpr int CP = RP / 4, JP = CP / 32;
+      float *cbase = (float *)p.c;
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) {
+#pragma unroll
+        for (int jg = 0; jg < MT_N / JP; ++jg) {
+#pragma unroll
+          for (int jj = 0; jj < JP; ++jj) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const v16f &a = acc[i][jg * JP + jj];
+              const v4f v = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+              const int chunk = jj * 8 + q * 2 + fg;
+              *(v4f *)(stage + fr * RP + ((chunk ^ (fr & (NCH - 1))) << 4)) = v;
+            }
+          }
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int r0 = 0; r0 < 32; r0 += RPI) {
+            const int r = r0 + lr;
+            const v4f v = *(const v4f *)(stage + r * RP + ((lc ^ (r & (NCH - 1))) << 4));
+            *(v4f *)(cbase + (int64_t)(wm0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 4) = v;
+          }
+          asm volatile("" ::: "memory");
+        }
+      }
+    }
+  };
+
+  // ---------------- prologue of the first tile ----------------
+  issue_g2l(0, 0, 0, 0, 0, A_LD);
+  issue_g2l(0, 1, 0, 1, 0, B_LD);
+  load_scales(0, 0);
+  issue_g2l(0, 0, 1, 2, 0, A_LD);
+  issue_g2l(0, 1, 1, 3, 0, B_LD);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(A_LD + B_LD));
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  canon_scales();
+  load_scales(0, 1);
+  read_frags(0, 1, 0, fa0, fb0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---------------- the tiles ----------------
+  // After the last tile the stream simply runs on into a repeat of that tile's
+  // first two K tiles (valid memory, never multiplied): one code path, no drain.
+  // The first tile is peeled off the loop: with it inside, the compiler's own
+  // waits (for the scale registers) would have to assume its store-free queue
+  // for every tile.
+  int sa = 0;
+  auto next_slot = [&](int s) { return s + 2 >= RING ? s + 2 - RING : s + 2; };
+  auto b_slot = [&](int s) { return s + 1 >= RING ? 0 : s + 1; };
+  auto run_tile = [&](auto pending_tag) -> bool {
+    const int npid = pid + (int)gridDim.x;
+    const bool has_next = set_tile(1, npid);
+    if (!has_next) {
+      m0[1] = m0[0], n0[1] = n0[0];
+      a_base[1] = a_base[0], b_base[1] = b_base[0], as_base[1] = as_base[0], bs_base[1] = bs_base[0];
+    }
+    k_tile(0, sa, b_slot(sa), std::integral_constant<int, kFirst>{}, pending_tag);
+    sa = next_slot(sa);
+    for (int j = 1; j < nkt - 2; ++j) {
+      k_tile(j, sa, b_slot(sa), std::integral_constant<int, kSteady>{}, pending_tag);
+      sa = next_slot(sa);
+    }
+    k_tile(nkt - 2, sa, b_slot(sa), std::integral_constant<int, kBound1>{}, pending_tag);
+    sa = next_slot(sa);
+    const int stage_slot = b_slot(sa);
+    k_tile(nkt - 1, sa, stage_slot, std::integral_constant<int, kBound2>{}, pending_tag);
+    // second half of B(1) of the next tile, ahead of the C stores (its first
+    // half went into slot `sa` in the last phase above)
+    issue_g2l(1, 1, 1, sa, B_LD / 2, B_LD);
+    sa = next_slot(sa);
+    __builtin_amdgcn_sched_barrier(0);
+    store_tile(stage_slot, m0[0], n0[0]);
+    if (!has_next) return false;
+    // the staging slot is the next target of the A stream: all waves must be done reading it
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    pid = npid;
+    m0[0] = m0[1], n0[0] = n0[1];
+    a_base[0] = a_base[1], b_base[0] = b_base[1], as_base[0] = as_base[1], bs_base[0] = bs_base[1];
+    return true;
+  };
+  if (run_tile(std::false_type{})) {
+    while (run_tile(std::true_type{})) {
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // the trailing DMA must not outlive the workgroup's LDS
+}
+
+template <class Cfg, bool OUT_BF16>
+__global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_kernel(const GemmParams p) {
+  persist_body<Cfg, OUT_BF16>(p);
+}
+
+template <class Cfg, bool OUT_BF16>
+static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_t stream) {
+  static bool attr_done = false;  // benign race: the attribute is idempotent
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  persist_gemm_kernel<Cfg, OUT_BF16><<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  return hipGetLastError();
+}
+
+template <class Cfg>
+static hipError_t launch_persist_cfg(const GemmParams &p, int grid_x, hipStream_t stream) {
+  return p.out_bf16 ? launch_persist_out<Cfg, true>(p, grid_x, stream) : launch_persist_out<Cfg, false>(p, grid_x, stream);
+}
+
+// Whether the persistent kernel serves this problem with `num_cus` CUs.
+bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
+  if (variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 && variant != WAVE_MXFP4_VARIANT_T256x256_W4x2) return false;
+  if (p.num_groups != 0 || p.splits != 1 || p.partial != nullptr) return false;
+  if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  if ((p.m & 255) != 0 || (p.n & 255) != 0 || (p.k & (kTileK - 1)) != 0 || p.k_tiles < 3) return false;
+  if (p.out_bf16 ? (p.n & 7) != 0 : (p.n & 3) != 0) return false;
+  // 32-bit offsets inside one operand tile, and more tiles than workgroups
+  if ((int64_t)256 * p.kp >= ((int64_t)1 << 31)) return false;
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  return grid >= kNumXcd && (int64_t)p.tiles_m * p.tiles_n > grid;
+}
+
+hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream) {
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_persist_cfg<TileCfg<256, 256, 2, 2>>(p, grid, stream);
+  return launch_persist_cfg<TileCfg<256, 256, 4, 2>>(p, grid, stream);
+}
+
+}  // namespace wave_mxfp4

@@ -171,7 +171,7 @@ def main():
         achieved = flops / per_launch / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_MXFP4_TFLOPS,
                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_MXFP4_TFLOPS, 4), "traffic": measured_traffic,
-                    "kernel": "tile_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
+                    "kernel": "persist_gemm_kernel" if (m % 256 == 0 and n % 256 == 0 and (m // 256) * (n // 256) > 256) else "tile_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
 
     result = {
         "metric": "MXFP4 GEMM TFLOPS + % of FP4 MFMA peak (8192^3); GB/s % HBM at M=16",

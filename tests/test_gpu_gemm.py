@@ -265,3 +265,32 @@ def test_persistent_path_more_tiles_than_cus(shape, vname, out_dtype):
     # and twice in a row into the same output (stale stores must not land late)
     got2 = run_gemm(x, xs, w_t, ws, out_dtype, variant=v)
     assert np.array_equal(got2, run_gemm(x, xs, w_t, ws, out_dtype, variant=v))
+
+
+@pytest.mark.parametrize("m,n", [(3, 69648), (16, 36864), (33, 40976), (64, 36880)])
+@pytest.mark.parametrize("layout", ["row_major", "mfma32_preshuffled"])
+def test_streaming_kernel_many_tiles_per_workgroup(m, n, layout):
+    """K = 8192 decode shapes whose N gives every workgroup more 16-row tiles
+    of B than it can hold finished sums for (8), so that C is also written in
+    the middle of the stream, with a ragged last tile and an uneven split of
+    tiles over workgroups."""
+    k = 8192
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=n + m, scale_lo=120, scale_hi=134)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    if layout == "row_major":
+        got = run_gemm(x, xs, w_t, ws, torch.bfloat16, variant=_lib.VARIANT_SKINNY)
+        assert_bf16_close(got, ref, "row-major")
+        got = run_gemm(x, xs, w_t, ws, torch.float32, variant=_lib.VARIANT_SKINNY)
+        assert_f32_close(got, ref, "row-major f32")
+    else:
+        (gw,) = to_gpu(w_t)
+        gwp = wave_amd.b_preshuffle(gw).cpu().numpy()
+        got = run_gemm(x, orc.mfma32_scale_layout(xs), gwp, orc.mfma32_scale_layout(ws), torch.float32,
+                       variant=_lib.VARIANT_SKINNY, a_scale_layout=_lib.SCALE_MFMA32,
+                       b_scale_layout=_lib.SCALE_MFMA32, b_layout=_lib.B_PRESHUFFLE)
+        assert_f32_close(got, ref, "MFMA32 scales, preshuffled B")
+        got = run_gemm(x, orc.e8m0_shuffle_padded(xs)[:(m + 31) // 32 * 32], w_t,
+                       orc.e8m0_shuffle_padded(ws)[:(n + 31) // 32 * 32], torch.bfloat16,
+                       variant=_lib.VARIANT_SKINNY, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
+                       b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
+        assert_bf16_close(got, ref, "shuffled scales")

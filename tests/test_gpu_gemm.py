@@ -294,3 +294,34 @@ def test_streaming_kernel_many_tiles_per_workgroup(m, n, layout):
                        variant=_lib.VARIANT_SKINNY, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
                        b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
         assert_bf16_close(got, ref, "shuffled scales")
+
+
+@pytest.mark.parametrize("k", [1024, 2048, 3072, 4096, 5120, 7168])
+@pytest.mark.parametrize("m", [5, 17])
+def test_streaming_kernel_fewer_k_tiles_per_wave(m, k):
+    """Decode shapes whose K gives each of the four waves 1..7 K tiles instead
+    of 8 (odd counts start odd waves on an odd K tile), in every scale layout;
+    NaN scales at the very end of a row must poison exactly their row/column,
+    also where lanes past the wave's range re-fetch that end."""
+    n = 8208
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=k + m, scale_lo=120, scale_hi=134)
+    ws[3, -1] = 255
+    ws[n - 1, -1] = 255
+    xs[m - 1, -1] = 255
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    assert np.isnan(ref[:, 3]).all() and np.isnan(ref[m - 1]).all() and not np.isnan(ref[0, 0])
+    got = run_gemm(x, xs, w_t, ws, torch.float32, variant=_lib.VARIANT_SKINNY)
+    assert_f32_close(got, ref, "row-major")
+    got = run_gemm(x, xs, w_t, ws, torch.bfloat16)
+    assert_bf16_close(got, ref, "row-major, auto, bf16")
+    (gw,) = to_gpu(w_t)
+    gwp = wave_amd.b_preshuffle(gw).cpu().numpy()
+    got = run_gemm(x, orc.mfma32_scale_layout(xs), gwp, orc.mfma32_scale_layout(ws), torch.float32,
+                   variant=_lib.VARIANT_SKINNY, a_scale_layout=_lib.SCALE_MFMA32,
+                   b_scale_layout=_lib.SCALE_MFMA32, b_layout=_lib.B_PRESHUFFLE)
+    assert_f32_close(got, ref, "MFMA32 scales, preshuffled B")
+    got = run_gemm(x, orc.e8m0_shuffle_padded(xs)[:(m + 31) // 32 * 32], w_t,
+                   orc.e8m0_shuffle_padded(ws)[:(n + 31) // 32 * 32], torch.float32,
+                   variant=_lib.VARIANT_SKINNY, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
+                   b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
+    assert_f32_close(got, ref, "shuffled scales")

@@ -61,7 +61,7 @@ __device__ __forceinline__ void stream_wait_vm() {
   __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// FULL: every wave owns exactly 8 whole K tiles and the scale rows are whole
+// FULL: every wave owns the same number (1..8) of whole K tiles and the scale rows are whole
 // 16-byte pieces, so every B tile costs the same number of DMA instructions,
 // nothing is predicated and waits can be counted.  Otherwise (K tails, fewer
 // K tiles) the same pipeline runs with predicated loads and full waits.
@@ -83,12 +83,14 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const int split = blockIdx.y;
   const int kt_begin = split * p.tiles_per_split;
   const int nkt = min(p.k_tiles, kt_begin + p.tiles_per_split) - kt_begin;
-  const int ktw = FULL ? kStreamKtPerWave : (nkt + kStreamWaves - 1) / kStreamWaves;  // <= kStreamKtPerWave
+  const int ktw = FULL ? nkt / kStreamWaves : (nkt + kStreamWaves - 1) / kStreamWaves;  // <= kStreamKtPerWave
   const int kt0 = kt_begin + wave * ktw;
-  const int my_nkt = FULL ? kStreamKtPerWave : max(0, min(ktw, kt_begin + nkt - kt0));
+  const int my_nkt = FULL ? ktw : max(0, min(ktw, kt_begin + nkt - kt0));
 
   const int kp = p.kp;
   const v4i zero = {0, 0, 0, 0};
+  // row-major scale pieces start 16-byte aligned: 8 bytes in front of the wave's first K tile if that is odd
+  const int sc_shift = FULL ? (kt0 & 1) * 8 : 0;
   const int tail_chunks = FULL ? 0 : (p.k & (kTileK - 1)) >> 5;  // valid chunks of a partial last K tile
   auto chunk_ok = [&](int kt, int chunk) {
     return FULL || tail_chunks == 0 || kt != p.k_tiles - 1 || chunk < tail_chunks;
@@ -104,18 +106,22 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const bool bpre = p.b_preshuffled != 0;
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t *>(p.b + (int64_t)nt_begin * 16 * kp), 0, 0x7FFFFFFF, 0x00020000);
+  const int b_voff = bpre ? lane * 16 : min(lane, ktw * 8 - 1) * 16;
   auto issue_rows = [&](int nt, int buf) {
     uint8_t *dst = lds.tile[wave][buf];
     const int tile_off = (nt - nt_begin) * 16 * kp;
     const int row_lim = p.n - 1 - nt * 16;
     if (FULL) {
       // one instruction per i, no control flow: the two layouts differ in scalars only
+      // With fewer than 8 K tiles per wave the lanes (row-major) or instructions
+      // (preshuffled) past the wave's range fetch its last chunk or K tile again:
+      // always the same 16 instructions, and what lands there meets zeros of A.
       const int pitch = bpre ? 1024 : kStreamRowPitch;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int soff = bpre ? tile_off + ((kt0 + (i >> 1)) * 4 + (i & 1) * 2) * 512
+        const int soff = bpre ? tile_off + ((kt0 + min(i >> 1, ktw - 1)) * 4 + (i & 1) * 2) * 512
                               : tile_off + min(i, row_lim) * kp + kt0 * kTileKBytes;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * pitch), 16, lane * 16, soff, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * pitch), 16, b_voff, soff, 0, 0);
       }
     } else if (bpre) {
 #pragma unroll
@@ -150,7 +156,8 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   //   row-major : 16 rows x 64 bytes starting at group kt0*8, stored piece-major (lane t -> row
   //               t%16, 16-byte piece t/16, so the 16 rows of a piece are 256 contiguous bytes and
   //               the reads below are conflict-free); K tiles 2q, 2q+1 of row fr are the 16 bytes
-  //               at q*256 + fr*16, step s of K tile j byte fg of dword (j%2)*2 + s.
+  //               at q*256 + fr*16, step s of K tile j byte fg of dword (j%2)*2 + s (one pair of
+  //               dwords later when the wave's first K tile is odd: see the alignment note below).
   //   MFMA32    : of each of the 8 consecutive 256-byte blocks (32 rows x one K tile) the two
   //               64-byte runs that hold this tile's 16 rows (lane t -> block t/8, piece t%8);
   //               K tile j of row r is the dword at j*128 + (fg&1)*64 + (r%16)*4, whose bytes
@@ -170,15 +177,20 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     const int blocked_off = (n0 >> 5) * sc_block_row_bytes + kt0 * 256;
     if (FULL) {
       // one instruction whatever the layout, a second one for the shuffled blocks
+      // (pieces and blocks past the wave's K tiles repeat its last one, and nothing is read past the tensor)
       const int row = min(n0 + (lane & 15), p.n - 1);
-      const int off_rm = row * p.ks + kt0 * 8 + (lane >> 4) * 16;
-      const int off_native = blocked_off + (lane >> 3) * 256 + ((lane & 7) >> 2) * 128 + ((n0 >> 4) & 1) * 64 +
-                             (lane & 3) * 16;
-      const int off_shuf = blocked_off + lane * 16;
+      // (the DMA wants 16-byte aligned sources: an odd first K tile starts its image 8 bytes early)
+      // (the last wave's pieces end exactly at the end of the row, so nothing is read past the tensor)
+      const int off_rm = row * p.ks + kt0 * 8 - sc_shift + min(lane >> 4, (sc_shift + ktw * 8 - 1) >> 4) * 16;
+      const int off_native = blocked_off + min(lane >> 3, ktw - 1) * 256 + ((lane & 7) >> 2) * 128 +
+                             ((n0 >> 4) & 1) * 64 + (lane & 3) * 16;
+      const int off_shuf = blocked_off + min(lane >> 4, ktw - 1) * 256 + (lane & 15) * 16;
       const int off = bsl == WAVE_MXFP4_SCALE_ROW_MAJOR ? off_rm : bsl == WAVE_MXFP4_SCALE_MFMA32 ? off_native : off_shuf;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, off, 0, 0, 0);
-      if (bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst + 1024), 16, off, 1024, 0, 0);
+      if (bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {
+        const int off2 = blocked_off + min(4 + (lane >> 4), ktw - 1) * 256 + (lane & 15) * 16;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst + 1024), 16, off2, 0, 0, 0);
+      }
     } else if (bsl == WAVE_MXFP4_SCALE_ROW_MAJOR) {
       const int row = min(n0 + (lane & 15), p.n - 1);
       const int64_t off = (int64_t)row * p.ks + (int64_t)kt0 * 8 + (lane >> 4) * 16;
@@ -256,22 +268,27 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       const int ao1 = min(i * 16 + 8 + (lane >> 3), p.m - 1) * kp + (lane & 7) * 16;
 #pragma unroll
       for (int j = 0; j < kStreamKtPerWave; ++j) {
-        a_frag[i][j][0] = load_b128(a_rsrc, ao0, (kt0 + j) * kTileKBytes);
-        a_frag[i][j][1] = load_b128(a_rsrc, ao1, (kt0 + j) * kTileKBytes);
+        a_frag[i][j][0] = load_b128(a_rsrc, ao0, (kt0 + min(j, ktw - 1)) * kTileKBytes);
+        a_frag[i][j][1] = load_b128(a_rsrc, ao1, (kt0 + min(j, ktw - 1)) * kTileKBytes);
       }
       // Both scale shapes are loaded, the one that does not apply from offset
       // 0: separate code paths per layout would make the compiler guard the
       // registers of the other path with waits in front of the stream.
       const bool rm = asl == WAVE_MXFP4_SCALE_ROW_MAJOR;
       // row-major: lane t holds row t/4, bytes 16*(t%4) .. +15 of the wave's 64 = K tiles 2*(t%4), 2*(t%4)+1
-      a_sq[i] = load_b128(as_rsrc, rm ? min(i * 16 + (lane >> 2), p.m - 1) * p.ks + (lane & 3) * 16 : 0, rm ? kt0 * 8 : 0);
+      // (16-byte aligned like the image of B's scales: 8 bytes early when the wave's first K tile is odd)
+      a_sq[i] = load_b128(as_rsrc,
+                          rm ? min(i * 16 + (lane >> 2), p.m - 1) * p.ks + kt0 * 8 - sc_shift +
+                                   min(lane & 3, (sc_shift + ktw * 8 - 1) >> 4) * 16
+                             : 0,
+                          0);
       // blocked: the dword of block (row/32, K tile) that holds this lane's two scale bytes
       const int row = i * 16 + fr;  // rows up to the next multiple of 32 exist in blocked layouts
       const int in_blk = asl == WAVE_MXFP4_SCALE_MFMA32 ? (((fg & 1) << 5) | (row & 31)) * 4 : fg * 64 + (row & 15) * 4;
       const int so = rm ? 0 : (row >> 5) * (p.ksp >> 3) * 256 + in_blk;
 #pragma unroll
       for (int j = 0; j < kStreamKtPerWave; ++j)
-        a_sc[i][j][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, so, rm ? 0 : (kt0 + j) * 256, 0);
+        a_sc[i][j][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, so, rm ? 0 : (kt0 + min(j, ktw - 1)) * 256, 0);
     }
   } else {
 #pragma unroll
@@ -346,6 +363,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
         a_frag[i][j][0] = *(const v4i *)(stage + rd);
         a_frag[i][j][1] = *(const v4i *)(stage + rd + 64);
         asm volatile("" ::: "memory");
+        if (j >= ktw) a_frag[i][j][0] = a_frag[i][j][1] = zero;  // K tiles the wave does not own
       }
       {
         // row-major: K tile j, step s of row fr is byte fg of dword (j%2)*2 + s held by lane fr*4 + j/2;
@@ -357,14 +375,23 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
         const int q[4] = {a_sq[i].x, a_sq[i].y, a_sq[i].z, a_sq[i].w};
 #pragma unroll
         for (int j = 0; j < kStreamKtPerWave; ++j) {
-          const int src = (fr * 4 + (j >> 1)) * 4;
-          const uint32_t d0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, q[(j & 1) * 2]);
-          const uint32_t d1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src, q[(j & 1) * 2 + 1]);
+          // (with the 8-byte shift K tile j is the (j+1)-th pair of dwords; both candidates are
+          // fetched and one is picked, so that no register array is indexed by a run-time value)
+          const bool sh = sc_shift != 0;
+          const int src0 = (fr * 4 + (j >> 1)) * 4, src1 = (fr * 4 + ((j + 1) >> 1)) * 4;
+          const uint32_t p0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src0, q[(j & 1) * 2]);
+          const uint32_t p1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src0, q[(j & 1) * 2 + 1]);
+          const uint32_t m0 = (uint32_t)__builtin_amdgcn_ds_bpermute(src1, q[((j + 1) & 1) * 2]);
+          const uint32_t m1 = (uint32_t)__builtin_amdgcn_ds_bpermute(src1, q[((j + 1) & 1) * 2 + 1]);
+          const uint32_t d0 = sh ? m0 : p0, d1 = sh ? m1 : p1;
           a_sc[i][j][0] = __builtin_amdgcn_perm(rm ? d1 : a_sc[i][j][0], rm ? d0 : a_sc[i][j][0], sel);
         }
       }
 #pragma unroll
-      for (int j = 0; j < kStreamKtPerWave; ++j) a_sc[i][j][1] = a_sc[i][j][0];
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        if (j >= ktw) a_sc[i][j][0] = 0x7F7Fu;
+        a_sc[i][j][1] = a_sc[i][j][0];
+      }
     }
     lds_barrier();  // the stage becomes the partial-tile area
     stream_wait_vm<17>();  // tile nt_begin has landed
@@ -439,11 +466,21 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     }
     if (sc_rowmajor) {
       const uint32_t sel = 0x0c0c0000u | (uint32_t)fg | ((uint32_t)(4 + fg) << 8);
+      uint32_t d[18];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const v4i d = *(const v4i *)(sc_img + q * 256 + fr * 16);
-        scb[2 * q] = __builtin_amdgcn_perm((uint32_t)d.y, (uint32_t)d.x, sel);
-        scb[2 * q + 1] = __builtin_amdgcn_perm((uint32_t)d.w, (uint32_t)d.z, sel);
+        const v4i v = *(const v4i *)(sc_img + q * 256 + fr * 16);
+        d[4 * q] = (uint32_t)v.x, d[4 * q + 1] = (uint32_t)v.y, d[4 * q + 2] = (uint32_t)v.z, d[4 * q + 3] = (uint32_t)v.w;
+      }
+      d[16] = d[17] = 0x7F7F7F7Fu;
+      const bool shifted = sc_shift != 0;  // K tile j then sits one dword pair further on
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) {
+        // (both candidates are formed and one is picked: an index that depends on
+        // `shifted` would put the array in scratch memory)
+        const uint32_t plain = __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], sel);
+        const uint32_t moved = __builtin_amdgcn_perm(d[2 * j + 3], d[2 * j + 2], sel);
+        scb[j] = shifted ? moved : plain;
       }
     } else {
       const bool native = bsl == WAVE_MXFP4_SCALE_MFMA32;
@@ -455,6 +492,14 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       for (int j = 0; j < kStreamKtPerWave; ++j) {
         const uint32_t d = img[j * stride];
         scb[j] = __builtin_amdgcn_perm(d, d, sel);
+      }
+    }
+
+    if (FULL) {
+      // K tiles the wave does not own: A is zero there, the scale must merely be finite
+#pragma unroll
+      for (int j = 1; j < kStreamKtPerWave; ++j) {
+        if (j >= ktw) scb[j] = 0x7F7Fu;
       }
     }
 
@@ -574,9 +619,9 @@ hipError_t launch_stream_gemm(const GemmParams &p, int num_cus, hipStream_t stre
   // ... and into A and both scale matrices (padded to 32-row blocks)
   if ((int64_t)p.m * p.kp >= ((int64_t)1 << 31) || ((int64_t)p.n + 32) * (p.ksp + 8) >= ((int64_t)1 << 31))
     return hipErrorInvalidValue;
-  // every wave of every split owns 8 whole K tiles
+  // every wave of every split owns the same number of whole K tiles
   // ... and every workgroup at least two tiles of B
-  const bool full = p.tiles_per_split == kStreamMaxKTiles && p.k_tiles % kStreamMaxKTiles == 0 &&
+  const bool full = p.tiles_per_split % kStreamWaves == 0 && p.k_tiles % p.tiles_per_split == 0 &&
                     (p.k & (kTileK - 1)) == 0 && nt_total >= 2 * grid_x;
   return full ? launch_stream_full<true>(p, grid_x, stream) : launch_stream_full<false>(p, grid_x, stream);
 }

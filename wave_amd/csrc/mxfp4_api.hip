@@ -228,18 +228,27 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? b_bytes : 0;
     if (ws_used + a_need + b_need <= workspace_bytes) {
       uint8_t *ws = (uint8_t *)workspace + ws_used;
-      if (a_need) {
-        e = launch_scale_convert(p.a_scale, p.a_scale_layout, ws, WAVE_MXFP4_SCALE_MFMA32, m, p.ks, stream);
-        if (e != hipSuccess) return record_hip(e);
+      // both operands row-major: one launch re-lays both
+      if (a_need && b_need && p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
+          p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
+          launch_scale_pair_to_mfma32(p.a_scale, ws, m, p.b_scale, ws + a_need, n, p.ks, stream) == hipSuccess) {
         p.a_scale = ws;
-        p.a_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
-        ws += a_need;
-      }
-      if (b_need) {
-        e = launch_scale_convert(p.b_scale, p.b_scale_layout, ws, WAVE_MXFP4_SCALE_MFMA32, n, p.ks, stream);
-        if (e != hipSuccess) return record_hip(e);
-        p.b_scale = ws;
-        p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+        p.b_scale = ws + a_need;
+        p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+      } else {
+        if (a_need) {
+          e = launch_scale_convert(p.a_scale, p.a_scale_layout, ws, WAVE_MXFP4_SCALE_MFMA32, m, p.ks, stream);
+          if (e != hipSuccess) return record_hip(e);
+          p.a_scale = ws;
+          p.a_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+          ws += a_need;
+        }
+        if (b_need) {
+          e = launch_scale_convert(p.b_scale, p.b_scale_layout, ws, WAVE_MXFP4_SCALE_MFMA32, n, p.ks, stream);
+          if (e != hipSuccess) return record_hip(e);
+          p.b_scale = ws;
+          p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+        }
       }
     }
   }

@@ -109,11 +109,19 @@ __global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_la
 // split with v_perm into the two dwords of its block (lanes r%32 and 32 + r%32),
 // a pass through LDS (block stride 65 dwords: conflict-free both ways), and
 // dword writes that walk the destination contiguously.
-__global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__restrict__ src,
-                                                              uint8_t *__restrict__ dst, int rows, int ks) {
+// blockIdx.z picks one of two tensors with the same ks (the A and B scales of a
+// GEMM go through one launch; rows1 = 0 for a single tensor).
+__global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__restrict__ src0,
+                                                              uint8_t *__restrict__ dst0, int rows0,
+                                                              const uint8_t *__restrict__ src1,
+                                                              uint8_t *__restrict__ dst1, int rows1, int ks) {
   __shared__ uint32_t stage[32 * 65];
+  const uint8_t *src = blockIdx.z ? src1 : src0;
+  uint8_t *dst = blockIdx.z ? dst1 : dst0;
+  const int rows = blockIdx.z ? rows1 : rows0;
   const int k_tiles = ks >> 3;
   const int rt = blockIdx.y, kt0 = blockIdx.x * 32;
+  if (rt * 32 >= rows) return;  // the grid is sized for the taller tensor
   const int t = threadIdx.x;
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
@@ -243,11 +251,25 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
   if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 7) == 0 &&
       ((uintptr_t)src & 7) == 0 && rows < ((int64_t)1 << 31) && ks < ((int64_t)1 << 31) && rows_p / 32 <= 65535) {
     dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)(rows_p / 32), 1);
-    scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, (int)ks);
+    scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks);
     return hipGetLastError();
   }
   scale_convert_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(src, src_layout, dst, dst_layout, rows,
                                                                         ks, rows_p, ksp);
+  return hipGetLastError();
+}
+
+// Row-major -> MFMA32 for the scales of both GEMM operands in one launch.
+// Returns hipErrorInvalidValue (nothing launched) when the fast kernel does not apply.
+hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
+                                       uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream) {
+  const int64_t rows_max = a_rows > b_rows ? a_rows : b_rows;
+  const int64_t rt = (rows_max + 31) / 32;
+  if ((ks & 7) != 0 || ks == 0 || (((uintptr_t)a_src | (uintptr_t)b_src) & 7) != 0 || rows_max >= ((int64_t)1 << 31) ||
+      ks >= ((int64_t)1 << 31) || rt > 65535 || a_rows <= 0 || b_rows <= 0)
+    return hipErrorInvalidValue;
+  dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)rt, 2);
+  scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks);
   return hipGetLastError();
 }
 

@@ -158,7 +158,7 @@ def main():
 
     # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this
     # command, scaled by a device copy of known size (profiles/pmc_*.txt); not measurable from here
-    measured_traffic = {"cfg2": 440e6 + 172e6, "cfg3_m16": 125.5e6 + 0.92e6}.get(args.workload) \
+    measured_traffic = {"cfg2": 435e6 + 134.2e6, "cfg3_m16": 125.5e6 + 0.92e6}.get(args.workload) \
         if args.variant == 0 else None
     flops, nbytes = gemm_flops(m, n, k), gemm_bytes(m, n, k, out_bytes)
     ms_per_step = wall / args.steps * 1e3

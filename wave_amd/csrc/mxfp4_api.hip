@@ -222,7 +222,8 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   // cache line per wave instruction; row-major scales cost 32 lines per
   // instruction.  With scratch available, re-lay both operands out first
   // (a few MB, microseconds) and run the native-scale kernel.
-  if (is_tile_variant(v) && k % kTileK == 0 && workspace) {
+  // (Not worth a second launch for short K: up to 8 K tiles per workgroup the direct reads cost less.)
+  if (is_tile_variant(v) && k % kTileK == 0 && workspace && p.tiles_per_split > 8) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
     const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? a_bytes : 0;
     const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? b_bytes : 0;

@@ -65,7 +65,7 @@ __device__ __forceinline__ void stream_wait_vm() {
 // 16-byte pieces, so every B tile costs the same number of DMA instructions,
 // nothing is predicated and waits can be counted.  Otherwise (K tails, fewer
 // K tiles) the same pipeline runs with predicated loads and full waits.
-template <int MT_M, bool FULL>
+template <int MT_M, bool FULL, int KW>
 __device__ __forceinline__ void stream_body(const GemmParams &p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_raw[];
   StreamLds &lds = *reinterpret_cast<StreamLds *>(smem_raw);
@@ -83,8 +83,18 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const int split = blockIdx.y;
   const int kt_begin = split * p.tiles_per_split;
   const int nkt = min(p.k_tiles, kt_begin + p.tiles_per_split) - kt_begin;
-  const int ktw = FULL ? nkt / kStreamWaves : (nkt + kStreamWaves - 1) / kStreamWaves;  // <= kStreamKtPerWave
-  const int kt0 = kt_begin + wave * ktw;
+  // The four waves form kw x nw: kw of them share a B tile along K, nw such
+  // groups take consecutive tiles (short K: a wave always fetches up to 1 KB of
+  // a row, and the fewer waves share a tile the less there is to add up).
+  constexpr int kw = FULL ? KW : kStreamWaves, nw = kStreamWaves / kw;
+  constexpr int kw_shift = kw == 4 ? 2 : kw == 2 ? 1 : 0;
+  const int kq = wave & (kw - 1), nq = wave >> kw_shift;
+  const int ktw = FULL ? nkt / kw : (nkt + kStreamWaves - 1) / kStreamWaves;  // <= kStreamKtPerWave
+  const int kt0 = kt_begin + kq * ktw;
+  const int ntiles = nt_end - nt_begin, steps = (ntiles + nw - 1) >> (2 - kw_shift);
+  // tile of this wave in step s (the last step may repeat the last tile: computed, not stored)
+  auto tile_of = [&](int s) { return nt_begin + min(s * nw + nq, ntiles - 1); };
+  auto tile_valid = [&](int s) { return s * nw + nq < ntiles; };
   const int my_nkt = FULL ? ktw : max(0, min(ktw, kt_begin + nkt - kt0));
 
   const int kp = p.kp;
@@ -230,7 +240,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
 
   // two B tiles in flight from the start (FULL mode is only launched with at
   // least two tiles per workgroup, which keeps this prologue branch-free)
-  issue_tile(nt_begin, 0);
+  issue_tile(tile_of(0), 0);
 
   // ---- A: resident fragments and scales; issued between the first two B tiles ----
   // All vector memory traffic of the kernel is buffer instructions: with a
@@ -315,14 +325,14 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   }
 
 
-  if (FULL || nt_begin + 1 < nt_end) issue_tile(nt_begin + 1, 1);
+  if (FULL || steps > 1) issue_tile(tile_of(1), 1);
 
   // Wait until tile nt has landed; tile nt+1 stays in flight.  In FULL mode a
   // tile is 17 DMA instructions (18 with e8m0_shuffle scales, whose first then
   // falls under the wait as well), and the youngest in the queue are those of
   // tile nt+1.
-  auto wait_tile = [&](int nt) {
-    if (FULL && nt + 1 < nt_end) {
+  auto wait_tile = [&](int s) {
+    if (FULL && s + 1 < steps) {
       stream_wait_vm<17>();
     } else {
       __builtin_amdgcn_s_waitcnt(0);
@@ -397,7 +407,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     stream_wait_vm<17>();  // tile nt_begin has landed
     asm volatile("" ::: "memory");
   } else {
-    wait_tile(nt_begin);
+    wait_tile(0);
   }
 
   auto store_tile = [&](int nt, int i, int l, const v4f &v) {
@@ -436,19 +446,19 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   // Per tile t: wait until it has landed (tile t+1 stays in flight), pull its
   // fragments and scales into registers, start the DMA of tile t+2 into the
   // buffer just emptied, multiply, add the four partial tiles through LDS.
-  // The sum of tile t is formed by wave t%4 and stays in its registers
-  // (kHold tiles per wave): C is written at the end of the kernel, by all four
-  // waves at once, so that in the common case no write traffic (16 partial
-  // lines per tile) is mixed into the read stream.  With more than 4*kHold
-  // tiles per workgroup the oldest held tile is stored just before the DMA
+  // The sum of a group's tile of step t is formed by its wave t % kw and stays
+  // in its registers (kHold tiles per wave): C is written at the end of the
+  // kernel, by all four waves at once, so that in the common case no write
+  // traffic (16 partial lines per tile) is mixed into the read stream.  With
+  // more than kw*kHold steps the oldest held tile is stored just before the DMA
   // issue of the iteration that replaces it: the stores are then older than
   // that DMA and the counted waits stay exact.
-  constexpr int kHold = FULL ? 2 : 1;
+  constexpr int kHold = FULL && (MT_M < 4 || KW == 4) ? 2 : 1;  // (64 rows of A leave few registers)
   v4f hold[kHold][MT_M];
-  const int ntiles = nt_end - nt_begin;
-  for (int nt = nt_begin; nt < nt_end; ++nt) {
-    const int buf = (nt - nt_begin) & 1;
-    if (nt > nt_begin) wait_tile(nt);
+  for (int t = 0; t < steps; ++t) {
+    const int nt = tile_of(t);
+    const int buf = t & 1;
+    if (t > 0) wait_tile(t);
 
     const int n_row = min(nt * 16 + fr, p.n - 1);
     const uint8_t *sc_img = lds.scales[wave][buf];
@@ -503,14 +513,14 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       }
     }
 
-    const int t = nt - nt_begin;
-    const int slot = (t >> 2) & (kHold - 1);
-    if (t >= 4 * kHold && wave == (t & 3)) {
+    const int reducer = t & (kw - 1);  // the wave of the group that adds up the tile of step t
+    const int slot = (t >> kw_shift) & (kHold - 1);
+    if (t >= kw * kHold && kq == reducer) {
 #pragma unroll
       for (int h = 0; h < kHold; ++h) {
         if (h == slot) {
 #pragma unroll
-          for (int i = 0; i < MT_M; ++i) store_tile(nt - 4 * kHold, i, lane, hold[h][i]);
+          for (int i = 0; i < MT_M; ++i) store_tile(tile_of(t - kw * kHold), i, lane, hold[h][i]);
         }
       }
     }
@@ -519,7 +529,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_waitcnt((7 << 4) | (3 << 14) | 15);  // lgkmcnt(0)
     asm volatile("" ::: "memory");
-    if (nt + 2 < nt_end) issue_tile(nt + 2, buf);
+    if (t + 2 < steps) issue_tile(tile_of(t + 2), buf);
 
     v4f acc[MT_M];
 #pragma unroll
@@ -541,19 +551,18 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       }
     }
 
-    // add the partial tiles: the other three waves hand theirs to wave t%4 through LDS
-    const int reducer = t & 3;
-    if (wave != reducer) {
+    // add the partial tiles: the other waves of the group hand theirs to the reducer through LDS
+    const int red0 = nq * (kw - 1);  // the group's share of the partial-tile area
+    if (kq != reducer) {
 #pragma unroll
-      for (int i = 0; i < MT_M; ++i) *(v4f *)lds.red[(wave - reducer - 1) & 3][i][lane] = acc[i];
+      for (int i = 0; i < MT_M; ++i) *(v4f *)lds.red[red0 + ((kq - reducer - 1) & (kw - 1))][i][lane] = acc[i];
     }
     lds_barrier();  // partials visible
-    if (wave == reducer) {
+    if (kq == reducer) {
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) {
         v4f v = acc[i];
-#pragma unroll
-        for (int w = 0; w < kStreamWaves - 1; ++w) v += *(const v4f *)lds.red[w][i][lane];
+        for (int w = 0; w < kw - 1; ++w) v += *(const v4f *)lds.red[red0 + w][i][lane];
 #pragma unroll
         for (int h = 0; h < kHold; ++h) {
           if (h == slot) hold[h][i] = v;
@@ -562,46 +571,46 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     }
     lds_barrier();  // red is free again
   }
-  // the tiles still held: the last 4*kHold (or fewer) of the workgroup
-  for (int t = max(0, ntiles - 4 * kHold); t < ntiles; ++t) {
-    if (wave == (t & 3)) {
+  // the tiles still held: those of the last kw*kHold (or fewer) steps
+  for (int t = max(0, steps - kw * kHold); t < steps; ++t) {
+    if (kq == (t & (kw - 1)) && tile_valid(t)) {
 #pragma unroll
       for (int h = 0; h < kHold; ++h) {
-        if (h == ((t >> 2) & (kHold - 1))) {
+        if (h == ((t >> kw_shift) & (kHold - 1))) {
 #pragma unroll
-          for (int i = 0; i < MT_M; ++i) store_tile(nt_begin + t, i, lane, hold[h][i]);
+          for (int i = 0; i < MT_M; ++i) store_tile(tile_of(t), i, lane, hold[h][i]);
         }
       }
     }
   }
 }
 
-template <int MT_M, bool FULL>
+template <int MT_M, bool FULL, int KW>
 __global__ void __launch_bounds__(kStreamWaves * 64, 1) stream_gemm_kernel(const GemmParams p) {
-  stream_body<MT_M, FULL>(p);
+  stream_body<MT_M, FULL, KW>(p);
 }
 
-template <int MT_M, bool FULL>
+template <int MT_M, bool FULL, int KW>
 static hipError_t launch_stream_mt(const GemmParams &p, int grid_x, hipStream_t stream) {
   static bool attr_done = false;
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)stream_gemm_kernel<MT_M, FULL>,
+    hipError_t e = hipFuncSetAttribute((const void *)stream_gemm_kernel<MT_M, FULL, KW>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(StreamLds));
     if (e != hipSuccess) return e;
     attr_done = true;
   }
   dim3 grid(grid_x, p.splits, 1);
-  stream_gemm_kernel<MT_M, FULL><<<grid, dim3(kStreamWaves * 64), sizeof(StreamLds), stream>>>(p);
+  stream_gemm_kernel<MT_M, FULL, KW><<<grid, dim3(kStreamWaves * 64), sizeof(StreamLds), stream>>>(p);
   return hipGetLastError();
 }
 
-template <bool FULL>
+template <bool FULL, int KW>
 static hipError_t launch_stream_full(const GemmParams &p, int grid_x, hipStream_t stream) {
   switch ((p.m + 15) / 16) {
-    case 1: return launch_stream_mt<1, FULL>(p, grid_x, stream);
-    case 2: return launch_stream_mt<2, FULL>(p, grid_x, stream);
-    case 3: return launch_stream_mt<3, FULL>(p, grid_x, stream);
-    case 4: return launch_stream_mt<4, FULL>(p, grid_x, stream);
+    case 1: return launch_stream_mt<1, FULL, KW>(p, grid_x, stream);
+    case 2: return launch_stream_mt<2, FULL, KW>(p, grid_x, stream);
+    case 3: return launch_stream_mt<3, FULL, KW>(p, grid_x, stream);
+    case 4: return launch_stream_mt<4, FULL, KW>(p, grid_x, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -619,11 +628,25 @@ hipError_t launch_stream_gemm(const GemmParams &p, int num_cus, hipStream_t stre
   // ... and into A and both scale matrices (padded to 32-row blocks)
   if ((int64_t)p.m * p.kp >= ((int64_t)1 << 31) || ((int64_t)p.n + 32) * (p.ksp + 8) >= ((int64_t)1 << 31))
     return hipErrorInvalidValue;
-  // every wave of every split owns the same number of whole K tiles
-  // ... and every workgroup at least two tiles of B
-  const bool full = p.tiles_per_split % kStreamWaves == 0 && p.k_tiles % p.tiles_per_split == 0 &&
-                    (p.k & (kTileK - 1)) == 0 && nt_total >= 2 * grid_x;
-  return full ? launch_stream_full<true>(p, grid_x, stream) : launch_stream_full<false>(p, grid_x, stream);
+  // Counted-wait mode: every wave owns the same number (at most 8) of whole K
+  // tiles and sees at least two tiles of B.  As few waves as possible share a
+  // tile along K.
+  int kw = 0;
+  if ((p.k & (kTileK - 1)) == 0 && p.k_tiles % p.tiles_per_split == 0) {
+    for (int c = 1; c <= kStreamWaves && kw == 0; c *= 2) {
+      if (p.tiles_per_split % c == 0 && p.tiles_per_split / c <= kStreamKtPerWave &&
+          nt_total >= 2 * (kStreamWaves / c) * grid_x)
+        kw = c;
+    }
+  }
+  if (kw != 0) {
+    switch (kw) {
+      case 1: return launch_stream_full<true, 1>(p, grid_x, stream);
+      case 2: return launch_stream_full<true, 2>(p, grid_x, stream);
+      default: return launch_stream_full<true, 4>(p, grid_x, stream);
+    }
+  }
+  return launch_stream_full<false, kStreamWaves>(p, grid_x, stream);
 }
 
 }  // namespace wave_mxfp4

@@ -67,6 +67,9 @@ typedef enum {
  * tagged_mxfp4_gemm.py:465-483); needs N % 16 == 0 and K % 64 == 0. */
 typedef enum { WAVE_MXFP4_B_ROW_MAJOR = 0, WAVE_MXFP4_B_PRESHUFFLE = 1 } wave_mxfp4_b_layout;
 
+/* Element type of the quantiser's input. */
+typedef enum { WAVE_MXFP4_IN_F32 = 0, WAVE_MXFP4_IN_BF16 = 1, WAVE_MXFP4_IN_F16 = 2 } wave_mxfp4_in_dtype;
+
 /* Kernel selection.  AUTO picks by shape.  The others force one kernel and
  * mirror the reference's (block_shape, wave_shape) template arguments
  * (tagged_mxfp4_gemm.py:38-48). */
@@ -149,6 +152,22 @@ int wave_mxfp4_scale_convert(const void *src, int src_layout, void *dst, int dst
 
 /* Device-side b_preshuffle (mxfp_utils.py:98-110); rows % 16 == 0, kp % 32 == 0. */
 int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, void *hip_stream);
+
+/* Activation / weight quantiser, the step in front of the GEMM:
+ * x [rows, k] (f32, bf16 or f16, row-major, 16-byte aligned) -> q [rows, k/2]
+ * packed e2m1 + one e8m0 scale per 32 elements of a row, written in
+ * `scale_layout` (row-major [rows, k/32], or a tiled layout over the padded
+ * buffer of wave_mxfp4_e8m0_shuffle_bytes(rows, k/32) bytes, padding written
+ * as 0), so that its outputs are the GEMM's A and A_scale (or B and B_scale)
+ * without a pass in between.  k % 32 == 0.
+ * Replaces aiter.get_triton_quant(QuantType.per_1x32)(x, shuffle=...) at the
+ * reference's call sites (wave_lang/kernel/wave/perf/bench_mxfp4_comparison.py:
+ * 1484-1486,1897-1899; shuffle=True is WAVE_MXFP4_SCALE_E8M0_SHUFFLE): scale
+ * 2^(floor(log2(amax rounded up at 1.75 of a binade)) - 2) clamped to
+ * 2^-127..2^127, elements rounded to nearest even, saturating at 6; NaN
+ * elements become +-6 under scale byte 254. */
+int wave_mxfp4_quantize(const void *x, int in_dtype, void *q, void *scale, int64_t rows, int64_t k,
+                        int scale_layout, void *hip_stream);
 
 /* Text for a status code; never NULL (the reference reports errors as
  * exceptions carrying hipGetErrorName/String, runtime.cpp:96-109). */

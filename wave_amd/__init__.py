@@ -11,6 +11,7 @@ from .mxfp4 import (
     mxfp4_gemm,
     mxfp4_gemm_grouped,
     mxfp4_to_f32,
+    quantize_mxfp4,
     scale_convert,
     workspace_bytes,
 )
@@ -23,6 +24,7 @@ __all__ = [
     "mxfp4_gemm",
     "mxfp4_gemm_grouped",
     "mxfp4_to_f32",
+    "quantize_mxfp4",
     "scale_convert",
     "workspace_bytes",
 ]

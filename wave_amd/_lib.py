@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # WAVE_MXFP4_LIB points at another build of the same ABI (e.g. an experiment)
 LIB_PATH = os.environ.get("WAVE_MXFP4_LIB") or os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # status codes of include/wave_mxfp4.h
 OK = 0
@@ -27,6 +27,7 @@ ERR_UNSUPPORTED = -8
 OUT_F32, OUT_BF16 = 0, 1
 SCALE_ROW_MAJOR, SCALE_E8M0_SHUFFLE, SCALE_MFMA32 = 0, 1, 2
 B_ROW_MAJOR, B_PRESHUFFLE = 0, 1
+IN_F32, IN_BF16, IN_F16 = 0, 1, 2
 
 VARIANT_AUTO = 0
 VARIANT_T256x256_W2x2 = 1
@@ -47,6 +48,7 @@ EXPORTS = (
     "wave_mxfp4_e8m0_shuffle_bytes",
     "wave_mxfp4_scale_convert",
     "wave_mxfp4_b_preshuffle",
+    "wave_mxfp4_quantize",
     "wave_mxfp4_status_string",
     "wave_mxfp4_last_hip_error",
     "wave_mxfp4_abi_version",
@@ -86,6 +88,8 @@ def load():
     lib.wave_mxfp4_scale_convert.restype = i32
     lib.wave_mxfp4_b_preshuffle.argtypes = [p, p, i64, i64, p]
     lib.wave_mxfp4_b_preshuffle.restype = i32
+    lib.wave_mxfp4_quantize.argtypes = [p, i32, p, p, i64, i64, i32, p]
+    lib.wave_mxfp4_quantize.restype = i32
     lib.wave_mxfp4_status_string.argtypes = [i32]
     lib.wave_mxfp4_status_string.restype = ctypes.c_char_p
     lib.wave_mxfp4_last_hip_error.argtypes = []

@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 2;
+constexpr int kAbiVersion = 3;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -372,6 +372,20 @@ int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, 
   if (!aligned(b, 16) || !aligned(out, 16)) return WAVE_MXFP4_ERR_MISALIGNED;
   return record_hip(
       launch_b_preshuffle((const uint8_t *)b, (uint8_t *)out, rows, kp, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_quantize(const void *x, int in_dtype, void *q, void *scale, int64_t rows, int64_t k,
+                        int scale_layout, void *hip_stream) {
+  if (rows < 0 || k < 0 || k % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (bad_enum(in_dtype, 3) || bad_enum(scale_layout, 3)) return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (rows == 0 || k == 0) return WAVE_MXFP4_OK;
+  if (!x || !q || !scale) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(x, 16) || !aligned(q, 4) || (scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && !aligned(scale, 4)))
+    return WAVE_MXFP4_ERR_MISALIGNED;
+  if (scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && (k / 32) % 4 == 0 && !aligned(scale, 4))
+    return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_quantize(x, in_dtype, (uint8_t *)q, (uint8_t *)scale, rows, k, scale_layout, device_cus(),
+                                    (hipStream_t)hip_stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,200 @@
+// Activation quantiser in front of the MXFP4 GEMM (gfx950): f32 / bf16 / f16
+// [rows, k] -> packed e2m1 [rows, k/2] + one e8m0 scale per 32 elements, written
+// in any of the GEMM's scale layouts.  HBM bound: the input is read once with
+// 16-byte loads that walk rows contiguously, the packed output is written once
+// with dword stores that do the same, and the scale bytes of a workgroup's tile
+// are gathered in LDS and written as whole dwords in the order of the layout.
+//
+// Arithmetic: the scale is taken from the group's largest magnitude, rounded up
+// to the next binade when its mantissa is at least 1.75, minus two binades; the
+// elements are divided by it and rounded to e2m1 (nearest, ties to even,
+// saturating at 6) by v_cvt_scalef32_pk_fp4_*, two elements per instruction.
+#include "mxfp4_common.h"
+
+namespace wave_mxfp4 {
+
+namespace {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kQuantRows = 32;  // rows of a workgroup's tile (one block of the tiled scale layouts)
+
+// Largest of the four lanes of a quad.
+__device__ __forceinline__ uint32_t quad_max(uint32_t v) {
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+  return v;
+}
+
+// f32 bit pattern of a group's largest magnitude -> e8m0 byte.
+__device__ __forceinline__ uint32_t scale_byte_of(uint32_t amax_bits) {
+  const uint32_t e = (amax_bits + 0x200000u) >> 23;  // up to 256: a NaN with a large mantissa carries out of the field
+  return e >= 255u ? 254u : (e > 2u ? e - 2u : 0u);
+}
+
+// The lane's 8 consecutive elements: DW dwords.
+template <int DT>
+struct Elems {
+  static constexpr int kBytes = DT == WAVE_MXFP4_IN_F32 ? 4 : 2;
+  static constexpr int kDwords = 2 * kBytes;
+  uint32_t d[kDwords];
+
+  __device__ __forceinline__ void load(const uint8_t *p, bool ok) {
+#pragma unroll
+    for (int i = 0; i < kDwords / 4; ++i) {
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (ok) v = *(const uint4 *)(p + 16 * i);
+      d[4 * i + 0] = v.x, d[4 * i + 1] = v.y, d[4 * i + 2] = v.z, d[4 * i + 3] = v.w;
+    }
+  }
+
+  // f32 bit pattern of the largest magnitude (NaN patterns compare above infinity)
+  __device__ __forceinline__ uint32_t amax_bits() const {
+    if constexpr (DT == WAVE_MXFP4_IN_F32) {
+      uint32_t m = 0;
+#pragma unroll
+      for (int i = 0; i < kDwords; ++i) m = max(m, d[i] & 0x7FFFFFFFu);
+      return m;
+    }
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < kDwords; ++i) {
+      lo = max(lo, d[i] & 0x7FFFu);
+      hi = max(hi, (d[i] >> 16) & 0x7FFFu);
+    }
+    const uint32_t h = max(lo, hi);
+    if constexpr (DT == WAVE_MXFP4_IN_BF16) return h << 16;
+    return __builtin_bit_cast(uint32_t, (float)__builtin_bit_cast(_Float16, (uint16_t)h));
+  }
+
+  // 8 e2m1 codes, element j in nibble j
+  __device__ __forceinline__ uint32_t convert(float scale) const {
+    uint32_t r = 0;
+    if constexpr (DT == WAVE_MXFP4_IN_F32) {
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, __builtin_bit_cast(float, d[0]), __builtin_bit_cast(float, d[1]), scale, 0);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, __builtin_bit_cast(float, d[2]), __builtin_bit_cast(float, d[3]), scale, 1);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, __builtin_bit_cast(float, d[4]), __builtin_bit_cast(float, d[5]), scale, 2);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, __builtin_bit_cast(float, d[6]), __builtin_bit_cast(float, d[7]), scale, 3);
+    } else if constexpr (DT == WAVE_MXFP4_IN_BF16) {
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, d[0]), scale, 0);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, d[1]), scale, 1);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, d[2]), scale, 2);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(r, __builtin_bit_cast(bf16x2, d[3]), scale, 3);
+    } else {
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, d[0]), scale, 0);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, d[1]), scale, 1);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, d[2]), scale, 2);
+      r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(r, __builtin_bit_cast(f16x2, d[3]), scale, 3);
+    }
+    return r;
+  }
+};
+
+// A workgroup of four waves takes 32 rows x TC K tiles (TC*256 columns); a wave
+// takes 8 of the rows.  Four lanes share a scale group (8 elements each); the 16
+// quads of a wave take 16 consecutive groups of a row per pass, so that one load
+// instruction covers up to 1 KB (bf16) and one store 256 B of a row.
+template <int DT, int TC>
+__global__ void __launch_bounds__(256) quantize_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ q,
+                                                       uint8_t *__restrict__ scale, int rows, int k,
+                                                       int scale_layout) {
+  constexpr int kEb = Elems<DT>::kBytes;
+  constexpr int kGroups = 8 * TC;              // scale groups of a tile row
+  constexpr int kPasses = 8 * kGroups / 16;    // per wave: 8 rows x kGroups groups, 16 per pass
+  constexpr int kBatch = DT == WAVE_MXFP4_IN_F32 ? 4 : 8;  // passes whose loads are in flight together
+  static_assert(kPasses % kBatch == 0 || kPasses < kBatch, "passes come in whole batches");
+  constexpr int kB = kPasses < kBatch ? kPasses : kBatch;
+  __shared__ uint32_t tile_scales[kQuantRows * kGroups / 4];
+  uint8_t *tile_bytes = (uint8_t *)tile_scales;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int quad = lane >> 2, sub = lane & 3;
+  const int ks = k >> 5, ksp = (ks + 7) & ~7;
+  const int col_tiles = (ks + kGroups - 1) / kGroups;
+  const int row_tile = blockIdx.x / col_tiles, col_tile = blockIdx.x - row_tile * col_tiles;
+  const int row0 = row_tile * kQuantRows, g0 = col_tile * kGroups;
+
+  for (int pb = 0; pb < kPasses; pb += kB) {
+    Elems<DT> e[kB];
+    int lrow[kB], lgrp[kB];
+#pragma unroll
+    for (int i = 0; i < kB; ++i) {
+      const int u = (pb + i) * 16 + quad;  // unit of the wave: (row, group)
+      lrow[i] = wave * 8 + u / kGroups;
+      lgrp[i] = u % kGroups;
+      const int row = row0 + lrow[i], g = g0 + lgrp[i];
+      const bool ok = row < rows && g < ks;
+      e[i].load(x + ((int64_t)row * k + (int64_t)g * 32 + sub * 8) * kEb, ok);
+    }
+#pragma unroll
+    for (int i = 0; i < kB; ++i) {
+      const int row = row0 + lrow[i], g = g0 + lgrp[i];
+      const uint32_t sb = scale_byte_of(quad_max(e[i].amax_bits()));
+      const float sf = __builtin_bit_cast(float, sb ? sb << 23 : 0x00400000u);  // 2^(sb-127)
+      const uint32_t codes = e[i].convert(sf);
+      if (row < rows && g < ks) *(uint32_t *)(q + (int64_t)row * (k >> 1) + g * 16 + sub * 4) = codes;
+      if (sub == 0) {
+        const int at = scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR
+                           ? lrow[i] * kGroups + lgrp[i]
+                           : (lgrp[i] >> 3) * 256 + (int)scale_offset(scale_layout, lrow[i], lgrp[i] & 7, 8, 8);
+        tile_bytes[at] = (uint8_t)sb;
+      }
+    }
+  }
+  __syncthreads();
+
+  if (scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR) {
+    // kGroups bytes of each row are contiguous
+    if ((ks & 3) == 0) {
+      for (int d = threadIdx.x; d < kQuantRows * kGroups / 4; d += 256) {
+        const int r = d / (kGroups / 4), gd = d % (kGroups / 4);
+        if (row0 + r < rows && g0 + gd * 4 < ks)
+          *(uint32_t *)(scale + (int64_t)(row0 + r) * ks + g0 + gd * 4) = tile_scales[d];
+      }
+    } else {
+      for (int b = threadIdx.x; b < kQuantRows * kGroups; b += 256) {
+        const int r = b / kGroups, g = b % kGroups;
+        if (row0 + r < rows && g0 + g < ks) scale[(int64_t)(row0 + r) * ks + g0 + g] = tile_bytes[b];
+      }
+    }
+  } else {
+    // the tile's TC blocks of 256 bytes follow one another (padding rows and groups hold 0)
+    const int k_tiles = ksp >> 3;
+    uint32_t *out = (uint32_t *)(scale + ((int64_t)row_tile * k_tiles + (int64_t)col_tile * TC) * 256);
+    for (int d = threadIdx.x; d < TC * 64; d += 256) {
+      if (col_tile * TC + (d >> 6) < k_tiles) out[d] = tile_scales[d];
+    }
+  }
+}
+
+template <int DT>
+hipError_t launch_quantize_dt(const void *x, uint8_t *q, uint8_t *scale, int rows, int k, int scale_layout,
+                              int num_cus, hipStream_t stream) {
+  const int ks = k >> 5;
+  const int64_t row_tiles = (rows + kQuantRows - 1) / kQuantRows;
+  // wide tiles (8 K tiles) when they still fill the chip twice over
+  const int64_t wide = row_tiles * ((ks + 63) / 64), narrow = row_tiles * ((ks + 7) / 8);
+  if (narrow > 0x7FFFFFFF) return hipErrorInvalidValue;
+  if (wide >= 2 * (int64_t)(num_cus > 0 ? num_cus : 256)) {
+    quantize_kernel<DT, 8><<<dim3((unsigned)wide), 256, 0, stream>>>((const uint8_t *)x, q, scale, rows, k, scale_layout);
+  } else {
+    quantize_kernel<DT, 1><<<dim3((unsigned)narrow), 256, 0, stream>>>((const uint8_t *)x, q, scale, rows, k, scale_layout);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_quantize(const void *x, int in_dtype, uint8_t *q, uint8_t *scale, int64_t rows, int64_t k,
+                           int scale_layout, int num_cus, hipStream_t stream) {
+  if (rows > 0x7FFFFFFF || k > 0x7FFFFFFF) return hipErrorInvalidValue;
+  switch (in_dtype) {
+    case WAVE_MXFP4_IN_F32: return launch_quantize_dt<WAVE_MXFP4_IN_F32>(x, q, scale, (int)rows, (int)k, scale_layout, num_cus, stream);
+    case WAVE_MXFP4_IN_BF16: return launch_quantize_dt<WAVE_MXFP4_IN_BF16>(x, q, scale, (int)rows, (int)k, scale_layout, num_cus, stream);
+    case WAVE_MXFP4_IN_F16: return launch_quantize_dt<WAVE_MXFP4_IN_F16>(x, q, scale, (int)rows, (int)k, scale_layout, num_cus, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace wave_mxfp4

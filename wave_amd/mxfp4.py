@@ -246,3 +246,41 @@ def b_preshuffle(b: torch.Tensor) -> torch.Tensor:
         st = lib.wave_mxfp4_b_preshuffle(b.data_ptr(), out.data_ptr(), rows, kp, _stream_ptr(b.device))
     _lib.check(st, "wave_mxfp4_b_preshuffle")
     return out
+
+
+_IN_DTYPES = {torch.float32: _lib.IN_F32, torch.bfloat16: _lib.IN_BF16, torch.float16: _lib.IN_F16}
+
+
+def quantize_mxfp4(x: torch.Tensor, *, shuffle: bool = False, scale_layout: int | None = None):
+    """``[R, K]`` f32 / bf16 / f16 -> ``(x_q [R, K/2] uint8, x_scales)``, the A
+    (or B) operand pair of :func:`mxfp4_gemm`.  Same call shape as the quantiser
+    the reference's benchmark uses, ``quant_func(x, shuffle=True)``
+    (wave_lang/kernel/wave/perf/bench_mxfp4_comparison.py:1484-1486):
+    ``shuffle=True`` writes the scales in ``e8m0_shuffle`` order.
+
+    ``x_scales`` is ``[R, K/32]`` for the row-major layout, otherwise the padded
+    buffer ``[ceil(R/32)*32, ceil(K/32/8)*8]`` in the tile order of
+    ``scale_layout``."""
+    lib = _lib.load()
+    if x.dim() != 2:
+        raise ValueError(f"x: expected [R, K], got shape {tuple(x.shape)}")
+    if x.dtype not in _IN_DTYPES:
+        raise ValueError(f"x: dtype {x.dtype} is not float32, bfloat16 or float16")
+    if x.device.type != "cuda":
+        raise ValueError("x: expected a device tensor")
+    layout = scale_layout if scale_layout is not None else (_lib.SCALE_E8M0_SHUFFLE if shuffle else _lib.SCALE_ROW_MAJOR)
+    x = x.contiguous()
+    rows, k = x.shape
+    if k % 32:
+        raise ValueError(f"x: K = {k} is not a multiple of 32")
+    ks = k // 32
+    q = torch.empty(rows, k // 2, dtype=torch.uint8, device=x.device)
+    if layout == _lib.SCALE_ROW_MAJOR:
+        scales = torch.empty(rows, ks, dtype=torch.uint8, device=x.device)
+    else:
+        scales = torch.empty((rows + 31) // 32 * 32, (ks + 7) // 8 * 8, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        st = lib.wave_mxfp4_quantize(x.data_ptr(), _IN_DTYPES[x.dtype], q.data_ptr(), scales.data_ptr(), rows, k,
+                                     layout, _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp4_quantize")
+    return q, scales

@@ -44,6 +44,9 @@ constexpr int kStreamRowBytes = kStreamKtPerWave * kTileKBytes;    // 1 KB of on
 constexpr int kStreamRowPitch = kStreamRowBytes + 32;              // LDS pitch (measured: fragment reads are conflict-free at 32 mod 64)
 constexpr int kStreamTileBytes = 16 * kStreamRowPitch;             // one 16-row B tile, one wave's K range
 constexpr int kStreamScaleBytes = 2048;                            // its scale image (1 KB used by two layouts)
+// Cache policy of the B data loads (the "nt" bit of the buffer instruction): B is read exactly once, and
+// marking it non-temporal keeps it from displacing A and the scales (measured: 25.4 -> 23.0 us at M=16).
+constexpr int kStreamOnce = 2;
 
 int stream_max_k_tiles() { return kStreamMaxKTiles; }
 
@@ -131,7 +134,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       for (int i = 0; i < 16; ++i) {
         const int soff = bpre ? tile_off + ((kt0 + min(i >> 1, ktw - 1)) * 4 + (i & 1) * 2) * 512
                               : tile_off + min(i, row_lim) * kp + kt0 * kTileKBytes;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * pitch), 16, b_voff, soff, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * pitch), 16, b_voff, soff, 0, kStreamOnce);
       }
     } else if (bpre) {
 #pragma unroll
@@ -140,7 +143,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
         if (j < my_nkt) {
           if (chunk_ok(kt0 + j, s * 4 + fg))
             __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * 1024), 16, lane * 16,
-                                                     tile_off + ((kt0 + j) * 4 + s * 2) * 512, 0, 0);
+                                                     tile_off + ((kt0 + j) * 4 + s * 2) * 512, 0, kStreamOnce);
           else
             *(v4i *)(dst + i * 1024 + lane * 16) = zero;
         }
@@ -151,7 +154,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
         if ((lane >> 3) < my_nkt) {
           if (chunk_ok(kt0 + (lane >> 3), lane & 7))
             __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(dst + i * kStreamRowPitch), 16, lane * 16,
-                                                     tile_off + min(i, row_lim) * kp + kt0 * kTileKBytes, 0, 0);
+                                                     tile_off + min(i, row_lim) * kp + kt0 * kTileKBytes, 0, kStreamOnce);
           else
             *(v4i *)(dst + i * kStreamRowPitch + lane * 16) = zero;
         }
@@ -196,10 +199,10 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
                              ((n0 >> 4) & 1) * 64 + (lane & 3) * 16;
       const int off_shuf = blocked_off + min(lane >> 4, ktw - 1) * 256 + (lane & 15) * 16;
       const int off = bsl == WAVE_MXFP4_SCALE_ROW_MAJOR ? off_rm : bsl == WAVE_MXFP4_SCALE_MFMA32 ? off_native : off_shuf;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, off, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, off, 0, 0, kStreamOnce);
       if (bsl == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {
         const int off2 = blocked_off + min(4 + (lane >> 4), ktw - 1) * 256 + (lane & 15) * 16;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst + 1024), 16, off2, 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst + 1024), 16, off2, 0, 0, kStreamOnce);
       }
     } else if (bsl == WAVE_MXFP4_SCALE_ROW_MAJOR) {
       const int row = min(n0 + (lane & 15), p.n - 1);
@@ -217,7 +220,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
     } else if (bsl == WAVE_MXFP4_SCALE_MFMA32) {
       const int blk = lane >> 3, piece = lane & 7;
       const int off = blocked_off + blk * 256 + (piece >> 2) * 128 + ((n0 >> 4) & 1) * 64 + (piece & 3) * 16;
-      if (kt0 + blk < p.k_tiles) __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, off, 0, 0, 0);
+      if (kt0 + blk < p.k_tiles) __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(dst), 16, off, 0, 0, kStreamOnce);
     } else {
       const int off = blocked_off + lane * 16;
 #pragma unroll

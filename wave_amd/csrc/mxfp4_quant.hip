@@ -43,8 +43,9 @@ struct Elems {
   __device__ __forceinline__ void load(const uint8_t *p, bool ok) {
 #pragma unroll
     for (int i = 0; i < kDwords / 4; ++i) {
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (ok) v = *(const uint4 *)(p + 16 * i);
+      v4i v = {0, 0, 0, 0};
+      // read once: 16-bit inputs bypass the caches; an f32 lane's two loads share lines and are faster through them
+      if (ok) v = kBytes == 2 ? __builtin_nontemporal_load((const v4i *)(p + 16 * i)) : *(const v4i *)(p + 16 * i);
       d[4 * i + 0] = v.x, d[4 * i + 1] = v.y, d[4 * i + 2] = v.z, d[4 * i + 3] = v.w;
     }
   }
@@ -133,7 +134,7 @@ __global__ void __launch_bounds__(256) quantize_kernel(const uint8_t *__restrict
       const uint32_t sb = scale_byte_of(quad_max(e[i].amax_bits()));
       const float sf = __builtin_bit_cast(float, sb ? sb << 23 : 0x00400000u);  // 2^(sb-127)
       const uint32_t codes = e[i].convert(sf);
-      if (row < rows && g < ks) *(uint32_t *)(q + (int64_t)row * (k >> 1) + g * 16 + sub * 4) = codes;
+      if (row < rows && g < ks) __builtin_nontemporal_store(codes, (uint32_t *)(q + (int64_t)row * (k >> 1) + g * 16 + sub * 4));
       if (sub == 0) {
         const int at = scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR
                            ? lrow[i] * kGroups + lgrp[i]

@@ -35,7 +35,7 @@ typedef enum {
   WAVE_MXFP4_ERR_BAD_SHAPE = -2,     /* negative dims, K % 32 != 0, layout divisibility */
   WAVE_MXFP4_ERR_BAD_ENUM = -3,      /* dtype / layout / variant out of range */
   WAVE_MXFP4_ERR_MISALIGNED = -4,    /* a pointer is not aligned as documented */
-  WAVE_MXFP4_ERR_WORKSPACE = -5,     /* split-K workspace missing or too small */
+  WAVE_MXFP4_ERR_WORKSPACE = -5,     /* workspace missing or too small (split-K, per-row scales) */
   WAVE_MXFP4_ERR_BAD_SPLIT = -6,     /* K per split < 256 or not a multiple of 256 */
   WAVE_MXFP4_ERR_HIP = -7,           /* a HIP call failed; see wave_mxfp4_last_hip_error */
   WAVE_MXFP4_ERR_UNSUPPORTED = -8
@@ -60,7 +60,14 @@ typedef enum {
    * byte count as the padded E8M0_SHUFFLE buffer.  Produced by
    * wave_mxfp4_scale_convert (no counterpart in the reference, whose
    * e8m0_shuffle is matched to the 16x16x128 instruction). */
-  WAVE_MXFP4_SCALE_MFMA32 = 2
+  WAVE_MXFP4_SCALE_MFMA32 = 2,
+  /* One e8m0 byte per row, [R], that holds for every 32-group of the row: the
+   * broadcast-scale kernel of the reference
+   * (wave_lang/kernel/wave/templates/test_kernels.py:75-135, a_scale: [M]
+   * broadcast to [M, K/32]).  Accepted as a_scale_layout of wave_mxfp4_gemm
+   * only; the call then needs the workspace, in which the library spreads the
+   * scales out before the GEMM. */
+  WAVE_MXFP4_SCALE_PER_ROW = 3
 } wave_mxfp4_scale_layout;
 
 /* B storage.  PRESHUFFLE is b_preshuffle (mxfp_utils.py:98-110,

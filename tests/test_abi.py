@@ -62,7 +62,10 @@ def test_gemm_argument_validation():
     assert gemm(lib, k=-32) == _lib.ERR_BAD_SHAPE
     assert gemm(lib, k=48) == _lib.ERR_BAD_SHAPE          # K % 32 != 0
     assert gemm(lib, od=2) == _lib.ERR_BAD_ENUM
-    assert gemm(lib, asl=3) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, asl=4) == _lib.ERR_BAD_ENUM
+    assert gemm(lib, bsl=3) == _lib.ERR_BAD_ENUM          # one scale per row is for A only
+    assert gemm(lib, asl=3) == _lib.ERR_WORKSPACE         # ... and needs the workspace
+    assert gemm(lib, asl=3, as_=P + 1, ws=P, wsb=16) == _lib.ERR_WORKSPACE
     assert gemm(lib, bsl=-1) == _lib.ERR_BAD_ENUM
     assert gemm(lib, bl=7) == _lib.ERR_BAD_ENUM
     assert gemm(lib, variant=99) == _lib.ERR_BAD_ENUM
@@ -121,6 +124,13 @@ def test_aux_argument_validation():
     assert lib.wave_mxfp4_b_preshuffle(P, P, 24, 32, None) == _lib.ERR_BAD_SHAPE
     assert lib.wave_mxfp4_b_preshuffle(P, P, 32, 48, None) == _lib.ERR_BAD_SHAPE
     assert lib.wave_mxfp4_b_preshuffle(P + 1, P, 32, 64, None) == _lib.ERR_MISALIGNED
+    assert lib.wave_mxfp4_quantize(P, 1, P, P, 4, 48, 0, None) == _lib.ERR_BAD_SHAPE
+    assert lib.wave_mxfp4_quantize(P, 3, P, P, 4, 64, 0, None) == _lib.ERR_BAD_ENUM
+    assert lib.wave_mxfp4_quantize(P, 1, P, P, 4, 64, 3, None) == _lib.ERR_BAD_ENUM
+    assert lib.wave_mxfp4_quantize(P, 1, None, P, 4, 64, 0, None) == _lib.ERR_NULL_POINTER
+    assert lib.wave_mxfp4_quantize(P + 8, 1, P, P, 4, 64, 0, None) == _lib.ERR_MISALIGNED
+    assert lib.wave_mxfp4_quantize(P, 1, P, P + 2, 4, 64, 1, None) == _lib.ERR_MISALIGNED
+    assert lib.wave_mxfp4_quantize(P, 1, P, P, 0, 64, 0, None) == _lib.OK
     assert lib.wave_mxfp4_e8m0_shuffle_bytes(4093, 224) == 4096 * 224
     assert lib.wave_mxfp4_e8m0_shuffle_bytes(33, 9) == 64 * 16
 
@@ -128,10 +138,11 @@ def test_aux_argument_validation():
 def test_workspace_bytes():
     lib = _lib.load()
     scales = 2 * 512 * 32                     # both operands re-laid out as MFMA32
-    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, 0) == scales
-    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 4, 3) == 4 * 512 * 512 * 4 + scales
-    assert lib.wave_mxfp4_workspace_bytes(16, 512, 1024, 1, 0) == 0      # skinny kernel: nothing to stage
-    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, _lib.VARIANT_NAIVE) == 0
+    spread = 512 * 32                         # room to spread per-row A scales over [M, K/32]
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, 0) == scales + spread
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 4, 3) == 4 * 512 * 512 * 4 + scales + spread
+    assert lib.wave_mxfp4_workspace_bytes(16, 512, 1024, 1, 0) == 16 * 32      # skinny kernel: nothing else to stage
+    assert lib.wave_mxfp4_workspace_bytes(512, 512, 1024, 1, _lib.VARIANT_NAIVE) == spread
     assert lib.wave_mxfp4_workspace_bytes(-1, 512, 1024, 4, 3) == 0
 
 

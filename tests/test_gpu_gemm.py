@@ -325,3 +325,40 @@ def test_streaming_kernel_fewer_k_tiles_per_wave(m, k):
                    variant=_lib.VARIANT_SKINNY, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
                    b_scale_layout=_lib.SCALE_E8M0_SHUFFLE)
     assert_f32_close(got, ref, "shuffled scales")
+
+
+@pytest.mark.parametrize("vname,m,split", [("auto", 16, 1), ("auto", 200, 1), ("t256x256_w2x2", 300, 1),
+                                           ("t128x128_w2x2", 384, 2), ("naive", 33, 1), ("auto", 4352, 1)])
+def test_one_scale_per_row_of_a(vname, m, split):
+    """a_scale [M], held for every 32-group of the row (the reference's
+    broadcast-scale kernel): same bits as the GEMM on the spread-out matrix, and
+    parity with the oracle on it."""
+    n, k = (4352, 768) if m > 1000 else (272, 2048)
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m, scale_lo=118, scale_hi=136)
+    per_row = np.ascontiguousarray(xs[:, 0])
+    spread = np.repeat(per_row[:, None], k // 32, axis=1)
+    v = ALL_VARIANTS[vname]
+    got = run_gemm(x, per_row, w_t, ws, torch.float32, variant=v, split_k=split)
+    same = run_gemm(x, spread, w_t, ws, torch.float32, variant=v, split_k=split)
+    assert np.array_equal(got, same)
+    if m <= 1000:
+        assert_f32_close(got, c_oracle.scaled_gemm_exact(x, w_t, spread, ws), vname)
+    # it needs the scratch buffer; without one the call is refused, nothing runs
+    gx, gs, gw, gws = to_gpu(x, per_row, w_t, ws)
+    out = torch.zeros(m, n, dtype=torch.float32, device=DEV)
+    with pytest.raises(ValueError, match="workspace"):
+        wave_amd.mxfp4_gemm(gx, gs, gw, gws, out, variant=v, workspace=False)
+    assert not bool(out.any())
+
+
+@pytest.mark.parametrize("batch,m,n,k", [(4, 96, 160, 512), (8, 1, 16384, 1664), (3, 16, 272, 8192)])
+def test_batched_a_with_shared_b(batch, m, n, k):
+    x, xs, w_t, ws = orc.make_inputs(batch * m, n, k, seed=batch + m)
+    gx, gxs, gw, gws = to_gpu(x.reshape(batch, m, k // 2), xs.reshape(batch, m, k // 32), w_t, ws)
+    out = torch.full((batch, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out)
+    torch.cuda.synchronize()
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    assert_f32_close(out.cpu().numpy().reshape(batch * m, n), ref)
+    with pytest.raises(ValueError, match="out"):
+        wave_amd.mxfp4_gemm(gx, gxs, gw, gws, torch.empty(batch * m, n, dtype=torch.float32, device=DEV))

@@ -149,3 +149,47 @@ def testScaledGemmMXFP4BatchedStyleM1():
     out = torch.zeros(1, 1024, dtype=torch.float32, device=DEV)
     gemm(x, x_scales, w.T.contiguous(), w_scales, out)
     torch.testing.assert_close(torchScaledGemmMXFP4(x, w, x_scales, w_scales), out.cpu(), check_dtype=False)
+
+
+@pytest.mark.parametrize("shape", [(512, 512, 512)])
+def testBroadcastedScaleGemmMXFP4(shape):
+    """tests/kernel/wave_gemm_mxfp_test.py:594-634."""
+    from wave_amd.kernel.wave.compile import WaveCompileOptions
+    from wave_amd.kernel.wave.templates import get_broadcasted_scale_gemm_mxfp4
+
+    broadcasted_scale_scaled_mma, hyperparams = get_broadcasted_scale_gemm_mxfp4(
+        shape, ScaledMMAType.F32_16x16x128_F8F6F4)
+    options = WaveCompileOptions(subs=hyperparams, canonicalize=True, schedule=None)
+    broadcasted_scale_scaled_mma = wave_compile(options, broadcasted_scale_scaled_mma)
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.float32, device=DEV)
+    compacted_x_scales = x_scales[:, 0].contiguous()
+    w_t = w.T.contiguous()
+    broadcasted_scale_scaled_mma(x, compacted_x_scales, w_t, w_scales, out)
+    broadcasted_compacted_x_scales = compacted_x_scales.view(-1, 1).repeat(1, x_scales.shape[-1]).contiguous()
+    torch_out = torchScaledGemmMXFP4(x, w, broadcasted_compacted_x_scales, w_scales)
+    torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+@pytest.mark.parametrize("batch", [4, 8])
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (1, 16384, 1664)])
+def testScaledBatchedGemmMXFP4(batch, shape):
+    """tests/kernel/wave_gemm_mxfp_test.py:302-339 (the 8192^3 and 16384^3
+    shapes of the reference need minutes of CPU oracle and are left to the
+    property tests)."""
+    from wave_amd.kernel.wave.templates import get_batched_scaled_gemm_template
+
+    options, batched_gemm = get_batched_scaled_gemm_template(shape, ScaledMMAType.F32_16x16x128_F8F6F4, None)
+    batched_gemm = wave_compile(options, batched_gemm)
+    linearized_shape = (batch * shape[0], shape[1], shape[2])
+    flat_x, w, flat_x_scales, w_scales = generate_gemm_afp4wfp4_inputs(linearized_shape, device=DEV)
+    w_t = w.T.contiguous()
+    x = flat_x.view(batch, shape[0], shape[2] // 2)
+    x_scales = flat_x_scales.view(batch, shape[0], shape[2] // 32)
+    w_t = w_t.view(shape[1], shape[2] // 2)
+    w_scales = w_scales.view(shape[1], shape[2] // 32)
+    out = torch.zeros(batch, shape[0], shape[1], dtype=torch.float32, device=DEV)
+    batched_gemm(x, x_scales, w_t, w_scales, out)
+    torch_flat_out = torchScaledGemmMXFP4(flat_x, w, flat_x_scales, w_scales)
+    torch_out = torch_flat_out.view(batch, shape[0], shape[1])
+    torch.testing.assert_close(torch_out, out.cpu())

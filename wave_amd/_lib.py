@@ -25,7 +25,7 @@ ERR_HIP = -7
 ERR_UNSUPPORTED = -8
 
 OUT_F32, OUT_BF16 = 0, 1
-SCALE_ROW_MAJOR, SCALE_E8M0_SHUFFLE, SCALE_MFMA32 = 0, 1, 2
+SCALE_ROW_MAJOR, SCALE_E8M0_SHUFFLE, SCALE_MFMA32, SCALE_PER_ROW = 0, 1, 2, 3
 B_ROW_MAJOR, B_PRESHUFFLE = 0, 1
 IN_F32, IN_BF16, IN_F16 = 0, 1, 2
 

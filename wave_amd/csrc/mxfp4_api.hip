@@ -29,15 +29,15 @@ int check_common(const void *a, const void *as, const void *b, const void *bs, c
                  int64_t n, int64_t k, int out_dtype, int asl, int bsl, int bl, int variant) {
   if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim) return WAVE_MXFP4_ERR_BAD_SHAPE;
   if (k % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
-  if (bad_enum(out_dtype, 2) || bad_enum(asl, 3) || bad_enum(bsl, 3) || bad_enum(bl, 2) ||
+  if (bad_enum(out_dtype, 2) || bad_enum(asl, 4) || bad_enum(bsl, 3) || bad_enum(bl, 2) ||
       bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
     return WAVE_MXFP4_ERR_BAD_ENUM;
   if (bl == WAVE_MXFP4_B_PRESHUFFLE && (n % 16 != 0 || k % 64 != 0)) return WAVE_MXFP4_ERR_BAD_SHAPE;
   if (m == 0 || n == 0) return WAVE_MXFP4_OK;  // nothing to read or write
   if (!c) return WAVE_MXFP4_ERR_NULL_POINTER;
   if (k > 0 && (!a || !as || !b || !bs)) return WAVE_MXFP4_ERR_NULL_POINTER;
-  if (!aligned(a, 16) || !aligned(b, 16) || !aligned(as, 8) || !aligned(bs, 8) || !aligned(c, 16))
-    return WAVE_MXFP4_ERR_MISALIGNED;
+  if (!aligned(a, 16) || !aligned(b, 16) || !aligned(bs, 8) || !aligned(c, 16)) return WAVE_MXFP4_ERR_MISALIGNED;
+  if (asl != WAVE_MXFP4_SCALE_PER_ROW && !aligned(as, 8)) return WAVE_MXFP4_ERR_MISALIGNED;
   // 32-bit offsets inside a tile: 256 rows of kp bytes must fit in 31 bits.
   if ((k / 2) * 256 >= ((int64_t)1 << 31)) return WAVE_MXFP4_ERR_UNSUPPORTED;
   return 1;  // proceed
@@ -146,7 +146,7 @@ const char *wave_mxfp4_status_string(int status) {
     case WAVE_MXFP4_ERR_BAD_SHAPE: return "bad shape (negative dims, K not a multiple of 32, or layout divisibility)";
     case WAVE_MXFP4_ERR_BAD_ENUM: return "dtype, layout or variant out of range";
     case WAVE_MXFP4_ERR_MISALIGNED: return "pointer not aligned as documented";
-    case WAVE_MXFP4_ERR_WORKSPACE: return "split-K workspace missing or too small";
+    case WAVE_MXFP4_ERR_WORKSPACE: return "workspace missing or too small (split-K, per-row scales)";
     case WAVE_MXFP4_ERR_BAD_SPLIT: return "K per split is below 256 or not a multiple of 256";
     case WAVE_MXFP4_ERR_HIP: return "HIP call failed";
     case WAVE_MXFP4_ERR_UNSUPPORTED: return "unsupported argument combination";
@@ -166,10 +166,10 @@ static size_t round_up_256(size_t v) { return (v + 255) / 256 * 256; }
 size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant) {
   if (m <= 0 || n <= 0 || k <= 0 || split_k < 0 || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_)) return 0;
   const int v = pick_variant(m, n, k, variant);
-  if (v == WAVE_MXFP4_VARIANT_NAIVE) return 0;
+  size_t bytes = round_up_256((size_t)m * (size_t)(k / 32));  // per-row A scales spread out to [M, K/32]
+  if (v == WAVE_MXFP4_VARIANT_NAIVE) return bytes;
   int splits = split_k;
   if (splits == 0) splits = auto_split(m, n, k, v);
-  size_t bytes = 0;
   if (splits > 1) bytes += round_up_256((size_t)splits * (size_t)m * (size_t)n * sizeof(float));
   if (is_tile_variant(v) && k % kTileK == 0)
     bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
@@ -218,6 +218,17 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   }
 
   hipError_t e;
+  if (p.a_scale_layout == WAVE_MXFP4_SCALE_PER_ROW) {
+    // one scale per row: spread it over the row's groups, then it is a row-major scale matrix
+    const size_t need = round_up_256((size_t)m * (size_t)p.ks);
+    if (!workspace || ws_used + need > workspace_bytes) return WAVE_MXFP4_ERR_WORKSPACE;
+    uint8_t *ws = (uint8_t *)workspace + ws_used;
+    e = launch_scale_spread_rows(p.a_scale, ws, m, p.ks, stream);
+    if (e != hipSuccess) return record_hip(e);
+    p.a_scale = ws;
+    p.a_scale_layout = WAVE_MXFP4_SCALE_ROW_MAJOR;
+    ws_used += need;
+  }
   // The tile kernels read MFMA32-ordered scales with one dword per lane and one
   // cache line per wave instruction; row-major scales cost 32 lines per
   // instruction.  With scratch available, re-lay both operands out first
@@ -283,6 +294,7 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   int rc = check_common(a, a_scale, b, b_scale, c, total_rows, n, k, out_dtype, a_scale_layout,
                         b_scale_layout, b_layout, variant);
   if (rc <= 0) return rc;
+  if (a_scale_layout == WAVE_MXFP4_SCALE_PER_ROW) return WAVE_MXFP4_ERR_UNSUPPORTED;
   if (num_groups == 0) return WAVE_MXFP4_OK;
   if (!offsets) return WAVE_MXFP4_ERR_NULL_POINTER;
   if (!aligned(offsets, 4)) return WAVE_MXFP4_ERR_MISALIGNED;

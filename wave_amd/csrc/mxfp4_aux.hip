@@ -141,6 +141,14 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
   }
 }
 
+// dst[r, g] = src[r]: one scale per row spread over the row's ks groups.
+__global__ void scale_spread_rows_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t rows,
+                                         int64_t ks) {
+  const int64_t total = rows * ks;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = src[i / ks];
+}
+
 // One thread per 16-byte chunk.
 __global__ void b_preshuffle_kernel(const uint8_t *__restrict__ b, uint8_t *__restrict__ out, int64_t rows,
                                     int64_t kp) {
@@ -270,6 +278,11 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
     return hipErrorInvalidValue;
   dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)rt, 2);
   scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks);
+  return hipGetLastError();
+}
+
+hipError_t launch_scale_spread_rows(const uint8_t *src, uint8_t *dst, int64_t rows, int64_t ks, hipStream_t stream) {
+  scale_spread_rows_kernel<<<blocks_for(rows * ks, 256), 256, 0, stream>>>(src, dst, rows, ks);
   return hipGetLastError();
 }
 

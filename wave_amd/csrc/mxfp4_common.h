@@ -108,6 +108,7 @@ hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus);
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream);
 hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);
+hipError_t launch_scale_spread_rows(const uint8_t *src, uint8_t *dst, int64_t rows, int64_t ks, hipStream_t stream);
 hipError_t launch_quantize(const void *x, int in_dtype, uint8_t *q, uint8_t *scale, int64_t rows, int64_t k,
                            int scale_layout, int num_cus, hipStream_t stream);
 hipError_t launch_stream_gemm(const GemmParams &p, int num_cus, hipStream_t stream);

@@ -81,7 +81,7 @@ class WaveKernel:
         if split > 1:
             # The library splits K in whole 256-element tiles; take the largest
             # split count not above the requested one that does.
-            k = x.shape[1] * 2
+            k = x.shape[-1] * 2
             while split > 1 and (k % split != 0 or (k // split) % 256 != 0):
                 split -= 1
         _ops.mxfp4_gemm(x, x_scales, w_t, w_scales, out, a_scale_layout=s.a_scale_layout,

@@ -44,6 +44,9 @@ def _scale_rows_ok(scale: torch.Tensor, rows: int, ks: int, layout: int, name: s
     if layout == _lib.SCALE_ROW_MAJOR:
         if tuple(scale.shape) != (rows, ks):
             raise ValueError(f"{name}: expected shape {(rows, ks)}, got {tuple(scale.shape)}")
+    elif layout == _lib.SCALE_PER_ROW:
+        if tuple(scale.shape) != (rows,):
+            raise ValueError(f"{name}: expected shape {(rows,)}, got {tuple(scale.shape)}")
     else:
         need = ((rows + 31) // 32 * 32) * ((ks + 7) // 8 * 8)
         if scale.numel() < need:
@@ -79,14 +82,34 @@ def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW
     Same arguments, in the same order, as the reference's compiled kernel
     (tests/kernel/wave_gemm_mxfp_test.py:194-201).  ``workspace`` is an optional
     uint8 GPU tensor of ``workspace_bytes(...)`` bytes; by default a buffer cached
-    per device and stream is used, ``False`` runs without scratch."""
+    per device and stream is used, ``False`` runs without scratch.
+
+    Two more call shapes of the reference are taken as they are:
+    * batched A with a shared B, ``x [B, M, K/2]``, ``x_scales [B, M, K/32]``,
+      ``out [B, M, N]`` (tests/kernel/wave_gemm_mxfp_test.py:205-339): the batch
+      is folded into the rows, which it is in memory;
+    * one scale per row of A, ``x_scales [M]``, held for the whole row
+      (wave_lang/kernel/wave/templates/test_kernels.py:75-135)."""
     lib = _lib.load()
     x = _as_u8(x, "x")
     w_t = _as_u8(w_t, "w_t")
     x_scales = _as_u8(x_scales, "x_scales")
     w_scales = _as_u8(w_scales, "w_scales")
+    if x.dim() == 3:
+        if a_scale_layout != _lib.SCALE_ROW_MAJOR:
+            raise ValueError("batched x: scales must be row-major [B, M, K/32]")
+        bsz, bm = x.shape[0], x.shape[1]
+        if x_scales.dim() != 3 or tuple(x_scales.shape[:2]) != (bsz, bm):
+            raise ValueError(f"x_scales: expected [{bsz}, {bm}, K/32], got {tuple(x_scales.shape)}")
+        if out.dim() != 3 or tuple(out.shape[:2]) != (bsz, bm) or not out.is_contiguous():
+            raise ValueError(f"out: expected a contiguous [{bsz}, {bm}, N], got {tuple(out.shape)}")
+        x = x.reshape(bsz * bm, x.shape[2])
+        x_scales = x_scales.reshape(bsz * bm, x_scales.shape[2])
+        out = out.view(bsz * bm, out.shape[2])
+    if x_scales.dim() == 1 and a_scale_layout == _lib.SCALE_ROW_MAJOR:
+        a_scale_layout = _lib.SCALE_PER_ROW
     if x.dim() != 2 or w_t.dim() != 2:
-        raise ValueError("x and w_t must be 2-D")
+        raise ValueError("x must be 2-D (or 3-D batched) and w_t 2-D")
     m, kp = x.shape
     n = w_t.shape[0]
     if w_t.shape[1] != kp:

@@ -176,6 +176,52 @@ int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, 
 int wave_mxfp4_quantize(const void *x, int in_dtype, void *q, void *scale, int64_t rows, int64_t k,
                         int scale_layout, void *hip_stream);
 
+/* The quantiser over gathered rows: output row r is the quantised row
+ * row_ids[r] / row_div of x [src_rows, k]; an id at or beyond src_rows * row_div
+ * (the padding value of wave_mxfp4_moe_align_block_size) gives a row of zeros
+ * with scale bytes 0.  With row_ids = sorted_ids and row_div = top_k this is the
+ * reference's per-expert gather of the repeated activations,
+ * a.view(m, -1, k).repeat(1, topk, 1)[mask] (tests/kernel/moe_test.py:113-127),
+ * fused into the quantiser: its outputs are the grouped GEMM's A and A_scale. */
+int wave_mxfp4_quantize_rows(const void *x, int in_dtype, int64_t src_rows, const int32_t *row_ids, int row_div,
+                             void *q, void *scale, int64_t rows, int64_t k, int scale_layout, void *hip_stream);
+
+/* Token alignment by expert, moe_align_block_size of the reference
+ * (tests/kernel/moe/torch_kernels.py:10-92): topk_ids holds num_entries =
+ * num_tokens * top_k expert ids (int32, or int64 as torch.topk returns them:
+ * ids_int64 = 1).  sorted_ids[sorted_len] receives, expert by expert, the flat
+ * indices of the entries routed to that expert in increasing order, each
+ * expert's run padded to a multiple of block_size with the value num_entries,
+ * which also fills the buffer past the padded total; expert_ids[b] the expert
+ * of block b below the padded total / block_size; num_tokens_post_pad[0] the
+ * padded total.  expert_offsets (may be NULL) receives the num_experts + 1
+ * running sums of the padded counts: with block_size = 1 they are the `offsets`
+ * argument of wave_mxfp4_gemm_grouped over the sorted rows (not an output of
+ * the reference function).  Ids outside [0, num_experts) are skipped.
+ * num_experts <= 1024; sorted_len >= num_entries. */
+int wave_mxfp4_moe_align_block_size(const void *topk_ids, int ids_int64, int64_t num_entries, int num_experts,
+                                    int block_size, int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids,
+                                    int64_t expert_ids_len, int32_t *num_tokens_post_pad, int32_t *expert_offsets,
+                                    void *hip_stream);
+
+/* out = gate * up / (1 + exp(-gate)), the gated activation between the two
+ * expert GEMMs (silu_and_mul_ref, tests/kernel/moe_test.py:39-40; kernel
+ * wave_lang/kernel/wave/templates/moe.py:89-145).  gate, up, out are
+ * [rows, n] of dtype WAVE_MXFP4_IN_BF16 or WAVE_MXFP4_IN_F16 with row strides
+ * ld_* in elements (so the two halves of a [rows, 2n] GEMM output can be
+ * passed as gate = x, up = x + n, ld = 2n); computed in f32, rounded once.
+ * n and the strides are multiples of 8, pointers 16-byte aligned. */
+int wave_mxfp4_silu_and_mul(const void *gate, const void *up, void *out, int64_t ld_gate, int64_t ld_up,
+                            int64_t ld_out, int dtype, int64_t rows, int64_t n, void *hip_stream);
+
+/* The same activation fused into the quantiser: q, scale = quantise(round to
+ * dtype(silu(gate) * up)), bit-identical to wave_mxfp4_silu_and_mul followed
+ * by wave_mxfp4_quantize without the [rows, n] round trip through memory.
+ * n % 32 == 0. */
+int wave_mxfp4_silu_and_mul_quantize(const void *gate, const void *up, int64_t ld_gate, int64_t ld_up, int dtype,
+                                     void *q, void *scale, int64_t rows, int64_t n, int scale_layout,
+                                     void *hip_stream);
+
 /* Text for a status code; never NULL (the reference reports errors as
  * exceptions carrying hipGetErrorName/String, runtime.cpp:96-109). */
 const char *wave_mxfp4_status_string(int status);

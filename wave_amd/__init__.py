@@ -10,8 +10,12 @@ from .mxfp4 import (
     e8m0_to_f32,
     mxfp4_gemm,
     mxfp4_gemm_grouped,
+    moe_align_block_size,
     mxfp4_to_f32,
     quantize_mxfp4,
+    quantize_mxfp4_rows,
+    silu_and_mul,
+    silu_and_mul_quantize,
     scale_convert,
     workspace_bytes,
 )
@@ -23,8 +27,12 @@ __all__ = [
     "e8m0_to_f32",
     "mxfp4_gemm",
     "mxfp4_gemm_grouped",
+    "moe_align_block_size",
     "mxfp4_to_f32",
     "quantize_mxfp4",
+    "quantize_mxfp4_rows",
+    "silu_and_mul",
+    "silu_and_mul_quantize",
     "scale_convert",
     "workspace_bytes",
 ]

@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 3;
+constexpr int kAbiVersion = 4;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -386,8 +386,8 @@ int wave_mxfp4_b_preshuffle(const void *b, void *out, int64_t rows, int64_t kp, 
       launch_b_preshuffle((const uint8_t *)b, (uint8_t *)out, rows, kp, (hipStream_t)hip_stream));
 }
 
-int wave_mxfp4_quantize(const void *x, int in_dtype, void *q, void *scale, int64_t rows, int64_t k,
-                        int scale_layout, void *hip_stream) {
+static int check_quantize(const void *x, int in_dtype, const void *q, const void *scale, int64_t rows, int64_t k,
+                          int scale_layout) {
   if (rows < 0 || k < 0 || k % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
   if (bad_enum(in_dtype, 3) || bad_enum(scale_layout, 3)) return WAVE_MXFP4_ERR_BAD_ENUM;
   if (rows == 0 || k == 0) return WAVE_MXFP4_OK;
@@ -396,8 +396,82 @@ int wave_mxfp4_quantize(const void *x, int in_dtype, void *q, void *scale, int64
     return WAVE_MXFP4_ERR_MISALIGNED;
   if (scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && (k / 32) % 4 == 0 && !aligned(scale, 4))
     return WAVE_MXFP4_ERR_MISALIGNED;
-  return record_hip(launch_quantize(x, in_dtype, (uint8_t *)q, (uint8_t *)scale, rows, k, scale_layout, device_cus(),
-                                    (hipStream_t)hip_stream));
+  return 1;  // proceed
+}
+
+int wave_mxfp4_quantize(const void *x, int in_dtype, void *q, void *scale, int64_t rows, int64_t k,
+                        int scale_layout, void *hip_stream) {
+  const int rc = check_quantize(x, in_dtype, q, scale, rows, k, scale_layout);
+  if (rc <= 0) return rc;
+  return record_hip(launch_quantize(x, in_dtype, nullptr, 1, rows, (uint8_t *)q, (uint8_t *)scale, rows, k,
+                                    scale_layout, device_cus(), (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_quantize_rows(const void *x, int in_dtype, int64_t src_rows, const int32_t *row_ids, int row_div,
+                             void *q, void *scale, int64_t rows, int64_t k, int scale_layout, void *hip_stream) {
+  if (src_rows < 0 || row_div < 1) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  const int rc = check_quantize(x, in_dtype, q, scale, rows, k, scale_layout);
+  if (rc <= 0) return rc;
+  if (!row_ids) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(row_ids, 4)) return WAVE_MXFP4_ERR_MISALIGNED;
+  if (src_rows * (int64_t)row_div > 0x7FFFFFFF) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  return record_hip(launch_quantize(x, in_dtype, row_ids, row_div, src_rows, (uint8_t *)q, (uint8_t *)scale, rows, k,
+                                    scale_layout, device_cus(), (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_moe_align_block_size(const void *topk_ids, int ids_int64, int64_t num_entries, int num_experts,
+                                    int block_size, int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids,
+                                    int64_t expert_ids_len, int32_t *num_tokens_post_pad, int32_t *expert_offsets,
+                                    void *hip_stream) {
+  if (num_entries < 0 || num_experts < 1 || block_size < 1 || sorted_len < num_entries || expert_ids_len < 0)
+    return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (num_experts > kMoeMaxExperts) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  // the padded total must fit the int32 outputs
+  if (num_entries + (int64_t)num_experts * (block_size - 1) > 0x7FFFFFFF || sorted_len > 0x7FFFFFFF ||
+      expert_ids_len > 0x7FFFFFFF)
+    return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (bad_enum(ids_int64, 2)) return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (!num_tokens_post_pad || (num_entries > 0 && !topk_ids) || (sorted_len > 0 && !sorted_ids) ||
+      (expert_ids_len > 0 && !expert_ids))
+    return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(topk_ids, ids_int64 ? 8 : 4) || !aligned(sorted_ids, 4) || !aligned(expert_ids, 4) ||
+      !aligned(num_tokens_post_pad, 4) || !aligned(expert_offsets, 4))
+    return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_moe_align(topk_ids, ids_int64, num_entries, num_experts, block_size, sorted_ids, sorted_len,
+                                     expert_ids, expert_ids_len, num_tokens_post_pad, expert_offsets,
+                                     (hipStream_t)hip_stream));
+}
+
+static int check_gated(const void *gate, const void *up, int64_t ld_gate, int64_t ld_up, int dtype, int64_t rows,
+                       int64_t n, int64_t mult) {
+  if (rows < 0 || n < 0 || n % mult != 0 || ld_gate < n || ld_up < n || ld_gate % 8 != 0 || ld_up % 8 != 0)
+    return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (dtype != WAVE_MXFP4_IN_BF16 && dtype != WAVE_MXFP4_IN_F16) return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (rows == 0 || n == 0) return WAVE_MXFP4_OK;
+  if (!gate || !up) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(gate, 16) || !aligned(up, 16)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return 1;
+}
+
+int wave_mxfp4_silu_and_mul(const void *gate, const void *up, void *out, int64_t ld_gate, int64_t ld_up,
+                            int64_t ld_out, int dtype, int64_t rows, int64_t n, void *hip_stream) {
+  const int rc = check_gated(gate, up, ld_gate, ld_up, dtype, rows, n, 8);
+  if (rc <= 0) return rc;
+  if (ld_out < n || ld_out % 8 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (!out) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(out, 16)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_silu_and_mul(gate, up, out, ld_gate, ld_up, ld_out, dtype, rows, n, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_silu_and_mul_quantize(const void *gate, const void *up, int64_t ld_gate, int64_t ld_up, int dtype,
+                                     void *q, void *scale, int64_t rows, int64_t n, int scale_layout,
+                                     void *hip_stream) {
+  int rc = check_gated(gate, up, ld_gate, ld_up, dtype, rows, n, 32);
+  if (rc <= 0) return rc;
+  rc = check_quantize(gate, dtype, q, scale, rows, n, scale_layout);
+  if (rc <= 0) return rc;
+  return record_hip(launch_silu_and_mul_quantize(gate, up, ld_gate, ld_up, dtype, (uint8_t *)q, (uint8_t *)scale, rows, n,
+                                                 scale_layout, device_cus(), (hipStream_t)hip_stream));
 }
 
 }  // extern "C"

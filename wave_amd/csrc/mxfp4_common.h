@@ -109,8 +109,18 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus);
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream);
 hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);
 hipError_t launch_scale_spread_rows(const uint8_t *src, uint8_t *dst, int64_t rows, int64_t ks, hipStream_t stream);
-hipError_t launch_quantize(const void *x, int in_dtype, uint8_t *q, uint8_t *scale, int64_t rows, int64_t k,
-                           int scale_layout, int num_cus, hipStream_t stream);
+hipError_t launch_quantize(const void *x, int in_dtype, const int32_t *row_ids, int row_div, int64_t src_rows,
+                           uint8_t *q, uint8_t *scale, int64_t rows, int64_t k, int scale_layout, int num_cus,
+                           hipStream_t stream);
+hipError_t launch_silu_and_mul_quantize(const void *gate, const void *up, int64_t ld_gate, int64_t ld_up, int in_dtype,
+                                        uint8_t *q, uint8_t *scale, int64_t rows, int64_t n, int scale_layout,
+                                        int num_cus, hipStream_t stream);
+hipError_t launch_silu_and_mul(const void *gate, const void *up, void *out, int64_t ld_gate, int64_t ld_up,
+                               int64_t ld_out, int in_dtype, int64_t rows, int64_t n, hipStream_t stream);
+constexpr int kMoeMaxExperts = 1024;  // experts the alignment kernel keeps counters for in LDS
+hipError_t launch_moe_align(const void *topk_ids, int ids_int64, int64_t n, int num_experts, int block_size,
+                            int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids, int64_t expert_ids_len,
+                            int32_t *total, int32_t *offsets, hipStream_t stream);
 hipError_t launch_stream_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
 int stream_max_k_tiles();
 hipError_t launch_naive_gemm(const GemmParams &p, hipStream_t stream);

@@ -1,0 +1,132 @@
+// Token alignment in front of the grouped (MoE) GEMM: sort the (token, slot)
+// entries of a top-k routing table by expert, keep their original order inside
+// an expert, pad every expert's run to a multiple of the block size.  Integer
+// work on a few thousand to a few hundred thousand entries: one workgroup of
+// sixteen waves does it in one launch (count, scan, place), everything but the
+// ids themselves in LDS.
+#include "mxfp4_common.h"
+
+namespace wave_mxfp4 {
+
+namespace {
+
+constexpr int kAlignWaves = 16;
+constexpr int kAlignThreads = kAlignWaves * 64;
+
+// Inclusive sum over the workgroup's 1024 threads (one value each).
+__device__ __forceinline__ int block_inclusive_scan(int v, int *wave_sums, int lane, int wave) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int o = __shfl_up(v, d, 64);
+    if (lane >= d) v += o;
+  }
+  if (lane == 63) wave_sums[wave] = v;
+  __syncthreads();
+  int before = 0;
+  for (int w = 0; w < wave; ++w) before += wave_sums[w];
+  __syncthreads();
+  return v + before;
+}
+
+template <typename IdT>
+__global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__restrict__ topk_ids, int n, int num_experts,
+                                                                  int block_size, int32_t *__restrict__ sorted_ids,
+                                                                  int sorted_len, int32_t *__restrict__ expert_ids,
+                                                                  int expert_ids_len, int32_t *__restrict__ total_out,
+                                                                  int32_t *__restrict__ offsets_out) {
+  extern __shared__ int lds[];
+  int *cnt = lds;                                // [kAlignWaves][E]: entries of expert e in wave w's segment, later
+                                                 // the next free position for them
+  int *wave_sums = lds + kAlignWaves * num_experts;  // [kAlignWaves]
+  const int E = num_experts;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+
+  for (int i = t; i < kAlignWaves * E; i += kAlignThreads) cnt[i] = 0;
+  __syncthreads();
+
+  // wave w owns the contiguous segment [seg0, seg1) of the flat table
+  const int per_wave = ((n + kAlignWaves - 1) / kAlignWaves + 63) & ~63;
+  const int seg0 = min(n, wave * per_wave), seg1 = min(n, seg0 + per_wave);
+  for (int i = seg0 + lane; i < seg1; i += 64) {
+    const int64_t e = (int64_t)topk_ids[i];
+    if (e >= 0 && e < E) atomicAdd(&cnt[wave * E + (int)e], 1);
+  }
+  __syncthreads();
+
+  // thread e: the expert's count, padded count and first position
+  int count = 0;
+  if (t < E) {
+    for (int w = 0; w < kAlignWaves; ++w) count += cnt[w * E + t];
+  }
+  const int blocks = (count + block_size - 1) / block_size, padded = blocks * block_size;
+  const int end = block_inclusive_scan(padded, wave_sums, lane, wave);  // also the total, in the last thread
+  const int start = end - padded;
+  if (t < E) {
+    int run = start;
+    for (int w = 0; w < kAlignWaves; ++w) {
+      const int c = cnt[w * E + t];
+      cnt[w * E + t] = run;
+      run += c;
+    }
+    for (int i = start + count; i < min(end, sorted_len); ++i) sorted_ids[i] = n;  // the run's padding
+    for (int b = start / block_size; b < min(end / block_size, expert_ids_len); ++b) expert_ids[b] = t;
+    if (offsets_out) offsets_out[t] = start;
+  }
+  if (t == kAlignThreads - 1) wave_sums[0] = end;
+  __syncthreads();
+  const int total = wave_sums[0];
+  if (t == 0) {
+    total_out[0] = total;
+    if (offsets_out) offsets_out[E] = total;
+  }
+  for (int i = total + t; i < sorted_len; i += kAlignThreads) sorted_ids[i] = n;  // past the padded total
+
+  // place: a wave walks its segment in order; the lanes of one expert take consecutive positions
+  volatile int *next = cnt + wave * E;
+  for (int base = seg0; base < seg1; base += 64) {
+    const int i = base + lane;
+    const int64_t e64 = i < seg1 ? (int64_t)topk_ids[i] : -1;
+    const bool valid = e64 >= 0 && e64 < E;
+    const int e = valid ? (int)e64 : -1;
+    uint64_t todo = __ballot(valid);
+    while (todo) {
+      const int leader = __ffsll((unsigned long long)todo) - 1;
+      const int e0 = __shfl(e, leader, 64);
+      const uint64_t same = __ballot(e == e0);
+      const int first = next[e0];
+      if (e == e0) {
+        const int pos = first + __popcll(same & ((1ull << lane) - 1));
+        if (pos < sorted_len) sorted_ids[pos] = i;
+      }
+      if (lane == leader) next[e0] = first + __popcll(same);
+      todo &= ~same;
+    }
+  }
+}
+
+}  // namespace
+
+hipError_t launch_moe_align(const void *topk_ids, int ids_int64, int64_t n, int num_experts, int block_size,
+                            int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids, int64_t expert_ids_len,
+                            int32_t *total, int32_t *offsets, hipStream_t stream) {
+  const size_t lds = (size_t)(kAlignWaves * num_experts + kAlignWaves) * sizeof(int);
+  static bool attr_done[2] = {false, false};
+  const void *fn = ids_int64 ? (const void *)moe_align_kernel<int64_t> : (const void *)moe_align_kernel<int32_t>;
+  if (!attr_done[ids_int64 ? 1 : 0]) {
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)((kAlignWaves * kMoeMaxExperts + kAlignWaves) * sizeof(int)));
+    if (e != hipSuccess) return e;
+    attr_done[ids_int64 ? 1 : 0] = true;
+  }
+  if (ids_int64)
+    moe_align_kernel<int64_t><<<1, kAlignThreads, lds, stream>>>((const int64_t *)topk_ids, (int)n, num_experts, block_size,
+                                                                 sorted_ids, (int)sorted_len, expert_ids,
+                                                                 (int)expert_ids_len, total, offsets);
+  else
+    moe_align_kernel<int32_t><<<1, kAlignThreads, lds, stream>>>((const int32_t *)topk_ids, (int)n, num_experts, block_size,
+                                                                 sorted_ids, (int)sorted_len, expert_ids,
+                                                                 (int)expert_ids_len, total, offsets);
+  return hipGetLastError();
+}
+
+}  // namespace wave_mxfp4

@@ -92,32 +92,70 @@ struct Elems {
   }
 };
 
+// What one quantiser launch reads and writes.
+struct QuantParams {
+  const uint8_t *x;        // [src_rows, ld_x] elements; with `up`, the gate operand
+  const uint8_t *up;       // null, or the second operand of the gated activation silu(x) * up
+  const int32_t *row_ids;  // null, or for each output row the id of its source: row_ids[r] / row_div
+  uint8_t *q;              // [rows, k/2]
+  uint8_t *scale;
+  int64_t ld_x, ld_up;     // row strides of x and up in elements
+  int rows, k;
+  int src_rows;            // rows of x (a row id at or beyond src_rows * row_div yields a zero row)
+  int row_div;
+  int scale_layout;
+};
+
+// silu(g) * u in f32, rounded to the 16-bit storage type (the value the unfused
+// pipeline would have stored between its two kernels).
+template <int DT>
+__device__ __forceinline__ uint32_t gated_pair(uint32_t g2, uint32_t u2) {
+  float g[2], u[2], r[2];
+  if constexpr (DT == WAVE_MXFP4_IN_BF16) {
+    g[0] = __builtin_bit_cast(float, g2 << 16), g[1] = __builtin_bit_cast(float, g2 & 0xFFFF0000u);
+    u[0] = __builtin_bit_cast(float, u2 << 16), u[1] = __builtin_bit_cast(float, u2 & 0xFFFF0000u);
+  } else {
+    const f16x2 gh = __builtin_bit_cast(f16x2, g2), uh = __builtin_bit_cast(f16x2, u2);
+    g[0] = (float)gh.x, g[1] = (float)gh.y, u[0] = (float)uh.x, u[1] = (float)uh.y;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) r[i] = g[i] * u[i] / (1.0f + expf(-g[i]));
+  if constexpr (DT == WAVE_MXFP4_IN_BF16) {
+    const bf16x2 o = {(__bf16)r[0], (__bf16)r[1]};
+    return __builtin_bit_cast(uint32_t, o);
+  } else {
+    const f16x2 o = {(_Float16)r[0], (_Float16)r[1]};
+    return __builtin_bit_cast(uint32_t, o);
+  }
+}
+
 // A workgroup of four waves takes 32 rows x TC K tiles (TC*256 columns); a wave
 // takes 8 of the rows.  Four lanes share a scale group (8 elements each); the 16
 // quads of a wave take 16 consecutive groups of a row per pass, so that one load
 // instruction covers up to 1 KB (bf16) and one store 256 B of a row.
-template <int DT, int TC>
-__global__ void __launch_bounds__(256) quantize_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ q,
-                                                       uint8_t *__restrict__ scale, int rows, int k,
-                                                       int scale_layout) {
+// GATED: the elements are silu(x) * up of two 16-bit operands.
+template <int DT, int TC, bool GATED>
+__global__ void __launch_bounds__(256) quantize_kernel(const QuantParams p) {
   constexpr int kEb = Elems<DT>::kBytes;
   constexpr int kGroups = 8 * TC;              // scale groups of a tile row
   constexpr int kPasses = 8 * kGroups / 16;    // per wave: 8 rows x kGroups groups, 16 per pass
-  constexpr int kBatch = DT == WAVE_MXFP4_IN_F32 ? 4 : 8;  // passes whose loads are in flight together
+  constexpr int kBatch = DT == WAVE_MXFP4_IN_F32 || GATED ? 4 : 8;  // passes whose loads are in flight together
   static_assert(kPasses % kBatch == 0 || kPasses < kBatch, "passes come in whole batches");
+  static_assert(!GATED || DT != WAVE_MXFP4_IN_F32, "the gated activation takes 16-bit operands");
   constexpr int kB = kPasses < kBatch ? kPasses : kBatch;
   __shared__ uint32_t tile_scales[kQuantRows * kGroups / 4];
   uint8_t *tile_bytes = (uint8_t *)tile_scales;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int quad = lane >> 2, sub = lane & 3;
+  const int rows = p.rows, k = p.k, scale_layout = p.scale_layout;
   const int ks = k >> 5, ksp = (ks + 7) & ~7;
   const int col_tiles = (ks + kGroups - 1) / kGroups;
   const int row_tile = blockIdx.x / col_tiles, col_tile = blockIdx.x - row_tile * col_tiles;
   const int row0 = row_tile * kQuantRows, g0 = col_tile * kGroups;
 
   for (int pb = 0; pb < kPasses; pb += kB) {
-    Elems<DT> e[kB];
+    Elems<DT> e[kB], eu[GATED ? kB : 1];
     int lrow[kB], lgrp[kB];
 #pragma unroll
     for (int i = 0; i < kB; ++i) {
@@ -125,16 +163,28 @@ __global__ void __launch_bounds__(256) quantize_kernel(const uint8_t *__restrict
       lrow[i] = wave * 8 + u / kGroups;
       lgrp[i] = u % kGroups;
       const int row = row0 + lrow[i], g = g0 + lgrp[i];
-      const bool ok = row < rows && g < ks;
-      e[i].load(x + ((int64_t)row * k + (int64_t)g * 32 + sub * 8) * kEb, ok);
+      bool ok = row < rows && g < ks;
+      int64_t src = row;
+      if (p.row_ids) {  // gathered rows
+        const uint32_t id = ok ? (uint32_t)p.row_ids[row] : 0u;
+        src = id / (uint32_t)p.row_div;
+        ok = ok && src < p.src_rows;
+      }
+      const int64_t col = (int64_t)g * 32 + sub * 8;
+      e[i].load(p.x + (src * p.ld_x + col) * kEb, ok);
+      if constexpr (GATED) eu[i].load(p.up + (src * p.ld_up + col) * kEb, ok);
     }
 #pragma unroll
     for (int i = 0; i < kB; ++i) {
       const int row = row0 + lrow[i], g = g0 + lgrp[i];
+      if constexpr (GATED) {
+#pragma unroll
+        for (int w = 0; w < Elems<DT>::kDwords; ++w) e[i].d[w] = gated_pair<DT>(e[i].d[w], eu[i].d[w]);
+      }
       const uint32_t sb = scale_byte_of(quad_max(e[i].amax_bits()));
       const float sf = __builtin_bit_cast(float, sb ? sb << 23 : 0x00400000u);  // 2^(sb-127)
       const uint32_t codes = e[i].convert(sf);
-      if (row < rows && g < ks) __builtin_nontemporal_store(codes, (uint32_t *)(q + (int64_t)row * (k >> 1) + g * 16 + sub * 4));
+      if (row < rows && g < ks) __builtin_nontemporal_store(codes, (uint32_t *)(p.q + (int64_t)row * (k >> 1) + g * 16 + sub * 4));
       if (sub == 0) {
         const int at = scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR
                            ? lrow[i] * kGroups + lgrp[i]
@@ -145,6 +195,7 @@ __global__ void __launch_bounds__(256) quantize_kernel(const uint8_t *__restrict
   }
   __syncthreads();
 
+  uint8_t *scale = p.scale;
   if (scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR) {
     // kGroups bytes of each row are contiguous
     if ((ks & 3) == 0) {
@@ -169,33 +220,90 @@ __global__ void __launch_bounds__(256) quantize_kernel(const uint8_t *__restrict
   }
 }
 
-template <int DT>
-hipError_t launch_quantize_dt(const void *x, uint8_t *q, uint8_t *scale, int rows, int k, int scale_layout,
-                              int num_cus, hipStream_t stream) {
-  const int ks = k >> 5;
-  const int64_t row_tiles = (rows + kQuantRows - 1) / kQuantRows;
+template <int DT, bool GATED>
+hipError_t launch_quantize_dt(const QuantParams &p, int num_cus, hipStream_t stream) {
+  const int ks = p.k >> 5;
+  const int64_t row_tiles = (p.rows + kQuantRows - 1) / kQuantRows;
   // wide tiles (8 K tiles) when they still fill the chip twice over
   const int64_t wide = row_tiles * ((ks + 63) / 64), narrow = row_tiles * ((ks + 7) / 8);
   if (narrow > 0x7FFFFFFF) return hipErrorInvalidValue;
   if (wide >= 2 * (int64_t)(num_cus > 0 ? num_cus : 256)) {
-    quantize_kernel<DT, 8><<<dim3((unsigned)wide), 256, 0, stream>>>((const uint8_t *)x, q, scale, rows, k, scale_layout);
+    quantize_kernel<DT, 8, GATED><<<dim3((unsigned)wide), 256, 0, stream>>>(p);
   } else {
-    quantize_kernel<DT, 1><<<dim3((unsigned)narrow), 256, 0, stream>>>((const uint8_t *)x, q, scale, rows, k, scale_layout);
+    quantize_kernel<DT, 1, GATED><<<dim3((unsigned)narrow), 256, 0, stream>>>(p);
   }
   return hipGetLastError();
 }
 
+// Elementwise silu(gate) * up, 8 elements per thread.
+template <int DT>
+__global__ void __launch_bounds__(256) silu_and_mul_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
+                                                           uint8_t *__restrict__ out, int64_t ld_gate, int64_t ld_up,
+                                                           int64_t ld_out, int rows, int n) {
+  const int chunks = n >> 3;  // per row
+  const int64_t total = (int64_t)rows * chunks;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / chunks, c = (i - r * chunks) * 8;
+    const v4i g = __builtin_nontemporal_load((const v4i *)(gate + (r * ld_gate + c) * 2));
+    const v4i u = __builtin_nontemporal_load((const v4i *)(up + (r * ld_up + c) * 2));
+    v4i o;
+    o.x = (int)gated_pair<DT>((uint32_t)g.x, (uint32_t)u.x);
+    o.y = (int)gated_pair<DT>((uint32_t)g.y, (uint32_t)u.y);
+    o.z = (int)gated_pair<DT>((uint32_t)g.z, (uint32_t)u.z);
+    o.w = (int)gated_pair<DT>((uint32_t)g.w, (uint32_t)u.w);
+    *(v4i *)(out + (r * ld_out + c) * 2) = o;
+  }
+}
+
 }  // namespace
 
-hipError_t launch_quantize(const void *x, int in_dtype, uint8_t *q, uint8_t *scale, int64_t rows, int64_t k,
-                           int scale_layout, int num_cus, hipStream_t stream) {
-  if (rows > 0x7FFFFFFF || k > 0x7FFFFFFF) return hipErrorInvalidValue;
+hipError_t launch_quantize(const void *x, int in_dtype, const int32_t *row_ids, int row_div, int64_t src_rows,
+                           uint8_t *q, uint8_t *scale, int64_t rows, int64_t k, int scale_layout, int num_cus,
+                           hipStream_t stream) {
+  if (rows > 0x7FFFFFFF || k > 0x7FFFFFFF || src_rows > 0x7FFFFFFF) return hipErrorInvalidValue;
+  QuantParams p = {};
+  p.x = (const uint8_t *)x, p.row_ids = row_ids, p.q = q, p.scale = scale;
+  p.ld_x = k, p.rows = (int)rows, p.k = (int)k, p.src_rows = (int)src_rows, p.row_div = row_div > 0 ? row_div : 1;
+  p.scale_layout = scale_layout;
   switch (in_dtype) {
-    case WAVE_MXFP4_IN_F32: return launch_quantize_dt<WAVE_MXFP4_IN_F32>(x, q, scale, (int)rows, (int)k, scale_layout, num_cus, stream);
-    case WAVE_MXFP4_IN_BF16: return launch_quantize_dt<WAVE_MXFP4_IN_BF16>(x, q, scale, (int)rows, (int)k, scale_layout, num_cus, stream);
-    case WAVE_MXFP4_IN_F16: return launch_quantize_dt<WAVE_MXFP4_IN_F16>(x, q, scale, (int)rows, (int)k, scale_layout, num_cus, stream);
+    case WAVE_MXFP4_IN_F32: return launch_quantize_dt<WAVE_MXFP4_IN_F32, false>(p, num_cus, stream);
+    case WAVE_MXFP4_IN_BF16: return launch_quantize_dt<WAVE_MXFP4_IN_BF16, false>(p, num_cus, stream);
+    case WAVE_MXFP4_IN_F16: return launch_quantize_dt<WAVE_MXFP4_IN_F16, false>(p, num_cus, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t launch_silu_and_mul_quantize(const void *gate, const void *up, int64_t ld_gate, int64_t ld_up, int in_dtype,
+                                        uint8_t *q, uint8_t *scale, int64_t rows, int64_t n, int scale_layout,
+                                        int num_cus, hipStream_t stream) {
+  if (rows > 0x7FFFFFFF || n > 0x7FFFFFFF) return hipErrorInvalidValue;
+  QuantParams p = {};
+  p.x = (const uint8_t *)gate, p.up = (const uint8_t *)up, p.q = q, p.scale = scale;
+  p.ld_x = ld_gate, p.ld_up = ld_up, p.rows = (int)rows, p.k = (int)n, p.src_rows = (int)rows, p.row_div = 1;
+  p.scale_layout = scale_layout;
+  switch (in_dtype) {
+    case WAVE_MXFP4_IN_BF16: return launch_quantize_dt<WAVE_MXFP4_IN_BF16, true>(p, num_cus, stream);
+    case WAVE_MXFP4_IN_F16: return launch_quantize_dt<WAVE_MXFP4_IN_F16, true>(p, num_cus, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t launch_silu_and_mul(const void *gate, const void *up, void *out, int64_t ld_gate, int64_t ld_up,
+                               int64_t ld_out, int in_dtype, int64_t rows, int64_t n, hipStream_t stream) {
+  if (rows > 0x7FFFFFFF || n > 0x7FFFFFFF) return hipErrorInvalidValue;
+  const int64_t work = rows * (n >> 3);
+  int64_t blocks = (work + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks < 1) blocks = 1;
+  if (in_dtype == WAVE_MXFP4_IN_BF16)
+    silu_and_mul_kernel<WAVE_MXFP4_IN_BF16><<<dim3((unsigned)blocks), 256, 0, stream>>>(
+        (const uint8_t *)gate, (const uint8_t *)up, (uint8_t *)out, ld_gate, ld_up, ld_out, (int)rows, (int)n);
+  else if (in_dtype == WAVE_MXFP4_IN_F16)
+    silu_and_mul_kernel<WAVE_MXFP4_IN_F16><<<dim3((unsigned)blocks), 256, 0, stream>>>(
+        (const uint8_t *)gate, (const uint8_t *)up, (uint8_t *)out, ld_gate, ld_up, ld_out, (int)rows, (int)n);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
 }
 
 }  // namespace wave_mxfp4

@@ -307,3 +307,111 @@ def quantize_mxfp4(x: torch.Tensor, *, shuffle: bool = False, scale_layout: int 
                                      layout, _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp4_quantize")
     return q, scales
+
+
+def _new_scales(rows: int, ks: int, layout: int, device) -> torch.Tensor:
+    if layout == _lib.SCALE_ROW_MAJOR:
+        return torch.empty(rows, ks, dtype=torch.uint8, device=device)
+    return torch.empty((rows + 31) // 32 * 32, (ks + 7) // 8 * 8, dtype=torch.uint8, device=device)
+
+
+def quantize_mxfp4_rows(x: torch.Tensor, row_ids: torch.Tensor, row_div: int = 1, *,
+                        scale_layout: int = _lib.SCALE_ROW_MAJOR):
+    """Quantise gathered rows: output row ``r`` is row ``row_ids[r] // row_div``
+    of ``x [R, K]``; ids at or beyond ``R * row_div`` (the padding value of
+    :func:`moe_align_block_size`) give zero rows.  With ``row_ids = sorted_ids``
+    and ``row_div = top_k`` this is the per-expert gather of the repeated
+    activations in the reference's MoE (tests/kernel/moe_test.py:113-127) fused
+    into the quantiser.  Returns ``(q [len(row_ids), K/2], scales)``."""
+    lib = _lib.load()
+    if x.dim() != 2 or x.dtype not in _IN_DTYPES or x.device.type != "cuda":
+        raise ValueError("x: expected a [R, K] float32 / bfloat16 / float16 device tensor")
+    if row_ids.dtype != torch.int32 or row_ids.dim() != 1 or row_ids.device != x.device:
+        raise ValueError("row_ids: expected a 1-D int32 tensor on x's device")
+    x = x.contiguous()
+    row_ids = row_ids.contiguous()
+    src_rows, k = x.shape
+    if k % 32:
+        raise ValueError(f"x: K = {k} is not a multiple of 32")
+    rows = row_ids.numel()
+    q = torch.empty(rows, k // 2, dtype=torch.uint8, device=x.device)
+    scales = _new_scales(rows, k // 32, scale_layout, x.device)
+    with torch.cuda.device(x.device):
+        st = lib.wave_mxfp4_quantize_rows(x.data_ptr(), _IN_DTYPES[x.dtype], src_rows, row_ids.data_ptr(), int(row_div),
+                                          q.data_ptr(), scales.data_ptr(), rows, k, scale_layout,
+                                          _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp4_quantize_rows")
+    return q, scales
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: int, sorted_ids: torch.Tensor,
+                         expert_ids: torch.Tensor, num_tokens_post_pad: torch.Tensor,
+                         expert_offsets: torch.Tensor | None = None) -> None:
+    """Same arguments as the reference's ``moe_align_block_size_pytorch``
+    (tests/kernel/moe/torch_kernels.py:10-92): all outputs are pre-allocated by
+    the caller (int32) and filled in place.  ``expert_offsets`` (optional,
+    ``num_experts + 1`` int32) receives the running sums of the padded counts."""
+    lib = _lib.load()
+    if topk_ids.dtype not in (torch.int32, torch.int64) or not topk_ids.is_cuda:
+        raise ValueError("topk_ids: expected an int32 or int64 device tensor")
+    for name, t in (("sorted_ids", sorted_ids), ("expert_ids", expert_ids),
+                    ("num_tokens_post_pad", num_tokens_post_pad), ("expert_offsets", expert_offsets)):
+        if t is not None and (t.dtype != torch.int32 or not t.is_contiguous() or t.device != topk_ids.device):
+            raise ValueError(f"{name}: expected a contiguous int32 tensor on topk_ids' device")
+    if expert_offsets is not None and expert_offsets.numel() < num_experts + 1:
+        raise ValueError("expert_offsets: needs num_experts + 1 entries")
+    if num_tokens_post_pad.numel() < 1:
+        raise ValueError("num_tokens_post_pad: needs one entry")
+    ids = topk_ids.contiguous()
+    with torch.cuda.device(ids.device):
+        st = lib.wave_mxfp4_moe_align_block_size(
+            ids.data_ptr(), 1 if ids.dtype == torch.int64 else 0, ids.numel(), int(num_experts), int(block_size),
+            sorted_ids.data_ptr(), sorted_ids.numel(), expert_ids.data_ptr(), expert_ids.numel(),
+            num_tokens_post_pad.data_ptr(), expert_offsets.data_ptr() if expert_offsets is not None else None,
+            _stream_ptr(ids.device))
+    _lib.check(st, "wave_mxfp4_moe_align_block_size")
+
+
+def _gated_args(gate: torch.Tensor, up: torch.Tensor):
+    if gate.dim() != 2 or gate.shape != up.shape or gate.dtype != up.dtype or gate.device != up.device:
+        raise ValueError("gate and up: expected two [M, N] tensors of one dtype on one device")
+    if gate.dtype not in (torch.bfloat16, torch.float16) or not gate.is_cuda:
+        raise ValueError(f"gate: expected a bfloat16 or float16 device tensor, got {gate.dtype}")
+    # row strides are passed through (the halves of a [M, 2N] tensor are fine); anything else is copied
+    gate = gate if gate.stride(1) == 1 else gate.contiguous()
+    up = up if up.stride(1) == 1 else up.contiguous()
+    return gate, up
+
+
+def silu_and_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``gate * up / (1 + exp(-gate))`` (tests/kernel/moe_test.py:39-40,69-79),
+    f32 inside, rounded once to the inputs' dtype."""
+    lib = _lib.load()
+    gate, up = _gated_args(gate, up)
+    rows, n = gate.shape
+    if out is None:
+        out = torch.empty(rows, n, dtype=gate.dtype, device=gate.device)
+    elif out.shape != gate.shape or out.dtype != gate.dtype or out.stride(1) != 1:
+        raise ValueError("out: expected the shape and dtype of gate, unit column stride")
+    with torch.cuda.device(gate.device):
+        st = lib.wave_mxfp4_silu_and_mul(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.stride(0), up.stride(0),
+                                         out.stride(0), _IN_DTYPES[gate.dtype], rows, n, _stream_ptr(gate.device))
+    _lib.check(st, "wave_mxfp4_silu_and_mul")
+    return out
+
+
+def silu_and_mul_quantize(gate: torch.Tensor, up: torch.Tensor, *, scale_layout: int = _lib.SCALE_ROW_MAJOR):
+    """:func:`silu_and_mul` followed by :func:`quantize_mxfp4` in one kernel
+    (same bits, no ``[M, N]`` round trip): the A operand of the second expert
+    GEMM.  Returns ``(q [M, N/2], scales)``."""
+    lib = _lib.load()
+    gate, up = _gated_args(gate, up)
+    rows, n = gate.shape
+    q = torch.empty(rows, n // 2, dtype=torch.uint8, device=gate.device)
+    scales = _new_scales(rows, n // 32, scale_layout, gate.device)
+    with torch.cuda.device(gate.device):
+        st = lib.wave_mxfp4_silu_and_mul_quantize(gate.data_ptr(), up.data_ptr(), gate.stride(0), up.stride(0),
+                                                  _IN_DTYPES[gate.dtype], q.data_ptr(), scales.data_ptr(), rows, n,
+                                                  scale_layout, _stream_ptr(gate.device))
+    _lib.check(st, "wave_mxfp4_silu_and_mul_quantize")
+    return q, scales

@@ -103,13 +103,42 @@ def cpu_baseline(torch, m, n, k, seed, scale_range, sample_rows):
     }
 
 
+def time_quantize(torch, wave_amd, rows, k, steps, warmup, device, shuffle=True):
+    """(seconds per launch, algorithmic bytes) of the bf16 -> MXFP4 quantiser on a [rows, k] activation; three
+    inputs are rotated so that none is cache resident (402 MB together at 8192 x 8192)."""
+    xs = [torch.randn(rows, k, device=device, dtype=torch.bfloat16) for _ in range(3)]
+    lib = wave_amd._lib.load()
+    q = torch.empty(rows, k // 2, dtype=torch.uint8, device=device)
+    sc = torch.empty((rows + 31) // 32 * 32, (k // 32 + 7) // 8 * 8, dtype=torch.uint8, device=device)
+    stream = torch.cuda.current_stream().cuda_stream
+    layout = wave_amd._lib.SCALE_E8M0_SHUFFLE if shuffle else wave_amd._lib.SCALE_ROW_MAJOR
+
+    def run(count):
+        for i in range(count):
+            st = lib.wave_mxfp4_quantize(xs[i % 3].data_ptr(), wave_amd._lib.IN_BF16, q.data_ptr(), sc.data_ptr(),
+                                         rows, k, layout, stream)
+            if st != 0:
+                raise RuntimeError(f"wave_mxfp4_quantize: status {st}")
+
+    run(warmup)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    run(steps)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / steps, rows * k * 2 + rows * k // 2 + rows * k // 32
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100,
                     help="untimed launches first; the GPU needs ~30 ms of load to reach its steady clocks")
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["quant_bf16"],
+                    help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
+                         "8192 x 8192 bf16 activation of cfg2")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode-shape leg")
@@ -146,6 +175,22 @@ def main():
                           "bytes_written_per_launch": nbytes, "launches": args.warmup + args.steps}))
         return
 
+    if args.workload == "quant_bf16":
+        rows, k = 8192, 8192
+        qper, qbytes = time_quantize(torch, wave_amd, rows, k, args.steps, args.warmup, dev)
+        gbps = qbytes / qper / 1e9
+        print(json.dumps({
+            "metric": "activation quantiser, GB/s % HBM", "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(qper * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in, e2m1 + e8m0 out",
+            "data": "synthetic (normal)",
+            "config": {"workload": f"quant_bf16: bf16 [{rows}, {k}] -> MXFP4, scales in e8m0_shuffle order, "
+                                   "3 inputs rotated"},
+            "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                         "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": 134.3e6 + 35.65e6, "kernel": "quantize_kernel",
+                         "launch_us": round(qper * 1e6, 2)}}))
+        return
+
     m, n, k, od, seed, srange = WORKLOADS[args.workload]
     out_dtype = torch.bfloat16 if od == "bf16" else torch.float32
     out_bytes = 2 if od == "bf16" else 4
@@ -158,7 +203,7 @@ def main():
 
     # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this
     # command, scaled by a device copy of known size (profiles/pmc_*.txt); not measurable from here
-    measured_traffic = {"cfg2": 435e6 + 134.2e6, "cfg3_m16": 125.5e6 + 0.92e6}.get(args.workload) \
+    measured_traffic = {"cfg2": 435e6 + 134.2e6, "cfg3_m16": 125.6e6 + 0.92e6}.get(args.workload) \
         if args.variant == 0 else None
     flops, nbytes = gemm_flops(m, n, k), gemm_bytes(m, n, k, out_bytes)
     ms_per_step = wall / args.steps * 1e3
@@ -208,6 +253,18 @@ def main():
             "bytes": dbytes,
         }
         del dsets, dout
+
+    if not args.no_decode and args.workload == "cfg2":
+        # the step in front of the GEMM: quantise the bf16 activation of this workload
+        qper, qbytes = time_quantize(torch, wave_amd, m, k, args.steps, args.warmup, dev)
+        result["quantize_a"] = {
+            "workload": f"bf16 [{m}, {k}] -> e2m1 + e8m0 (e8m0_shuffle order), 3 inputs rotated",
+            "kernel": "quantize_kernel",
+            "launch_us": round(qper * 1e6, 2),
+            "gbps": round(qbytes / qper / 1e9, 1),
+            "frac_of_hbm_peak": round(qbytes / qper / 1e9 / PEAK_HBM_GBPS, 4),
+            "bytes": qbytes,
+        }
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, m, n, k, seed, srange, args.cpu_rows)

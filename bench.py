@@ -21,6 +21,7 @@ if ROOT not in sys.path:
 
 PEAK_MXFP4_TFLOPS = 10100.0   # MI355X dense FP4 MFMA
 PEAK_HBM_GBPS = 8000.0        # MI355X HBM3E
+PEAK_MXFP8_TFLOPS = 5000.0    # MI355X dense FP8 MFMA
 
 WORKLOADS = {
     # name: (m, n, k, out dtype, seed, scale range)
@@ -136,9 +137,9 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100,
                     help="untimed launches first; the GPU needs ~30 ms of load to reach its steady clocks")
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["quant_bf16"],
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["quant_bf16", "mxfp8"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
-                         "8192 x 8192 bf16 activation of cfg2")
+                         "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode-shape leg")
@@ -189,6 +190,40 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": 134.3e6 + 35.65e6, "kernel": "quantize_kernel",
                          "launch_us": round(qper * 1e6, 2)}}))
+        return
+
+    if args.workload == "mxfp8":
+        # tests/kernel/wave_gemm_mxfp_test.py:416-501 at its larger shape: e5m2 operands, scales 124..127, f32 out
+        m = n = k = 8192
+        g = torch.Generator(device=dev).manual_seed(5)
+        x = torch.randn(m, k, device=dev, generator=g).to(torch.float8_e5m2)
+        w_t = torch.randn(n, k, device=dev, generator=g).to(torch.float8_e5m2)
+        xs = torch.randint(124, 128, (m, k // 32), dtype=torch.uint8, device=dev, generator=g)
+        ws = torch.randint(124, 128, (n, k // 32), dtype=torch.uint8, device=dev, generator=g)
+        out = torch.empty(m, n, dtype=torch.float32, device=dev)
+
+        def run(count):
+            for _ in range(count):
+                wave_amd.mxfp8_gemm(x, xs, w_t, ws, out, variant=args.variant)
+
+        run(args.warmup)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        run(args.steps)
+        e1.record()
+        torch.cuda.synchronize()
+        per = e0.elapsed_time(e1) * 1e-3 / args.steps
+        tflops = 2.0 * m * n * k / per / 1e12
+        print(json.dumps({
+            "metric": "MXFP8 GEMM TFLOPS + % of FP8 MFMA peak (8192^3)", "value": round(tflops, 2), "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "mxfp8 (e5m2 x e8m0) in, f32 accumulate, f32 out", "data": "synthetic (normal values, seeded)",
+            "config": {"workload": f"mxfp8: M={m} N={n} K={k} f32 out seed 5", "variant": args.variant},
+            "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_MXFP8_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tflops / PEAK_MXFP8_TFLOPS, 4), "traffic": None, "kernel": "tile_gemm_kernel",
+                         "launch_us": round(per * 1e6, 2)}}))
         return
 
     m, n, k, od, seed, srange = WORKLOADS[args.workload]

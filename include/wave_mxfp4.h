@@ -132,6 +132,19 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
                             int64_t n, int64_t k, int out_dtype, int a_scale_layout,
                             int b_scale_layout, int b_layout, int variant, void *hip_stream);
 
+/* Element format of the MXFP8 operands (OCP MX: e4m3 is the "fn" variant without
+ * infinities, e5m2 is IEEE-like). */
+typedef enum { WAVE_MXFP8_E4M3 = 0, WAVE_MXFP8_E5M2 = 1 } wave_mxfp8_format;
+
+/* The same block-scaled GEMM on MXFP8 operands: A [M, K] and B [N, K] one byte
+ * per element (both of elem_format), scales [R, K/32] e8m0 row-major, C f32 or
+ * bf16.  Replaces the kernel of tests/kernel/wave_gemm_mxfp_test.py:416-501
+ * (tkl.f8e5m2 operands through the same scaled MFMA).  K % 128 == 0; variant
+ * AUTO, T256x256_W2x2 or T128x128_W2x2. */
+int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
+                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, int variant,
+                    void *hip_stream);
+
 /* Packed e2m1 [rows, kp] -> f32 [rows, 2*kp] through the 16-entry table, code 8
  * gives -0.0 (mxfp_utils.py:60-83).  Bit-exact. */
 int wave_mxfp4_to_f32(const void *q, float *out, int64_t rows, int64_t kp, void *hip_stream);

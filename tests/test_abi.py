@@ -16,7 +16,7 @@ HEADER = os.path.join(ROOT, "include", "wave_mxfp4.h")
 def declared_symbols():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(wave_mxfp4_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(wave_mxfp[48]_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():

@@ -1,0 +1,119 @@
+"""GPU: the MXFP8 block-scaled GEMM through the C ABI against the oracle
+(oracle/mxfp8_oracle.py).  Floating point: the products are exact and only the
+accumulation differs.  Bound: max|C - Cref| <= 1e-3 * max|Cref| (the reference's
+own test, tests/kernel/wave_gemm_mxfp_test.py:416-501, uses atol 2e-3, rtol
+1e-3), and the tighter 1e-4 * max|Cref| that the hardware's fp8 dot-product
+tree keeps in practice (it aligns the products of one instruction to their
+largest exponent before adding, so widely spread e5m2 magnitudes and scales lose
+more low bits than an f32 running sum would: 2.5e-5 measured with scales
+120..134)."""
+
+import numpy as np
+import pytest
+import torch
+
+import wave_amd
+from oracle import mxfp8_oracle as o8
+from wave_amd import _lib
+
+from gpu_util import DEV, assert_bf16_close, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+def assert_f32_close(c, ref, what=""):
+    ref = np.asarray(ref, dtype=np.float64)
+    c = np.asarray(c, dtype=np.float64)
+    assert c.shape == ref.shape and not np.isnan(c).any(), what
+    scale = np.abs(ref).max()
+    err = np.abs(c - ref).max()
+    assert err <= 1e-3 * scale, f"{what}: max err {err:g} > 1e-3 * {scale:g}"
+    assert err <= 1e-4 * scale, f"{what}: max err {err:g} > 1e-4 * {scale:g}"
+
+
+VARIANTS = {"auto": _lib.VARIANT_AUTO, "t256": _lib.VARIANT_T256x256_W2x2, "t128": _lib.VARIANT_T128x128_W2x2}
+
+
+def run(x, xs, w_t, ws, fmt, out_dtype=torch.float32, variant=_lib.VARIANT_AUTO):
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    out = torch.full((x.shape[0], w_t.shape[0]), float("nan"), dtype=out_dtype, device=DEV)
+    wave_amd.mxfp8_gemm(gx, gxs, gw, gws, out, elem_format=fmt, variant=variant)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("fmt", [o8.E5M2, o8.E4M3], ids=["e5m2", "e4m3"])
+@pytest.mark.parametrize("vname", sorted(VARIANTS))
+@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (256, 256, 512), (300, 200, 384), (1, 40, 256), (257, 33, 1152),
+                                   (1024, 1024, 1024)])
+def test_mxfp8_against_oracle(m, n, k, vname, fmt):
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=m + n + k, fmt=fmt, scale_lo=120, scale_hi=134)
+    ref = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, fmt)
+    assert_f32_close(run(x, xs, w_t, ws, fmt, variant=VARIANTS[vname]), ref, f"{vname} {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("fmt", [o8.E5M2, o8.E4M3], ids=["e5m2", "e4m3"])
+def test_mxfp8_bf16_output_and_every_code(fmt):
+    """Every finite byte value of the format appears in both operands."""
+    m, n, k = 256, 384, 256
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=7, fmt=fmt)
+    table = o8.E5M2_TABLE if fmt == o8.E5M2 else o8.E4M3_TABLE
+    finite = np.nonzero(np.isfinite(table) & (np.abs(table) < 64))[0].astype(np.uint8)
+    x[0, : len(finite)] = finite
+    w_t[5, : len(finite)] = finite[::-1]
+    ref = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, fmt)
+    assert_f32_close(run(x, xs, w_t, ws, fmt), ref)
+    assert_bf16_close(run(x, xs, w_t, ws, fmt, torch.bfloat16), ref)
+
+
+def test_mxfp8_one_hot_rows_read_back_b():
+    """A row of A that is 1.0 at one position picks out a column of dequantised B exactly."""
+    fmt = o8.E5M2
+    m, n, k = 128, 160, 256
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=3, fmt=fmt)
+    x[:] = 0
+    xs[:] = 127
+    one = int(np.nonzero(o8.E5M2_TABLE == 1.0)[0][0])
+    for r in range(m):
+        x[r, (r * 5) % k] = one
+    got = run(x, xs, w_t, ws, fmt)
+    deq = o8.fp8_to_f64(w_t, fmt) * np.exp2(ws.astype(np.float64) - 127).repeat(32, axis=1)
+    want = np.stack([deq[:, (r * 5) % k] for r in range(m)])
+    assert np.array_equal(got.astype(np.float64), want)
+
+
+def test_mxfp8_reference_style_and_torch_float8_inputs():
+    """tests/kernel/wave_gemm_mxfp_test.py:64-91,416-501 with float8 tensors passed as they are."""
+    shape = (1024, 1024, 1024)
+    torch.manual_seed(5)
+    x = torch.randn(shape[0], shape[2], device=DEV).to(torch.float8_e5m2)
+    w_t = torch.randn(shape[1], shape[2], device=DEV).to(torch.float8_e5m2)
+    x_scales = torch.randint(124, 128, (shape[0], shape[2] // 32), dtype=torch.uint8, device=DEV)
+    w_scales = torch.randint(124, 128, (shape[1], shape[2] // 32), dtype=torch.uint8, device=DEV)
+    out = torch.zeros(shape[0], shape[1], dtype=torch.float32, device=DEV)
+    wave_amd.mxfp8_gemm(x, x_scales, w_t, w_scales, out)
+    out2 = torch.zeros_like(out)
+    wave_amd.mxfp8_gemm(x.view(torch.int8), x_scales, w_t.view(torch.int8), w_scales, out2)   # the reference's call
+    assert torch.equal(out, out2)
+    xf = x.float().cpu() * torch.exp2(x_scales.cpu().float() - 127).repeat_interleave(32, 1)
+    wf = w_t.float().cpu() * torch.exp2(w_scales.cpu().float() - 127).repeat_interleave(32, 1)
+    torch.testing.assert_close(torch.mm(xf, wf.T), out.cpu(), atol=2e-3, rtol=1e-3)
+
+
+def test_mxfp8_argument_errors():
+    lib = _lib.load()
+    P = 0x1000
+    g = lambda **kw: lib.wave_mxfp8_gemm(*[kw.get(k, d) for k, d in (
+        ("a", P), ("as_", P), ("b", P), ("bs", P), ("c", P), ("m", 128), ("n", 128), ("k", 256), ("fmt", 1), ("od", 0),
+        ("variant", 0), ("stream", None))])
+    assert g(k=192) == _lib.ERR_BAD_SHAPE
+    assert g(m=-1) == _lib.ERR_BAD_SHAPE
+    assert g(fmt=2) == _lib.ERR_BAD_ENUM
+    assert g(od=3) == _lib.ERR_BAD_ENUM
+    assert g(variant=_lib.VARIANT_SKINNY) == _lib.ERR_UNSUPPORTED
+    assert g(a=None) == _lib.ERR_NULL_POINTER
+    assert g(b=P + 8) == _lib.ERR_MISALIGNED
+    assert g(m=0, a=None, c=None) == _lib.OK
+    with pytest.raises(ValueError):
+        wave_amd.mxfp8_gemm(torch.zeros(4, 96, dtype=torch.uint8, device=DEV), torch.zeros(4, 3, dtype=torch.uint8, device=DEV),
+                            torch.zeros(4, 96, dtype=torch.uint8, device=DEV), torch.zeros(4, 3, dtype=torch.uint8, device=DEV),
+                            torch.zeros(4, 4, device=DEV))

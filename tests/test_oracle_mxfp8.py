@@ -1,0 +1,50 @@
+"""CPU: pins of the MXFP8 oracle (oracle/mxfp8_oracle.py): the element decode
+against the library routine the reference relies on (``tensor.to(float32)`` of a
+float8 tensor, tests/kernel/wave_gemm_mxfp_test.py:82-83) over all byte values,
+the GEMM against a brute-force loop in exact rationals."""
+
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mxfp8_oracle as o8
+
+
+@pytest.mark.parametrize("fmt,dtype", [(o8.E5M2, torch.float8_e5m2), (o8.E4M3, torch.float8_e4m3fn)])
+def test_decode_every_byte_equals_torch(fmt, dtype):
+    b = torch.arange(256, dtype=torch.uint8)
+    want = b.view(dtype).to(torch.float32).numpy().astype(np.float64)
+    got = o8.fp8_to_f64(b.numpy(), fmt)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok], want[ok]) and np.array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
+
+
+def test_known_values():
+    assert o8.E5M2_TABLE[0x3C] == 1.0 and o8.E5M2_TABLE[0x7B] == 57344.0 and o8.E5M2_TABLE[0x01] == 2.0 ** -16
+    assert np.isinf(o8.E5M2_TABLE[0x7C]) and np.isnan(o8.E5M2_TABLE[0x7D])
+    assert o8.E4M3_TABLE[0x38] == 1.0 and o8.E4M3_TABLE[0x7E] == 448.0 and o8.E4M3_TABLE[0x01] == 2.0 ** -9
+    assert np.isnan(o8.E4M3_TABLE[0x7F]) and o8.E4M3_TABLE[0x78] == 256.0     # no infinity in e4m3fn
+
+
+@pytest.mark.parametrize("fmt", [o8.E5M2, o8.E4M3])
+def test_gemm_equals_brute_force(fmt):
+    m, n, k = 3, 4, 64
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=1, fmt=fmt, scale_lo=100, scale_hi=150)
+    got = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, fmt)
+    table = o8.E5M2_TABLE if fmt == o8.E5M2 else o8.E4M3_TABLE
+    for i in range(m):
+        for j in range(n):
+            acc = Fraction(0)
+            for kk in range(k):
+                acc += (Fraction(float(table[x[i, kk]])) * Fraction(2) ** (int(xs[i, kk // 32]) - 127)
+                        * Fraction(float(table[w_t[j, kk]])) * Fraction(2) ** (int(ws[j, kk // 32]) - 127))
+            assert abs(Fraction(float(got[i, j])) - acc) <= abs(acc) * Fraction(1, 2 ** 45)
+
+
+def test_generator_rounds_to_nearest_code():
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(8, 8, 128, seed=0, fmt=o8.E4M3)
+    assert x.dtype == np.uint8 and xs.shape == (8, 4) and np.isfinite(o8.fp8_to_f64(x, o8.E4M3)).all()
+    assert ((xs >= 124) & (xs <= 127)).all()

@@ -12,6 +12,7 @@ from .mxfp4 import (
     mxfp4_gemm_grouped,
     moe_align_block_size,
     mxfp4_to_f32,
+    mxfp8_gemm,
     quantize_mxfp4,
     quantize_mxfp4_rows,
     silu_and_mul,
@@ -29,6 +30,7 @@ __all__ = [
     "mxfp4_gemm_grouped",
     "moe_align_block_size",
     "mxfp4_to_f32",
+    "mxfp8_gemm",
     "quantize_mxfp4",
     "quantize_mxfp4_rows",
     "silu_and_mul",

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # WAVE_MXFP4_LIB points at another build of the same ABI (e.g. an experiment)
 LIB_PATH = os.environ.get("WAVE_MXFP4_LIB") or os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 # status codes of include/wave_mxfp4.h
 OK = 0
@@ -28,6 +28,7 @@ OUT_F32, OUT_BF16 = 0, 1
 SCALE_ROW_MAJOR, SCALE_E8M0_SHUFFLE, SCALE_MFMA32, SCALE_PER_ROW = 0, 1, 2, 3
 B_ROW_MAJOR, B_PRESHUFFLE = 0, 1
 IN_F32, IN_BF16, IN_F16 = 0, 1, 2
+MXFP8_E4M3, MXFP8_E5M2 = 0, 1
 
 VARIANT_AUTO = 0
 VARIANT_T256x256_W2x2 = 1
@@ -41,6 +42,7 @@ EXPORTS = (
     "wave_mxfp4_gemm",
     "wave_mxfp4_workspace_bytes",
     "wave_mxfp4_gemm_grouped",
+    "wave_mxfp8_gemm",
     "wave_mxfp4_to_f32",
     "wave_mxfp4_e8m0_to_f32",
     "wave_mxfp4_dequant",
@@ -78,6 +80,8 @@ def load():
     lib.wave_mxfp4_workspace_bytes.restype = sz
     lib.wave_mxfp4_gemm_grouped.argtypes = [p, p, p, p, p, p, i32, i64, i64, i64, i32, i32, i32, i32, i32, p]
     lib.wave_mxfp4_gemm_grouped.restype = i32
+    lib.wave_mxfp8_gemm.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.wave_mxfp8_gemm.restype = i32
     lib.wave_mxfp4_to_f32.argtypes = [p, p, i64, i64, p]
     lib.wave_mxfp4_to_f32.restype = i32
     lib.wave_mxfp4_e8m0_to_f32.argtypes = [p, p, i64, p]

@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 4;
+constexpr int kAbiVersion = 5;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -284,6 +284,50 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (e != hipSuccess) return record_hip(e);
   if (splits > 1) e = launch_splitk_reduce(p.partial, c, m * n, splits, p.out_bf16, stream);
   return record_hip(e);
+}
+
+int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
+                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, int variant,
+                    void *hip_stream) {
+  if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim || k % 128 != 0)
+    return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (bad_enum(elem_format, 2) || bad_enum(out_dtype, 2) || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
+    return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (variant != WAVE_MXFP4_VARIANT_AUTO && variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 &&
+      variant != WAVE_MXFP4_VARIANT_T128x128_W2x2)
+    return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (m == 0 || n == 0) return WAVE_MXFP4_OK;
+  if (!c) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (k > 0 && (!a || !a_scale || !b || !b_scale)) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(a, 16) || !aligned(b, 16) || !aligned(a_scale, 4) || !aligned(b_scale, 4) || !aligned(c, 16))
+    return WAVE_MXFP4_ERR_MISALIGNED;
+  if (k * 256 >= ((int64_t)1 << 31)) return WAVE_MXFP4_ERR_UNSUPPORTED;  // 32-bit offsets inside a tile
+  hipStream_t stream = (hipStream_t)hip_stream;
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t *)a, p.a_scale = (const uint8_t *)a_scale;
+  p.b = (const uint8_t *)b, p.b_scale = (const uint8_t *)b_scale;
+  p.c = c;
+  p.m = (int)m, p.n = (int)n, p.k = (int)k;
+  p.kp = (int)k;  // bytes per operand row
+  p.ks = (int)(k / 32);
+  p.ksp = (p.ks + 7) / 8 * 8;
+  p.k_tiles = (int)(k / 128);  // a K tile is 128 bytes of a row
+  p.tiles_per_split = p.k_tiles;
+  p.splits = 1;
+  p.out_bf16 = out_dtype == WAVE_MXFP4_OUT_BF16;
+  if (k == 0) {  // empty reduction: C = 0 (the naive kernel never touches the operands)
+    p.kp = 0;
+    return record_hip(launch_naive_gemm(p, stream));
+  }
+  int v = variant;
+  if (v == WAVE_MXFP4_VARIANT_AUTO)
+    v = ((m + 255) / 256) * ((n + 255) / 256) >= 128 ? WAVE_MXFP4_VARIANT_T256x256_W2x2 : WAVE_MXFP4_VARIANT_T128x128_W2x2;
+  int bm, bn;
+  tile_variant_shape(v, &bm, &bn);
+  p.tiles_m = (int)((m + bm - 1) / bm);
+  p.tiles_n = (int)((n + bn - 1) / bn);
+  return record_hip(launch_tile_gemm_fp8(p, v, elem_format == WAVE_MXFP8_E5M2, stream));
 }
 
 int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,

@@ -102,10 +102,19 @@ __device__ __forceinline__ const uint8_t *scale_tile_base(const uint8_t *base, i
 // rows that are not 8-byte multiples (K % 256 != 0).
 enum TileMode { kDirect = 0, kNative = 1, kGenericK = 2 };
 
-template <class Cfg, int MODE>
+// FMT is the element format code of the scaled MFMA: 4 = e2m1 (MXFP4, everything
+// described above), 0 = e4m3, 1 = e5m2 (MXFP8: tkl.f8e5m2 operands through the
+// same instruction, tests/kernel/wave_gemm_mxfp_test.py:416-501).  An MXFP8 row
+// holds one byte per element, so the same 128-byte K tile is 128 elements = two
+// 64-wide K steps of 32 bytes per lane = four scale groups; the byte geometry of
+// the ring, the DMA and the swizzle is unchanged.  MXFP8 takes row-major scales,
+// row-major B and kDirect only.
+template <class Cfg, int MODE, int FMT = 4>
 __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   constexpr bool GENERIC_K = MODE == kGenericK;
   constexpr bool NATIVE = MODE == kNative;
+  constexpr bool FP8 = FMT != 4;
+  static_assert(!FP8 || MODE == kDirect, "MXFP8 is built for directly read row-major scales only");
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
   constexpr int SLOT = Cfg::SLOT_BYTES, RING = Cfg::RING_SLOTS;
@@ -210,19 +219,42 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   // t*2 + l/32 of the LDS row.  Wave and tile row bases are multiples of 32,
   // so swz(row) only depends on the lane.
   const int fr = lane & 31, fg = lane >> 5;
+  // (MXFP8: K step s takes 32 bytes per lane in two halves, like the two 32-deep passes the instruction makes:
+  //  registers 0-3 hold K 16*(l/32) .. +15 of the step, registers 4-7 K 32 + 16*(l/32) .. +15, i.e. chunks
+  //  4s + l/32 and 4s + 2 + l/32; foff[2s + h] is half h.  The scale of lane l still belongs to the 32-block l/32.)
   uint32_t foff[4];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) foff[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
+  for (int t = 0; t < 4; ++t) {
+    const int chunk = FP8 ? (t >> 1) * 4 + (t & 1) * 2 + fg : t * 2 + fg;
+    foff[t] = (uint32_t)(fr * kTileKBytes + ((chunk ^ ((fr >> 1) & 7)) << 4));
+  }
   const uint32_t a_fbase = (uint32_t)(wave_m * Cfg::WM * kTileKBytes);
   const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
 
-  auto read_frags = [&](int slot_a, int slot_b, int t, v4i(&fa)[MT_M], v4i(&fb)[MT_N]) {
-    const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
-    const uint8_t *bb = smem + slot_b * SLOT + b_fbase + foff[t];
+  typedef typename std::conditional<FP8, v8i, v4i>::type Frag;
+  auto read_frags = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], Frag(&fb)[MT_N]) {
+    if constexpr (FP8) {
+      const uint8_t *ta = smem + slot_a * SLOT + a_fbase, *tb = smem + slot_b * SLOT + b_fbase;
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(ba + i * 32 * kTileKBytes);
+      for (int i = 0; i < MT_M; ++i) {
+        const v4i lo = *(const v4i *)(ta + foff[2 * t] + i * 32 * kTileKBytes);
+        const v4i hi = *(const v4i *)(ta + foff[2 * t + 1] + i * 32 * kTileKBytes);
+        fa[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
 #pragma unroll
-    for (int j = 0; j < MT_N; ++j) fb[j] = *(const v4i *)(bb + j * 32 * kTileKBytes);
+      for (int j = 0; j < MT_N; ++j) {
+        const v4i lo = *(const v4i *)(tb + foff[2 * t] + j * 32 * kTileKBytes);
+        const v4i hi = *(const v4i *)(tb + foff[2 * t + 1] + j * 32 * kTileKBytes);
+        fb[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+    } else {
+      const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
+      const uint8_t *bb = smem + slot_b * SLOT + b_fbase + foff[t];
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(ba + i * 32 * kTileKBytes);
+#pragma unroll
+      for (int j = 0; j < MT_N; ++j) fb[j] = *(const v4i *)(bb + j * 32 * kTileKBytes);
+    }
   };
 
   // ---------------- scales ----------------
@@ -238,8 +270,16 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   for (int j = 0; j < MT_N; ++j)
     scale_lane_setup(p.b_scale_layout, min(n0 + wave_n * Cfg::WN + j * 32 + fr, p.n - 1), n0, fg, p.ks, p.ksp,
                      b_soff[j], b_ssel[j]);
-  const ScaleAddr a_sa = scale_addr(p.a_scale_layout);
-  const ScaleAddr b_sa = scale_addr(p.b_scale_layout);
+  if constexpr (FP8) {
+    // row-major [R, K/32]: the K tile's four groups are one dword of the row; byte s of the canonical
+    // register is group 2s + fg
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) a_ssel[i] = fg ? 0x0c0c0301u : 0x0c0c0200u;
+#pragma unroll
+    for (int j = 0; j < MT_N; ++j) b_ssel[j] = fg ? 0x0c0c0301u : 0x0c0c0200u;
+  }
+  const ScaleAddr a_sa = FP8 ? ScaleAddr{4, 0} : scale_addr(p.a_scale_layout);
+  const ScaleAddr b_sa = FP8 ? ScaleAddr{4, 0} : scale_addr(p.b_scale_layout);
   const uint8_t *as_base = scale_tile_base(p.a_scale, p.a_scale_layout, m0, p.ks, p.ksp);
   const uint8_t *bs_base = scale_tile_base(bs_ptr, p.b_scale_layout, n0, p.ks, p.ksp);
   const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc(as_base);
@@ -280,13 +320,13 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
       raw_a[i][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, (int)a_soff[i], ao, 0);
-      if (!NATIVE)
+      if (!NATIVE && !FP8)
         raw_a[i][1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, (int)a_soff[i], ao + a_sa.delta, 0);
     }
 #pragma unroll
     for (int j = 0; j < MT_N; ++j) {
       raw_b[j][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(bs_rsrc, (int)b_soff[j], bo, 0);
-      if (!NATIVE)
+      if (!NATIVE && !FP8)
         raw_b[j][1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(bs_rsrc, (int)b_soff[j], bo + b_sa.delta, 0);
     }
   };
@@ -306,10 +346,10 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
     }
 #pragma unroll
     for (int i = 0; i < MT_M; ++i)
-      sc_a[i] = a_bytes ? raw_a[i][0] : perm_bytes(raw_a[i][1], raw_a[i][0], a_ssel[i]);
+      sc_a[i] = a_bytes ? raw_a[i][0] : perm_bytes(FP8 ? 0u : raw_a[i][1], raw_a[i][0], a_ssel[i]);
 #pragma unroll
     for (int j = 0; j < MT_N; ++j)
-      sc_b[j] = b_bytes ? raw_b[j][0] : perm_bytes(raw_b[j][1], raw_b[j][0], b_ssel[j]);
+      sc_b[j] = b_bytes ? raw_b[j][0] : perm_bytes(FP8 ? 0u : raw_b[j][1], raw_b[j][0], b_ssel[j]);
   };
 
   // ---------------- accumulators ----------------
@@ -321,16 +361,20 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
 #pragma unroll
       for (int g = 0; g < 16; ++g) acc[i][j][g] = 0.f;
 
-  auto mfma_block = [&](const v4i(&fa)[MT_M], const v4i(&fb)[MT_N], auto t_tag) {
+  auto mfma_block = [&](const Frag(&fa)[MT_M], const Frag(&fb)[MT_N], auto t_tag) {
     constexpr int T = decltype(t_tag)::value;
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
-      const v8i va = {fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
+      v8i va;
+      if constexpr (FP8) va = fa[i];
+      else va = v8i{fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
-        const v8i vb = {fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
+        v8i vb;
+        if constexpr (FP8) vb = fb[j];
+        else vb = v8i{fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
         // first port = B rows (N index), second port = A rows (M index)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][j], 4, 4, T,
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][j], FMT, FMT, T,
                                                                      (int)sc_b[j], T, (int)sc_a[i]);
       }
     }
@@ -369,7 +413,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   // After it all waves have finished reading tile j, which frees the slots of
   // A(j) (-> B(j+2), issued from P3 on) and B(j) (-> A(j+3)).
   // Fragments are double-buffered in registers across the K steps.
-  v4i fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  Frag fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
   constexpr int kWaitSteady = GENERIC_K ? 0 : A_LD;
   constexpr int kWaitPrologue = GENERIC_K ? 0 : A_LD + B_LD / 2;
 
@@ -400,6 +444,29 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
     const int sa1 = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
     const int sb1 = sa + 3 >= RING ? sa + 3 - RING : sa + 3;
     const int sa2 = sa + 4 >= RING ? sa + 4 - RING : sa + 4;
+    if constexpr (FP8) {
+      // two K steps per tile: the same DMA sequence folded into two phases
+      read_frags(sa, sb, 1, fa1, fb1);
+      mfma_block(fa0, fb0, T0{});
+      if (HAS1) issue_g2l(1, kt + 1, sb1, B_LD / 2, B_LD);
+      if (HAS2) issue_g2l(0, kt + 2, sa2, 0, A_LD);
+      __builtin_amdgcn_sched_barrier(0);
+      if (HAS1) {
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(HAS2 ? kWaitSteady : 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(sa1, sb1, 0, fa0, fb0);
+      }
+      mfma_block(fa1, fb1, T1{});
+      if (HAS2) issue_g2l(1, kt + 2, sa, 0, B_LD / 2);
+      __builtin_amdgcn_sched_barrier(0);
+      if (HAS1) canon_scales();
+      if (HAS2) load_scales(kt + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
     read_frags(sa, sb, 1, fa1, fb1);
     mfma_block(fa0, fb0, T0{});
     if (HAS1) issue_g2l(1, kt + 1, sb1, B_LD / 2, B_LD);
@@ -557,9 +624,9 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   }
 }
 
-template <class Cfg, int MODE>
+template <class Cfg, int MODE, int FMT>
 __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams p) {
-  tile_gemm_body<Cfg, MODE>(p);
+  tile_gemm_body<Cfg, MODE, FMT>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -578,11 +645,11 @@ void tile_variant_shape(int variant, int *bm, int *bn) {
   }
 }
 
-template <class Cfg, int MODE>
+template <class Cfg, int MODE, int FMT = 4>
 static hipError_t launch_cfg(const GemmParams &p, hipStream_t stream) {
   static bool attr_done = false;  // benign race: the attribute is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)tile_gemm_kernel<Cfg, MODE>,
+    hipError_t e = hipFuncSetAttribute((const void *)tile_gemm_kernel<Cfg, MODE, FMT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
@@ -590,7 +657,7 @@ static hipError_t launch_cfg(const GemmParams &p, hipStream_t stream) {
   const int total = p.tiles_m * p.tiles_n;
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
   dim3 grid(per_xcd * kNumXcd, p.splits, 1);
-  tile_gemm_kernel<Cfg, MODE><<<grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  tile_gemm_kernel<Cfg, MODE, FMT><<<grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
   return hipGetLastError();
 }
 
@@ -612,6 +679,15 @@ hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream
     case WAVE_MXFP4_VARIANT_T128x128_W2x2: return launch_by_scales<Cfg128x128w4>(p, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+// MXFP8: `p` describes the byte geometry (kp = K bytes per row, ks = K/32, k_tiles = K/128).
+hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int e5m2, hipStream_t stream) {
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2)
+    return e5m2 ? launch_cfg<Cfg256x256w4, kDirect, 1>(p, stream) : launch_cfg<Cfg256x256w4, kDirect, 0>(p, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2)
+    return e5m2 ? launch_cfg<Cfg128x128w4, kDirect, 1>(p, stream) : launch_cfg<Cfg128x128w4, kDirect, 0>(p, stream);
+  return hipErrorInvalidValue;
 }
 
 }  // namespace wave_mxfp4

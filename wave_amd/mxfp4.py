@@ -415,3 +415,44 @@ def silu_and_mul_quantize(gate: torch.Tensor, up: torch.Tensor, *, scale_layout:
                                                   scale_layout, _stream_ptr(gate.device))
     _lib.check(st, "wave_mxfp4_silu_and_mul_quantize")
     return q, scales
+
+
+_FP8_FORMATS = {torch.float8_e4m3fn: _lib.MXFP8_E4M3, torch.float8_e5m2: _lib.MXFP8_E5M2}
+
+
+def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format: int | None = None,
+               variant=_lib.VARIANT_AUTO) -> None:
+    """``out[M, N] = (x * scales) @ (w_t * scales).T`` for MXFP8 operands:
+    ``x [M, K]``, ``w_t [N, K]`` one byte per element, scales ``[R, K/32]`` e8m0
+    (tests/kernel/wave_gemm_mxfp_test.py:416-501, which passes
+    ``x.view(torch.int8)`` of ``float8_e5m2`` tensors).  float8 tensors carry
+    their format; for uint8 / int8 views pass ``elem_format`` (default e5m2, the
+    reference's ``tkl.f8e5m2``)."""
+    lib = _lib.load()
+    fmt = elem_format
+    ops = []
+    for name, t in (("x", x), ("w_t", w_t)):
+        if t.dtype in _FP8_FORMATS:
+            if fmt is not None and fmt != _FP8_FORMATS[t.dtype]:
+                raise ValueError(f"{name}: {t.dtype} does not match elem_format {fmt}")
+            fmt = _FP8_FORMATS[t.dtype]
+            t = t.view(torch.uint8)
+        ops.append(_as_u8(t, name))
+    x, w_t = ops
+    if fmt is None:
+        fmt = _lib.MXFP8_E5M2
+    x_scales = _as_u8(x_scales, "x_scales")
+    w_scales = _as_u8(w_scales, "w_scales")
+    if x.dim() != 2 or w_t.dim() != 2 or x.shape[1] != w_t.shape[1]:
+        raise ValueError("x must be [M, K] and w_t [N, K]")
+    m, k = x.shape
+    n = w_t.shape[0]
+    if k % 128:
+        raise ValueError(f"K = {k} must be a multiple of 128")
+    _scale_rows_ok(x_scales, m, k // 32, _lib.SCALE_ROW_MAJOR, "x_scales")
+    _scale_rows_ok(w_scales, n, k // 32, _lib.SCALE_ROW_MAJOR, "w_scales")
+    od = _check_out(out, (m, n))
+    with torch.cuda.device(x.device):
+        st = lib.wave_mxfp8_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
+                                 out.data_ptr(), m, n, k, fmt, od, variant, _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp8_gemm")

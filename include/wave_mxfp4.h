@@ -140,10 +140,13 @@ typedef enum { WAVE_MXFP8_E4M3 = 0, WAVE_MXFP8_E5M2 = 1 } wave_mxfp8_format;
  * per element (both of elem_format), scales [R, K/32] e8m0 row-major, C f32 or
  * bf16.  Replaces the kernel of tests/kernel/wave_gemm_mxfp_test.py:416-501
  * (tkl.f8e5m2 operands through the same scaled MFMA).  K % 128 == 0; variant
- * AUTO, T256x256_W2x2 or T128x128_W2x2. */
+ * AUTO, T256x256_W2x2 or T128x128_W2x2.  `workspace` is optional scratch of
+ * wave_mxfp8_workspace_bytes(m, n, k) bytes (256-byte aligned): with it, and
+ * K % 256 == 0, the scales are first re-laid out for one-dword-per-lane reads. */
 int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
-                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, int variant,
-                    void *hip_stream);
+                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, void *workspace,
+                    size_t workspace_bytes, int variant, void *hip_stream);
+size_t wave_mxfp8_workspace_bytes(int64_t m, int64_t n, int64_t k);
 
 /* Packed e2m1 [rows, kp] -> f32 [rows, 2*kp] through the 16-entry table, code 8
  * gives -0.0 (mxfp_utils.py:60-83).  Bit-exact. */

@@ -34,10 +34,14 @@ VARIANTS = {"auto": _lib.VARIANT_AUTO, "t256": _lib.VARIANT_T256x256_W2x2, "t128
 
 
 def run(x, xs, w_t, ws, fmt, out_dtype=torch.float32, variant=_lib.VARIANT_AUTO):
+    """With the scratch buffer (scales re-laid out first) and without (read as given): same bits."""
     gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
     out = torch.full((x.shape[0], w_t.shape[0]), float("nan"), dtype=out_dtype, device=DEV)
     wave_amd.mxfp8_gemm(gx, gxs, gw, gws, out, elem_format=fmt, variant=variant)
+    direct = torch.full_like(out, float("nan"))
+    wave_amd.mxfp8_gemm(gx, gxs, gw, gws, direct, elem_format=fmt, variant=variant, workspace=False)
     torch.cuda.synchronize()
+    assert torch.equal(out, direct)
     return out.float().cpu().numpy()
 
 
@@ -104,7 +108,7 @@ def test_mxfp8_argument_errors():
     P = 0x1000
     g = lambda **kw: lib.wave_mxfp8_gemm(*[kw.get(k, d) for k, d in (
         ("a", P), ("as_", P), ("b", P), ("bs", P), ("c", P), ("m", 128), ("n", 128), ("k", 256), ("fmt", 1), ("od", 0),
-        ("variant", 0), ("stream", None))])
+        ("ws", None), ("wsb", 0), ("variant", 0), ("stream", None))])
     assert g(k=192) == _lib.ERR_BAD_SHAPE
     assert g(m=-1) == _lib.ERR_BAD_SHAPE
     assert g(fmt=2) == _lib.ERR_BAD_ENUM

@@ -43,6 +43,7 @@ EXPORTS = (
     "wave_mxfp4_workspace_bytes",
     "wave_mxfp4_gemm_grouped",
     "wave_mxfp8_gemm",
+    "wave_mxfp8_workspace_bytes",
     "wave_mxfp4_to_f32",
     "wave_mxfp4_e8m0_to_f32",
     "wave_mxfp4_dequant",
@@ -80,7 +81,9 @@ def load():
     lib.wave_mxfp4_workspace_bytes.restype = sz
     lib.wave_mxfp4_gemm_grouped.argtypes = [p, p, p, p, p, p, i32, i64, i64, i64, i32, i32, i32, i32, i32, p]
     lib.wave_mxfp4_gemm_grouped.restype = i32
-    lib.wave_mxfp8_gemm.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p]
+    lib.wave_mxfp8_gemm.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, p, sz, i32, p]
+    lib.wave_mxfp8_workspace_bytes.argtypes = [i64, i64, i64]
+    lib.wave_mxfp8_workspace_bytes.restype = sz
     lib.wave_mxfp8_gemm.restype = i32
     lib.wave_mxfp4_to_f32.argtypes = [p, p, i64, i64, p]
     lib.wave_mxfp4_to_f32.restype = i32

@@ -286,9 +286,14 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   return record_hip(e);
 }
 
+size_t wave_mxfp8_workspace_bytes(int64_t m, int64_t n, int64_t k) {
+  if (m <= 0 || n <= 0 || k <= 0 || k % 256 != 0) return 0;
+  return round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
+}
+
 int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
-                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, int variant,
-                    void *hip_stream) {
+                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, void *workspace,
+                    size_t workspace_bytes, int variant, void *hip_stream) {
   if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim || k % 128 != 0)
     return WAVE_MXFP4_ERR_BAD_SHAPE;
   if (bad_enum(elem_format, 2) || bad_enum(out_dtype, 2) || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
@@ -302,6 +307,7 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (!aligned(a, 16) || !aligned(b, 16) || !aligned(a_scale, 4) || !aligned(b_scale, 4) || !aligned(c, 16))
     return WAVE_MXFP4_ERR_MISALIGNED;
   if (k * 256 >= ((int64_t)1 << 31)) return WAVE_MXFP4_ERR_UNSUPPORTED;  // 32-bit offsets inside a tile
+  if (workspace && !aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
   hipStream_t stream = (hipStream_t)hip_stream;
   GemmParams p;
   memset(&p, 0, sizeof(p));
@@ -327,6 +333,15 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   tile_variant_shape(v, &bm, &bn);
   p.tiles_m = (int)((m + bm - 1) / bm);
   p.tiles_n = (int)((n + bn - 1) / bn);
+  // with scratch, re-lay both scale tensors out in MFMA32 order first (one launch), as the MXFP4 path does
+  const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k));
+  if (workspace && k % 256 == 0 && workspace_bytes >= wave_mxfp8_workspace_bytes(m, n, k) &&
+      launch_scale_pair_to_mfma32(p.a_scale, (uint8_t *)workspace, m, p.b_scale, (uint8_t *)workspace + a_bytes, n,
+                                  p.ks, stream) == hipSuccess) {
+    p.a_scale = (const uint8_t *)workspace;
+    p.b_scale = (const uint8_t *)workspace + a_bytes;
+    p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+  }
   return record_hip(launch_tile_gemm_fp8(p, v, elem_format == WAVE_MXFP8_E5M2, stream));
 }
 

@@ -107,14 +107,16 @@ enum TileMode { kDirect = 0, kNative = 1, kGenericK = 2 };
 // same instruction, tests/kernel/wave_gemm_mxfp_test.py:416-501).  An MXFP8 row
 // holds one byte per element, so the same 128-byte K tile is 128 elements = two
 // 64-wide K steps of 32 bytes per lane = four scale groups; the byte geometry of
-// the ring, the DMA and the swizzle is unchanged.  MXFP8 takes row-major scales,
-// row-major B and kDirect only.
+// the ring, the DMA and the swizzle is unchanged.  MXFP8 takes row-major B and
+// scales that are row-major (kDirect) or MFMA32-ordered (kNative: an MFMA32 block
+// covers 8 groups = two MXFP8 K tiles, the odd one's bytes sit in the upper half
+// of the lane's dword).
 template <class Cfg, int MODE, int FMT = 4>
 __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   constexpr bool GENERIC_K = MODE == kGenericK;
   constexpr bool NATIVE = MODE == kNative;
   constexpr bool FP8 = FMT != 4;
-  static_assert(!FP8 || MODE == kDirect, "MXFP8 is built for directly read row-major scales only");
+  static_assert(!FP8 || MODE != kGenericK, "MXFP8 needs whole K tiles");
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
   constexpr int SLOT = Cfg::SLOT_BYTES, RING = Cfg::RING_SLOTS;
@@ -270,7 +272,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   for (int j = 0; j < MT_N; ++j)
     scale_lane_setup(p.b_scale_layout, min(n0 + wave_n * Cfg::WN + j * 32 + fr, p.n - 1), n0, fg, p.ks, p.ksp,
                      b_soff[j], b_ssel[j]);
-  if constexpr (FP8) {
+  if constexpr (FP8 && !NATIVE) {
     // row-major [R, K/32]: the K tile's four groups are one dword of the row; byte s of the canonical
     // register is group 2s + fg
 #pragma unroll
@@ -278,8 +280,8 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
 #pragma unroll
     for (int j = 0; j < MT_N; ++j) b_ssel[j] = fg ? 0x0c0c0301u : 0x0c0c0200u;
   }
-  const ScaleAddr a_sa = FP8 ? ScaleAddr{4, 0} : scale_addr(p.a_scale_layout);
-  const ScaleAddr b_sa = FP8 ? ScaleAddr{4, 0} : scale_addr(p.b_scale_layout);
+  const ScaleAddr a_sa = FP8 && !NATIVE ? ScaleAddr{4, 0} : scale_addr(p.a_scale_layout);
+  const ScaleAddr b_sa = FP8 && !NATIVE ? ScaleAddr{4, 0} : scale_addr(p.b_scale_layout);
   const uint8_t *as_base = scale_tile_base(p.a_scale, p.a_scale_layout, m0, p.ks, p.ksp);
   const uint8_t *bs_base = scale_tile_base(bs_ptr, p.b_scale_layout, n0, p.ks, p.ksp);
   const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc(as_base);
@@ -316,7 +318,8 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
       }
       return;
     }
-    const int ao = kt * a_sa.kt_stride, bo = kt * b_sa.kt_stride;
+    const int blk = FP8 && NATIVE ? kt >> 1 : kt;  // MXFP8: one MFMA32 block serves two K tiles
+    const int ao = blk * a_sa.kt_stride, bo = blk * b_sa.kt_stride;
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
       raw_a[i][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(as_rsrc, (int)a_soff[i], ao, 0);
@@ -330,7 +333,17 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
         raw_b[j][1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(bs_rsrc, (int)b_soff[j], bo + b_sa.delta, 0);
     }
   };
-  auto canon_scales = [&]() {
+  auto canon_scales = [&](int kt) {
+    if constexpr (FP8 && NATIVE) {
+      // bytes 0, 1 of the canonical register: the tile's K steps; they are bytes 2, 3 of the block's dword for
+      // the odd tile of a pair.  A pinned instruction, for the reason given below.
+      const int shift = (kt & 1) * 16;
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(sc_a[i]) : "s"(shift), "v"(raw_a[i][0]));
+#pragma unroll
+      for (int j = 0; j < MT_N; ++j) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(sc_b[j]) : "s"(shift), "v"(raw_b[j][0]));
+      return;
+    }
     const bool a_bytes = GENERIC_K && (p.ks & 7) != 0 && p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
     const bool b_bytes = GENERIC_K && (p.ks & 7) != 0 && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
     if (NATIVE) {
@@ -430,7 +443,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  canon_scales();
+  canon_scales(kt_begin);
   if (nkt > 1) load_scales(kt_begin + 1);
   read_frags(0, 1, 0, fa0, fb0);
   __builtin_amdgcn_sched_barrier(0);
@@ -462,7 +475,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
       mfma_block(fa1, fb1, T1{});
       if (HAS2) issue_g2l(1, kt + 2, sa, 0, B_LD / 2);
       __builtin_amdgcn_sched_barrier(0);
-      if (HAS1) canon_scales();
+      if (HAS1) canon_scales(kt + 1);
       if (HAS2) load_scales(kt + 2);
       __builtin_amdgcn_sched_barrier(0);
       return;
@@ -494,7 +507,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
     if (HAS2) issue_g2l(1, kt + 2, sa, 0, B_LD / 2);
     order_phase();
     __builtin_amdgcn_sched_barrier(0);
-    if (HAS1) canon_scales();
+    if (HAS1) canon_scales(kt + 1);
     if (HAS2) load_scales(kt + 2);
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -682,11 +695,18 @@ hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream
 }
 
 // MXFP8: `p` describes the byte geometry (kp = K bytes per row, ks = K/32, k_tiles = K/128).
+template <class Cfg, int FMT>
+static hipError_t launch_fp8_by_scales(const GemmParams &p, hipStream_t stream) {
+  const bool native =
+      p.a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+  return native ? launch_cfg<Cfg, kNative, FMT>(p, stream) : launch_cfg<Cfg, kDirect, FMT>(p, stream);
+}
+
 hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int e5m2, hipStream_t stream) {
   if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2)
-    return e5m2 ? launch_cfg<Cfg256x256w4, kDirect, 1>(p, stream) : launch_cfg<Cfg256x256w4, kDirect, 0>(p, stream);
+    return e5m2 ? launch_fp8_by_scales<Cfg256x256w4, 1>(p, stream) : launch_fp8_by_scales<Cfg256x256w4, 0>(p, stream);
   if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2)
-    return e5m2 ? launch_cfg<Cfg128x128w4, kDirect, 1>(p, stream) : launch_cfg<Cfg128x128w4, kDirect, 0>(p, stream);
+    return e5m2 ? launch_fp8_by_scales<Cfg128x128w4, 1>(p, stream) : launch_fp8_by_scales<Cfg128x128w4, 0>(p, stream);
   return hipErrorInvalidValue;
 }
 

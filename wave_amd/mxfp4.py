@@ -421,13 +421,13 @@ _FP8_FORMATS = {torch.float8_e4m3fn: _lib.MXFP8_E4M3, torch.float8_e5m2: _lib.MX
 
 
 def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format: int | None = None,
-               variant=_lib.VARIANT_AUTO) -> None:
+               variant=_lib.VARIANT_AUTO, workspace=None) -> None:
     """``out[M, N] = (x * scales) @ (w_t * scales).T`` for MXFP8 operands:
     ``x [M, K]``, ``w_t [N, K]`` one byte per element, scales ``[R, K/32]`` e8m0
     (tests/kernel/wave_gemm_mxfp_test.py:416-501, which passes
     ``x.view(torch.int8)`` of ``float8_e5m2`` tensors).  float8 tensors carry
     their format; for uint8 / int8 views pass ``elem_format`` (default e5m2, the
-    reference's ``tkl.f8e5m2``)."""
+    reference's ``tkl.f8e5m2``).  ``workspace`` as in :func:`mxfp4_gemm`."""
     lib = _lib.load()
     fmt = elem_format
     ops = []
@@ -452,7 +452,14 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format: int | None = Non
     _scale_rows_ok(x_scales, m, k // 32, _lib.SCALE_ROW_MAJOR, "x_scales")
     _scale_rows_ok(w_scales, n, k // 32, _lib.SCALE_ROW_MAJOR, "w_scales")
     od = _check_out(out, (m, n))
+    ws_ptr, ws_bytes = None, 0
+    if workspace is None:
+        workspace = _workspace(x.device, int(lib.wave_mxfp8_workspace_bytes(m, n, k)))
+    elif workspace is False:
+        workspace = None
+    if workspace is not None:
+        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     with torch.cuda.device(x.device):
         st = lib.wave_mxfp8_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
-                                 out.data_ptr(), m, n, k, fmt, od, variant, _stream_ptr(x.device))
+                                 out.data_ptr(), m, n, k, fmt, od, ws_ptr, ws_bytes, variant, _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp8_gemm")

@@ -362,3 +362,28 @@ def test_batched_a_with_shared_b(batch, m, n, k):
     assert_f32_close(out.cpu().numpy().reshape(batch * m, n), ref)
     with pytest.raises(ValueError, match="out"):
         wave_amd.mxfp4_gemm(gx, gxs, gw, gws, torch.empty(batch * m, n, dtype=torch.float32, device=DEV))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("vname", ["t256x256_w2x2", "t256x256_w4x2"])
+@pytest.mark.parametrize("m", [4352 - 255, 4352 - 3, 4097])
+def test_persistent_path_ragged_m(m, vname, out_dtype):
+    """More tiles than CUs with a last tile row that runs past M: the rows past M
+    are read as zeros and never stored (a canary behind C stays intact)."""
+    n, k = 4352, 768
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m, scale_lo=120, scale_hi=134)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    buf = torch.full(((m + 300) * n,), 7.0, dtype=out_dtype, device=DEV)
+    out = buf[: m * n].view(m, n)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out, variant=ALL_VARIANTS[vname])
+    torch.cuda.synchronize()
+    assert bool((buf[m * n:] == 7.0).all())
+    rows = np.r_[0:64, m - 300:m]              # the oracle on the first rows and on the last two tile rows
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    assert_close(out.float().cpu().numpy()[rows], ref, out_dtype, f"{vname} M={m}")
+    # the one-tile-per-workgroup kernel (no scratch: scales read as given) agrees on every element
+    other = torch.empty_like(out)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, other, variant=ALL_VARIANTS[vname], workspace=False)
+    torch.cuda.synchronize()
+    diff = (out.float() - other.float()).abs().max().item()
+    assert diff <= (2e-6 if out_dtype == torch.float32 else 2.0 ** -7) * out.float().abs().max().item()

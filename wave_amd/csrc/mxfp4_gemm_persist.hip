@@ -15,7 +15,8 @@
 // behind the loads it needs; from the second K tile on the stores must have
 // drained, which by then they have had a whole K tile of time to do.
 //
-// Taken for M % 256 == 0, N % 256 == 0, K % 256 == 0, K >= 768, MFMA-native
+// Taken for N % 256 == 0, K % 256 == 0, K >= 768 (any M: the last tile row reads
+// and writes through descriptors that end with the tensors), MFMA-native
 // scales for both operands, no grouping, no split.  Everything else runs the
 // one-tile-per-workgroup kernel.  The reference writes one tile per workgroup
 // (wave_lang/kernel/wave/templates/tagged_mxfp4_gemm.py:38-145); the result
@@ -54,8 +55,11 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // ---------------- the tile sequence of this workgroup ----------------
   // Workgroup w takes ids w, w + grid, w + 2*grid, ...: the grid is a multiple
   // of the XCD count, so all of them map to the same XCD's run of tiles.
+  // a_lim / as_lim: bytes of A and of its scale blocks from the tile's first row to the end of the tensor
+  // (M need not be a multiple of the tile: rows past it read zeros and are never stored)
   const uint8_t *a_base[2], *b_base[2], *as_base[2], *bs_base[2];
-  int m0[2], n0[2];
+  int m0[2], n0[2], a_lim[2], as_lim[2];
+  const int m_blocks = (p.m + 31) >> 5;
   auto set_tile = [&](int which, int pid) -> bool {
     int tm, tn;
     if (pid >= padded || !map_tile(pid, p.tiles_m, p.tiles_n, tm, tn)) return false;
@@ -65,6 +69,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     b_base[which] = p.b + (int64_t)n0[which] * kp;
     as_base[which] = p.a_scale + (int64_t)(m0[which] >> 5) * k_tiles_blocks;
     bs_base[which] = p.b_scale + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
+    a_lim[which] = (int)min((int64_t)(p.m - m0[which]) * kp, (int64_t)0x7FFFFFFF);
+    as_lim[which] = (int)min((int64_t)(m_blocks - (m0[which] >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
     return true;
   };
   int pid = blockIdx.x;
@@ -86,7 +92,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // output tile `which` (0 = current, 1 = next), into ring slot `slot`.
   auto issue_g2l = [&](int which, int op, int kt, int slot, int d0, int d1) {
     uint8_t *dst_tile = smem + slot * SLOT;
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(op == 0 ? a_base[which] : b_base[which]);
+    const __amdgpu_buffer_rsrc_t rsrc =
+        op == 0 ? make_rsrc_n(a_base[which], a_lim[which]) : make_rsrc(b_base[which]);
     const int soff = op == 0 ? kt * kTileKBytes : kt * b_kt_stride;
 #pragma unroll
     for (int d = d0; d < d1; ++d) {
@@ -117,7 +124,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   const int s_lane = lane * 4;
   uint32_t raw_a[MT_M], raw_b[MT_N], sc_a[MT_M], sc_b[MT_N];
   auto load_scales = [&](int which, int kt) {
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(as_base[which]), rb = make_rsrc(bs_base[which]);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc_n(as_base[which], as_lim[which]), rb = make_rsrc(bs_base[which]);
 #pragma unroll
     for (int i = 0; i < MT_M; ++i)
       raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, s_lane, a_srow + i * k_tiles_blocks + kt * 256, 0);
@@ -248,7 +255,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     constexpr int NCH = RP / 16;       // chunks per row
     constexpr int LPR = NCH, RPI = 64 / LPR;
     uint8_t *stage = smem + slot * SLOT + wave * SW;
-    const int wm0 = tm0 + wave_m * Cfg::WM, wn0 = tn0 + wave_n * Cfg::WN;
+    const int wn0 = tn0 + wave_n * Cfg::WN;
     // Staging addresses are recomputed from the lane id at every tile: hoisted
     // out of the tile loop they would sit in registers through the main loop,
     // which has none to spare (a spill there costs a wait for the whole queue).
@@ -256,11 +263,16 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     asm volatile("" : "+v"(lane_v));
     const int fr = lane_v & 31, fg = lane_v >> 5;
     const int lr = lane_v / LPR, lc = lane_v % LPR;
-    const int64_t ldc = p.n;
+    // C goes out through a descriptor that ends with row M - 1: the rows of a last tile row past M are dropped
+    const int ldc = p.n;
+    constexpr int ELT = OUT_BF16 ? 2 : 4;
+    const __amdgpu_buffer_rsrc_t c_rsrc =
+        make_rsrc_n((uint8_t *)p.c + (int64_t)tm0 * ldc * ELT,
+                    (int)min((int64_t)(p.m - tm0) * ldc * ELT, (int64_t)0x7FFFFFFF));
+    const int wr0 = wave_m * Cfg::WM;  // the wave's first row inside the tile
     if (out_bf16) {
       constexpr int CP = RP / 2, JP = CP / 32;  // columns, 32-column tiles per pass
       typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
-      __bf16 *cbase = (__bf16 *)p.c;
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) {
 #pragma unroll
@@ -280,14 +292,14 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
           for (int r0 = 0; r0 < 32; r0 += RPI) {
             const int r = r0 + lr;
             const v4i v = *(const v4i *)(stage + r * RP + ((lc ^ (r & (NCH - 1))) << 4));
-            *(v4i *)(cbase + (int64_t)(wm0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 8) = v;
+            __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, ((wr0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 8) * 2,
+                                                       0, 0);
           }
           asm volatile("" ::: "memory");
         }
       }
     } else {
       constexpr int CP = RP / 4, JP = CP / 32;
-      float *cbase = (float *)p.c;
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) {
 #pragma unroll
@@ -307,7 +319,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
           for (int r0 = 0; r0 < 32; r0 += RPI) {
             const int r = r0 + lr;
             const v4f v = *(const v4f *)(stage + r * RP + ((lc ^ (r & (NCH - 1))) << 4));
-            *(v4f *)(cbase + (int64_t)(wm0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 4) = v;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc,
+                                                       ((wr0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 4) * 4, 0, 0);
           }
           asm volatile("" ::: "memory");
         }
@@ -343,7 +356,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const int npid = pid + (int)gridDim.x;
     const bool has_next = set_tile(1, npid);
     if (!has_next) {
-      m0[1] = m0[0], n0[1] = n0[0];
+      m0[1] = m0[0], n0[1] = n0[0], a_lim[1] = a_lim[0], as_lim[1] = as_lim[0];
       a_base[1] = a_base[0], b_base[1] = b_base[0], as_base[1] = as_base[0], bs_base[1] = bs_base[0];
     }
     k_tile(0, sa, b_slot(sa), std::integral_constant<int, kFirst>{}, pending_tag);
@@ -370,7 +383,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     pid = npid;
-    m0[0] = m0[1], n0[0] = n0[1];
+    m0[0] = m0[1], n0[0] = n0[1], a_lim[0] = a_lim[1], as_lim[0] = as_lim[1];
     a_base[0] = a_base[1], b_base[0] = b_base[1], as_base[0] = as_base[1], bs_base[0] = bs_base[1];
     return true;
   };
@@ -409,10 +422,10 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
   if (variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 && variant != WAVE_MXFP4_VARIANT_T256x256_W4x2) return false;
   if (p.num_groups != 0 || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
-  if ((p.m & 255) != 0 || (p.n & 255) != 0 || (p.k & (kTileK - 1)) != 0 || p.k_tiles < 3) return false;
+  if ((p.n & 255) != 0 || (p.k & (kTileK - 1)) != 0 || p.k_tiles < 3) return false;  // any M
   if (p.out_bf16 ? (p.n & 7) != 0 : (p.n & 3) != 0) return false;
   // 32-bit offsets inside one operand tile, and more tiles than workgroups
-  if ((int64_t)256 * p.kp >= ((int64_t)1 << 31)) return false;
+  if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31)) return false;
   const int grid = num_cus / kNumXcd * kNumXcd;
   return grid >= kNumXcd && (int64_t)p.tiles_m * p.tiles_n > grid;
 }

@@ -55,6 +55,13 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7FFFFFFF, 0x00020000);
 }
 
+// The same over [base, base + bytes): accesses past the end read zeros and drop
+// their stores, which is how the persistent kernel handles a last tile row that
+// runs past M without per-lane clamps or guards.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc_n(const void *base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
 // s_waitcnt immediate that waits for vmcnt <= n and lgkmcnt == 0 (gfx9
 // encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14).
 __host__ __device__ constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | (7 << 4) | ((n >> 4) << 14); }

@@ -137,9 +137,10 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100,
                     help="untimed launches first; the GPU needs ~30 ms of load to reach its steady clocks")
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["quant_bf16", "mxfp8"],
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
-                         "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out")
+                         "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out; "
+                         "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode-shape leg")
@@ -190,6 +191,45 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": 134.3e6 + 35.65e6, "kernel": "quantize_kernel",
                          "launch_us": round(qper * 1e6, 2)}}))
+        return
+
+    if args.workload == "cfg4":
+        # E = 8 experts, 4096 tokens x top-2 = 8192 rows dealt multinomially, rows sorted by expert, bf16 out, seed 3
+        import numpy as np
+
+        E, n, k, rows = 8, 14336, 4096, 8192
+        counts = np.random.default_rng(3).multinomial(rows, np.ones(E) / E)
+        offs = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).to(dev)
+        g = torch.Generator(device=dev).manual_seed(3)
+        x = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, device=dev, generator=g)
+        xs = torch.randint(124, 131, (rows, k // 32), dtype=torch.uint8, device=dev, generator=g)
+        w = torch.randint(0, 256, (E, n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+        ws = torch.randint(124, 131, (E, n, k // 32), dtype=torch.uint8, device=dev, generator=g)
+        out = torch.empty(rows, n, dtype=torch.bfloat16, device=dev)
+
+        def run(count):
+            for _ in range(count):
+                wave_amd.mxfp4_gemm_grouped(x, xs, w, ws, offs, out, variant=args.variant)
+
+        run(args.warmup)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        run(args.steps)
+        e1.record()
+        torch.cuda.synchronize()
+        per = e0.elapsed_time(e1) * 1e-3 / args.steps
+        tflops = 2.0 * rows * n * k / per / 1e12
+        print(json.dumps({
+            "metric": "grouped (MoE) MXFP4 GEMM TFLOPS", "value": round(tflops, 2), "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out", "data": "synthetic (seeded uniform)",
+            "config": {"workload": f"cfg4: E={E} N={n} K={k} rows={rows} (counts {counts.tolist()}) bf16 out seed 3",
+                       "variant": args.variant},
+            "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tflops / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "tile_gemm_kernel",
+                         "launch_us": round(per * 1e6, 2)}}))
         return
 
     if args.workload == "mxfp8":

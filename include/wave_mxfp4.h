@@ -126,11 +126,17 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
  * E shuffled buffers of ceil(N/32)*32 x ceil(K/256)*8 bytes each.
  * The reference has no grouped MXFP4 kernel: this replaces its per-expert
  * Python loop over single GEMMs (tests/kernel/moe_test.py:175-246).
+ * `workspace` is optional scratch (256-byte aligned) of
+ * wave_mxfp4_grouped_workspace_bytes(...) bytes: with it the scales of both
+ * operands are first re-laid out for one-dword-per-lane reads, as in
+ * wave_mxfp4_gemm (N % 32 == 0 and K % 256 == 0; otherwise it is not used).
  */
 int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,
                             void *c, const int32_t *offsets, int num_groups, int64_t total_rows,
                             int64_t n, int64_t k, int out_dtype, int a_scale_layout,
-                            int b_scale_layout, int b_layout, int variant, void *hip_stream);
+                            int b_scale_layout, int b_layout, int variant, void *workspace,
+                            size_t workspace_bytes, void *hip_stream);
+size_t wave_mxfp4_grouped_workspace_bytes(int64_t total_rows, int64_t n, int64_t k, int num_groups);
 
 /* Element format of the MXFP8 operands (OCP MX: e4m3 is the "fn" variant without
  * infinities, e5m2 is IEEE-like). */

@@ -92,7 +92,7 @@ def test_grouped_argument_validation():
     def grouped(a=P, as_=P, b=P, bs=P, c=P, off=P, e=4, rows=256, n=64, k=256, od=1, asl=0, bsl=0, bl=0,
                 variant=0):
         return lib.wave_mxfp4_gemm_grouped(a, as_, b, bs, c, off, e, rows, n, k, od, asl, bsl, bl, variant,
-                                           None)
+                                           None, 0, None)
 
     assert grouped(off=None) == _lib.ERR_NULL_POINTER
     assert grouped(a=None) == _lib.ERR_NULL_POINTER

@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 5;
+constexpr int kAbiVersion = 6;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -345,10 +345,16 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   return record_hip(launch_tile_gemm_fp8(p, v, elem_format == WAVE_MXFP8_E5M2, stream));
 }
 
+size_t wave_mxfp4_grouped_workspace_bytes(int64_t total_rows, int64_t n, int64_t k, int num_groups) {
+  if (total_rows <= 0 || n <= 0 || k <= 0 || num_groups <= 0 || k % kTileK != 0 || n % 32 != 0) return 0;
+  return round_up_256(scale_buffer_bytes(total_rows, k)) + round_up_256((size_t)num_groups * scale_buffer_bytes(n, k));
+}
+
 int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,
                             void *c, const int32_t *offsets, int num_groups, int64_t total_rows,
                             int64_t n, int64_t k, int out_dtype, int a_scale_layout,
-                            int b_scale_layout, int b_layout, int variant, void *hip_stream) {
+                            int b_scale_layout, int b_layout, int variant, void *workspace,
+                            size_t workspace_bytes, void *hip_stream) {
   if (num_groups < 0 || num_groups > 65536) return WAVE_MXFP4_ERR_BAD_SHAPE;
   int rc = check_common(a, a_scale, b, b_scale, c, total_rows, n, k, out_dtype, a_scale_layout,
                         b_scale_layout, b_layout, variant);
@@ -381,6 +387,32 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   // sum over groups of ceil(rows_e / bm) <= total_rows / bm + num_groups
   p.tiles_m = (int)(total_rows / bm + num_groups);
   p.tiles_n = (int)((n + bn - 1) / bn);
+  // With scratch: both scale tensors into the MFMA32 order first.  The experts' B scales are one
+  // [E * N, K/32] matrix whose 32-row blocks do not straddle experts when N % 32 == 0.
+  if (workspace && !aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
+  const size_t ws_need = wave_mxfp4_grouped_workspace_bytes(total_rows, n, k, num_groups);
+  if (workspace && ws_need != 0 && workspace_bytes >= ws_need && (int64_t)num_groups * n <= 0x7FFFFFFF) {
+    uint8_t *ws_a = (uint8_t *)workspace, *ws_b = ws_a + round_up_256(scale_buffer_bytes(total_rows, k));
+    hipError_t e = hipSuccess;
+    if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR) {
+      e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, total_rows, p.b_scale, ws_b, (int64_t)num_groups * n, p.ks, stream);
+    } else {
+      if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32)
+        e = launch_scale_convert(p.a_scale, p.a_scale_layout, ws_a, WAVE_MXFP4_SCALE_MFMA32, total_rows, p.ks, stream);
+      else
+        ws_a = const_cast<uint8_t *>(p.a_scale);
+      if (e == hipSuccess && p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32)
+        e = launch_scale_convert(p.b_scale, p.b_scale_layout, ws_b, WAVE_MXFP4_SCALE_MFMA32, (int64_t)num_groups * n,
+                                 p.ks, stream);
+      else if (e == hipSuccess)
+        ws_b = const_cast<uint8_t *>(p.b_scale);
+    }
+    if (e != hipSuccess) return record_hip(e);
+    p.a_scale = ws_a;
+    p.b_scale = ws_b;
+    p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+    p.b_scale_group_stride = n * (int64_t)p.ksp;  // N % 32 == 0: no padding rows between experts
+  }
   return record_hip(launch_tile_gemm(p, v, stream));
 }
 

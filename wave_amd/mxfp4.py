@@ -137,11 +137,11 @@ def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW
 
 def mxfp4_gemm_grouped(x, x_scales, w_t, w_scales, offsets, out, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,
                        b_scale_layout=_lib.SCALE_ROW_MAJOR, b_layout=_lib.B_ROW_MAJOR,
-                       variant=_lib.VARIANT_AUTO) -> None:
+                       variant=_lib.VARIANT_AUTO, workspace=None) -> None:
     """Grouped (MoE) GEMM: rows ``offsets[e]:offsets[e+1]`` of ``x`` times
     expert ``e``'s ``w_t[e]`` ``[N, K/2]``; ``offsets`` is an int32 GPU tensor
     of E+1 entries.  ``out`` is ``[rows, N]``; rows past ``offsets[-1]`` are
-    left untouched."""
+    left untouched.  ``workspace`` as in :func:`mxfp4_gemm`."""
     lib = _lib.load()
     x = _as_u8(x, "x")
     w_t = _as_u8(w_t, "w_t")
@@ -170,11 +170,18 @@ def mxfp4_gemm_grouped(x, x_scales, w_t, w_scales, offsets, out, *, a_scale_layo
         if w_scales.numel() < need:
             raise ValueError(f"w_scales: shuffled scales need {need} bytes, got {w_scales.numel()}")
     od = _check_out(out, (rows, n))
+    ws_ptr, ws_bytes = None, 0
+    if workspace is None:
+        workspace = _workspace(x.device, int(lib.wave_mxfp4_grouped_workspace_bytes(rows, n, k, e)))
+    elif workspace is False:
+        workspace = None
+    if workspace is not None:
+        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     with torch.cuda.device(x.device):
         st = lib.wave_mxfp4_gemm_grouped(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(),
                                          w_scales.data_ptr(), out.data_ptr(), offsets.data_ptr(), e, rows,
                                          n, k, od, a_scale_layout, b_scale_layout, b_layout, variant,
-                                         _stream_ptr(x.device))
+                                         ws_ptr, ws_bytes, _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp4_gemm_grouped")
 
 

@@ -345,9 +345,18 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   return record_hip(launch_tile_gemm_fp8(p, v, elem_format == WAVE_MXFP8_E5M2, stream));
 }
 
+// Scratch of a grouped call: [M tile table | A scales, one 256-row slab per possible M tile | B scales].
+static size_t grouped_table_bytes(int64_t total_rows, int num_groups) {
+  return round_up_256((size_t)(1 + total_rows / 256 + num_groups) * 16);
+}
+static size_t grouped_a_scale_bytes(int64_t total_rows, int64_t k, int num_groups) {
+  return round_up_256(scale_buffer_bytes((total_rows / 256 + num_groups) * 256, k));
+}
+
 size_t wave_mxfp4_grouped_workspace_bytes(int64_t total_rows, int64_t n, int64_t k, int num_groups) {
   if (total_rows <= 0 || n <= 0 || k <= 0 || num_groups <= 0 || k % kTileK != 0 || n % 32 != 0) return 0;
-  return round_up_256(scale_buffer_bytes(total_rows, k)) + round_up_256((size_t)num_groups * scale_buffer_bytes(n, k));
+  return grouped_table_bytes(total_rows, num_groups) + grouped_a_scale_bytes(total_rows, k, num_groups) +
+         round_up_256((size_t)num_groups * scale_buffer_bytes(n, k));
 }
 
 int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,
@@ -392,8 +401,32 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   if (workspace && !aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
   const size_t ws_need = wave_mxfp4_grouped_workspace_bytes(total_rows, n, k, num_groups);
   if (workspace && ws_need != 0 && workspace_bytes >= ws_need && (int64_t)num_groups * n <= 0x7FFFFFFF) {
-    uint8_t *ws_a = (uint8_t *)workspace, *ws_b = ws_a + round_up_256(scale_buffer_bytes(total_rows, k));
+    int32_t *table = (int32_t *)workspace;
+    uint8_t *ws_a = (uint8_t *)workspace + grouped_table_bytes(total_rows, num_groups);
+    uint8_t *ws_b = ws_a + grouped_a_scale_bytes(total_rows, k, num_groups);
     hipError_t e = hipSuccess;
+    // Large problems on the 256x256 tiles: the persistent kernel over a device-built table of M tiles, with
+    // A's scales laid out per tile (a group may start at any row).
+    GemmParams q = p;
+    q.tile_table = table;
+    q.a_scale_layout = q.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+    if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
+        (p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR || p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32) &&
+        persist_gemm_applies(q, v, device_cus())) {
+      e = launch_grouped_tile_table(offsets, num_groups, 256, table, stream);
+      if (e != hipSuccess) return record_hip(e);
+      const bool b_native = p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+      e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, total_rows, p.b_scale, ws_b, b_native ? 0 : (int64_t)num_groups * n,
+                                      p.ks, stream, table, total_rows / 256 + num_groups);
+      if (e == hipSuccess) {
+        q.a_scale = ws_a;
+        if (!b_native) q.b_scale = ws_b;
+        q.b_scale_group_stride = n * (int64_t)p.ksp;
+        return record_hip(launch_persist_gemm(q, v, device_cus(), stream));
+      }
+      // (the fast re-layout does not apply: fall through to the one-tile-per-workgroup kernel)
+      e = hipSuccess;
+    }
     if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR) {
       e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, total_rows, p.b_scale, ws_b, (int64_t)num_groups * n, p.ks, stream);
     } else {

@@ -111,22 +111,36 @@ __global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_la
 // dword writes that walk the destination contiguously.
 // blockIdx.z picks one of two tensors with the same ks (the A and B scales of a
 // GEMM go through one launch; rows1 = 0 for a single tensor).
+// With `tiles0` (the M tile table of a grouped GEMM: entry 0 = {count}, entry
+// 1 + t = {first row, rows, expert}) tensor 0 is written tile by tile instead:
+// the 8 blocks of tile t hold rows first .. first + 255 (zeros past the tile's
+// rows), so that a tile's scales are block aligned wherever its group starts.
 __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__restrict__ src0,
                                                               uint8_t *__restrict__ dst0, int rows0,
                                                               const uint8_t *__restrict__ src1,
-                                                              uint8_t *__restrict__ dst1, int rows1, int ks) {
+                                                              uint8_t *__restrict__ dst1, int rows1, int ks,
+                                                              const int32_t *__restrict__ tiles0) {
   __shared__ uint32_t stage[32 * 65];
   const uint8_t *src = blockIdx.z ? src1 : src0;
   uint8_t *dst = blockIdx.z ? dst1 : dst0;
-  const int rows = blockIdx.z ? rows1 : rows0;
+  int rows = blockIdx.z ? rows1 : rows0;
   const int k_tiles = ks >> 3;
   const int rt = blockIdx.y, kt0 = blockIdx.x * 32;
-  if (rt * 32 >= rows) return;  // the grid is sized for the taller tensor
+  int row_base = rt * 32;
+  if (tiles0 != nullptr && blockIdx.z == 0) {
+    const int tile = rt >> 3;
+    if (tile >= tiles0[0]) return;
+    const int first = tiles0[4 * (1 + tile)], count = tiles0[4 * (1 + tile) + 1];
+    row_base = first + (rt & 7) * 32;
+    rows = first + count;
+  } else if (rt * 32 >= rows) {
+    return;  // the grid is sized for the taller tensor
+  }
   const int t = threadIdx.x;
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int unit = t + 256 * u, r = unit >> 5, ktl = unit & 31;
-    const int row = rt * 32 + r, kt = kt0 + ktl;
+    const int row = row_base + r, kt = kt0 + ktl;
     uint2 v = make_uint2(0u, 0u);
     if (row < rows && kt < k_tiles) v = *(const uint2 *)(src + (int64_t)row * ks + (int64_t)kt * 8);
     stage[ktl * 65 + r] = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u);       // groups 0, 2, 4, 6
@@ -259,7 +273,7 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
   if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 7) == 0 &&
       ((uintptr_t)src & 7) == 0 && rows < ((int64_t)1 << 31) && ks < ((int64_t)1 << 31) && rows_p / 32 <= 65535) {
     dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)(rows_p / 32), 1);
-    scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks);
+    scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks, nullptr);
     return hipGetLastError();
   }
   scale_convert_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(src, src_layout, dst, dst_layout, rows,
@@ -269,15 +283,19 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
 
 // Row-major -> MFMA32 for the scales of both GEMM operands in one launch.
 // Returns hipErrorInvalidValue (nothing launched) when the fast kernel does not apply.
+// With `a_tiles` (and room for a_tile_cap tiles of 256 rows in a_dst) A's scales are written per M tile of a
+// grouped GEMM, see the kernel.
 hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
-                                       uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream) {
-  const int64_t rows_max = a_rows > b_rows ? a_rows : b_rows;
+                                       uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream,
+                                       const int32_t *a_tiles, int64_t a_tile_cap) {
+  const int64_t a_rows_out = a_tiles ? a_tile_cap * 256 : a_rows;
+  const int64_t rows_max = a_rows_out > b_rows ? a_rows_out : b_rows;
   const int64_t rt = (rows_max + 31) / 32;
-  if ((ks & 7) != 0 || ks == 0 || (((uintptr_t)a_src | (uintptr_t)b_src) & 7) != 0 || rows_max >= ((int64_t)1 << 31) ||
-      ks >= ((int64_t)1 << 31) || rt > 65535 || a_rows <= 0 || b_rows <= 0)
+  if ((ks & 7) != 0 || ks == 0 || ((uintptr_t)a_src & 7) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 7) != 0) ||
+      rows_max >= ((int64_t)1 << 31) || ks >= ((int64_t)1 << 31) || rt > 65535 || a_rows <= 0 || b_rows < 0)
     return hipErrorInvalidValue;
-  dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)rt, 2);
-  scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks);
+  dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)rt, b_rows > 0 ? 2 : 1);  // b_rows == 0: A alone
+  scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks, a_tiles);
   return hipGetLastError();
 }
 

@@ -34,6 +34,8 @@ struct GemmParams {
   void *c;                 // [M, N] f32 / bf16
   float *partial;          // split-K slices [splits, M, N] f32, or null
   const int32_t *offsets;  // grouped: device [E+1]; else null
+  const int32_t *tile_table;  // grouped, persistent kernel: device table of M tiles (int32 x 4 each: entry 0 =
+                              // {count}, entry 1 + t = {first row, rows, expert}); A's scales are laid out per tile
   int m, n, k;
   int kp;              // K / 2
   int ks;              // K / 32
@@ -136,7 +138,9 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
 hipError_t launch_e8m0_shuffle(const uint8_t *scale, uint8_t *out, int64_t rows, int64_t ks,
                                hipStream_t stream);
 hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
-                                       uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream);
+                                       uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream,
+                                       const int32_t *a_tiles = nullptr, int64_t a_tile_cap = 0);
+hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int32_t *table, hipStream_t stream);
 hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t kp,
                                hipStream_t stream);
 

@@ -17,7 +17,8 @@
 //
 // Taken for N % 256 == 0, K % 256 == 0, K >= 768 (any M: the last tile row reads
 // and writes through descriptors that end with the tensors), MFMA-native
-// scales for both operands, no grouping, no split.  Everything else runs the
+// scales for both operands, no split; grouped (MoE) problems by way of a table
+// of M tiles.  Everything else runs the
 // one-tile-per-workgroup kernel.  The reference writes one tile per workgroup
 // (wave_lang/kernel/wave/templates/tagged_mxfp4_gemm.py:38-145); the result
 // contract is the same.
@@ -37,7 +38,10 @@ enum KtKind {
 // OUT_BF16 is a template parameter so that the C stores are straight-line code:
 // behind a run-time branch the compiler's wait insertion has to assume the
 // store-free path and waits for the stores long before it must.
-template <class Cfg, bool OUT_BF16>
+// GROUPED: the M tiles come from a table (first row, rows, expert) built on the
+// device from the group offsets; a tile's rows past its group are computed and
+// dropped like rows past M, and A's scales are laid out per tile (8 blocks each).
+template <class Cfg, bool OUT_BF16, bool GROUPED>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
@@ -48,7 +52,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
   const int kp = p.kp, nkt = p.k_tiles;
-  const int total = p.tiles_m * p.tiles_n;
+  const int tiles_m = GROUPED ? p.tile_table[0] : p.tiles_m;
+  const int total = tiles_m * p.tiles_n;
   const int padded = (total + kNumXcd - 1) / kNumXcd * kNumXcd;
   const int k_tiles_blocks = (p.ksp >> 3) * 256;  // bytes of one 32-row scale tile row
 
@@ -58,19 +63,33 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // a_lim / as_lim: bytes of A and of its scale blocks from the tile's first row to the end of the tensor
   // (M need not be a multiple of the tile: rows past it read zeros and are never stored)
   const uint8_t *a_base[2], *b_base[2], *as_base[2], *bs_base[2];
-  int m0[2], n0[2], a_lim[2], as_lim[2];
+  // c_rows: rows of the tile that are stored
+  int m0[2], n0[2], a_lim[2], as_lim[2], c_rows[2];
   const int m_blocks = (p.m + 31) >> 5;
   auto set_tile = [&](int which, int pid) -> bool {
     int tm, tn;
-    if (pid >= padded || !map_tile(pid, p.tiles_m, p.tiles_n, tm, tn)) return false;
-    m0[which] = tm * BM;
+    if (pid >= padded || !map_tile(pid, tiles_m, p.tiles_n, tm, tn)) return false;
     n0[which] = tn * BN;
+    if (GROUPED) {
+      const int32_t *ent = p.tile_table + 4 * (1 + tm);
+      const int first = __builtin_amdgcn_readfirstlane(ent[0]), rows = __builtin_amdgcn_readfirstlane(ent[1]);
+      const int expert = __builtin_amdgcn_readfirstlane(ent[2]);
+      m0[which] = first;
+      c_rows[which] = rows;
+      b_base[which] = p.b + (int64_t)expert * p.b_group_stride + (int64_t)n0[which] * kp;
+      bs_base[which] = p.b_scale + (int64_t)expert * p.b_scale_group_stride + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
+      as_base[which] = p.a_scale + (int64_t)tm * (BM / 32) * k_tiles_blocks;
+      as_lim[which] = (BM / 32) * k_tiles_blocks;
+    } else {
+      m0[which] = tm * BM;
+      c_rows[which] = p.m - m0[which];
+      b_base[which] = p.b + (int64_t)n0[which] * kp;
+      bs_base[which] = p.b_scale + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
+      as_base[which] = p.a_scale + (int64_t)(m0[which] >> 5) * k_tiles_blocks;
+      as_lim[which] = (int)min((int64_t)(m_blocks - (m0[which] >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
+    }
     a_base[which] = p.a + (int64_t)m0[which] * kp;
-    b_base[which] = p.b + (int64_t)n0[which] * kp;
-    as_base[which] = p.a_scale + (int64_t)(m0[which] >> 5) * k_tiles_blocks;
-    bs_base[which] = p.b_scale + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
     a_lim[which] = (int)min((int64_t)(p.m - m0[which]) * kp, (int64_t)0x7FFFFFFF);
-    as_lim[which] = (int)min((int64_t)(m_blocks - (m0[which] >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
     return true;
   };
   int pid = blockIdx.x;
@@ -249,7 +268,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // chunk c sits at position c ^ (row % chunks per row) (conflict-free 16-byte
   // reads, two-way on the 8-byte writes), written pass by pass and read back as
   // whole rows, 16 bytes per lane.
-  auto store_tile = [&](int slot, int tm0, int tn0) {
+  auto store_tile = [&](int slot, int tm0, int tn0, int rows) {
     constexpr int SW = SLOT / NWAVES;  // staging bytes of a wave
     constexpr int RP = SW / 32;        // row pitch
     constexpr int NCH = RP / 16;       // chunks per row
@@ -263,12 +282,13 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     asm volatile("" : "+v"(lane_v));
     const int fr = lane_v & 31, fg = lane_v >> 5;
     const int lr = lane_v / LPR, lc = lane_v % LPR;
-    // C goes out through a descriptor that ends with row M - 1: the rows of a last tile row past M are dropped
+    // C goes out through a descriptor that ends with the tile's last valid row: rows past M (or past the
+    // tile's group) are dropped
     const int ldc = p.n;
     constexpr int ELT = OUT_BF16 ? 2 : 4;
     const __amdgpu_buffer_rsrc_t c_rsrc =
         make_rsrc_n((uint8_t *)p.c + (int64_t)tm0 * ldc * ELT,
-                    (int)min((int64_t)(p.m - tm0) * ldc * ELT, (int64_t)0x7FFFFFFF));
+                    (int)min((int64_t)rows * ldc * ELT, (int64_t)0x7FFFFFFF));
     const int wr0 = wave_m * Cfg::WM;  // the wave's first row inside the tile
     if (out_bf16) {
       constexpr int CP = RP / 2, JP = CP / 32;  // columns, 32-column tiles per pass
@@ -356,7 +376,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const int npid = pid + (int)gridDim.x;
     const bool has_next = set_tile(1, npid);
     if (!has_next) {
-      m0[1] = m0[0], n0[1] = n0[0], a_lim[1] = a_lim[0], as_lim[1] = as_lim[0];
+      m0[1] = m0[0], n0[1] = n0[0], a_lim[1] = a_lim[0], as_lim[1] = as_lim[0], c_rows[1] = c_rows[0];
       a_base[1] = a_base[0], b_base[1] = b_base[0], as_base[1] = as_base[0], bs_base[1] = bs_base[0];
     }
     k_tile(0, sa, b_slot(sa), std::integral_constant<int, kFirst>{}, pending_tag);
@@ -374,7 +394,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     issue_g2l(1, 1, 1, sa, B_LD / 2, B_LD);
     sa = next_slot(sa);
     __builtin_amdgcn_sched_barrier(0);
-    store_tile(stage_slot, m0[0], n0[0]);
+    store_tile(stage_slot, m0[0], n0[0], c_rows[0]);
     if (!has_next) return false;
     // the staging slot is the next target of the A stream: all waves must be done reading it
     asm volatile("" ::: "memory");
@@ -383,7 +403,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     pid = npid;
-    m0[0] = m0[1], n0[0] = n0[1], a_lim[0] = a_lim[1], as_lim[0] = as_lim[1];
+    m0[0] = m0[1], n0[0] = n0[1], a_lim[0] = a_lim[1], as_lim[0] = as_lim[1], c_rows[0] = c_rows[1];
     a_base[0] = a_base[1], b_base[0] = b_base[1], as_base[0] = as_base[1], bs_base[0] = bs_base[1];
     return true;
   };
@@ -394,40 +414,47 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   __builtin_amdgcn_s_waitcnt(0);  // the trailing DMA must not outlive the workgroup's LDS
 }
 
-template <class Cfg, bool OUT_BF16>
+template <class Cfg, bool OUT_BF16, bool GROUPED>
 __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_kernel(const GemmParams p) {
-  persist_body<Cfg, OUT_BF16>(p);
+  persist_body<Cfg, OUT_BF16, GROUPED>(p);
 }
 
-template <class Cfg, bool OUT_BF16>
+template <class Cfg, bool OUT_BF16, bool GROUPED>
 static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_t stream) {
   static bool attr_done = false;  // benign race: the attribute is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16>,
+    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  persist_gemm_kernel<Cfg, OUT_BF16><<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  persist_gemm_kernel<Cfg, OUT_BF16, GROUPED><<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
   return hipGetLastError();
 }
 
 template <class Cfg>
 static hipError_t launch_persist_cfg(const GemmParams &p, int grid_x, hipStream_t stream) {
-  return p.out_bf16 ? launch_persist_out<Cfg, true>(p, grid_x, stream) : launch_persist_out<Cfg, false>(p, grid_x, stream);
+  if (p.tile_table != nullptr)
+    return p.out_bf16 ? launch_persist_out<Cfg, true, true>(p, grid_x, stream)
+                      : launch_persist_out<Cfg, false, true>(p, grid_x, stream);
+  return p.out_bf16 ? launch_persist_out<Cfg, true, false>(p, grid_x, stream)
+                    : launch_persist_out<Cfg, false, false>(p, grid_x, stream);
 }
 
 // Whether the persistent kernel serves this problem with `num_cus` CUs.
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
   if (variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 && variant != WAVE_MXFP4_VARIANT_T256x256_W4x2) return false;
-  if (p.num_groups != 0 || p.splits != 1 || p.partial != nullptr) return false;
+  // (a grouped problem comes with its M tile table and per-tile A scales, or not at all)
+  if ((p.num_groups != 0) != (p.tile_table != nullptr) || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
   if ((p.n & 255) != 0 || (p.k & (kTileK - 1)) != 0 || p.k_tiles < 3) return false;  // any M
   if (p.out_bf16 ? (p.n & 7) != 0 : (p.n & 3) != 0) return false;
   // 32-bit offsets inside one operand tile, and more tiles than workgroups
   if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31)) return false;
   const int grid = num_cus / kNumXcd * kNumXcd;
-  return grid >= kNumXcd && (int64_t)p.tiles_m * p.tiles_n > grid;
+  // (grouped: tiles_m is an upper bound, the rows give the estimate)
+  const int64_t tiles_m = p.num_groups != 0 ? p.m / 256 : p.tiles_m;
+  return grid >= kNumXcd && tiles_m * p.tiles_n > grid;
 }
 
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream) {

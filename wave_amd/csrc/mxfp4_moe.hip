@@ -104,7 +104,45 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
   }
 }
 
+// M tile table of a grouped GEMM: group e's rows offsets[e] .. offsets[e+1]-1 cut into tiles of bm rows.
+// Entry 0 = {number of tiles}; entry 1 + t = {first row, rows, group, 0}, in group order.
+__global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const int32_t *__restrict__ offsets,
+                                                                           int num_groups, int bm,
+                                                                           int32_t *__restrict__ table) {
+  __shared__ int wave_sums[kAlignWaves];
+  __shared__ int carry;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  if (t == 0) carry = 0;
+  __syncthreads();
+  for (int e0 = 0; e0 < num_groups; e0 += kAlignThreads) {
+    const int e = e0 + t;
+    int lo = 0, tiles = 0, hi = 0;
+    if (e < num_groups) {
+      lo = offsets[e], hi = offsets[e + 1];
+      tiles = hi > lo ? (hi - lo + bm - 1) / bm : 0;
+    }
+    const int base = carry;  // read before anyone moves it on
+    const int end = block_inclusive_scan(tiles, wave_sums, lane, wave);
+    for (int i = 0; i < tiles; ++i) {
+      int32_t *ent = table + 4 * (1 + base + end - tiles + i);
+      ent[0] = lo + i * bm;
+      ent[1] = min(bm, hi - lo - i * bm);
+      ent[2] = e;
+      ent[3] = 0;
+    }
+    __syncthreads();
+    if (t == kAlignThreads - 1) carry = base + end;
+    __syncthreads();
+  }
+  if (t == 0) table[0] = carry;
+}
+
 }  // namespace
+
+hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int32_t *table, hipStream_t stream) {
+  grouped_tile_table_kernel<<<1, kAlignThreads, 0, stream>>>(offsets, num_groups, bm, table);
+  return hipGetLastError();
+}
 
 hipError_t launch_moe_align(const void *topk_ids, int ids_int64, int64_t n, int num_experts, int block_size,
                             int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids, int64_t expert_ids_len,

@@ -137,10 +137,11 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100,
                     help="untimed launches first; the GPU needs ~30 ms of load to reach its steady clocks")
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8"],
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
                          "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out; "
-                         "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096")
+                         "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096; moe_glue: the steps around "
+                         "it at the same sizes (token alignment, gathered quantiser, gated activation + quantiser)")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode-shape leg")
@@ -191,6 +192,64 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": 134.3e6 + 35.65e6, "kernel": "quantize_kernel",
                          "launch_us": round(qper * 1e6, 2)}}))
+        return
+
+    if args.workload == "moe_glue":
+        # the steps around cfg4: 4096 tokens x top-2 of 8 experts, hidden 4096, intermediate 14336, bf16
+        tokens, topk, E, hidden, inter = 4096, 2, 8, 4096, 14336
+        g = torch.Generator(device=dev).manual_seed(3)
+        ids = torch.stack([torch.randperm(E, device=dev, generator=g)[:topk] for _ in range(tokens)]).to(torch.int32)
+        n_ent = tokens * topk
+        sorted_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
+        expert_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
+        total = torch.empty(1, dtype=torch.int32, device=dev)
+        offs = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        acts = [torch.randn(tokens, hidden, device=dev, generator=g).to(torch.bfloat16) for _ in range(3)]
+        gemm1 = [torch.randn(n_ent, 2 * inter, device=dev, generator=g).to(torch.bfloat16) for _ in range(2)]
+
+        def timed(fn):
+            for i in range(args.warmup):
+                fn(i)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(args.steps):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / args.steps
+
+        # straight through the C ABI with outputs allocated once: the kernels are shorter than a Python wrapper call
+        lib, st = _lib.load(), torch.cuda.current_stream().cuda_stream
+        q1 = torch.empty(n_ent, hidden // 2, dtype=torch.uint8, device=dev)
+        s1 = torch.empty(n_ent, hidden // 32, dtype=torch.uint8, device=dev)
+        q2 = torch.empty(n_ent, inter // 2, dtype=torch.uint8, device=dev)
+        s2 = torch.empty(n_ent, inter // 32, dtype=torch.uint8, device=dev)
+        t_align = timed(lambda i: lib.wave_mxfp4_moe_align_block_size(
+            ids.data_ptr(), 0, n_ent, E, 1, sorted_ids.data_ptr(), n_ent, expert_ids.data_ptr(), n_ent,
+            total.data_ptr(), offs.data_ptr(), st))
+        t_gather = timed(lambda i: lib.wave_mxfp4_quantize_rows(
+            acts[i % 3].data_ptr(), _lib.IN_BF16, tokens, sorted_ids.data_ptr(), topk, q1.data_ptr(), s1.data_ptr(),
+            n_ent, hidden, _lib.SCALE_ROW_MAJOR, st))
+        t_act = timed(lambda i: lib.wave_mxfp4_silu_and_mul_quantize(
+            gemm1[i % 2].data_ptr(), gemm1[i % 2].data_ptr() + 2 * inter, 2 * inter, 2 * inter, _lib.IN_BF16,
+            q2.data_ptr(), s2.data_ptr(), n_ent, inter, _lib.SCALE_ROW_MAJOR, st))
+        b_gather = n_ent * hidden * 2 + n_ent * hidden // 2 + n_ent * hidden // 32   # every source row is read top_k times
+        b_act = n_ent * inter * 4 + n_ent * inter // 2 + n_ent * inter // 32
+        gbps = b_act / t_act / 1e9
+        print(json.dumps({
+            "metric": "MoE glue: gated activation + quantiser GB/s % HBM", "value": round(gbps, 1), "unit": "GB/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t_act * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in, e2m1 + e8m0 out",
+            "data": "synthetic (normal)",
+            "config": {"workload": f"moe_glue: {tokens} tokens x top-{topk} of {E} experts, hidden {hidden}, "
+                                   f"intermediate {inter}"},
+            "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                         "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": None,
+                         "kernel": "quantize_kernel (gated)", "launch_us": round(t_act * 1e6, 2)},
+            "moe_align_block_size_us": round(t_align * 1e6, 2),
+            "gathered_quantiser": {"launch_us": round(t_gather * 1e6, 2), "gbps": round(b_gather / t_gather / 1e9, 1),
+                                   "bytes": b_gather}}))
         return
 
     if args.workload == "cfg4":

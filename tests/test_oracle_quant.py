@@ -105,3 +105,13 @@ def test_zero_group_and_shapes():
     assert not q[0].any()
     with pytest.raises(ValueError):
         qo.quantize_mxfp4(np.zeros((1, 48), dtype=np.float32))
+
+
+def test_committed_fixture_matches_the_oracle():
+    """tests/golden/q_quantize_37x320.npz is what the oracle says today."""
+    import os
+
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "q_quantize_37x320.npz"))
+    q, s = qo.quantize_mxfp4(g["x_f32_bits"].view(np.float32))
+    assert np.array_equal(q, g["q"]) and np.array_equal(s, g["scales"])
+    assert np.array_equal(orc.e8m0_shuffle_padded(s), g["scales_shuffled"])

@@ -38,6 +38,7 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
   int *cnt = lds;                                // [kAlignWaves][E]: entries of expert e in wave w's segment, later
                                                  // the next free position for them
   int *wave_sums = lds + kAlignWaves * num_experts;  // [kAlignWaves]
+  int *starts = wave_sums + kAlignWaves;             // [E + 1]: first position of every expert's run, then the total
   const int E = num_experts;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
@@ -47,9 +48,17 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
   // wave w owns the contiguous segment [seg0, seg1) of the flat table
   const int per_wave = ((n + kAlignWaves - 1) / kAlignWaves + 63) & ~63;
   const int seg0 = min(n, wave * per_wave), seg1 = min(n, seg0 + per_wave);
-  for (int i = seg0 + lane; i < seg1; i += 64) {
-    const int64_t e = (int64_t)topk_ids[i];
-    if (e >= 0 && e < E) atomicAdd(&cnt[wave * E + (int)e], 1);
+  // (8 steps of 64 ids are fetched together: a step at a time would pay a memory round trip each)
+  for (int base = seg0; base < seg1; base += 8 * 64) {
+    int64_t e[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int i = base + s * 64 + lane;
+      e[s] = i < seg1 ? (int64_t)topk_ids[i] : -1;
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+      if (e[s] >= 0 && e[s] < E) atomicAdd(&cnt[wave * E + (int)e[s]], 1);
   }
   __syncthreads();
 
@@ -68,38 +77,66 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
       cnt[w * E + t] = run;
       run += c;
     }
-    for (int i = start + count; i < min(end, sorted_len); ++i) sorted_ids[i] = n;  // the run's padding
-    for (int b = start / block_size; b < min(end / block_size, expert_ids_len); ++b) expert_ids[b] = t;
+    for (int i = start + count; i < min(end, sorted_len); ++i) sorted_ids[i] = n;  // the run's padding (< block_size)
+    starts[t] = start;
     if (offsets_out) offsets_out[t] = start;
   }
-  if (t == kAlignThreads - 1) wave_sums[0] = end;
+  if (t == kAlignThreads - 1) starts[E] = end;
   __syncthreads();
-  const int total = wave_sums[0];
+  const int total = starts[E];
   if (t == 0) {
     total_out[0] = total;
     if (offsets_out) offsets_out[E] = total;
   }
   for (int i = total + t; i < sorted_len; i += kAlignThreads) sorted_ids[i] = n;  // past the padded total
+  // the expert of every block, all threads together: the last expert whose run starts at or before the block
+  for (int b = t; b < min(total / block_size, expert_ids_len); b += kAlignThreads) {
+    const int pos = b * block_size;
+    int lo = 0, hi = E - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (starts[mid] <= pos) lo = mid; else hi = mid - 1;
+    }
+    // (an empty expert shares its start with the next one; "the last" steps past it)
+    expert_ids[b] = lo;
+  }
 
   // place: a wave walks its segment in order; the lanes of one expert take consecutive positions
+  // Up to 64 experts the wave keeps "next free position of expert e" in lane e's register (a readlane per
+  // look-up); beyond that in its row of cnt (an LDS round trip per look-up).
+  const bool in_regs = E <= 64;
   volatile int *next = cnt + wave * E;
-  for (int base = seg0; base < seg1; base += 64) {
-    const int i = base + lane;
-    const int64_t e64 = i < seg1 ? (int64_t)topk_ids[i] : -1;
-    const bool valid = e64 >= 0 && e64 < E;
-    const int e = valid ? (int)e64 : -1;
-    uint64_t todo = __ballot(valid);
-    while (todo) {
-      const int leader = __ffsll((unsigned long long)todo) - 1;
-      const int e0 = __shfl(e, leader, 64);
-      const uint64_t same = __ballot(e == e0);
-      const int first = next[e0];
-      if (e == e0) {
-        const int pos = first + __popcll(same & ((1ull << lane) - 1));
-        if (pos < sorted_len) sorted_ids[pos] = i;
+  int next_reg = in_regs && lane < E ? cnt[wave * E + lane] : 0;
+  for (int base8 = seg0; base8 < seg1; base8 += 8 * 64) {
+    int64_t e8[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int i = base8 + s * 64 + lane;
+      e8[s] = i < seg1 ? (int64_t)topk_ids[i] : -1;
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int i = base8 + s * 64 + lane;
+      const bool valid = e8[s] >= 0 && e8[s] < E;
+      const int e = valid ? (int)e8[s] : -1;
+      uint64_t todo = __ballot(valid);
+      while (todo) {
+        const int leader = __ffsll((unsigned long long)todo) - 1;
+        const int e0 = __builtin_amdgcn_readlane(e, leader);
+        const uint64_t same = __ballot(e == e0);
+        const int first = in_regs ? __builtin_amdgcn_readlane(next_reg, e0) : next[e0];
+        if (e == e0) {
+          const int pos = first + __popcll(same & ((1ull << lane) - 1));
+          if (pos < sorted_len) sorted_ids[pos] = i;
+        }
+        const int taken = __popcll(same);
+        if (in_regs) {
+          if (lane == e0) next_reg += taken;
+        } else if (lane == leader) {
+          next[e0] = first + taken;
+        }
+        todo &= ~same;
       }
-      if (lane == leader) next[e0] = first + __popcll(same);
-      todo &= ~same;
     }
   }
 }
@@ -147,12 +184,12 @@ hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int
 hipError_t launch_moe_align(const void *topk_ids, int ids_int64, int64_t n, int num_experts, int block_size,
                             int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids, int64_t expert_ids_len,
                             int32_t *total, int32_t *offsets, hipStream_t stream) {
-  const size_t lds = (size_t)(kAlignWaves * num_experts + kAlignWaves) * sizeof(int);
+  const size_t lds = (size_t)(kAlignWaves * num_experts + kAlignWaves + num_experts + 1) * sizeof(int);
   static bool attr_done[2] = {false, false};
   const void *fn = ids_int64 ? (const void *)moe_align_kernel<int64_t> : (const void *)moe_align_kernel<int32_t>;
   if (!attr_done[ids_int64 ? 1 : 0]) {
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)((kAlignWaves * kMoeMaxExperts + kAlignWaves) * sizeof(int)));
+                                       (int)((kAlignWaves * kMoeMaxExperts + kAlignWaves + kMoeMaxExperts + 1) * sizeof(int)));
     if (e != hipSuccess) return e;
     attr_done[ids_int64 ? 1 : 0] = true;
   }

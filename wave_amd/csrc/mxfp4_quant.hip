@@ -107,7 +107,10 @@ struct QuantParams {
 };
 
 // silu(g) * u in f32, rounded to the 16-bit storage type (the value the unfused
-// pipeline would have stored between its two kernels).
+// pipeline would have stored between its two kernels).  Hardware exp2 and
+// reciprocal (about 1 ulp of f32 each, far below the 8 or 11 bits that are kept):
+// the accurate expf and IEEE division cost more than the memory time of the
+// kernel.
 template <int DT>
 __device__ __forceinline__ uint32_t gated_pair(uint32_t g2, uint32_t u2) {
   float g[2], u[2], r[2];
@@ -119,7 +122,8 @@ __device__ __forceinline__ uint32_t gated_pair(uint32_t g2, uint32_t u2) {
     g[0] = (float)gh.x, g[1] = (float)gh.y, u[0] = (float)uh.x, u[1] = (float)uh.y;
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) r[i] = g[i] * u[i] / (1.0f + expf(-g[i]));
+  for (int i = 0; i < 2; ++i)
+    r[i] = g[i] * u[i] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g[i] * -1.44269504088896340736f));
   if constexpr (DT == WAVE_MXFP4_IN_BF16) {
     const bf16x2 o = {(__bf16)r[0], (__bf16)r[1]};
     return __builtin_bit_cast(uint32_t, o);
@@ -154,6 +158,13 @@ __global__ void __launch_bounds__(256) quantize_kernel(const QuantParams p) {
   const int row_tile = blockIdx.x / col_tiles, col_tile = blockIdx.x - row_tile * col_tiles;
   const int row0 = row_tile * kQuantRows, g0 = col_tile * kGroups;
 
+  // gathered rows: the ids of the wave's 8 rows, one per lane, fetched once (a load per unit would put two
+  // dependent memory round trips in front of every batch)
+  // ... and divided once: wave_src is the source row, or one past the last for "no such row"
+  uint32_t wave_src = (uint32_t)p.src_rows;
+  if (p.row_ids != nullptr && lane < 8 && row0 + wave * 8 + lane < rows)
+    wave_src = min((uint32_t)p.row_ids[row0 + wave * 8 + lane] / (uint32_t)p.row_div, (uint32_t)p.src_rows);
+
   for (int pb = 0; pb < kPasses; pb += kB) {
     Elems<DT> e[kB], eu[GATED ? kB : 1];
     int lrow[kB], lgrp[kB];
@@ -166,8 +177,7 @@ __global__ void __launch_bounds__(256) quantize_kernel(const QuantParams p) {
       bool ok = row < rows && g < ks;
       int64_t src = row;
       if (p.row_ids) {  // gathered rows
-        const uint32_t id = ok ? (uint32_t)p.row_ids[row] : 0u;
-        src = id / (uint32_t)p.row_div;
+        src = (uint32_t)__shfl((int)wave_src, u / kGroups, 64);
         ok = ok && src < p.src_rows;
       }
       const int64_t col = (int64_t)g * 32 + sub * 8;

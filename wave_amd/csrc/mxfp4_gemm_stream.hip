@@ -623,7 +623,7 @@ hipError_t launch_stream_gemm(const GemmParams &p, int num_cus, hipStream_t stre
   if (p.tiles_per_split > kStreamMaxKTiles) return hipErrorInvalidValue;
   const int nt_total = (p.n + 15) / 16;
   int grid_x = num_cus > 0 ? num_cus : 256;
-  if (p.splits > 1) grid_x = (grid_x + p.splits - 1) / p.splits;
+  if (p.splits > 1) grid_x = grid_x / p.splits;  // all splits resident at once: one workgroup fills a CU's LDS
   if (grid_x > nt_total) grid_x = nt_total;
   if (grid_x < 1) grid_x = 1;
   // 32-bit DMA offsets inside a workgroup's range of B rows

@@ -77,7 +77,7 @@ class WaveKernel:
         want = s.output_dtype.torch_dtype
         if out.dtype != want:
             raise ValueError(f"kernel was built for {want} output, got {out.dtype}")
-        split = s.num_splits
+        split = s.num_splits if s.num_splits > 1 else 0  # a plain template leaves the choice to the library
         if split > 1:
             # The library splits K in whole 256-element tiles; take the largest
             # split count not above the requested one that does.

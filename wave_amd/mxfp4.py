@@ -76,13 +76,15 @@ def _workspace(device, nbytes: int):
 
 
 def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,
-               b_scale_layout=_lib.SCALE_ROW_MAJOR, b_layout=_lib.B_ROW_MAJOR, split_k=1,
+               b_scale_layout=_lib.SCALE_ROW_MAJOR, b_layout=_lib.B_ROW_MAJOR, split_k=0,
                variant=_lib.VARIANT_AUTO, workspace=None) -> None:
     """``out[M, N] = dequant(x[M, K/2]) @ dequant(w_t[N, K/2]).T`` in place.
     Same arguments, in the same order, as the reference's compiled kernel
     (tests/kernel/wave_gemm_mxfp_test.py:194-201).  ``workspace`` is an optional
     uint8 GPU tensor of ``workspace_bytes(...)`` bytes; by default a buffer cached
-    per device and stream is used, ``False`` runs without scratch.
+    per device and stream is used, ``False`` runs without scratch.  ``split_k``: 0 lets the
+    library split K where that pays (decode shapes with K > 8192, few-tile shapes with long K; the
+    result is overwritten either way), 1 never splits, n > 1 splits n ways.
 
     Two more call shapes of the reference are taken as they are:
     * batched A with a shared B, ``x [B, M, K/2]``, ``x_scales [B, M, K/32]``,

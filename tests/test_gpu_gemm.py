@@ -387,3 +387,29 @@ def test_persistent_path_ragged_m(m, vname, out_dtype):
     torch.cuda.synchronize()
     diff = (out.float() - other.float()).abs().max().item()
     assert diff <= (2e-6 if out_dtype == torch.float32 else 2.0 ** -7) * out.float().abs().max().item()
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("vname", sorted(TILE_VARIANTS))
+@pytest.mark.parametrize("m,n,k", [(300, 520, 1248), (512, 512, 800), (257, 264, 288), (128, 128, 32 + 256 * 3)])
+def test_partial_last_k_tile_every_tile_kernel(m, n, k, vname, out_dtype):
+    """K % 256 != 0: with scratch the scales are re-laid out and the lanes past the end of K fetch zeros from beyond
+    the buffer descriptor (any tile kernel); without scratch the generic 128x128 kernel runs.  Both against the
+    oracle.  A NaN scale in the last group that exists must still poison its row."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=k + m, scale_lo=118, scale_hi=136)
+    xs[3, -1] = 255
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    v = ALL_VARIANTS[vname]
+    assert_close(run_gemm(x, xs, w_t, ws, out_dtype, variant=v), ref, out_dtype, f"{vname} with scratch")
+    assert_close(run_gemm(x, xs, w_t, ws, out_dtype, variant=v, workspace=False), ref, out_dtype, f"{vname} without")
+
+
+def test_partial_last_k_tile_full_size_sampled_rows():
+    """8192 x 8192 x 16000 (a shape of the reference's benchmark list,
+    wave_lang/kernel/wave/perf/mxfp4_shapes_macrotiles.csv): sampled rows against the oracle."""
+    m, n, k = 8192, 8192, 16000
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=16)
+    rows = np.r_[0:8, 4093:4099, 8184:8192]
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    got = run_gemm(x, xs, w_t, ws, torch.bfloat16)
+    assert_bf16_close(got[rows], ref)

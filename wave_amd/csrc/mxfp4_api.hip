@@ -91,13 +91,18 @@ bool is_tile_variant(int v) {
   return bm != 0;
 }
 
-// K % 256 != 0 is only built for the 128x128 tile kernel.
 int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
   int v = variant;
   if (v == WAVE_MXFP4_VARIANT_AUTO)
     v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
-  if (is_tile_variant(v) && k % kTileK != 0) v = WAVE_MXFP4_VARIANT_T128x128_W2x2;
   return v;
+}
+
+// A partial last K tile with scales that are not (or cannot be brought) in MFMA32 order is only built for the
+// 128x128 tile kernel.
+bool needs_generic_k(const GemmParams &p) {
+  return (p.k % kTileK) != 0 && (p.b_preshuffled || p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ||
+                                 p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32);
 }
 
 // Split the library takes by itself for a tile kernel: only when the tile
@@ -171,8 +176,7 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
   int splits = split_k;
   if (splits == 0) splits = auto_split(m, n, k, v);
   if (splits > 1) bytes += round_up_256((size_t)splits * (size_t)m * (size_t)n * sizeof(float));
-  if (is_tile_variant(v) && k % kTileK == 0)
-    bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
+  if (is_tile_variant(v)) bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
   return bytes;
 }
 
@@ -233,8 +237,9 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   // cache line per wave instruction; row-major scales cost 32 lines per
   // instruction.  With scratch available, re-lay both operands out first
   // (a few MB, microseconds) and run the native-scale kernel.
-  // (Not worth a second launch for short K: up to 8 K tiles per workgroup the direct reads cost less.)
-  if (is_tile_variant(v) && k % kTileK == 0 && workspace && p.tiles_per_split > 8) {
+  // (Not worth a second launch for a small problem with short K: there the direct reads cost less.)
+  const bool small_short = p.tiles_per_split <= 8 && (int64_t)m * n <= (int64_t)2048 * 2048 && k % kTileK == 0;
+  if (is_tile_variant(v) && workspace && !small_short && !(p.b_preshuffled && k % kTileK != 0)) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
     const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? a_bytes : 0;
     const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? b_bytes : 0;
@@ -275,11 +280,12 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     if (e == hipErrorInvalidValue) e = launch_skinny_gemm(p, stream);
   } else {
     int bm, bn;
-    tile_variant_shape(v, &bm, &bn);
+    const int tv = needs_generic_k(p) ? WAVE_MXFP4_VARIANT_T128x128_W2x2 : v;
+    tile_variant_shape(tv, &bm, &bn);
     p.tiles_m = (int)((m + bm - 1) / bm);
     p.tiles_n = (int)((n + bn - 1) / bn);
-    e = persist_gemm_applies(p, v, device_cus()) ? launch_persist_gemm(p, v, device_cus(), stream)
-                                                 : launch_tile_gemm(p, v, stream);
+    e = persist_gemm_applies(p, tv, device_cus()) ? launch_persist_gemm(p, tv, device_cus(), stream)
+                                                  : launch_tile_gemm(p, tv, stream);
   }
   if (e != hipSuccess) return record_hip(e);
   if (splits > 1) e = launch_splitk_reduce(p.partial, c, m * n, splits, p.out_bf16, stream);
@@ -392,10 +398,13 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
                                                    : pick_variant(total_rows, n, k, variant);
   if (v == WAVE_MXFP4_VARIANT_NAIVE) return record_hip(launch_naive_gemm(p, stream));
   int bm, bn;
-  tile_variant_shape(v, &bm, &bn);
-  // sum over groups of ceil(rows_e / bm) <= total_rows / bm + num_groups
-  p.tiles_m = (int)(total_rows / bm + num_groups);
-  p.tiles_n = (int)((n + bn - 1) / bn);
+  auto size_grid = [&](int tile_variant) {
+    tile_variant_shape(tile_variant, &bm, &bn);
+    // sum over groups of ceil(rows_e / bm) <= total_rows / bm + num_groups
+    p.tiles_m = (int)(total_rows / bm + num_groups);
+    p.tiles_n = (int)((n + bn - 1) / bn);
+  };
+  size_grid(v);
   // With scratch: both scale tensors into the MFMA32 order first.  The experts' B scales are one
   // [E * N, K/32] matrix whose 32-row blocks do not straddle experts when N % 32 == 0.
   if (workspace && !aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
@@ -446,7 +455,9 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
     p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
     p.b_scale_group_stride = n * (int64_t)p.ksp;  // N % 32 == 0: no padding rows between experts
   }
-  return record_hip(launch_tile_gemm(p, v, stream));
+  const int tv = needs_generic_k(p) ? WAVE_MXFP4_VARIANT_T128x128_W2x2 : v;
+  size_grid(tv);
+  return record_hip(launch_tile_gemm(p, tv, stream));
 }
 
 int wave_mxfp4_to_f32(const void *q, float *out, int64_t rows, int64_t kp, void *hip_stream) {

@@ -191,6 +191,25 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   }
   const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
   const int tail_chunks = GENERIC_K ? ((p.k & (kTileK - 1)) >> 5) : 0;  // valid chunks of a partial last tile
+  // kNative with a partial last K tile (MXFP4 only): the lanes whose chunk lies past the end of K fetch from
+  // beyond the descriptor instead, which lands zeros in LDS: the same instructions as for a whole tile, so the
+  // counted waits hold.  (The padded scale groups of the MFMA32 buffer are finite and meet those zeros.)
+  // The per-lane offsets are redirected in place just before the last K tile is issued, nothing is selected
+  // per instruction: part 0 = A and the first half of B, part 1 = the second half of B (issued a K tile later).
+  const int native_tail = NATIVE && !FP8 ? ((p.k & (kTileK - 1)) >> 5) : 0;
+  const bool tail_lane = native_tail != 0 && ld_chunk >= native_tail;
+  auto arm_tail = [&](int part) {
+    if (!NATIVE || FP8) return;
+    if (part == 0) {
+#pragma unroll
+      for (int d = 0; d < A_LD; ++d) a_goff[d] = tail_lane ? (int)0x80000000 : a_goff[d];
+#pragma unroll
+      for (int d = 0; d < B_LD / 2; ++d) b_goff[d] = tail_lane ? (int)0x80000000 : b_goff[d];
+    } else {
+#pragma unroll
+      for (int d = B_LD / 2; d < B_LD; ++d) b_goff[d] = tail_lane ? (int)0x80000000 : b_goff[d];
+    }
+  };
 
   // DMA instructions [d0, d1) of operand tile `op` (0 = A, 1 = B) of K tile
   // `kt` into ring slot `slot`.
@@ -430,10 +449,14 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   constexpr int kWaitSteady = GENERIC_K ? 0 : A_LD;
   constexpr int kWaitPrologue = GENERIC_K ? 0 : A_LD + B_LD / 2;
 
+  // (the last K tile of the problem is the last of the last split only)
+  const bool has_tail = native_tail != 0 && kt_end == p.k_tiles;
+  if (has_tail && nkt == 1) arm_tail(0), arm_tail(1);
   issue_g2l(0, kt_begin, 0, 0, A_LD);
   issue_g2l(1, kt_begin, 1, 0, B_LD);
   load_scales(kt_begin);
   if (nkt > 1) {
+    if (has_tail && nkt == 2) arm_tail(0);
     issue_g2l(0, kt_begin + 1, 2, 0, A_LD);
     issue_g2l(1, kt_begin + 1, 3, 0, B_LD / 2);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kWaitPrologue));
@@ -512,11 +535,19 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
     __builtin_amdgcn_sched_barrier(0);
   };
   int j = 0, sa = 0;
-  for (; j < nkt - 2; ++j) {
+  for (; j < nkt - 3; ++j) {
     const int sb = sa + 1 >= RING ? 0 : sa + 1;
     k_tile(j, sa, sb, std::true_type{}, std::true_type{});
     sa = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
   }
+  if (j < nkt - 2) {  // K tile nkt - 3 issues A and the first half of B of the last K tile
+    if (has_tail) arm_tail(0);
+    const int sb = sa + 1 >= RING ? 0 : sa + 1;
+    k_tile(j, sa, sb, std::true_type{}, std::true_type{});
+    sa = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
+    ++j;
+  }
+  if (has_tail && nkt >= 2) arm_tail(1);  // K tile nkt - 2 issues the second half of B of the last K tile
   if (j < nkt - 1) {
     const int sb = sa + 1 >= RING ? 0 : sa + 1;
     k_tile(j, sa, sb, std::true_type{}, std::false_type{});
@@ -682,10 +713,14 @@ static hipError_t launch_by_scales(const GemmParams &p, hipStream_t stream) {
 }
 
 // K % 256 != 0 (partial last K tile, scale rows that are not 8-byte multiples)
-// is served by one extra instantiation of the 128x128 kernel; the caller maps
-// every tile variant onto it for such K.
+// with scales that are not in MFMA32 order is served by one extra instantiation
+// of the 128x128 kernel; the caller sizes its grid for 128x128 tiles then.
 hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream) {
-  if ((p.k & (kTileK - 1)) != 0) return launch_cfg<Cfg128x128w4, kGenericK>(p, stream);
+  const bool native =
+      p.a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+  // (with both scale tensors in MFMA32 order every tile kernel takes a partial last K tile;
+  //  preshuffled B keeps whole 64-element K steps only, which the generic kernel handles)
+  if ((p.k & (kTileK - 1)) != 0 && (!native || p.b_preshuffled)) return launch_cfg<Cfg128x128w4, kGenericK>(p, stream);
   switch (variant) {
     case WAVE_MXFP4_VARIANT_T256x256_W2x2: return launch_by_scales<Cfg256x256w4>(p, stream);
     case WAVE_MXFP4_VARIANT_T256x256_W4x2: return launch_by_scales<Cfg256x256w8>(p, stream);

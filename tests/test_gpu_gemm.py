@@ -413,3 +413,20 @@ def test_partial_last_k_tile_full_size_sampled_rows():
     ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
     got = run_gemm(x, xs, w_t, ws, torch.bfloat16)
     assert_bf16_close(got[rows], ref)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("vname", ["t256x256_w2x2", "t256x256_w4x2"])
+@pytest.mark.parametrize("k", [1024 + 128, 1024 + 32, 2048 - 32])
+def test_persistent_path_partial_last_k_tile(k, vname, out_dtype):
+    """More tiles than CUs and K % 256 != 0 (128 is the remainder of K = 16000, the K of the reference's
+    benchmark shapes); ragged M on top.  A NaN scale in the last existing group must poison its row and column."""
+    m, n = 4352 - 100, 4352
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=k, scale_lo=120, scale_hi=134)
+    xs[7, -1] = 255
+    ws[9, -1] = 255
+    rows = np.r_[0:40, m - 200:m]
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    got = run_gemm(x, xs, w_t, ws, out_dtype, variant=ALL_VARIANTS[vname])
+    assert_close(got[rows], ref, out_dtype, f"{vname} K={k}")
+    assert np.isnan(got[7]).all() and np.isnan(got[:, 9]).all() and not np.isnan(np.delete(np.delete(got, 7, 0), 9, 1)).any()

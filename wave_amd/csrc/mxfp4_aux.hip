@@ -103,7 +103,7 @@ __global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_la
   }
 }
 
-// Row-major -> MFMA32 for ks % 8 == 0, the conversion in front of every tile
+// Row-major -> MFMA32 for ks % 4 == 0, the conversion in front of every tile
 // GEMM with row-major scales.  A workgroup takes 32 rows x 32 K tiles: 8-byte
 // reads that walk each row contiguously, the even and odd groups of a K tile
 // split with v_perm into the two dwords of its block (lanes r%32 and 32 + r%32),
@@ -124,7 +124,7 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
   const uint8_t *src = blockIdx.z ? src1 : src0;
   uint8_t *dst = blockIdx.z ? dst1 : dst0;
   int rows = blockIdx.z ? rows1 : rows0;
-  const int k_tiles = ks >> 3;
+  const int k_tiles = (ks + 7) >> 3;  // ks % 4 == 0: the last K tile may hold 4 groups only (the rest is written as 0)
   const int rt = blockIdx.y, kt0 = blockIdx.x * 32;
   int row_base = rt * 32;
   if (tiles0 != nullptr && blockIdx.z == 0) {
@@ -142,7 +142,11 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
     const int unit = t + 256 * u, r = unit >> 5, ktl = unit & 31;
     const int row = row_base + r, kt = kt0 + ktl;
     uint2 v = make_uint2(0u, 0u);
-    if (row < rows && kt < k_tiles) v = *(const uint2 *)(src + (int64_t)row * ks + (int64_t)kt * 8);
+    if (row < rows && kt < k_tiles) {
+      const uint8_t *at = src + (int64_t)row * ks + (int64_t)kt * 8;
+      v.x = *(const uint32_t *)at;
+      if (kt * 8 + 4 < ks) v.y = *(const uint32_t *)(at + 4);
+    }
     stage[ktl * 65 + r] = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u);       // groups 0, 2, 4, 6
     stage[ktl * 65 + 32 + r] = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);  // groups 1, 3, 5, 7
   }
@@ -270,9 +274,9 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
   const int64_t rows_p = (rows + 31) / 32 * 32, ksp = (ks + 7) / 8 * 8;
   const int64_t n = rows_p * (ksp / 4);
   if (n == 0) return hipSuccess;
-  if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 7) == 0 &&
-      ((uintptr_t)src & 7) == 0 && rows < ((int64_t)1 << 31) && ks < ((int64_t)1 << 31) && rows_p / 32 <= 65535) {
-    dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)(rows_p / 32), 1);
+  if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 3) == 0 &&
+      ((uintptr_t)src & 3) == 0 && rows < ((int64_t)1 << 31) && ks < ((int64_t)1 << 31) && rows_p / 32 <= 65535) {
+    dim3 grid((unsigned)((ksp / 8 + 31) / 32), (unsigned)(rows_p / 32), 1);
     scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks, nullptr);
     return hipGetLastError();
   }
@@ -291,10 +295,10 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
   const int64_t a_rows_out = a_tiles ? a_tile_cap * 256 : a_rows;
   const int64_t rows_max = a_rows_out > b_rows ? a_rows_out : b_rows;
   const int64_t rt = (rows_max + 31) / 32;
-  if ((ks & 7) != 0 || ks == 0 || ((uintptr_t)a_src & 7) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 7) != 0) ||
+  if ((ks & 3) != 0 || ks == 0 || ((uintptr_t)a_src & 3) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 3) != 0) ||
       rows_max >= ((int64_t)1 << 31) || ks >= ((int64_t)1 << 31) || rt > 65535 || a_rows <= 0 || b_rows < 0)
     return hipErrorInvalidValue;
-  dim3 grid((unsigned)((ks / 8 + 31) / 32), (unsigned)rt, b_rows > 0 ? 2 : 1);  // b_rows == 0: A alone
+  dim3 grid((unsigned)(((ks + 7) / 8 + 31) / 32), (unsigned)rt, b_rows > 0 ? 2 : 1);  // b_rows == 0: A alone
   scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks, a_tiles);
   return hipGetLastError();
 }

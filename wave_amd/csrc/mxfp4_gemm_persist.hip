@@ -15,7 +15,8 @@
 // behind the loads it needs; from the second K tile on the stores must have
 // drained, which by then they have had a whole K tile of time to do.
 //
-// Taken for N % 256 == 0, K % 256 == 0, K >= 768 (any M: the last tile row reads
+// Taken for N % 256 == 0, K >= 768 (K % 256 != 0 with a partial last K tile from
+// K = 1024 on; any M: the last tile row reads
 // and writes through descriptors that end with the tensors), MFMA-native
 // scales for both operands, no split; grouped (MoE) problems by way of a table
 // of M tiles.  Everything else runs the
@@ -29,6 +30,7 @@
 namespace wave_mxfp4 {
 
 enum KtKind {
+  kSteadyTail = 4,  // kSteady whose K tile j+2 is a partial last K tile (TAIL kernels: j = nkt - 3)
   kSteady = 0,  // K tiles j+1, j+2 belong to this output tile
   kFirst = 1,   // first K tile of an output tile (B(1) was fetched whole ahead of it)
   kBound1 = 2,  // K tile j+2 is K tile 0 of the next output tile
@@ -41,7 +43,12 @@ enum KtKind {
 // GROUPED: the M tiles come from a table (first row, rows, expert) built on the
 // device from the group offsets; a tile's rows past its group are computed and
 // dropped like rows past M, and A's scales are laid out per tile (8 blocks each).
-template <class Cfg, bool OUT_BF16, bool GROUPED>
+// TAIL: K % 256 != 0.  The lanes whose 16-byte chunk lies past the end of K fetch
+// the last K tile from beyond the buffer descriptor (zeros land in LDS): their
+// offset gets its top bit flipped just before that tile's DMA is issued and
+// flipped back after it, at fixed places of two peeled K tiles, so the steady
+// loop and the instruction counts the waits rely on are untouched.
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
@@ -100,11 +107,13 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   const int ld_chunk = (lane & 7) ^ ((ld_row0 >> 1) & 7);
   // DMA instruction d of a wave fills rows 8*NWAVES*d further down: one per-lane
   // offset per operand, the rest is scalar (registers are what this kernel is short of).
-  const int a_goff = ld_row0 * kp + ld_chunk * 16;
-  const int b_goff = p.b_preshuffled ? (ld_row0 >> 4) * 16 * kp + (ld_row0 & 15) * 16 + (ld_chunk >> 1) * 512 +
+  int a_goff = ld_row0 * kp + ld_chunk * 16;
+  int b_goff = p.b_preshuffled ? (ld_row0 >> 4) * 16 * kp + (ld_row0 & 15) * 16 + (ld_chunk >> 1) * 512 +
                                            (ld_chunk & 1) * 256
                                      : ld_row0 * kp + ld_chunk * 16;
   const int ld_step = NWAVES * 8 * kp;  // bytes between consecutive d, either layout (8*NWAVES is a multiple of 16)
+  const bool tail_lane = TAIL && ld_chunk >= ((p.k & (kTileK - 1)) >> 5);
+  auto flip_tail = [&](int &goff) { goff ^= tail_lane ? (int)0x80000000 : 0; };
   const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
 
   // DMA instructions [d0, d1) of operand `op` (0 = A, 1 = B), K tile `kt` of
@@ -216,6 +225,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   auto k_tile = [&](int j, int sa, int sb, auto kind_tag, auto pending_tag) {
     constexpr int KIND = decltype(kind_tag)::value;
     constexpr bool PENDING = decltype(pending_tag)::value;
+    static_assert(TAIL || KIND != kSteadyTail, "kSteadyTail belongs to the TAIL kernels");
     constexpr int W1 = KIND == kBound2 ? 1 : 0;                      // output tile of K tile j+1
     constexpr int W2 = (KIND == kBound1 || KIND == kBound2) ? 1 : 0;  // ... of K tile j+2
     const int kt1 = KIND == kBound2 ? 0 : j + 1;
@@ -228,6 +238,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     read_frags(sa, sb, 1, fa1, fb1);
     mfma_block(fa0, fb0, T0{}, Zero{});
     if (KIND != kFirst) issue_g2l(W1, 1, kt1, sb1, B_LD / 2, B_LD);
+    if (TAIL && KIND == kBound1) flip_tail(b_goff);  // the second half of B of the partial K tile is out: back
+    if (TAIL && KIND == kSteadyTail) flip_tail(a_goff);
     order_phase();
     __builtin_amdgcn_sched_barrier(0);
     read_frags(sa, sb, 2, fa0, fb0);
@@ -238,6 +250,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     read_frags(sa, sb, 3, fa1, fb1);
     mfma_block(fa0, fb0, T2{}, Keep{});
     issue_g2l(W2, 0, kt2, sa2, A_LD / 2, A_LD);
+    if (TAIL && KIND == kSteadyTail) flip_tail(a_goff), flip_tail(b_goff);  // A back; B until kBound1's first phase
     order_phase();
     __builtin_amdgcn_sched_barrier(0);
     // Everything this wave issued up to B(j+1) has landed.  Younger than that:
@@ -381,8 +394,12 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     }
     k_tile(0, sa, b_slot(sa), std::integral_constant<int, kFirst>{}, pending_tag);
     sa = next_slot(sa);
-    for (int j = 1; j < nkt - 2; ++j) {
+    for (int j = 1; j < nkt - (TAIL ? 3 : 2); ++j) {
       k_tile(j, sa, b_slot(sa), std::integral_constant<int, kSteady>{}, pending_tag);
+      sa = next_slot(sa);
+    }
+    if constexpr (TAIL) {  // nkt >= 4
+      k_tile(nkt - 3, sa, b_slot(sa), std::integral_constant<int, kSteadyTail>{}, pending_tag);
       sa = next_slot(sa);
     }
     k_tile(nkt - 2, sa, b_slot(sa), std::integral_constant<int, kBound1>{}, pending_tag);
@@ -414,31 +431,34 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   __builtin_amdgcn_s_waitcnt(0);  // the trailing DMA must not outlive the workgroup's LDS
 }
 
-template <class Cfg, bool OUT_BF16, bool GROUPED>
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL>
 __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_kernel(const GemmParams p) {
-  persist_body<Cfg, OUT_BF16, GROUPED>(p);
+  persist_body<Cfg, OUT_BF16, GROUPED, TAIL>(p);
 }
 
-template <class Cfg, bool OUT_BF16, bool GROUPED>
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL>
 static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_t stream) {
   static bool attr_done = false;  // benign race: the attribute is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED>,
+    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  persist_gemm_kernel<Cfg, OUT_BF16, GROUPED><<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL><<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
   return hipGetLastError();
 }
 
 template <class Cfg>
 static hipError_t launch_persist_cfg(const GemmParams &p, int grid_x, hipStream_t stream) {
   if (p.tile_table != nullptr)
-    return p.out_bf16 ? launch_persist_out<Cfg, true, true>(p, grid_x, stream)
-                      : launch_persist_out<Cfg, false, true>(p, grid_x, stream);
-  return p.out_bf16 ? launch_persist_out<Cfg, true, false>(p, grid_x, stream)
-                    : launch_persist_out<Cfg, false, false>(p, grid_x, stream);
+    return p.out_bf16 ? launch_persist_out<Cfg, true, true, false>(p, grid_x, stream)
+                      : launch_persist_out<Cfg, false, true, false>(p, grid_x, stream);
+  if ((p.k & (kTileK - 1)) != 0)
+    return p.out_bf16 ? launch_persist_out<Cfg, true, false, true>(p, grid_x, stream)
+                      : launch_persist_out<Cfg, false, false, true>(p, grid_x, stream);
+  return p.out_bf16 ? launch_persist_out<Cfg, true, false, false>(p, grid_x, stream)
+                    : launch_persist_out<Cfg, false, false, false>(p, grid_x, stream);
 }
 
 // Whether the persistent kernel serves this problem with `num_cus` CUs.
@@ -447,7 +467,9 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
   // (a grouped problem comes with its M tile table and per-tile A scales, or not at all)
   if ((p.num_groups != 0) != (p.tile_table != nullptr) || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
-  if ((p.n & 255) != 0 || (p.k & (kTileK - 1)) != 0 || p.k_tiles < 3) return false;  // any M
+  if ((p.n & 255) != 0 || p.k_tiles < 3) return false;  // any M
+  // a partial last K tile: dense problems with row-major B and at least four K tiles
+  if ((p.k & (kTileK - 1)) != 0 && (p.num_groups != 0 || p.b_preshuffled || p.k_tiles < 4)) return false;
   if (p.out_bf16 ? (p.n & 7) != 0 : (p.n & 3) != 0) return false;
   // 32-bit offsets inside one operand tile, and more tiles than workgroups
   if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31)) return false;

@@ -33,6 +33,28 @@ WORKLOADS = {
     "cfg5": (4093, 6144, 7168, "f32", 4, (100, 154)),
 }
 
+# (M, N) pairs of the reference's benchmark shape list, all at K = 16000
+# (wave_lang/kernel/wave/perf/mxfp4_shapes_macrotiles.csv, columns M,N,K; 103 distinct pairs)
+REF_SHAPES_K = 16000
+REF_SHAPES_MN = {
+    512: [512, 1024, 2048, 8192],
+    1024: [512, 1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 12288, 16384, 20480, 24576, 28672, 32768],
+    1536: [8192],
+    2048: [512, 1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 12288, 16384, 20480, 24576, 28672, 32768],
+    2560: [8192],
+    3072: [1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 12288, 16384, 20480],
+    3584: [8192],
+    4096: [1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 12288, 16384],
+    4608: [8192],
+    5120: [1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192, 12288],
+    5632: [8192],
+    6144: [1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192],
+    6656: [8192],
+    7168: [1024, 2048, 3072, 4096, 5120, 6144, 7168, 8192],
+    7680: [8192],
+    8192: [512, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 4608, 5120, 5632, 6144, 6656, 7168, 7680, 8192],
+}
+
 
 def gemm_flops(m, n, k):
     return 2 * m * n * k
@@ -137,7 +159,7 @@ def main():
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=100,
                     help="untimed launches first; the GPU needs ~30 ms of load to reach its steady clocks")
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue"],
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue", "ref_shapes"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
                          "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out; "
                          "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096; moe_glue: the steps around "
@@ -192,6 +214,35 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": 134.3e6 + 35.65e6, "kernel": "quantize_kernel",
                          "launch_us": round(qper * 1e6, 2)}}))
+        return
+
+    if args.workload == "ref_shapes":
+        # every (M, N) of the reference's benchmark list at its K = 16000 (a partial last K tile), bf16 out
+        import math
+
+        k = REF_SHAPES_K
+        rows = []
+        for m in sorted(REF_SHAPES_MN):
+            for n in REF_SHAPES_MN[m]:
+                sets = make_gpu_inputs(torch, m, n, k, 1, (124, 130), dev, copies=1)
+                out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+                flops = gemm_flops(m, n, k)
+                steps = max(10, min(args.steps, int(0.05 / (flops / 4.0e15))))
+                _, per = time_gemm(torch, wave_amd, sets, out, steps, max(5, steps // 3), variant=args.variant)
+                rows.append((m, n, per, flops / per / 1e12))
+                del sets, out
+        geo = math.exp(sum(math.log(r[3]) for r in rows) / len(rows))
+        big = [r for r in rows if r[0] * r[1] >= 4096 * 4096]
+        geo_big = math.exp(sum(math.log(r[3]) for r in big) / len(big))
+        print(json.dumps({
+            "metric": "MXFP4 GEMM TFLOPS over the reference's benchmark shapes (K = 16000), geometric mean",
+            "value": round(geo, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(sum(r[2] for r in rows) * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out",
+            "data": "synthetic (seeded uniform nibbles and scales)",
+            "config": {"workload": f"ref_shapes: {len(rows)} (M, N) pairs, K = {k}, bf16 out, seed 1"},
+            "geomean_tflops_mn_ge_4096x4096": round(geo_big, 1),
+            "shapes": [{"m": r[0], "n": r[1], "us": round(r[2] * 1e6, 1), "tflops": round(r[3], 1)} for r in rows]}))
         return
 
     if args.workload == "moe_glue":

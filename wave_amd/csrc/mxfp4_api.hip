@@ -118,9 +118,9 @@ int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
   }
   int bm, bn;
   tile_variant_shape(variant, &bm, &bn);
-  if (bm == 0 || k % kTileK != 0) return 1;
+  if (bm == 0) return 1;
   const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
-  const int64_t k_tiles = k / kTileK;
+  const int64_t k_tiles = (k + kTileK - 1) / kTileK;  // a partial last K tile belongs to the last split
   if (tiles >= 128 || k_tiles < 8) return 1;
   int s = (int)(256 / tiles);
   if (s > 8) s = 8;

@@ -199,8 +199,10 @@ def test_config5_edge_shape_shuffled_scales_f32_seed4():
     assert np.array_equal(shuffled, plain)                          # same arithmetic, same bits
     direct = run(xs_sh, ws_sh, a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
                  workspace=False)
-    assert np.array_equal(direct, plain)                            # read in place, no pre-pass
-    assert np.array_equal(run(gxs, gws, workspace=False), plain)
+    # read in place, no pre-pass.  (With scratch the library may cut the tiles of a sparsely filled last round
+    # along K, which changes the order of the sums: compared within f32 accumulation noise, not bit for bit.)
+    assert_f32_close(direct, plain, "no scratch vs scratch")
+    assert np.array_equal(run(gxs, gws, workspace=False), direct)
     # and with preshuffled B on top
     gwp = wave_amd.b_preshuffle(gw)
     out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)

@@ -430,3 +430,26 @@ def test_persistent_path_partial_last_k_tile(k, vname, out_dtype):
     got = run_gemm(x, xs, w_t, ws, out_dtype, variant=ALL_VARIANTS[vname])
     assert_close(got[rows], ref, out_dtype, f"{vname} K={k}")
     assert np.isnan(got[7]).all() and np.isnan(got[:, 9]).all() and not np.isnan(np.delete(np.delete(got, 7, 0), 9, 1)).any()
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(4608, 4096, 4096 + 128), (4608 - 70, 4096, 2304), (2560, 8192, 1024 + 64 * 32)])
+def test_persistent_path_last_round_cut_along_k(m, n, k, out_dtype):
+    """288 or 320 tiles on 256 CUs: the tiles of the last round are cut along K over the idle workgroups and
+    summed afterwards (with and without a partial last K tile, ragged M).  Two rows of every tile row against
+    the oracle, and every element against the one-tile-per-workgroup kernel."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + k, scale_lo=120, scale_hi=134)
+    rows = np.array(sorted({min(m - 1, b * 256 + o) for b in range((m + 255) // 256) for o in (3, 250)}))
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    buf = torch.full(((m + 64) * n,), 7.0, dtype=out_dtype, device=DEV)
+    out = buf[: m * n].view(m, n)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out, variant=_lib.VARIANT_T256x256_W4x2)
+    torch.cuda.synchronize()
+    assert bool((buf[m * n:] == 7.0).all())
+    assert_close(out.float().cpu().numpy()[rows], ref, out_dtype, f"{m}x{n}x{k}")
+    other = torch.empty_like(out)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, other, variant=_lib.VARIANT_T128x128_W2x2)
+    torch.cuda.synchronize()
+    diff = (out.float() - other.float()).abs().max().item()
+    assert diff <= (4e-6 if out_dtype == torch.float32 else 2.0 ** -7) * out.float().abs().max().item()

@@ -177,6 +177,17 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
   if (splits == 0) splits = auto_split(m, n, k, v);
   if (splits > 1) bytes += round_up_256((size_t)splits * (size_t)m * (size_t)n * sizeof(float));
   if (is_tile_variant(v)) bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
+  if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && n % 256 == 0 && splits <= 1) {
+    // the parts of the tiles of a sparsely filled last round (persistent kernel)
+    const int grid = device_cus() / 8 * 8;
+    const int64_t tiles = ((m + 255) / 256) * (n / 256);
+    const int64_t rest = grid > 0 && tiles % grid != 0 ? (tiles + 7) / 8 * 8 - tiles / grid * grid : 0;
+    if (tiles > grid && rest != 0 && rest * 2 <= grid) {
+      int64_t parts = grid / rest;
+      if (parts > 8) parts = 8;
+      bytes += (size_t)(rest * parts) * 256 * 256 * sizeof(float);
+    }
+  }
   return bytes;
 }
 
@@ -222,6 +233,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   }
 
   hipError_t e;
+  size_t ws_scales_end = 0;  // first free byte of the workspace behind partials and re-laid scales
   if (p.a_scale_layout == WAVE_MXFP4_SCALE_PER_ROW) {
     // one scale per row: spread it over the row's groups, then it is a row-major scale matrix
     const size_t need = round_up_256((size_t)m * (size_t)p.ks);
@@ -245,6 +257,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? b_bytes : 0;
     if (ws_used + a_need + b_need <= workspace_bytes) {
       uint8_t *ws = (uint8_t *)workspace + ws_used;
+      ws_scales_end = ws_used + a_need + b_need;
       // both operands row-major: one launch re-lays both
       if (a_need && b_need && p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
           p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
@@ -270,6 +283,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     }
   }
 
+  if (ws_scales_end < ws_used) ws_scales_end = ws_used;
   if (v == WAVE_MXFP4_VARIANT_NAIVE) {
     e = launch_naive_gemm(p, stream);
   } else if (v == WAVE_MXFP4_VARIANT_SKINNY) {
@@ -284,8 +298,18 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     tile_variant_shape(tv, &bm, &bn);
     p.tiles_m = (int)((m + bm - 1) / bm);
     p.tiles_n = (int)((n + bn - 1) / bn);
-    e = persist_gemm_applies(p, tv, device_cus()) ? launch_persist_gemm(p, tv, device_cus(), stream)
-                                                  : launch_tile_gemm(p, tv, stream);
+    if (persist_gemm_applies(p, tv, device_cus())) {
+      // a last round of tiles that would leave most workgroups idle is cut along K instead, if there is scratch
+      size_t part_bytes = 0;
+      const int parts = persist_tail_parts(p, tv, device_cus(), &part_bytes);
+      if (parts > 1 && workspace && ws_scales_end + part_bytes <= workspace_bytes) {
+        p.tail_parts = parts;
+        p.tail_partial = (float *)((uint8_t *)workspace + ws_scales_end);
+      }
+      e = launch_persist_gemm(p, tv, device_cus(), stream);
+    } else {
+      e = launch_tile_gemm(p, tv, stream);
+    }
   }
   if (e != hipSuccess) return record_hip(e);
   if (splits > 1) e = launch_splitk_reduce(p.partial, c, m * n, splits, p.out_bf16, stream);

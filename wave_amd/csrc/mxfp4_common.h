@@ -46,6 +46,9 @@ struct GemmParams {
   int out_bf16;
   int a_scale_layout, b_scale_layout;  // wave_mxfp4_scale_layout
   int b_preshuffled;
+  int tail_parts;      // persistent kernel: the tiles of the last, partly filled round are cut along K into this
+                       // many parts (1 = not), one part per workgroup, summed afterwards from tail_partial
+  float *tail_partial; // [tiles of the last round][tail_parts][256][256] f32
   int num_groups;      // 0 = dense
   int tiles_m, tiles_n;
   int64_t b_group_stride;        // bytes between experts in b
@@ -110,6 +113,7 @@ hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream
 hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int e5m2, hipStream_t stream);
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus);
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream);
+int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *partial_bytes);
 hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);
 hipError_t launch_scale_spread_rows(const uint8_t *src, uint8_t *dst, int64_t rows, int64_t ks, hipStream_t stream);
 hipError_t launch_quantize(const void *x, int in_dtype, const int32_t *row_ids, int row_div, int64_t src_rows,

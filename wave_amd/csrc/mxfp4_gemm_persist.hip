@@ -48,7 +48,12 @@ enum KtKind {
 // offset gets its top bit flipped just before that tile's DMA is issued and
 // flipped back after it, at fixed places of two peeled K tiles, so the steady
 // loop and the instruction counts the waits rely on are untouched.
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL>
+// SPLIT: the tiles of the last round, which only part of the workgroups would
+// get one of, are cut along K into p.tail_parts parts instead, one part per
+// workgroup (its last item); the parts go to p.tail_partial as f32 tiles and a
+// small kernel adds them up.  A 288-tile problem on 256 CUs then takes 1 + 1/8
+// tile times instead of 2.
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
@@ -71,11 +76,32 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // (M need not be a multiple of the tile: rows past it read zeros and are never stored)
   const uint8_t *a_base[2], *b_base[2], *as_base[2], *bs_base[2];
   // c_rows: rows of the tile that are stored
-  int m0[2], n0[2], a_lim[2], as_lim[2], c_rows[2];
+  // nkt_of / part_of / tail_on: K tiles of the item, its slot in tail_partial (-1: a whole tile), and whether
+  // its K range ends with the (partial) last K tile of the problem
+  int m0[2], n0[2], a_lim[2], as_lim[2], c_rows[2], nkt_of[2], part_of[2];
+  bool tail_on[2];
   const int m_blocks = (p.m + 31) >> 5;
+  const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
   auto set_tile = [&](int which, int pid) -> bool {
-    int tm, tn;
-    if (pid >= padded || !map_tile(pid, tiles_m, p.tiles_n, tm, tn)) return false;
+    int tm, tn, kt_lo = 0;
+    nkt_of[which] = nkt;
+    part_of[which] = -1;
+    if (SPLIT && pid >= total / (int)gridDim.x * (int)gridDim.x) {
+      // the last round: workgroup w takes part w % parts of tile (whole rounds) + w / parts
+      const int whole = total / (int)gridDim.x * (int)gridDim.x, w = pid - whole;
+      if (w >= (int)gridDim.x) return false;
+      const int r = w / p.tail_parts, i = w - r * p.tail_parts;
+      if (whole + r >= padded) return false;  // (ids up to `padded`: map_tile skips the padding ids among them)
+      pid = whole + r;
+      const int base = nkt / p.tail_parts, rem = nkt - base * p.tail_parts;
+      nkt_of[which] = base + (i < rem ? 1 : 0);
+      kt_lo = i * base + min(i, rem);
+      part_of[which] = r * p.tail_parts + i;
+      if (!map_tile(pid, tiles_m, p.tiles_n, tm, tn)) return false;
+    } else if (pid >= padded || !map_tile(pid, tiles_m, p.tiles_n, tm, tn)) {
+      return false;
+    }
+    tail_on[which] = TAIL && kt_lo + nkt_of[which] == nkt;
     n0[which] = tn * BN;
     if (GROUPED) {
       const int32_t *ent = p.tile_table + 4 * (1 + tm);
@@ -97,6 +123,14 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     }
     a_base[which] = p.a + (int64_t)m0[which] * kp;
     a_lim[which] = (int)min((int64_t)(p.m - m0[which]) * kp, (int64_t)0x7FFFFFFF);
+    if (SPLIT) {  // the item's K range starts at K tile kt_lo: move the bases there
+      a_base[which] += kt_lo * kTileKBytes;
+      a_lim[which] = max(a_lim[which] - kt_lo * kTileKBytes, 0);
+      b_base[which] += (int64_t)kt_lo * b_kt_stride;
+      as_base[which] += kt_lo * 256;
+      as_lim[which] = max(as_lim[which] - kt_lo * 256, 0);
+      bs_base[which] += kt_lo * 256;
+    }
     return true;
   };
   int pid = blockIdx.x;
@@ -113,8 +147,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
                                      : ld_row0 * kp + ld_chunk * 16;
   const int ld_step = NWAVES * 8 * kp;  // bytes between consecutive d, either layout (8*NWAVES is a multiple of 16)
   const bool tail_lane = TAIL && ld_chunk >= ((p.k & (kTileK - 1)) >> 5);
-  auto flip_tail = [&](int &goff) { goff ^= tail_lane ? (int)0x80000000 : 0; };
-  const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
+  auto flip_tail = [&](int &goff) { goff ^= tail_lane && (!SPLIT || tail_on[0]) ? (int)0x80000000 : 0; };
 
   // DMA instructions [d0, d1) of operand `op` (0 = A, 1 = B), K tile `kt` of
   // output tile `which` (0 = current, 1 = next), into ring slot `slot`.
@@ -215,7 +248,6 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   constexpr int NS_BF16 = Cfg::WM * Cfg::WN * 2 / 1024, NS_F32 = Cfg::WM * Cfg::WN * 4 / 1024;
   constexpr int kWaitFirstBf16 = NS_BF16 + A_LD > 63 ? 63 : NS_BF16 + A_LD;
   constexpr int kWaitFirstF32 = NS_F32 + A_LD > 63 ? 63 : NS_F32 + A_LD;
-  constexpr bool out_bf16 = OUT_BF16;
 
   // ---------------- one K tile (phases as in the one-tile kernel) ----------------
   //   P0: second half of B(j+1)      P1, P2: A(j+2)      P3: barrier, first half of B(j+2)
@@ -281,7 +313,9 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // chunk c sits at position c ^ (row % chunks per row) (conflict-free 16-byte
   // reads, two-way on the 8-byte writes), written pass by pass and read back as
   // whole rows, 16 bytes per lane.
-  auto store_tile = [&](int slot, int tm0, int tn0, int rows) {
+  // `cbase`: the tile's first row; `f32_tag`: store f32 whatever the kernel's output type (the parts of SPLIT)
+  auto store_tile = [&](int slot, uint8_t *cbase, int ldc, int tn0, int rows, auto f32_tag) {
+    constexpr bool out_bf16 = OUT_BF16 && !decltype(f32_tag)::value;
     constexpr int SW = SLOT / NWAVES;  // staging bytes of a wave
     constexpr int RP = SW / 32;        // row pitch
     constexpr int NCH = RP / 16;       // chunks per row
@@ -297,11 +331,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const int lr = lane_v / LPR, lc = lane_v % LPR;
     // C goes out through a descriptor that ends with the tile's last valid row: rows past M (or past the
     // tile's group) are dropped
-    const int ldc = p.n;
-    constexpr int ELT = OUT_BF16 ? 2 : 4;
-    const __amdgpu_buffer_rsrc_t c_rsrc =
-        make_rsrc_n((uint8_t *)p.c + (int64_t)tm0 * ldc * ELT,
-                    (int)min((int64_t)rows * ldc * ELT, (int64_t)0x7FFFFFFF));
+    constexpr int ELT = out_bf16 ? 2 : 4;
+    const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc_n(cbase, (int)min((int64_t)rows * ldc * ELT, (int64_t)0x7FFFFFFF));
     const int wr0 = wave_m * Cfg::WM;  // the wave's first row inside the tile
     if (out_bf16) {
       constexpr int CP = RP / 2, JP = CP / 32;  // columns, 32-column tiles per pass
@@ -382,7 +413,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // The first tile is peeled off the loop: with it inside, the compiler's own
   // waits (for the scale registers) would have to assume its store-free queue
   // for every tile.
-  int sa = 0;
+  int sa = 0, part_stage = -1;
   auto next_slot = [&](int s) { return s + 2 >= RING ? s + 2 - RING : s + 2; };
   auto b_slot = [&](int s) { return s + 1 >= RING ? 0 : s + 1; };
   auto run_tile = [&](auto pending_tag) -> bool {
@@ -390,28 +421,35 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const bool has_next = set_tile(1, npid);
     if (!has_next) {
       m0[1] = m0[0], n0[1] = n0[0], a_lim[1] = a_lim[0], as_lim[1] = as_lim[0], c_rows[1] = c_rows[0];
+      nkt_of[1] = nkt_of[0], part_of[1] = part_of[0], tail_on[1] = tail_on[0];
       a_base[1] = a_base[0], b_base[1] = b_base[0], as_base[1] = as_base[0], bs_base[1] = bs_base[0];
     }
+    const int nk = SPLIT ? nkt_of[0] : nkt;  // K tiles of this item
     k_tile(0, sa, b_slot(sa), std::integral_constant<int, kFirst>{}, pending_tag);
     sa = next_slot(sa);
-    for (int j = 1; j < nkt - (TAIL ? 3 : 2); ++j) {
+    for (int j = 1; j < nk - (TAIL ? 3 : 2); ++j) {
       k_tile(j, sa, b_slot(sa), std::integral_constant<int, kSteady>{}, pending_tag);
       sa = next_slot(sa);
     }
-    if constexpr (TAIL) {  // nkt >= 4
-      k_tile(nkt - 3, sa, b_slot(sa), std::integral_constant<int, kSteadyTail>{}, pending_tag);
+    if constexpr (TAIL) {  // nk >= 4
+      k_tile(nk - 3, sa, b_slot(sa), std::integral_constant<int, kSteadyTail>{}, pending_tag);
       sa = next_slot(sa);
     }
-    k_tile(nkt - 2, sa, b_slot(sa), std::integral_constant<int, kBound1>{}, pending_tag);
+    k_tile(nk - 2, sa, b_slot(sa), std::integral_constant<int, kBound1>{}, pending_tag);
     sa = next_slot(sa);
     const int stage_slot = b_slot(sa);
-    k_tile(nkt - 1, sa, stage_slot, std::integral_constant<int, kBound2>{}, pending_tag);
+    k_tile(nk - 1, sa, stage_slot, std::integral_constant<int, kBound2>{}, pending_tag);
     // second half of B(1) of the next tile, ahead of the C stores (its first
     // half went into slot `sa` in the last phase above)
     issue_g2l(1, 1, 1, sa, B_LD / 2, B_LD);
     sa = next_slot(sa);
     __builtin_amdgcn_sched_barrier(0);
-    store_tile(stage_slot, m0[0], n0[0], c_rows[0]);
+    if (SPLIT && part_of[0] >= 0) {  // a part of a tile of the last round: always the workgroup's last item,
+      part_stage = stage_slot;       // stored after the loop (a second store path in here costs the loop registers)
+      return false;
+    }
+    store_tile(stage_slot, (uint8_t *)p.c + (int64_t)m0[0] * p.n * (OUT_BF16 ? 2 : 4), p.n, n0[0], c_rows[0],
+               std::false_type{});
     if (!has_next) return false;
     // the staging slot is the next target of the A stream: all waves must be done reading it
     asm volatile("" ::: "memory");
@@ -421,6 +459,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     __builtin_amdgcn_sched_barrier(0);
     pid = npid;
     m0[0] = m0[1], n0[0] = n0[1], a_lim[0] = a_lim[1], as_lim[0] = as_lim[1], c_rows[0] = c_rows[1];
+    nkt_of[0] = nkt_of[1], part_of[0] = part_of[1], tail_on[0] = tail_on[1];
     a_base[0] = a_base[1], b_base[0] = b_base[1], as_base[0] = as_base[1], bs_base[0] = bs_base[1];
     return true;
   };
@@ -428,37 +467,106 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     while (run_tile(std::true_type{})) {
     }
   }
+  if (SPLIT && part_stage >= 0)
+    store_tile(part_stage, (uint8_t *)(p.tail_partial + (int64_t)part_of[0] * BM * BN), BN, 0, BM, std::true_type{});
   __builtin_amdgcn_s_waitcnt(0);  // the trailing DMA must not outlive the workgroup's LDS
 }
 
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL>
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
 __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_kernel(const GemmParams p) {
-  persist_body<Cfg, OUT_BF16, GROUPED, TAIL>(p);
+  persist_body<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>(p);
 }
 
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL>
+// Adds up the parts of the tiles of the last round (SPLIT) and writes them to C: one workgroup per 32 rows of a
+// tile, a thread per 4 columns and row.
+template <class Cfg>
+__global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams p, int grid_main) {
+  constexpr int BM = Cfg::BM, BN = Cfg::BN;
+  const int total = p.tiles_m * p.tiles_n, whole = total / grid_main * grid_main;
+  const int r = blockIdx.x / (BM / 32), band = blockIdx.x % (BM / 32);
+  int tm, tn;
+  if (!map_tile(whole + r, p.tiles_m, p.tiles_n, tm, tn)) return;  // a padding id
+  const float *part = p.tail_partial + (int64_t)r * p.tail_parts * BM * BN;
+  for (int e = threadIdx.x; e < 32 * BN / 4; e += 256) {
+    const int row = band * 32 + e / (BN / 4), col = (e % (BN / 4)) * 4;
+    const int m = tm * BM + row, n = tn * BN + col;
+    if (m >= p.m) continue;
+    v4f sum = *(const v4f *)(part + (int64_t)row * BN + col);
+    for (int i = 1; i < p.tail_parts; ++i) sum += *(const v4f *)(part + ((int64_t)i * BM + row) * BN + col);
+    if (p.out_bf16) {
+      typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+      *(bf4 *)((__bf16 *)p.c + (int64_t)m * p.n + n) = bf4{(__bf16)sum.x, (__bf16)sum.y, (__bf16)sum.z, (__bf16)sum.w};
+    } else {
+      *(v4f *)((float *)p.c + (int64_t)m * p.n + n) = sum;
+    }
+  }
+}
+
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
 static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_t stream) {
   static bool attr_done = false;  // benign race: the attribute is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL>,
+    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL><<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
-  return hipGetLastError();
+  persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>
+      <<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  hipError_t e = hipGetLastError();
+  if (SPLIT && e == hipSuccess) {
+    const int total = p.tiles_m * p.tiles_n;
+    const int ids = (total + kNumXcd - 1) / kNumXcd * kNumXcd - total / grid_x * grid_x;  // tile ids of the last round
+    persist_tail_sum_kernel<Cfg><<<dim3(ids * (Cfg::BM / 32)), 256, 0, stream>>>(p, grid_x);
+    e = hipGetLastError();
+  }
+  return e;
+}
+
+template <class Cfg, bool OUT_BF16>
+static hipError_t launch_persist_dense(const GemmParams &p, int grid_x, hipStream_t stream) {
+  const bool tail = (p.k & (kTileK - 1)) != 0;
+  if constexpr (Cfg::NWAVES == 8) {  // (the 4-wave kernel has no registers to spare for the split bookkeeping)
+    if (p.tail_parts > 1)
+      return tail ? launch_persist_out<Cfg, OUT_BF16, false, true, true>(p, grid_x, stream)
+                  : launch_persist_out<Cfg, OUT_BF16, false, false, true>(p, grid_x, stream);
+  }
+  return tail ? launch_persist_out<Cfg, OUT_BF16, false, true, false>(p, grid_x, stream)
+              : launch_persist_out<Cfg, OUT_BF16, false, false, false>(p, grid_x, stream);
 }
 
 template <class Cfg>
 static hipError_t launch_persist_cfg(const GemmParams &p, int grid_x, hipStream_t stream) {
   if (p.tile_table != nullptr)
-    return p.out_bf16 ? launch_persist_out<Cfg, true, true, false>(p, grid_x, stream)
-                      : launch_persist_out<Cfg, false, true, false>(p, grid_x, stream);
-  if ((p.k & (kTileK - 1)) != 0)
-    return p.out_bf16 ? launch_persist_out<Cfg, true, false, true>(p, grid_x, stream)
-                      : launch_persist_out<Cfg, false, false, true>(p, grid_x, stream);
-  return p.out_bf16 ? launch_persist_out<Cfg, true, false, false>(p, grid_x, stream)
-                    : launch_persist_out<Cfg, false, false, false>(p, grid_x, stream);
+    return p.out_bf16 ? launch_persist_out<Cfg, true, true, false, false>(p, grid_x, stream)
+                      : launch_persist_out<Cfg, false, true, false, false>(p, grid_x, stream);
+  return p.out_bf16 ? launch_persist_dense<Cfg, true>(p, grid_x, stream) : launch_persist_dense<Cfg, false>(p, grid_x, stream);
+}
+
+// How many parts the tiles of the last round should be cut into along K (1 = leave them whole), and the bytes
+// of f32 scratch that takes.  Only when less than half of the workgroups would get a tile in that round,
+// every part keeps at least four K tiles and the estimate says it pays.
+int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *partial_bytes) {
+  *partial_bytes = 0;
+  if (variant != WAVE_MXFP4_VARIANT_T256x256_W4x2 || p.num_groups != 0 || !persist_gemm_applies(p, variant, num_cus))
+    return 1;
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
+  if (total % grid == 0) return 1;
+  // tile ids of the last round, the XCD padding ids among them included (they get a slot and stay unused)
+  const int rest = (int)((total + kNumXcd - 1) / kNumXcd * kNumXcd - total / grid * grid);
+  if (rest * 2 > grid) return 1;
+  // Cost of the last round in us: a tile's K tiles at the measured 1.85 us each, divided among the parts, plus
+  // writing and re-reading the f32 parts (about 4 TB/s) and the launch of the kernel that sums them.
+  const double tile_us = 1.85 * p.k_tiles;
+  int parts = 1;
+  double best = tile_us;
+  for (int c = 2; c <= 8 && c * rest <= grid && p.k_tiles / c >= 4; ++c) {
+    const double us = tile_us / c + 2.0 * rest * c * (256 * 256 * 4) / 4.0e6 + 6.0;
+    if (us < best * 0.9) best = us, parts = c;
+  }
+  if (parts > 1) *partial_bytes = (size_t)rest * parts * 256 * 256 * sizeof(float);
+  return parts;
 }
 
 // Whether the persistent kernel serves this problem with `num_cus` CUs.

@@ -10,6 +10,8 @@ call returns None."""
 
 from __future__ import annotations
 
+import functools
+
 import torch
 
 from . import _lib
@@ -19,6 +21,26 @@ _OUT_DTYPES = {torch.float32: _lib.OUT_F32, torch.bfloat16: _lib.OUT_BF16}
 
 def _stream_ptr(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """``torch.cuda.device(d)`` only when ``d`` is not the current device already (the context manager costs
+    several microseconds of host time per call, which shows on small problems)."""
+
+    __slots__ = ("_ctx",)
+
+    def __init__(self, device):
+        idx = device.index if device.index is not None else torch.cuda.current_device()
+        self._ctx = None if idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            self._ctx.__exit__(*exc)
+        return False
 
 
 def _as_u8(t: torch.Tensor, name: str) -> torch.Tensor:
@@ -54,6 +76,7 @@ def _scale_rows_ok(scale: torch.Tensor, rows: int, ks: int, layout: int, name: s
                 f"{name}: shuffled scales need {need} bytes (rows padded to 32, groups to 8), got {scale.numel()}")
 
 
+@functools.lru_cache(maxsize=4096)
 def workspace_bytes(m: int, n: int, k: int, split_k: int = 0, variant: int = _lib.VARIANT_AUTO) -> int:
     return int(_lib.load().wave_mxfp4_workspace_bytes(m, n, k, split_k, variant))
 
@@ -130,7 +153,7 @@ def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW
         workspace = None
     if workspace is not None:
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.wave_mxfp4_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
                                  out.data_ptr(), m, n, k, od, a_scale_layout, b_scale_layout, b_layout,
                                  split_k, ws_ptr, ws_bytes, variant, _stream_ptr(x.device))
@@ -179,7 +202,7 @@ def mxfp4_gemm_grouped(x, x_scales, w_t, w_scales, offsets, out, *, a_scale_layo
         workspace = None
     if workspace is not None:
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.wave_mxfp4_gemm_grouped(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(),
                                          w_scales.data_ptr(), out.data_ptr(), offsets.data_ptr(), e, rows,
                                          n, k, od, a_scale_layout, b_scale_layout, b_layout, variant,
@@ -194,7 +217,7 @@ def mxfp4_to_f32(x: torch.Tensor) -> torch.Tensor:
     x = _as_u8(x, "x")
     rows, kp = x.shape
     out = torch.empty(rows, kp * 2, dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.wave_mxfp4_to_f32(x.data_ptr(), out.data_ptr(), rows, kp, _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp4_to_f32")
     return out
@@ -206,7 +229,7 @@ def e8m0_to_f32(s: torch.Tensor) -> torch.Tensor:
     lib = _lib.load()
     s = _as_u8(s, "s")
     out = torch.empty(s.shape, dtype=torch.float32, device=s.device)
-    with torch.cuda.device(s.device):
+    with _on_device(s.device):
         st = lib.wave_mxfp4_e8m0_to_f32(s.data_ptr(), out.data_ptr(), s.numel(), _stream_ptr(s.device))
     _lib.check(st, "wave_mxfp4_e8m0_to_f32")
     return out
@@ -223,7 +246,7 @@ def dequant(x: torch.Tensor, scales: torch.Tensor, scale_layout=_lib.SCALE_ROW_M
     k = kp * 2
     _scale_rows_ok(scales, rows, k // 32, scale_layout, "scales")
     out = torch.empty(rows, k, dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.wave_mxfp4_dequant(x.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, k, scale_layout,
                                     _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp4_dequant")
@@ -241,7 +264,7 @@ def scale_convert(scale: torch.Tensor, rows: int, ks: int, src_layout: int, dst_
         out = torch.empty(rows, ks, dtype=torch.uint8, device=scale.device)
     else:
         out = torch.empty((rows + 31) // 32 * 32, (ks + 7) // 8 * 8, dtype=torch.uint8, device=scale.device)
-    with torch.cuda.device(scale.device):
+    with _on_device(scale.device):
         st = lib.wave_mxfp4_scale_convert(scale.data_ptr(), src_layout, out.data_ptr(), dst_layout, rows, ks,
                                           _stream_ptr(scale.device))
     _lib.check(st, "wave_mxfp4_scale_convert")
@@ -260,7 +283,7 @@ def e8m0_shuffle(scale: torch.Tensor) -> torch.Tensor:
     scale = _as_u8(scale, "scale")
     rows, ks = scale.shape
     out = torch.empty((rows + 31) // 32 * 32, (ks + 7) // 8 * 8, dtype=torch.uint8, device=scale.device)
-    with torch.cuda.device(scale.device):
+    with _on_device(scale.device):
         st = lib.wave_mxfp4_e8m0_shuffle(scale.data_ptr(), out.data_ptr(), rows, ks, _stream_ptr(scale.device))
     _lib.check(st, "wave_mxfp4_e8m0_shuffle")
     return out
@@ -274,7 +297,7 @@ def b_preshuffle(b: torch.Tensor) -> torch.Tensor:
     b = _as_u8(b, "b")
     rows, kp = b.shape
     out = torch.empty_like(b)
-    with torch.cuda.device(b.device):
+    with _on_device(b.device):
         st = lib.wave_mxfp4_b_preshuffle(b.data_ptr(), out.data_ptr(), rows, kp, _stream_ptr(b.device))
     _lib.check(st, "wave_mxfp4_b_preshuffle")
     return out
@@ -311,7 +334,7 @@ def quantize_mxfp4(x: torch.Tensor, *, shuffle: bool = False, scale_layout: int 
         scales = torch.empty(rows, ks, dtype=torch.uint8, device=x.device)
     else:
         scales = torch.empty((rows + 31) // 32 * 32, (ks + 7) // 8 * 8, dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.wave_mxfp4_quantize(x.data_ptr(), _IN_DTYPES[x.dtype], q.data_ptr(), scales.data_ptr(), rows, k,
                                      layout, _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp4_quantize")
@@ -345,7 +368,7 @@ def quantize_mxfp4_rows(x: torch.Tensor, row_ids: torch.Tensor, row_div: int = 1
     rows = row_ids.numel()
     q = torch.empty(rows, k // 2, dtype=torch.uint8, device=x.device)
     scales = _new_scales(rows, k // 32, scale_layout, x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.wave_mxfp4_quantize_rows(x.data_ptr(), _IN_DTYPES[x.dtype], src_rows, row_ids.data_ptr(), int(row_div),
                                           q.data_ptr(), scales.data_ptr(), rows, k, scale_layout,
                                           _stream_ptr(x.device))
@@ -372,7 +395,7 @@ def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: i
     if num_tokens_post_pad.numel() < 1:
         raise ValueError("num_tokens_post_pad: needs one entry")
     ids = topk_ids.contiguous()
-    with torch.cuda.device(ids.device):
+    with _on_device(ids.device):
         st = lib.wave_mxfp4_moe_align_block_size(
             ids.data_ptr(), 1 if ids.dtype == torch.int64 else 0, ids.numel(), int(num_experts), int(block_size),
             sorted_ids.data_ptr(), sorted_ids.numel(), expert_ids.data_ptr(), expert_ids.numel(),
@@ -402,7 +425,7 @@ def silu_and_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor | None 
         out = torch.empty(rows, n, dtype=gate.dtype, device=gate.device)
     elif out.shape != gate.shape or out.dtype != gate.dtype or out.stride(1) != 1:
         raise ValueError("out: expected the shape and dtype of gate, unit column stride")
-    with torch.cuda.device(gate.device):
+    with _on_device(gate.device):
         st = lib.wave_mxfp4_silu_and_mul(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.stride(0), up.stride(0),
                                          out.stride(0), _IN_DTYPES[gate.dtype], rows, n, _stream_ptr(gate.device))
     _lib.check(st, "wave_mxfp4_silu_and_mul")
@@ -418,7 +441,7 @@ def silu_and_mul_quantize(gate: torch.Tensor, up: torch.Tensor, *, scale_layout:
     rows, n = gate.shape
     q = torch.empty(rows, n // 2, dtype=torch.uint8, device=gate.device)
     scales = _new_scales(rows, n // 32, scale_layout, gate.device)
-    with torch.cuda.device(gate.device):
+    with _on_device(gate.device):
         st = lib.wave_mxfp4_silu_and_mul_quantize(gate.data_ptr(), up.data_ptr(), gate.stride(0), up.stride(0),
                                                   _IN_DTYPES[gate.dtype], q.data_ptr(), scales.data_ptr(), rows, n,
                                                   scale_layout, _stream_ptr(gate.device))
@@ -468,7 +491,7 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format: int | None = Non
         workspace = None
     if workspace is not None:
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = lib.wave_mxfp8_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
                                  out.data_ptr(), m, n, k, fmt, od, ws_ptr, ws_bytes, variant, _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp8_gemm")

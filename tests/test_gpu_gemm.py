@@ -453,3 +453,20 @@ def test_persistent_path_last_round_cut_along_k(m, n, k, out_dtype):
     torch.cuda.synchronize()
     diff = (out.float() - other.float()).abs().max().item()
     assert diff <= (4e-6 if out_dtype == torch.float32 else 2.0 ** -7) * out.float().abs().max().item()
+
+
+@pytest.mark.parametrize("vname", ["t128x128_w2x2", "t256x256_w4x2"])
+@pytest.mark.parametrize("m,n,k", [(300, 528, 1248 - 32), (4352 - 100, 4352, 1024 + 128)])
+def test_partial_last_k_tile_preshuffled_b_and_shuffled_scales(m, n, k, vname):
+    """The reference's fastest templates (preshuffled B, e8m0_shuffle scales) at K % 256 != 0 (K % 64 == 0 as
+    b_preshuffle needs): same bits as the row-major operands on the same kernel."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=n + k, scale_lo=120, scale_hi=134)
+    v = ALL_VARIANTS[vname]
+    plain = run_gemm(x, xs, w_t, ws, torch.float32, variant=v)
+    rows = np.r_[0:32, m - 40:m]
+    assert_f32_close(plain[rows], c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows), vname)
+    pre = run_gemm(x, orc.e8m0_shuffle_padded(xs)[: (m + 31) // 32 * 32], orc.b_preshuffle(w_t),
+                   orc.e8m0_shuffle_padded(ws)[: (n + 31) // 32 * 32], torch.float32, variant=v,
+                   a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
+                   b_layout=_lib.B_PRESHUFFLE)
+    assert np.array_equal(pre, plain)

@@ -101,8 +101,8 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
 // A partial last K tile with scales that are not (or cannot be brought) in MFMA32 order is only built for the
 // 128x128 tile kernel.
 bool needs_generic_k(const GemmParams &p) {
-  return (p.k % kTileK) != 0 && (p.b_preshuffled || p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ||
-                                 p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32);
+  return (p.k % kTileK) != 0 &&
+         (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32);
 }
 
 // Split the library takes by itself for a tile kernel: only when the tile
@@ -251,7 +251,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   // (a few MB, microseconds) and run the native-scale kernel.
   // (Not worth a second launch for a small problem with short K: there the direct reads cost less.)
   const bool small_short = p.tiles_per_split <= 8 && (int64_t)m * n <= (int64_t)2048 * 2048 && k % kTileK == 0;
-  if (is_tile_variant(v) && workspace && !small_short && !(p.b_preshuffled && k % kTileK != 0)) {
+  if (is_tile_variant(v) && workspace && !small_short) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
     const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? a_bytes : 0;
     const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? b_bytes : 0;
@@ -262,6 +262,13 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
       if (a_need && b_need && p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
           p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
           launch_scale_pair_to_mfma32(p.a_scale, ws, m, p.b_scale, ws + a_need, n, p.ks, stream) == hipSuccess) {
+        p.a_scale = ws;
+        p.b_scale = ws + a_need;
+        p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+      } else if (a_need && b_need && p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE &&
+                 p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE &&
+                 launch_scale_pair_shuffle_to_mfma32(p.a_scale, ws, m, p.b_scale, ws + a_need, n, p.ks, stream) ==
+                     hipSuccess) {
         p.a_scale = ws;
         p.b_scale = ws + a_need;
         p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;

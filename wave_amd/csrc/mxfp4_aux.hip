@@ -159,6 +159,25 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
   }
 }
 
+// e8m0_shuffle -> MFMA32: both keep one 256-byte block per (32 rows, K tile) in the same block order, so the
+// conversion permutes bytes inside a block.  One thread per destination dword (lane (g%2)*32 + r%32, bytes
+// t = 0..3 = groups 2t + g%2): its bytes come from the two source dwords (g%4)*16 + r%16 for g%4 = g%2 and
+// 2 + g%2, byte (g/4)*2 + (r%32)/16 of each.  blockIdx.y picks one of two tensors.
+__global__ void __launch_bounds__(256) scale_shuffle_to_mfma32_kernel(const uint32_t *__restrict__ src0,
+                                                                      uint32_t *__restrict__ dst0, int64_t dwords0,
+                                                                      const uint32_t *__restrict__ src1,
+                                                                      uint32_t *__restrict__ dst1, int64_t dwords1) {
+  const uint32_t *src = blockIdx.y ? src1 : src0;
+  uint32_t *dst = blockIdx.y ? dst1 : dst0;
+  const int64_t dwords = blockIdx.y ? dwords1 : dwords0;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < dwords; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t blk = i >> 6;
+    const int lane = (int)(i & 63), r32 = lane & 31, gpar = lane >> 5;
+    const uint32_t d0 = src[blk * 64 + gpar * 16 + (r32 & 15)], d1 = src[blk * 64 + (2 + gpar) * 16 + (r32 & 15)];
+    dst[i] = __builtin_amdgcn_perm(d1, d0, (r32 >> 4) ? 0x07030501u : 0x06020400u);
+  }
+}
+
 // dst[r, g] = src[r]: one scale per row spread over the row's ks groups.
 __global__ void scale_spread_rows_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int64_t rows,
                                          int64_t ks) {
@@ -280,8 +299,24 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
     scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks, nullptr);
     return hipGetLastError();
   }
+  if (src_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && ((uintptr_t)src & 3) == 0) {
+    scale_shuffle_to_mfma32_kernel<<<dim3(blocks_for(n, kThreads), 1), kThreads, 0, stream>>>(
+        (const uint32_t *)src, (uint32_t *)dst, n, nullptr, nullptr, 0);
+    return hipGetLastError();
+  }
   scale_convert_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(src, src_layout, dst, dst_layout, rows,
                                                                         ks, rows_p, ksp);
+  return hipGetLastError();
+}
+
+// e8m0_shuffle -> MFMA32 for the scales of both GEMM operands in one launch.
+hipError_t launch_scale_pair_shuffle_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
+                                               uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream) {
+  if ((((uintptr_t)a_src | (uintptr_t)b_src) & 3) != 0) return hipErrorInvalidValue;
+  const int64_t ksp = (ks + 7) / 8 * 8;
+  const int64_t na = (a_rows + 31) / 32 * 32 * (ksp / 4), nb = (b_rows + 31) / 32 * 32 * (ksp / 4);
+  scale_shuffle_to_mfma32_kernel<<<dim3(blocks_for(na > nb ? na : nb, kThreads), 2), kThreads, 0, stream>>>(
+      (const uint32_t *)a_src, (uint32_t *)a_dst, na, (const uint32_t *)b_src, (uint32_t *)b_dst, nb);
   return hipGetLastError();
 }
 

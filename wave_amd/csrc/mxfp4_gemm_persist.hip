@@ -576,8 +576,8 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
   if ((p.num_groups != 0) != (p.tile_table != nullptr) || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
   if ((p.n & 255) != 0 || p.k_tiles < 3) return false;  // any M
-  // a partial last K tile: dense problems with row-major B and at least four K tiles
-  if ((p.k & (kTileK - 1)) != 0 && (p.num_groups != 0 || p.b_preshuffled || p.k_tiles < 4)) return false;
+  // a partial last K tile: dense problems with at least four K tiles
+  if ((p.k & (kTileK - 1)) != 0 && (p.num_groups != 0 || p.k_tiles < 4)) return false;
   if (p.out_bf16 ? (p.n & 7) != 0 : (p.n & 3) != 0) return false;
   // 32-bit offsets inside one operand tile, and more tiles than workgroups
   if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31)) return false;

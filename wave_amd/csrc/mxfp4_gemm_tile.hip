@@ -718,9 +718,8 @@ static hipError_t launch_by_scales(const GemmParams &p, hipStream_t stream) {
 hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream) {
   const bool native =
       p.a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
-  // (with both scale tensors in MFMA32 order every tile kernel takes a partial last K tile;
-  //  preshuffled B keeps whole 64-element K steps only, which the generic kernel handles)
-  if ((p.k & (kTileK - 1)) != 0 && (!native || p.b_preshuffled)) return launch_cfg<Cfg128x128w4, kGenericK>(p, stream);
+  // (with both scale tensors in MFMA32 order every tile kernel takes a partial last K tile)
+  if ((p.k & (kTileK - 1)) != 0 && !native) return launch_cfg<Cfg128x128w4, kGenericK>(p, stream);
   switch (variant) {
     case WAVE_MXFP4_VARIANT_T256x256_W2x2: return launch_by_scales<Cfg256x256w4>(p, stream);
     case WAVE_MXFP4_VARIANT_T256x256_W4x2: return launch_by_scales<Cfg256x256w8>(p, stream);

@@ -142,15 +142,16 @@ size_t wave_mxfp4_grouped_workspace_bytes(int64_t total_rows, int64_t n, int64_t
  * infinities, e5m2 is IEEE-like). */
 typedef enum { WAVE_MXFP8_E4M3 = 0, WAVE_MXFP8_E5M2 = 1 } wave_mxfp8_format;
 
-/* The same block-scaled GEMM on MXFP8 operands: A [M, K] and B [N, K] one byte
- * per element (both of elem_format), scales [R, K/32] e8m0 row-major, C f32 or
+/* The same block-scaled GEMM on MXFP8 operands: A [M, K] of a_format and
+ * B [N, K] of b_format, one byte per element (the formats may differ: cbsz /
+ * blgp 0 / 1 of the instruction), scales [R, K/32] e8m0 row-major, C f32 or
  * bf16.  Replaces the kernel of tests/kernel/wave_gemm_mxfp_test.py:416-501
  * (tkl.f8e5m2 operands through the same scaled MFMA).  K % 128 == 0; variant
  * AUTO, T256x256_W2x2 or T128x128_W2x2.  `workspace` is optional scratch of
  * wave_mxfp8_workspace_bytes(m, n, k) bytes (256-byte aligned): with it, and
  * K % 256 == 0, the scales are first re-laid out for one-dword-per-lane reads. */
 int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
-                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, void *workspace,
+                    int64_t m, int64_t n, int64_t k, int a_format, int b_format, int out_dtype, void *workspace,
                     size_t workspace_bytes, int variant, void *hip_stream);
 size_t wave_mxfp8_workspace_bytes(int64_t m, int64_t n, int64_t k);
 

@@ -49,34 +49,38 @@ def fp8_to_f64(x: np.ndarray, fmt: int) -> np.ndarray:
     return table[np.asarray(x, dtype=np.uint8)]
 
 
-def scaled_gemm_mxfp8(x, w_t, x_scales, w_scales, fmt: int) -> np.ndarray:
+def scaled_gemm_mxfp8(x, w_t, x_scales, w_scales, fmt) -> np.ndarray:
     """x [M, K], w_t [N, K] uint8 codes, scales [R, K/32] e8m0 -> C [M, N] float64
-    (tests/kernel/wave_gemm_mxfp_test.py:80-91 with w_t = w.T)."""
+    (tests/kernel/wave_gemm_mxfp_test.py:80-91 with w_t = w.T).  ``fmt`` is one
+    format for both operands or a pair (x format, w_t format)."""
+    fmt_x, fmt_w = fmt if isinstance(fmt, (tuple, list)) else (fmt, fmt)
     xs = e8m0_to_f32(np.asarray(x_scales, dtype=np.uint8)).astype(np.float64).repeat(SCALE_GROUP_SIZE, axis=1)
     ws = e8m0_to_f32(np.asarray(w_scales, dtype=np.uint8)).astype(np.float64).repeat(SCALE_GROUP_SIZE, axis=1)
-    a = fp8_to_f64(x, fmt) * xs
-    b = fp8_to_f64(w_t, fmt) * ws
+    a = fp8_to_f64(x, fmt_x) * xs
+    b = fp8_to_f64(w_t, fmt_w) * ws
     return a @ b.T
 
 
-def make_inputs_mxfp8(m, n, k, seed, fmt: int, scale_lo=124, scale_hi=127):
+def make_inputs_mxfp8(m, n, k, seed, fmt, scale_lo=124, scale_hi=127):
     """Seeded operands in the manner of generate_gemm_afp8wfp8_inputs
     (tests/kernel/wave_gemm_mxfp_test.py:64-77): normal values rounded to the
-    format, scales uniform in [scale_lo, scale_hi].  Returns codes, not floats."""
+    format (one for both operands, or a pair), scales uniform in
+    [scale_lo, scale_hi].  Returns codes, not floats."""
     rng = np.random.default_rng(seed)
-    table = E5M2_TABLE if fmt == E5M2 else E4M3_TABLE
-    finite = np.nonzero(np.isfinite(table))[0]
-    vals = table[finite]
-    order = np.argsort(vals, kind="stable")
-    vals, codes = vals[order], finite[order].astype(np.uint8)
+    fmt_x, fmt_w = fmt if isinstance(fmt, (tuple, list)) else (fmt, fmt)
 
-    def quantise(v):
+    def quantise(v, f):
+        table = E5M2_TABLE if f == E5M2 else E4M3_TABLE
+        finite = np.nonzero(np.isfinite(table))[0]
+        vals = table[finite]
+        order = np.argsort(vals, kind="stable")
+        vals, codes = vals[order], finite[order].astype(np.uint8)
         idx = np.clip(np.searchsorted(vals, v), 1, len(vals) - 1)
         lower = (v - vals[idx - 1]) <= (vals[idx] - v)
         return codes[np.where(lower, idx - 1, idx)]
 
-    x = quantise(rng.standard_normal((m, k)))
-    w_t = quantise(rng.standard_normal((n, k)))
+    x = quantise(rng.standard_normal((m, k)), fmt_x)
+    w_t = quantise(rng.standard_normal((n, k)), fmt_w)
     xs = rng.integers(scale_lo, scale_hi + 1, size=(m, k // 32), dtype=np.uint8)
     ws = rng.integers(scale_lo, scale_hi + 1, size=(n, k // 32), dtype=np.uint8)
     return x, xs, w_t, ws

@@ -55,6 +55,35 @@ def test_mxfp8_against_oracle(m, n, k, vname, fmt):
     assert_f32_close(run(x, xs, w_t, ws, fmt, variant=VARIANTS[vname]), ref, f"{vname} {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("fmt", [(o8.E4M3, o8.E5M2), (o8.E5M2, o8.E4M3)], ids=["e4m3_x_e5m2", "e5m2_x_e4m3"])
+@pytest.mark.parametrize("vname", sorted(VARIANTS))
+@pytest.mark.parametrize("m,n,k", [(256, 256, 512), (300, 200, 384), (1024, 1024, 1024)])
+def test_mxfp8_mixed_formats_against_oracle(m, n, k, vname, fmt):
+    """Activations and weights in different 8-bit formats (each operand of the instruction carries its own)."""
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=m + n + k + 1, fmt=fmt, scale_lo=120, scale_hi=134)
+    ref = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, fmt)
+    assert_f32_close(run(x, xs, w_t, ws, fmt, variant=VARIANTS[vname]), ref, f"{vname} {m}x{n}x{k}")
+
+
+def test_mxfp8_mixed_formats_from_torch_dtypes():
+    """float8 tensors carry their own format: e4m3 activations against e5m2 weights, exact on one-hot rows."""
+    m, n, k = 128, 96, 256
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=11, fmt=(o8.E4M3, o8.E5M2))
+    x[:] = 0
+    xs[:] = 127
+    one = int(np.nonzero(o8.E4M3_TABLE == 1.0)[0][0])
+    for r in range(m):
+        x[r, (r * 7) % k] = one
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    out = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    wave_amd.mxfp8_gemm(gx.view(torch.float8_e4m3fn), gxs, gw.view(torch.float8_e5m2), gws, out)
+    deq = o8.fp8_to_f64(w_t, o8.E5M2) * np.exp2(ws.astype(np.float64) - 127).repeat(32, axis=1)
+    want = np.stack([deq[:, (r * 7) % k] for r in range(m)])
+    assert np.array_equal(out.cpu().numpy().astype(np.float64), want)
+    with pytest.raises(ValueError):
+        wave_amd.mxfp8_gemm(gx.view(torch.float8_e4m3fn), gxs, gw, gws, out, elem_format=(o8.E5M2, o8.E5M2))
+
+
 @pytest.mark.parametrize("fmt", [o8.E5M2, o8.E4M3], ids=["e5m2", "e4m3"])
 def test_mxfp8_bf16_output_and_every_code(fmt):
     """Every finite byte value of the format appears in both operands."""
@@ -107,11 +136,12 @@ def test_mxfp8_argument_errors():
     lib = _lib.load()
     P = 0x1000
     g = lambda **kw: lib.wave_mxfp8_gemm(*[kw.get(k, d) for k, d in (
-        ("a", P), ("as_", P), ("b", P), ("bs", P), ("c", P), ("m", 128), ("n", 128), ("k", 256), ("fmt", 1), ("od", 0),
+        ("a", P), ("as_", P), ("b", P), ("bs", P), ("c", P), ("m", 128), ("n", 128), ("k", 256), ("fmt", 1), ("fmt_b", 1), ("od", 0),
         ("ws", None), ("wsb", 0), ("variant", 0), ("stream", None))])
     assert g(k=192) == _lib.ERR_BAD_SHAPE
     assert g(m=-1) == _lib.ERR_BAD_SHAPE
     assert g(fmt=2) == _lib.ERR_BAD_ENUM
+    assert g(fmt_b=-1) == _lib.ERR_BAD_ENUM
     assert g(od=3) == _lib.ERR_BAD_ENUM
     assert g(variant=_lib.VARIANT_SKINNY) == _lib.ERR_UNSUPPORTED
     assert g(a=None) == _lib.ERR_NULL_POINTER

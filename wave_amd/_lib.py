@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # WAVE_MXFP4_LIB points at another build of the same ABI (e.g. an experiment)
 LIB_PATH = os.environ.get("WAVE_MXFP4_LIB") or os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 # status codes of include/wave_mxfp4.h
 OK = 0
@@ -84,7 +84,7 @@ def load():
     lib.wave_mxfp4_grouped_workspace_bytes.argtypes = [i64, i64, i64, i32]
     lib.wave_mxfp4_grouped_workspace_bytes.restype = sz
     lib.wave_mxfp4_gemm_grouped.restype = i32
-    lib.wave_mxfp8_gemm.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, p, sz, i32, p]
+    lib.wave_mxfp8_gemm.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, p, sz, i32, p]
     lib.wave_mxfp8_workspace_bytes.argtypes = [i64, i64, i64]
     lib.wave_mxfp8_workspace_bytes.restype = sz
     lib.wave_mxfp8_gemm.restype = i32

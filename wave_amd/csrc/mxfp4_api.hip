@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 6;
+constexpr int kAbiVersion = 7;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -329,11 +329,12 @@ size_t wave_mxfp8_workspace_bytes(int64_t m, int64_t n, int64_t k) {
 }
 
 int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
-                    int64_t m, int64_t n, int64_t k, int elem_format, int out_dtype, void *workspace,
+                    int64_t m, int64_t n, int64_t k, int a_format, int b_format, int out_dtype, void *workspace,
                     size_t workspace_bytes, int variant, void *hip_stream) {
   if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim || k % 128 != 0)
     return WAVE_MXFP4_ERR_BAD_SHAPE;
-  if (bad_enum(elem_format, 2) || bad_enum(out_dtype, 2) || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
+  if (bad_enum(a_format, 2) || bad_enum(b_format, 2) || bad_enum(out_dtype, 2) ||
+      bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
     return WAVE_MXFP4_ERR_BAD_ENUM;
   if (variant != WAVE_MXFP4_VARIANT_AUTO && variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 &&
       variant != WAVE_MXFP4_VARIANT_T128x128_W2x2)
@@ -379,7 +380,7 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
     p.b_scale = (const uint8_t *)workspace + a_bytes;
     p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
   }
-  return record_hip(launch_tile_gemm_fp8(p, v, elem_format == WAVE_MXFP8_E5M2, stream));
+  return record_hip(launch_tile_gemm_fp8(p, v, a_format == WAVE_MXFP8_E5M2, b_format == WAVE_MXFP8_E5M2, stream));
 }
 
 // Scratch of a grouped call: [M tile table | A scales, one 256-row slab per possible M tile | B scales].

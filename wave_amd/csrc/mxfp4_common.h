@@ -110,7 +110,7 @@ __device__ __host__ __forceinline__ int64_t b_preshuffle_offset(int64_t n, int64
 
 // ---- launchers (defined in the .hip files, called from the C ABI) ----
 hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream);
-hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int e5m2, hipStream_t stream);
+hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_e5m2, hipStream_t stream);
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus);
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream);
 int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *partial_bytes);

@@ -111,8 +111,11 @@ enum TileMode { kDirect = 0, kNative = 1, kGenericK = 2 };
 // scales that are row-major (kDirect) or MFMA32-ordered (kNative: an MFMA32 block
 // covers 8 groups = two MXFP8 K tiles, the odd one's bytes sit in the upper half
 // of the lane's dword).
-template <class Cfg, int MODE, int FMT = 4>
+// FMT is A's format, FMT_B B's (MXFP8 operands may differ: e4m3 activations against e5m2 weights or the other
+// way round, cbsz / blgp 0 / 1 of the instruction).
+template <class Cfg, int MODE, int FMT = 4, int FMT_B = FMT>
 __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
+  static_assert((FMT == 4) == (FMT_B == 4), "MXFP4 x MXFP8 operands are not built");
   constexpr bool GENERIC_K = MODE == kGenericK;
   constexpr bool NATIVE = MODE == kNative;
   constexpr bool FP8 = FMT != 4;
@@ -406,7 +409,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
         if constexpr (FP8) vb = fb[j];
         else vb = v8i{fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
         // first port = B rows (N index), second port = A rows (M index)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][j], FMT, FMT, T,
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][j], FMT_B, FMT, T,
                                                                      (int)sc_b[j], T, (int)sc_a[i]);
       }
     }
@@ -668,9 +671,9 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   }
 }
 
-template <class Cfg, int MODE, int FMT>
+template <class Cfg, int MODE, int FMT, int FMT_B>
 __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams p) {
-  tile_gemm_body<Cfg, MODE, FMT>(p);
+  tile_gemm_body<Cfg, MODE, FMT, FMT_B>(p);
 }
 
 // ---------------------------------------------------------------------------
@@ -689,11 +692,11 @@ void tile_variant_shape(int variant, int *bm, int *bn) {
   }
 }
 
-template <class Cfg, int MODE, int FMT = 4>
+template <class Cfg, int MODE, int FMT = 4, int FMT_B = FMT>
 static hipError_t launch_cfg(const GemmParams &p, hipStream_t stream) {
   static bool attr_done = false;  // benign race: the attribute is idempotent
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)tile_gemm_kernel<Cfg, MODE, FMT>,
+    hipError_t e = hipFuncSetAttribute((const void *)tile_gemm_kernel<Cfg, MODE, FMT, FMT_B>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
@@ -701,7 +704,7 @@ static hipError_t launch_cfg(const GemmParams &p, hipStream_t stream) {
   const int total = p.tiles_m * p.tiles_n;
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
   dim3 grid(per_xcd * kNumXcd, p.splits, 1);
-  tile_gemm_kernel<Cfg, MODE, FMT><<<grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  tile_gemm_kernel<Cfg, MODE, FMT, FMT_B><<<grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
   return hipGetLastError();
 }
 
@@ -729,18 +732,23 @@ hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream
 }
 
 // MXFP8: `p` describes the byte geometry (kp = K bytes per row, ks = K/32, k_tiles = K/128).
-template <class Cfg, int FMT>
+template <class Cfg, int FMT_A, int FMT_B>
 static hipError_t launch_fp8_by_scales(const GemmParams &p, hipStream_t stream) {
   const bool native =
       p.a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
-  return native ? launch_cfg<Cfg, kNative, FMT>(p, stream) : launch_cfg<Cfg, kDirect, FMT>(p, stream);
+  return native ? launch_cfg<Cfg, kNative, FMT_A, FMT_B>(p, stream) : launch_cfg<Cfg, kDirect, FMT_A, FMT_B>(p, stream);
 }
 
-hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int e5m2, hipStream_t stream) {
-  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2)
-    return e5m2 ? launch_fp8_by_scales<Cfg256x256w4, 1>(p, stream) : launch_fp8_by_scales<Cfg256x256w4, 0>(p, stream);
-  if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2)
-    return e5m2 ? launch_fp8_by_scales<Cfg128x128w4, 1>(p, stream) : launch_fp8_by_scales<Cfg128x128w4, 0>(p, stream);
+template <class Cfg>
+static hipError_t launch_fp8_formats(const GemmParams &p, int a_e5m2, int b_e5m2, hipStream_t stream) {
+  if (a_e5m2) return b_e5m2 ? launch_fp8_by_scales<Cfg, 1, 1>(p, stream) : launch_fp8_by_scales<Cfg, 1, 0>(p, stream);
+  return b_e5m2 ? launch_fp8_by_scales<Cfg, 0, 1>(p, stream) : launch_fp8_by_scales<Cfg, 0, 0>(p, stream);
+}
+
+// MXFP8: `p` describes the byte geometry (kp = K bytes per row, ks = K/32, k_tiles = K/128).
+hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_e5m2, hipStream_t stream) {
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_fp8_formats<Cfg256x256w4>(p, a_e5m2, b_e5m2, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2) return launch_fp8_formats<Cfg128x128w4>(p, a_e5m2, b_e5m2, stream);
   return hipErrorInvalidValue;
 }
 

@@ -452,27 +452,29 @@ def silu_and_mul_quantize(gate: torch.Tensor, up: torch.Tensor, *, scale_layout:
 _FP8_FORMATS = {torch.float8_e4m3fn: _lib.MXFP8_E4M3, torch.float8_e5m2: _lib.MXFP8_E5M2}
 
 
-def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format: int | None = None,
+def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
                variant=_lib.VARIANT_AUTO, workspace=None) -> None:
     """``out[M, N] = (x * scales) @ (w_t * scales).T`` for MXFP8 operands:
     ``x [M, K]``, ``w_t [N, K]`` one byte per element, scales ``[R, K/32]`` e8m0
     (tests/kernel/wave_gemm_mxfp_test.py:416-501, which passes
     ``x.view(torch.int8)`` of ``float8_e5m2`` tensors).  float8 tensors carry
-    their format; for uint8 / int8 views pass ``elem_format`` (default e5m2, the
+    their format; for uint8 / int8 views pass ``elem_format``, one value for both
+    operands or a pair ``(x format, w_t format)`` (default e5m2, the
     reference's ``tkl.f8e5m2``).  ``workspace`` as in :func:`mxfp4_gemm`."""
     lib = _lib.load()
-    fmt = elem_format
-    ops = []
-    for name, t in (("x", x), ("w_t", w_t)):
+    given = tuple(elem_format) if isinstance(elem_format, (tuple, list)) else (elem_format, elem_format)
+    if len(given) != 2:
+        raise ValueError("elem_format is one format or a pair (x, w_t)")
+    ops, fmts = [], []
+    for name, t, fmt in (("x", x, given[0]), ("w_t", w_t, given[1])):
         if t.dtype in _FP8_FORMATS:
             if fmt is not None and fmt != _FP8_FORMATS[t.dtype]:
                 raise ValueError(f"{name}: {t.dtype} does not match elem_format {fmt}")
             fmt = _FP8_FORMATS[t.dtype]
             t = t.view(torch.uint8)
         ops.append(_as_u8(t, name))
+        fmts.append(_lib.MXFP8_E5M2 if fmt is None else fmt)
     x, w_t = ops
-    if fmt is None:
-        fmt = _lib.MXFP8_E5M2
     x_scales = _as_u8(x_scales, "x_scales")
     w_scales = _as_u8(w_scales, "w_scales")
     if x.dim() != 2 or w_t.dim() != 2 or x.shape[1] != w_t.shape[1]:
@@ -493,5 +495,6 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format: int | None = Non
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
     with _on_device(x.device):
         st = lib.wave_mxfp8_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
-                                 out.data_ptr(), m, n, k, fmt, od, ws_ptr, ws_bytes, variant, _stream_ptr(x.device))
+                                 out.data_ptr(), m, n, k, fmts[0], fmts[1], od, ws_ptr, ws_bytes, variant,
+                                 _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp8_gemm")

@@ -470,3 +470,17 @@ def test_partial_last_k_tile_preshuffled_b_and_shuffled_scales(m, n, k, vname):
                    a_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_scale_layout=_lib.SCALE_E8M0_SHUFFLE,
                    b_layout=_lib.B_PRESHUFFLE)
     assert np.array_equal(pre, plain)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(1024, 2048, 16000), (1000, 1920, 48 * 256 + 256), (512, 640, 9 * 256),
+                                   (384, 512, 11 * 256 + 64)])
+def test_automatic_split_with_uneven_parts(m, n, k, out_dtype):
+    """Few tiles and a long K whose tile count the split count does not divide (63 K tiles in 2 parts, 9 in 8 ...):
+    the last part is shorter and owns the partial last K tile.  Sampled rows against the oracle."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + k, scale_lo=122, scale_hi=132)
+    rows = np.r_[0:6, m // 2 - 3:m // 2 + 3, m - 6:m]
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    got = run_gemm(x, xs, w_t, ws, out_dtype)
+    assert not np.isnan(got).any()
+    assert_close(got[rows], ref, out_dtype, f"{m}x{n}x{k}")

@@ -68,7 +68,9 @@ void fill_params(GemmParams &p, const void *a, const void *as, const void *b, co
 
 int pick_tile_variant(int64_t m, int64_t n) {
   const int64_t t256 = ((m + 255) / 256) * ((n + 255) / 256);
-  if (t256 >= 128) return WAVE_MXFP4_VARIANT_T256x256_W4x2;  // 8 waves: measured 4-5 % ahead of 4 at 8192^3
+  // 8 waves: measured 4-5 % ahead of 4 at 8192^3.  Up to 128 tiles of 256x256 leave half the CUs idle; the same
+  // problem as up to 512 tiles of 128x128 fills them with two workgroups each (1024 x 8192 x 16384: 87 -> 82 us).
+  if (t256 > 128) return WAVE_MXFP4_VARIANT_T256x256_W4x2;
   return WAVE_MXFP4_VARIANT_T128x128_W2x2;
 }
 
@@ -121,10 +123,13 @@ int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
   if (bm == 0) return 1;
   const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
   const int64_t k_tiles = (k + kTileK - 1) / kTileK;  // a partial last K tile belongs to the last split
-  if (tiles >= 128 || k_tiles < 8) return 1;
+  if (tiles > 128 || k_tiles < 8) return 1;
+  if (tiles > 64 && k_tiles < 48) return 1;  // two splits only pay for a long K (1024 x 2048: K = 16384 44 -> 36 us,
+                                             // K = 8192 no gain)
   int s = (int)(256 / tiles);
   if (s > 8) s = 8;
-  while (s > 1 && (k_tiles % s != 0 || k_tiles / s < 2)) --s;
+  // splits take ceil(k_tiles / s) K tiles each, the last one what is left (at least one)
+  while (s > 1 && (k_tiles / s < 2 || (s - 1) * ((k_tiles + s - 1) / s) >= k_tiles)) --s;
   return s < 1 ? 1 : s;
 }
 
@@ -219,7 +224,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
       splits = auto_split(m, n, k, v);
       const size_t need = (size_t)splits * m * n * sizeof(float);
       if (splits > 1 && (!workspace || workspace_bytes < need)) splits = 1;  // no scratch: no split
-      if (splits > 1) p.tiles_per_split = p.k_tiles / splits;
+      if (splits > 1) p.tiles_per_split = (p.k_tiles + splits - 1) / splits;
     }
   }
   size_t ws_used = 0;

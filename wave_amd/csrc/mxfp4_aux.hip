@@ -214,6 +214,38 @@ __global__ void splitk_reduce_kernel(const float *__restrict__ partial, void *__
   }
 }
 
+// The same, four consecutive elements per thread (16-byte loads of every split in flight together, one 8- or
+// 16-byte store); mn % 4 == 0, c 16-byte aligned.  SPLITS > 0 fixes the count at compile time.
+template <int SPLITS, bool OUT_BF16>
+__global__ void __launch_bounds__(256) splitk_reduce4_kernel(const float *__restrict__ partial, void *__restrict__ c,
+                                                             int64_t mn4, int splits_rt) {
+  const int splits = SPLITS > 0 ? SPLITS : splits_rt;
+  const v4f *src = (const v4f *)partial;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < mn4; i += (int64_t)gridDim.x * blockDim.x) {
+    v4f acc;
+    if constexpr (SPLITS > 0) {
+      v4f part[SPLITS];
+#pragma unroll
+      for (int s = 0; s < SPLITS; ++s) part[s] = __builtin_nontemporal_load(src + (int64_t)s * mn4 + i);
+      acc = part[0];
+#pragma unroll
+      for (int s = 1; s < SPLITS; ++s) acc += part[s];  // the order of the one-element kernel
+    } else {
+      acc = __builtin_nontemporal_load(src + i);
+      for (int s = 1; s < splits; ++s) acc += __builtin_nontemporal_load(src + (int64_t)s * mn4 + i);
+    }
+    if constexpr (OUT_BF16) {
+      typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+      bf4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (__bf16)acc[e];
+      ((bf4 *)c)[i] = o;
+    } else {
+      ((v4f *)c)[i] = acc;
+    }
+  }
+}
+
 // One thread per C element: table decode, f32 multiply-add in K order.  Slow;
 // exists so the MFMA kernels can be checked on the device at any shape.
 __global__ void naive_gemm_kernel(const GemmParams p) {
@@ -354,6 +386,23 @@ hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int
 hipError_t launch_splitk_reduce(const float *partial, void *c, int64_t mn, int splits, int out_bf16,
                                 hipStream_t stream) {
   if (mn == 0) return hipSuccess;
+  if (mn % 4 == 0 && ((uintptr_t)c & 15) == 0 && ((uintptr_t)partial & 15) == 0) {
+    const int64_t mn4 = mn / 4;
+    const unsigned grid = blocks_for(mn4, kThreads);
+#define WAVE_REDUCE4(S)                                                                                    \
+  (out_bf16 ? splitk_reduce4_kernel<S, true><<<grid, kThreads, 0, stream>>>(partial, c, mn4, splits)       \
+            : splitk_reduce4_kernel<S, false><<<grid, kThreads, 0, stream>>>(partial, c, mn4, splits))
+    switch (splits) {
+      case 2: WAVE_REDUCE4(2); break;
+      case 3: WAVE_REDUCE4(3); break;
+      case 4: WAVE_REDUCE4(4); break;
+      case 6: WAVE_REDUCE4(6); break;
+      case 8: WAVE_REDUCE4(8); break;
+      default: WAVE_REDUCE4(0); break;
+    }
+#undef WAVE_REDUCE4
+    return hipGetLastError();
+  }
   splitk_reduce_kernel<<<blocks_for(mn, kThreads), kThreads, 0, stream>>>(partial, c, mn, splits, out_bf16);
   return hipGetLastError();
 }

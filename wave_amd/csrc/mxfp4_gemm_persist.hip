@@ -82,6 +82,20 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   bool tail_on[2];
   const int m_blocks = (p.m + 31) >> 5;
   const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
+  static_assert(!(GROUPED && SPLIT), "the K cut of the last round is for dense problems");
+  // Grouped: the same XCD regrouping as map_tile, but the bands the sequence walks column by column are the
+  // table's (at most 8 tiles of one expert), not fixed runs of 8 tile rows.
+  auto map_grouped = [&](int id, int &tm, int &tn) -> bool {
+    const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
+    const int seq = (id % kNumXcd) * per_xcd + id / kNumXcd;
+    if (seq >= total) return false;
+    const int band = __builtin_amdgcn_readfirstlane(p.tile_table[4 * (1 + seq / p.tiles_n) + 3]);
+    const int start = band >> 4, height = band & 15;
+    const int in_band = seq - start * p.tiles_n;
+    tn = in_band / height;
+    tm = start + in_band - tn * height;
+    return true;
+  };
   auto set_tile = [&](int which, int pid) -> bool {
     int tm, tn, kt_lo = 0;
     nkt_of[which] = nkt;
@@ -98,7 +112,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       kt_lo = i * base + min(i, rem);
       part_of[which] = r * p.tail_parts + i;
       if (!map_tile(pid, tiles_m, p.tiles_n, tm, tn)) return false;
-    } else if (pid >= padded || !map_tile(pid, tiles_m, p.tiles_n, tm, tn)) {
+    } else if (pid >= padded || !(GROUPED ? map_grouped(pid, tm, tn) : map_tile(pid, tiles_m, p.tiles_n, tm, tn))) {
       return false;
     }
     tail_on[which] = TAIL && kt_lo + nkt_of[which] == nkt;

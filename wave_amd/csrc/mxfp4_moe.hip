@@ -142,7 +142,10 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
 }
 
 // M tile table of a grouped GEMM: group e's rows offsets[e] .. offsets[e+1]-1 cut into tiles of bm rows.
-// Entry 0 = {number of tiles}; entry 1 + t = {first row, rows, group, 0}, in group order.
+// Entry 0 = {number of tiles}; entry 1 + t = {first row, rows, group, band}, in group order.
+// band = 16 * (first tile of the tile's band) + (tiles in the band): a group's tiles form bands of at most 8
+// (as equal as possible), the unit inside which the GEMM walks column by column, so that the tiles running
+// together share one expert's B panels.
 __global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const int32_t *__restrict__ offsets,
                                                                            int num_groups, int bm,
                                                                            int32_t *__restrict__ table) {
@@ -160,12 +163,17 @@ __global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const
     }
     const int base = carry;  // read before anyone moves it on
     const int end = block_inclusive_scan(tiles, wave_sums, lane, wave);
+    const int nb = (tiles + 7) >> 3;  // bands of the group: `rem` of height hb + 1, then the rest of height hb
+    const int hb = nb ? tiles / nb : 0, rem = nb ? tiles - hb * nb : 0;
+    const int first_tile = base + end - tiles;
     for (int i = 0; i < tiles; ++i) {
-      int32_t *ent = table + 4 * (1 + base + end - tiles + i);
+      int32_t *ent = table + 4 * (1 + first_tile + i);
       ent[0] = lo + i * bm;
       ent[1] = min(bm, hi - lo - i * bm);
       ent[2] = e;
-      ent[3] = 0;
+      const int tall = rem * (hb + 1);
+      const int start = i < tall ? i / (hb + 1) * (hb + 1) : tall + (i - tall) / hb * hb;
+      ent[3] = 16 * (first_tile + start) + (i < tall ? hb + 1 : hb);
     }
     __syncthreads();
     if (t == kAlignThreads - 1) carry = base + end;

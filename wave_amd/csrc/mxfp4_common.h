@@ -110,6 +110,24 @@ __device__ __host__ __forceinline__ int64_t b_preshuffle_offset(int64_t n, int64
 
 // ---- launchers (defined in the .hip files, called from the C ABI) ----
 hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream);
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) once per kernel and device: the attribute belongs to the
+// device's copy of the kernel.  `once` is a static of the calling launcher (one per kernel instantiation); two
+// threads that both find it unset both set the attribute, which is idempotent.
+constexpr int kMaxDevices = 64;
+struct LdsAttrOnce {
+  bool done[kMaxDevices] = {};
+};
+inline hipError_t allow_dynamic_lds(LdsAttrOnce &once, const void *kernel, int bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  if (tracked && once.done[dev]) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && tracked) once.done[dev] = true;
+  return e;
+}
+
 hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_e5m2, hipStream_t stream);
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus);
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream);

@@ -518,16 +518,13 @@ __global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams 
 
 template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
 static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_t stream) {
-  static bool attr_done = false;  // benign race: the attribute is idempotent
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    attr_done = true;
-  }
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, (const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>,
+                                   Cfg::LDS_BYTES);
+  if (e != hipSuccess) return e;
   persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>
       <<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
-  hipError_t e = hipGetLastError();
+  e = hipGetLastError();
   if (SPLIT && e == hipSuccess) {
     const int total = p.tiles_m * p.tiles_n;
     const int ids = (total + kNumXcd - 1) / kNumXcd * kNumXcd - total / grid_x * grid_x;  // tile ids of the last round

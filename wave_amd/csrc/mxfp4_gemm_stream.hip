@@ -595,13 +595,9 @@ __global__ void __launch_bounds__(kStreamWaves * 64, 1) stream_gemm_kernel(const
 
 template <int MT_M, bool FULL, int KW>
 static hipError_t launch_stream_mt(const GemmParams &p, int grid_x, hipStream_t stream) {
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)stream_gemm_kernel<MT_M, FULL, KW>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(StreamLds));
-    if (e != hipSuccess) return e;
-    attr_done = true;
-  }
+  static LdsAttrOnce once;
+  const hipError_t e = allow_dynamic_lds(once, (const void *)stream_gemm_kernel<MT_M, FULL, KW>, (int)sizeof(StreamLds));
+  if (e != hipSuccess) return e;
   dim3 grid(grid_x, p.splits, 1);
   stream_gemm_kernel<MT_M, FULL, KW><<<grid, dim3(kStreamWaves * 64), sizeof(StreamLds), stream>>>(p);
   return hipGetLastError();

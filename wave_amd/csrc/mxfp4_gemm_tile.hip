@@ -694,13 +694,9 @@ void tile_variant_shape(int variant, int *bm, int *bn) {
 
 template <class Cfg, int MODE, int FMT = 4, int FMT_B = FMT>
 static hipError_t launch_cfg(const GemmParams &p, hipStream_t stream) {
-  static bool attr_done = false;  // benign race: the attribute is idempotent
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)tile_gemm_kernel<Cfg, MODE, FMT, FMT_B>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    attr_done = true;
-  }
+  static LdsAttrOnce once;
+  const hipError_t e = allow_dynamic_lds(once, (const void *)tile_gemm_kernel<Cfg, MODE, FMT, FMT_B>, Cfg::LDS_BYTES);
+  if (e != hipSuccess) return e;
   const int total = p.tiles_m * p.tiles_n;
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
   dim3 grid(per_xcd * kNumXcd, p.splits, 1);

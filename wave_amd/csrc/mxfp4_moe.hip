@@ -193,14 +193,11 @@ hipError_t launch_moe_align(const void *topk_ids, int ids_int64, int64_t n, int 
                             int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids, int64_t expert_ids_len,
                             int32_t *total, int32_t *offsets, hipStream_t stream) {
   const size_t lds = (size_t)(kAlignWaves * num_experts + kAlignWaves + num_experts + 1) * sizeof(int);
-  static bool attr_done[2] = {false, false};
+  static LdsAttrOnce once[2];
   const void *fn = ids_int64 ? (const void *)moe_align_kernel<int64_t> : (const void *)moe_align_kernel<int32_t>;
-  if (!attr_done[ids_int64 ? 1 : 0]) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)((kAlignWaves * kMoeMaxExperts + kAlignWaves + kMoeMaxExperts + 1) * sizeof(int)));
-    if (e != hipSuccess) return e;
-    attr_done[ids_int64 ? 1 : 0] = true;
-  }
+  const hipError_t e = allow_dynamic_lds(
+      once[ids_int64 ? 1 : 0], fn, (int)((kAlignWaves * kMoeMaxExperts + kAlignWaves + kMoeMaxExperts + 1) * sizeof(int)));
+  if (e != hipSuccess) return e;
   if (ids_int64)
     moe_align_kernel<int64_t><<<1, kAlignThreads, lds, stream>>>((const int64_t *)topk_ids, (int)n, num_experts, block_size,
                                                                  sorted_ids, (int)sorted_len, expert_ids,

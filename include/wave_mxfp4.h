@@ -87,6 +87,7 @@ typedef enum {
   WAVE_MXFP4_VARIANT_T128x128_W2x2 = 3, /* 128x128x256 tile, 4 waves */
   WAVE_MXFP4_VARIANT_SKINNY = 4,        /* M <= 64 streaming kernel */
   WAVE_MXFP4_VARIANT_NAIVE = 5,         /* one thread per C element, for cross-checks */
+  WAVE_MXFP4_VARIANT_T128x256_W2x2 = 6, /* 128x256x256 tile, 4 waves */
   WAVE_MXFP4_VARIANT_COUNT_
 } wave_mxfp4_variant;
 

@@ -71,4 +71,5 @@ TILE_VARIANTS = {
     "t256x256_w2x2": _lib.VARIANT_T256x256_W2x2,
     "t256x256_w4x2": _lib.VARIANT_T256x256_W4x2,
     "t128x128_w2x2": _lib.VARIANT_T128x128_W2x2,
+    "t128x256_w2x2": _lib.VARIANT_T128x256_W2x2,
 }

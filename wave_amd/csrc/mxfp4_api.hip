@@ -71,6 +71,10 @@ int pick_tile_variant(int64_t m, int64_t n) {
   // 8 waves: measured 4-5 % ahead of 4 at 8192^3.  Up to 128 tiles of 256x256 leave half the CUs idle; the same
   // problem as up to 512 tiles of 128x128 fills them with two workgroups each (1024 x 8192 x 16384: 87 -> 82 us).
   if (t256 > 128) return WAVE_MXFP4_VARIANT_T256x256_W4x2;
+  // 129..256 tiles of 128x256: one workgroup per CU on at least half of them, at nearly twice the MFMA duty of
+  // the 128x128 kernel (1024 x 5120 x 16000: 72 -> 60 us; 1024 x 8192: 80 -> 76 us)
+  const int64_t t128x256 = ((m + 127) / 128) * ((n + 255) / 256);
+  if (t128x256 > 128 && t128x256 <= 256) return WAVE_MXFP4_VARIANT_T128x256_W2x2;
   return WAVE_MXFP4_VARIANT_T128x128_W2x2;
 }
 

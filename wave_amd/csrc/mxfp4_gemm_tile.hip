@@ -682,12 +682,14 @@ __global__ void __launch_bounds__(Cfg::NT, 1) tile_gemm_kernel(const GemmParams 
 typedef TileCfg<256, 256, 2, 2> Cfg256x256w4;
 typedef TileCfg<256, 256, 4, 2> Cfg256x256w8;
 typedef TileCfg<128, 128, 2, 2> Cfg128x128w4;
+typedef TileCfg<128, 256, 2, 2> Cfg128x256w4;
 
 void tile_variant_shape(int variant, int *bm, int *bn) {
   switch (variant) {
     case WAVE_MXFP4_VARIANT_T256x256_W2x2:
     case WAVE_MXFP4_VARIANT_T256x256_W4x2: *bm = 256; *bn = 256; break;
     case WAVE_MXFP4_VARIANT_T128x128_W2x2: *bm = 128; *bn = 128; break;
+    case WAVE_MXFP4_VARIANT_T128x256_W2x2: *bm = 128; *bn = 256; break;
     default: *bm = 0; *bn = 0; break;
   }
 }
@@ -723,6 +725,7 @@ hipError_t launch_tile_gemm(const GemmParams &p, int variant, hipStream_t stream
     case WAVE_MXFP4_VARIANT_T256x256_W2x2: return launch_by_scales<Cfg256x256w4>(p, stream);
     case WAVE_MXFP4_VARIANT_T256x256_W4x2: return launch_by_scales<Cfg256x256w8>(p, stream);
     case WAVE_MXFP4_VARIANT_T128x128_W2x2: return launch_by_scales<Cfg128x128w4>(p, stream);
+    case WAVE_MXFP4_VARIANT_T128x256_W2x2: return launch_by_scales<Cfg128x256w4>(p, stream);
     default: return hipErrorInvalidValue;
   }
 }

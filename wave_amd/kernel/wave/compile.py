@@ -52,6 +52,7 @@ _TILE_VARIANTS = {
     ((256, 256), (2, 2)): _lib.VARIANT_T256x256_W2x2,
     ((256, 256), (4, 2)): _lib.VARIANT_T256x256_W4x2,
     ((128, 128), (2, 2)): _lib.VARIANT_T128x128_W2x2,
+    ((128, 256), (2, 2)): _lib.VARIANT_T128x256_W2x2,
 }
 
 

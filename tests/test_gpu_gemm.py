@@ -484,3 +484,17 @@ def test_automatic_split_with_uneven_parts(m, n, k, out_dtype):
     got = run_gemm(x, xs, w_t, ws, out_dtype)
     assert not np.isnan(got).any()
     assert_close(got[rows], ref, out_dtype, f"{m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("k_tiles", [1, 2, 7, 16, 17])
+def test_row_major_scales_without_scratch_short_and_long_k(k_tiles):
+    """Without scratch the 128x128 kernel copies the row-major scale rows of its tile into LDS when the workgroup
+    has at most 16 K tiles and reads them from global memory per K tile otherwise; ragged M and N (rows past the
+    tensors are clamped), odd K tile counts (the LDS row pitch depends on their parity)."""
+    m, n, k = 300, 250, 256 * k_tiles
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=k_tiles, scale_lo=110, scale_hi=140)
+    xs[5, 0] = 255
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    got = run_gemm(x, xs, w_t, ws, torch.float32, variant=_lib.VARIANT_T128x128_W2x2, workspace=False)
+    assert np.isnan(got[5]).all() and not np.isnan(np.delete(got, 5, 0)).any()
+    assert_f32_close(np.delete(got, 5, 0), np.delete(ref, 5, 0), f"{k_tiles} K tiles")

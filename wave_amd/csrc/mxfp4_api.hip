@@ -128,8 +128,23 @@ int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
   const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
   const int64_t k_tiles = (k + kTileK - 1) / kTileK;  // a partial last K tile belongs to the last split
   if (tiles > 128 || k_tiles < 8) return 1;
-  if (tiles > 64 && k_tiles < 48) return 1;  // two splits only pay for a long K (1024 x 2048: K = 16384 44 -> 36 us,
-                                             // K = 8192 no gain)
+  if (bm == 128 && bn == 128) {
+    // Estimate in us, fixed launch time left out: a workgroup's K tiles at the measured 0.52 us each while every
+    // CU holds at most one workgroup (1.28 us for the two of a CU beyond that), plus, for a split, the launch that
+    // sums the parts and their f32 traffic.  (1024 x 1024: K = 2048 stays whole, K = 8192 and 16384 take 4 parts.)
+    int best = 1;
+    double best_us = 0.52 * (double)k_tiles;
+    for (int s = 2; s <= 8; ++s) {
+      const int64_t per = (k_tiles + s - 1) / s;
+      if (k_tiles / s < 2 || (s - 1) * per >= k_tiles) continue;  // every part at least one K tile, most two
+      const int64_t wgs = tiles * s;
+      const double step = wgs <= 256 ? 0.52 : 1.28 * (double)((wgs + 511) / 512);
+      const double us = step * (double)per + 3.5 + (double)s * (double)m * (double)n * 4.0 / 8.0e6;
+      if (us < 0.9 * best_us) best = s, best_us = us;
+    }
+    return best;
+  }
+  if (tiles > 64 && k_tiles < 48) return 1;  // two splits only pay for a long K
   int s = (int)(256 / tiles);
   if (s > 8) s = 8;
   // splits take ceil(k_tiles / s) K tiles each, the last one what is left (at least one)
@@ -258,8 +273,11 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   // cache line per wave instruction; row-major scales cost 32 lines per
   // instruction.  With scratch available, re-lay both operands out first
   // (a few MB, microseconds) and run the native-scale kernel.
-  // (Not worth a second launch for a small problem with short K: there the direct reads cost less.)
-  const bool small_short = p.tiles_per_split <= 8 && (int64_t)m * n <= (int64_t)2048 * 2048 && k % kTileK == 0;
+  // (Not worth a second launch for a short K range on the 128x128 tiles: there the kernel stages the row-major
+  // scale rows of its tile through LDS itself, 0.1-0.2 us per K tile slower than with re-laid scales: break-even
+  // measured near 13 K tiles.)
+  const bool small_short = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 && p.tiles_per_split <= 12 && k % kTileK == 0 &&
+                           p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
   if (is_tile_variant(v) && workspace && !small_short) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
     const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? a_bytes : 0;

@@ -1,0 +1,55 @@
+"""Seeded random shapes, layouts, split counts and scratch on/off through the library's own choice of kernel,
+against the exact oracle: the dispatch rules (tile shape by tile count, automatic and explicit splits with uneven
+parts, scale staging, streaming kernel) are exercised at shapes nobody picked by hand."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import mxfp4_oracle as orc
+from wave_amd import _lib
+
+from gpu_util import assert_close, run_gemm
+
+pytestmark = pytest.mark.gpu
+
+
+def _cases(count, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        kind = rng.integers(0, 4)
+        if kind == 0:    # decode-like
+            m, n, k = int(rng.integers(1, 65)), int(rng.integers(1, 3000)), 32 * int(rng.integers(1, 160))
+        elif kind == 1:  # small and ragged
+            m, n, k = int(rng.integers(1, 400)), int(rng.integers(1, 400)), 32 * int(rng.integers(1, 64))
+        elif kind == 2:  # few tiles, long K (automatic split)
+            m, n, k = int(rng.integers(65, 700)), int(rng.integers(100, 700)), 256 * int(rng.integers(8, 40))
+        else:            # many tiles, short K
+            m, n, k = int(rng.integers(500, 2200)), int(rng.integers(500, 2200)), 32 * int(rng.integers(4, 24))
+        out.append((i, m, n, k, int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2)),
+                    bool(rng.integers(0, 2)), bool(rng.integers(0, 4) > 0)))
+    return out
+
+
+@pytest.mark.parametrize("case", _cases(48, seed=20), ids=lambda c: f"{c[0]}-{c[1]}x{c[2]}x{c[3]}")
+def test_random_shape_against_oracle(case):
+    i, m, n, k, a_layout, b_layout, preshuffle, bf16, scratch = case
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=1000 + i, scale_lo=118, scale_hi=136)
+    rows = np.unique(np.r_[0:min(m, 4), m // 2, max(0, m - 3):m])
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    layouts = [_lib.SCALE_ROW_MAJOR, _lib.SCALE_E8M0_SHUFFLE, _lib.SCALE_MFMA32]
+    conv = {_lib.SCALE_ROW_MAJOR: lambda s: s, _lib.SCALE_E8M0_SHUFFLE: orc.e8m0_shuffle_padded,
+            _lib.SCALE_MFMA32: orc.mfma32_scale_layout}
+    kw = dict(a_scale_layout=layouts[a_layout], b_scale_layout=layouts[b_layout])
+    if preshuffle and n % 16 == 0 and k % 64 == 0:
+        w_in, kw["b_layout"] = orc.b_preshuffle(w_t), _lib.B_PRESHUFFLE
+    else:
+        w_in = w_t
+    if not scratch:
+        kw["workspace"] = False
+    out_dtype = torch.bfloat16 if bf16 else torch.float32
+    got = run_gemm(x, conv[layouts[a_layout]](xs), w_in, conv[layouts[b_layout]](ws), out_dtype, **kw)
+    assert not np.isnan(got).any()
+    assert_close(got[rows], ref, out_dtype, f"case {case}")

@@ -1,0 +1,56 @@
+"""The library's launches under HIP graph capture: every entry point takes its scratch from the caller and
+enqueues kernels only (no allocation, no memset node, no synchronisation), so a captured sequence replays with the
+eager results, bit for bit, also with eager work of the program between the replays."""
+
+import numpy as np
+import pytest
+import torch
+
+import wave_amd
+from oracle import mxfp4_oracle as orc
+from wave_amd import _lib
+
+from gpu_util import DEV, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+
+def test_captured_gemm_sequence_replays_with_eager_results():
+    shapes = [(1024, 1024, 8192), (16, 4096, 4096), (512, 768, 16384), (300, 200, 1248), (2304, 2304, 1024)]
+    ops = []
+    for i, (m, n, k) in enumerate(shapes):
+        x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=40 + i, scale_lo=120, scale_hi=134)
+        ops.append(to_gpu(x, xs, w_t, ws) + (torch.empty(m, n, dtype=torch.bfloat16 if i % 2 else torch.float32, device=DEV),))
+    act = torch.randn(512, 4096, device=DEV, dtype=torch.bfloat16)
+
+    def sequence():
+        for gx, gxs, gw, gws, out in ops:
+            wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out)
+        return wave_amd.quantize_mxfp4(act, scale_layout=_lib.SCALE_MFMA32)
+
+    q_eager, s_eager = sequence()  # also sizes the cached scratch buffers, so nothing is allocated under capture
+    torch.cuda.synchronize()
+    eager = [o[4].clone() for o in ops]
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        sequence()  # warm-up on the capture stream
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            q_graph, s_graph = sequence()
+    torch.cuda.current_stream().wait_stream(stream)
+    for replay in range(3):
+        for o in ops:
+            o[4].fill_(float("nan"))
+        q_graph.zero_()
+        s_graph.zero_()
+        # eager work of the program between the replays, on the same scratch
+        wave_amd.mxfp4_gemm(*ops[(replay + 1) % len(ops)][:4], torch.empty_like(ops[(replay + 1) % len(ops)][4]))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for want, o in zip(eager, ops):
+            assert torch.equal(want, o[4]), f"replay {replay}: {tuple(want.shape)}"
+        assert torch.equal(q_graph, q_eager) and torch.equal(s_graph, s_eager)

@@ -11,7 +11,7 @@ import torch
 import wave_amd.kernel.lang as tkl
 from oracle.torch_oracle import torch_scaled_gemm_mxfp4
 from wave_amd.kernel.lang import TORCH_DTYPE_TO_WAVE
-from wave_amd.kernel.wave.compile import wave_compile
+from wave_amd.kernel.wave.compile import WaveCompileOptions, wave_compile
 from wave_amd.kernel.wave.constraints import ScaledMMAType
 from wave_amd.kernel.wave.schedules import (
     get_mxfp4_asymmetric_schedule,
@@ -169,6 +169,22 @@ def testBroadcastedScaleGemmMXFP4(shape):
     broadcasted_compacted_x_scales = compacted_x_scales.view(-1, 1).repeat(1, x_scales.shape[-1]).contiguous()
     torch_out = torchScaledGemmMXFP4(x, w, broadcasted_compacted_x_scales, w_scales)
     torch.testing.assert_close(torch_out, out.cpu(), check_dtype=False)
+
+
+def test_scaled_gemm_kernel_template():
+    """tests/kernel/wave/water_e2e_test.py:172-230: the plain template of templates/gemm.py, compiled from its
+    hyperparameters and checked against the torch dequant + matmul."""
+    from wave_amd.kernel.wave.templates.gemm import get_scaled_gemm_kernel
+
+    shape = (1024, 1024, 1024)
+    scaled_gemm, hyperparams = get_scaled_gemm_kernel(shape=shape, mfma_variant=ScaledMMAType.F32_16x16x128_F8F6F4)
+    options = WaveCompileOptions(subs=hyperparams, canonicalize=True)
+    compiled = wave_compile(options, scaled_gemm)
+    x, w, x_scales, w_scales = generate_gemm_afp4wfp4_inputs(shape, device=DEV)
+    out = torch.zeros(shape[0], shape[1], dtype=torch.float32, device=DEV)
+    compiled(x, x_scales, w.T.contiguous(), w_scales, out)
+    expected = torchScaledGemmMXFP4(x, w, x_scales, w_scales)
+    torch.testing.assert_close(out.cpu(), expected, rtol=1e-3, atol=1e-3, check_dtype=False)
 
 
 @pytest.mark.parametrize("batch", [4, 8])

@@ -148,7 +148,7 @@ typedef enum { WAVE_MXFP8_E4M3 = 0, WAVE_MXFP8_E5M2 = 1 } wave_mxfp8_format;
  * blgp 0 / 1 of the instruction), scales [R, K/32] e8m0 row-major, C f32 or
  * bf16.  Replaces the kernel of tests/kernel/wave_gemm_mxfp_test.py:416-501
  * (tkl.f8e5m2 operands through the same scaled MFMA).  K % 128 == 0; variant
- * AUTO, T256x256_W2x2 or T128x128_W2x2.  `workspace` is optional scratch of
+ * AUTO, T256x256_W2x2, T256x256_W4x2 or T128x128_W2x2.  `workspace` is optional scratch of
  * wave_mxfp8_workspace_bytes(m, n, k) bytes (256-byte aligned): with it, and
  * K % 256 == 0, the scales are first re-laid out for one-dword-per-lane reads. */
 int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,

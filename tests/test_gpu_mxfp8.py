@@ -30,7 +30,8 @@ def assert_f32_close(c, ref, what=""):
     assert err <= 1e-4 * scale, f"{what}: max err {err:g} > 1e-4 * {scale:g}"
 
 
-VARIANTS = {"auto": _lib.VARIANT_AUTO, "t256": _lib.VARIANT_T256x256_W2x2, "t128": _lib.VARIANT_T128x128_W2x2}
+VARIANTS = {"auto": _lib.VARIANT_AUTO, "t256": _lib.VARIANT_T256x256_W2x2, "t256w8": _lib.VARIANT_T256x256_W4x2,
+            "t128": _lib.VARIANT_T128x128_W2x2}
 
 
 def run(x, xs, w_t, ws, fmt, out_dtype=torch.float32, variant=_lib.VARIANT_AUTO):

@@ -364,7 +364,7 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
       bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
     return WAVE_MXFP4_ERR_BAD_ENUM;
   if (variant != WAVE_MXFP4_VARIANT_AUTO && variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 &&
-      variant != WAVE_MXFP4_VARIANT_T128x128_W2x2)
+      variant != WAVE_MXFP4_VARIANT_T256x256_W4x2 && variant != WAVE_MXFP4_VARIANT_T128x128_W2x2)
     return WAVE_MXFP4_ERR_UNSUPPORTED;
   if (m == 0 || n == 0) return WAVE_MXFP4_OK;
   if (!c) return WAVE_MXFP4_ERR_NULL_POINTER;
@@ -393,7 +393,8 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   }
   int v = variant;
   if (v == WAVE_MXFP4_VARIANT_AUTO)
-    v = ((m + 255) / 256) * ((n + 255) / 256) >= 128 ? WAVE_MXFP4_VARIANT_T256x256_W2x2 : WAVE_MXFP4_VARIANT_T128x128_W2x2;
+    v = ((m + 255) / 256) * ((n + 255) / 256) >= 128 ? WAVE_MXFP4_VARIANT_T256x256_W4x2  // 8 waves: 498 -> 476 us at 8192^3
+                                                     : WAVE_MXFP4_VARIANT_T128x128_W2x2;
   int bm, bn;
   tile_variant_shape(v, &bm, &bn);
   p.tiles_m = (int)((m + bm - 1) / bm);

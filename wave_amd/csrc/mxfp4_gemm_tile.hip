@@ -821,6 +821,7 @@ static hipError_t launch_fp8_formats(const GemmParams &p, int a_e5m2, int b_e5m2
 // MXFP8: `p` describes the byte geometry (kp = K bytes per row, ks = K/32, k_tiles = K/128).
 hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_e5m2, hipStream_t stream) {
   if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_fp8_formats<Cfg256x256w4>(p, a_e5m2, b_e5m2, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W4x2) return launch_fp8_formats<Cfg256x256w8>(p, a_e5m2, b_e5m2, stream);
   if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2) return launch_fp8_formats<Cfg128x128w4>(p, a_e5m2, b_e5m2, stream);
   return hipErrorInvalidValue;
 }

@@ -182,7 +182,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this operator runs on one GPU; --gpus N with N > 1 is not supported "
-              "(the path shards by N or M with no exchange, see DESIGN.md)", file=sys.stderr)
+              "(the operator shards over GPUs by splitting N or M, with no exchange between them)", file=sys.stderr)
         sys.exit(2)
 
     import torch

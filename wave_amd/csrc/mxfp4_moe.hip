@@ -12,6 +12,7 @@ namespace {
 
 constexpr int kAlignWaves = 16;
 constexpr int kAlignThreads = kAlignWaves * 64;
+constexpr int kFewExperts = 16;
 
 // Inclusive sum over the workgroup's 1024 threads (one value each).
 __device__ __forceinline__ int block_inclusive_scan(int v, int *wave_sums, int lane, int wave) {
@@ -39,6 +40,7 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
                                                  // the next free position for them
   int *wave_sums = lds + kAlignWaves * num_experts;  // [kAlignWaves]
   int *starts = wave_sums + kAlignWaves;             // [E + 1]: first position of every expert's run, then the total
+  int *counts = starts + num_experts + 1;            // [E]: entries of every expert
   const int E = num_experts;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
 
@@ -77,8 +79,8 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
       cnt[w * E + t] = run;
       run += c;
     }
-    for (int i = start + count; i < min(end, sorted_len); ++i) sorted_ids[i] = n;  // the run's padding (< block_size)
     starts[t] = start;
+    counts[t] = count;
     if (offsets_out) offsets_out[t] = start;
   }
   if (t == kAlignThreads - 1) starts[E] = end;
@@ -89,6 +91,11 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
     if (offsets_out) offsets_out[E] = total;
   }
   for (int i = total + t; i < sorted_len; i += kAlignThreads) sorted_ids[i] = n;  // past the padded total
+  // every run's padding (fewer than block_size entries): one wave per expert, a lane per entry
+  for (int e = wave; e < E; e += kAlignWaves) {
+    const int from = starts[e] + counts[e], to = min(starts[e + 1], sorted_len);
+    for (int i = from + lane; i < to; i += 64) sorted_ids[i] = n;
+  }
   // the expert of every block, all threads together: the last expert whose run starts at or before the block
   for (int b = t; b < min(total / block_size, expert_ids_len); b += kAlignThreads) {
     const int pos = b * block_size;
@@ -119,6 +126,21 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
       const int i = base8 + s * 64 + lane;
       const bool valid = e8[s] >= 0 && e8[s] < E;
       const int e = valid ? (int)e8[s] : -1;
+      if (E <= kFewExperts) {
+        // few experts: one ballot per expert, no search for the experts that occur
+        int pos = -1;
+#pragma unroll
+        for (int x = 0; x < kFewExperts; ++x) {
+          if (x < E) {
+            const uint64_t same = __ballot(e == x);
+            const int first = __builtin_amdgcn_readlane(next_reg, x);
+            if (e == x) pos = first + __popcll(same & ((1ull << lane) - 1));
+            if (lane == x) next_reg += __popcll(same);
+          }
+        }
+        if (pos >= 0 && pos < sorted_len) sorted_ids[pos] = i;
+        continue;
+      }
       uint64_t todo = __ballot(valid);
       while (todo) {
         const int leader = __ffsll((unsigned long long)todo) - 1;
@@ -192,11 +214,11 @@ hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int
 hipError_t launch_moe_align(const void *topk_ids, int ids_int64, int64_t n, int num_experts, int block_size,
                             int32_t *sorted_ids, int64_t sorted_len, int32_t *expert_ids, int64_t expert_ids_len,
                             int32_t *total, int32_t *offsets, hipStream_t stream) {
-  const size_t lds = (size_t)(kAlignWaves * num_experts + kAlignWaves + num_experts + 1) * sizeof(int);
+  const size_t lds = (size_t)(kAlignWaves * num_experts + kAlignWaves + 2 * num_experts + 1) * sizeof(int);
   static LdsAttrOnce once[2];
   const void *fn = ids_int64 ? (const void *)moe_align_kernel<int64_t> : (const void *)moe_align_kernel<int32_t>;
   const hipError_t e = allow_dynamic_lds(
-      once[ids_int64 ? 1 : 0], fn, (int)((kAlignWaves * kMoeMaxExperts + kAlignWaves + kMoeMaxExperts + 1) * sizeof(int)));
+      once[ids_int64 ? 1 : 0], fn, (int)((kAlignWaves * kMoeMaxExperts + kAlignWaves + 2 * kMoeMaxExperts + 1) * sizeof(int)));
   if (e != hipSuccess) return e;
   if (ids_int64)
     moe_align_kernel<int64_t><<<1, kAlignThreads, lds, stream>>>((const int64_t *)topk_ids, (int)n, num_experts, block_size,

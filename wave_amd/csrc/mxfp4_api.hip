@@ -274,9 +274,11 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   // instruction.  With scratch available, re-lay both operands out first
   // (a few MB, microseconds) and run the native-scale kernel.
   // (Not worth a second launch for a short K range on the 128x128 tiles: there the kernel stages the row-major
-  // scale rows of its tile through LDS itself, 0.1-0.2 us per K tile slower than with re-laid scales: break-even
-  // measured near 13 K tiles.)
-  const bool small_short = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 && p.tiles_per_split <= 12 && k % kTileK == 0 &&
+  // scale rows of its tile through LDS itself, 0.1-0.2 us per K tile slower than with re-laid scales: with a split,
+  // whose parts are summed by a launch of their own anyway, the break-even was measured near 13 K tiles; without,
+  // 16 K tiles - all the kernel stages - still win: 1024 x 1024 x 4096 12.3 against 16.3 us.)
+  const bool small_short = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 && p.tiles_per_split <= (splits > 1 ? 12 : 16) &&
+                           k % kTileK == 0 &&
                            p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
   if (is_tile_variant(v) && workspace && !small_short) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));

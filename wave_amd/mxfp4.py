@@ -85,6 +85,8 @@ def workspace_bytes(m: int, n: int, k: int, split_k: int = 0, variant: int = _li
 # sums and the re-laid-out scales of a call live there.  Calls on one stream are
 # ordered, so they can share it; different streams get different buffers.
 _scratch: dict = {}
+# signatures of mxfp4_gemm calls that passed every check: -> (m, n, k, out dtype code, a scale layout, scratch bytes)
+_checked: dict = {}
 
 
 def _workspace(device, nbytes: int):
@@ -116,6 +118,30 @@ def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW
     * one scale per row of A, ``x_scales [M]``, held for the whole row
       (wave_lang/kernel/wave/templates/test_kernels.py:75-135)."""
     lib = _lib.load()
+    # A call whose shapes, types, device and options were checked before skips the checks (they cost more host
+    # time than the launch of a small problem): contiguity is the one property a tensor of the same shape can lose.
+    key = (x.shape, x_scales.shape, w_t.shape, w_scales.shape, out.shape, x.dtype, x_scales.dtype, w_t.dtype,
+           w_scales.dtype, out.dtype, x.device, w_t.device, out.device, a_scale_layout, b_scale_layout, b_layout,
+           split_k, variant)
+    plan = _checked.get(key)
+    if (plan is not None and workspace is None and x.is_contiguous() and x_scales.is_contiguous()
+            and w_t.is_contiguous() and w_scales.is_contiguous() and out.is_contiguous()
+            and x_scales.device == x.device and w_scales.device == x.device):
+        m, n, k, od, asl, nbytes = plan
+        device = x.device
+        stream = torch.cuda.current_stream(device).cuda_stream
+        ws_ptr = None
+        if nbytes:
+            buf = _scratch.get((device, stream))
+            if buf is None or buf.numel() < nbytes:
+                buf = _workspace(device, nbytes)
+            ws_ptr = buf.data_ptr()
+        with _on_device(device):
+            st = lib.wave_mxfp4_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
+                                     out.data_ptr(), m, n, k, od, asl, b_scale_layout, b_layout, split_k, ws_ptr,
+                                     nbytes if ws_ptr is not None else 0, variant, stream)
+        _lib.check(st, "wave_mxfp4_gemm")
+        return
     x = _as_u8(x, "x")
     w_t = _as_u8(w_t, "w_t")
     x_scales = _as_u8(x_scales, "x_scales")
@@ -147,17 +173,24 @@ def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW
     _scale_rows_ok(w_scales, n, ks, b_scale_layout, "w_scales")
     od = _check_out(out, (m, n))
     ws_ptr, ws_bytes = None, 0
+    default_scratch = workspace is None
     if workspace is None:
         workspace = _workspace(x.device, workspace_bytes(m, n, k, split_k, variant))
     elif workspace is False:  # run without scratch: scales are read in the layout given
         workspace = None
     if workspace is not None:
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    if w_t.device != x.device or out.device != x.device or x_scales.device != x.device or w_scales.device != x.device:
+        raise ValueError("all tensors must be on the same device")
     with _on_device(x.device):
         st = lib.wave_mxfp4_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
                                  out.data_ptr(), m, n, k, od, a_scale_layout, b_scale_layout, b_layout,
                                  split_k, ws_ptr, ws_bytes, variant, _stream_ptr(x.device))
     _lib.check(st, "wave_mxfp4_gemm")
+    if default_scratch:  # remember the checked signature (as given by the caller: before any reshaping above)
+        if len(_checked) > 4096:
+            _checked.clear()
+        _checked[key] = (m, n, k, od, a_scale_layout, workspace_bytes(m, n, k, split_k, variant))
 
 
 def mxfp4_gemm_grouped(x, x_scales, w_t, w_scales, offsets, out, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,

@@ -498,3 +498,30 @@ def test_row_major_scales_without_scratch_short_and_long_k(k_tiles):
     got = run_gemm(x, xs, w_t, ws, torch.float32, variant=_lib.VARIANT_T128x128_W2x2, workspace=False)
     assert np.isnan(got[5]).all() and not np.isnan(np.delete(got, 5, 0)).any()
     assert_f32_close(np.delete(got, 5, 0), np.delete(ref, 5, 0), f"{k_tiles} K tiles")
+
+
+def test_repeated_calls_with_one_signature():
+    """The wrapper checks a signature (shapes, types, device, options) once and then only contiguity: later calls
+    with new contents, a non-contiguous operand of the same shape, and other options on the same tensors must all
+    give their own right answers."""
+    m, n, k = 300, 260, 1024
+    outs = []
+    for seed in (1, 2, 3):
+        x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=seed, scale_lo=120, scale_hi=134)
+        ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+        assert_f32_close(run_gemm(x, xs, w_t, ws, torch.float32), ref, f"seed {seed}")
+        outs.append(ref)
+    assert not np.array_equal(outs[0], outs[1])
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    wide = torch.zeros(n, k, dtype=torch.uint8, device=DEV)
+    wide[:, ::2] = gw
+    out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm(gx, gxs, wide[:, ::2], gws, out)          # same shape, strided: copied, not misread
+    assert_f32_close(out.cpu().numpy(), ref, "strided w_t")
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, out, split_k=2)          # same tensors, another option
+    assert_f32_close(out.cpu().numpy(), ref, "split_k=2")
+    bf = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, bf)                      # same shapes, another output type
+    assert_bf16_close(bf.float().cpu().numpy(), ref, "bf16 out")
+    with pytest.raises(ValueError):
+        wave_amd.mxfp4_gemm(gx, gxs, gw, gws, torch.empty(m, n, dtype=torch.float16, device=DEV))

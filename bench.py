@@ -468,19 +468,22 @@ def main():
         del xs32, ws32
 
     if not args.no_decode and args.workload == "cfg2":
-        dm, dn, dk, _, dseed, drange = WORKLOADS["cfg3_m16"]
-        dsets = make_gpu_inputs(torch, dm, dn, dk, dseed, drange, dev, copies=4)
-        dout = torch.empty(dm, dn, dtype=torch.bfloat16, device=dev)
-        dwall, dper = time_gemm(torch, wave_amd, dsets, dout, max(args.steps, 20) * 4, args.warmup)
-        dbytes = gemm_bytes(dm, dn, dk, 2)
-        result["decode_m16"] = {
-            "workload": f"cfg3_m16: M={dm} N={dn} K={dk} bf16 out seed {dseed}, 4 operand sets rotated (HBM-cold B)",
-            "launch_us": round(dper * 1e6, 2),
-            "gbps": round(dbytes / dper / 1e9, 1),
-            "frac_of_hbm_peak": round(dbytes / dper / 1e9 / PEAK_HBM_GBPS, 4),
-            "bytes": dbytes,
-        }
-        del dsets, dout
+        # the decode shapes of the metric's second half: M = 16 (its target), and M = 1 and 32 beside it
+        for name in ("cfg3_m16", "cfg3_m1", "cfg3_m32"):
+            dm, dn, dk, _, dseed, drange = WORKLOADS[name]
+            dsets = make_gpu_inputs(torch, dm, dn, dk, dseed, drange, dev, copies=4)
+            dout = torch.empty(dm, dn, dtype=torch.bfloat16, device=dev)
+            dsteps = max(args.steps, 20) * (4 if name == "cfg3_m16" else 1)
+            dwall, dper = time_gemm(torch, wave_amd, dsets, dout, dsteps, args.warmup)
+            dbytes = gemm_bytes(dm, dn, dk, 2)
+            result["decode_m%d" % dm] = {
+                "workload": f"{name}: M={dm} N={dn} K={dk} bf16 out seed {dseed}, 4 operand sets rotated (HBM-cold B)",
+                "launch_us": round(dper * 1e6, 2),
+                "gbps": round(dbytes / dper / 1e9, 1),
+                "frac_of_hbm_peak": round(dbytes / dper / 1e9 / PEAK_HBM_GBPS, 4),
+                "bytes": dbytes,
+            }
+            del dsets, dout
 
     if not args.no_decode and args.workload == "cfg2":
         # the step in front of the GEMM: quantise the bf16 activation of this workload

@@ -514,6 +514,9 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
       for (int j = 1; j < kStreamKtPerWave; ++j) {
         if (j >= ktw) scb[j] = 0x7F7Fu;
       }
+      // (all eight selects here, ahead of the MFMAs: one directly in front of the MFMA that reads it costs wait states)
+#pragma unroll
+      for (int j = 0; j < kStreamKtPerWave; ++j) asm volatile("" : "+v"(scb[j]));
     }
 
     const int reducer = t & (kw - 1);  // the wave of the group that adds up the tile of step t

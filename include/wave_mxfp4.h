@@ -123,7 +123,10 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
  * are multiplied by expert e's B[e] [N, K/2] with B_scale[e]; C is
  * [total_rows, N].  `offsets` is a DEVICE array of num_groups+1 int32,
  * non-decreasing, offsets[0] = 0, offsets[num_groups] <= total_rows; empty
- * groups are allowed.  B is [E, N, K/2]; B_scale is [E, N, K/32] row-major, or
+ * groups are allowed.  The array lives on the device, so it is clamped there,
+ * not validated: each group's range is cut to [0, total_rows] with end >=
+ * begin, which keeps every access inside the buffers; what a malformed array
+ * computes is unspecified.  B is [E, N, K/2]; B_scale is [E, N, K/32] row-major, or
  * E shuffled buffers of ceil(N/32)*32 x ceil(K/256)*8 bytes each.
  * The reference has no grouped MXFP4 kernel: this replaces its per-expert
  * Python loop over single GEMMs (tests/kernel/moe_test.py:175-246).

@@ -152,3 +152,13 @@ def test_check_maps_status_to_exceptions():
     with pytest.raises(RuntimeError, match="HIP call failed"):
         _lib.check(_lib.ERR_HIP, "x")
     _lib.check(_lib.OK, "x")
+
+
+def test_explicit_split_must_leave_no_split_empty():
+    """ceil(K / splits) can be a whole number of K tiles while the last splits own none: K = 299 K tiles in 300
+    splits of one K tile each.  An empty split would leave its slice of the partial sums unwritten."""
+    lib = _lib.load()
+    k = 299 * 256
+    assert gemm(lib, m=128, k=k, split=300, variant=3, ws=P, wsb=1 << 40) == _lib.ERR_BAD_SPLIT
+    assert gemm(lib, m=128, k=k, split=1000, variant=3, ws=P, wsb=1 << 40) == _lib.ERR_BAD_SPLIT
+    assert gemm(lib, m=128, k=1024, split=8, variant=3, ws=P, wsb=1 << 40) == _lib.ERR_BAD_SPLIT   # 128 per split

@@ -1,10 +1,10 @@
 """GPU parity at the five benchmark configurations, full size.
 
-Where the whole exact oracle is too slow on host cores, rows are sampled
-(tile corners, tile interiors, the last row) against the exact oracle, every
-element is compared with the independent one-thread-per-element device kernel
-(itself pinned against the oracle on the sampled rows), and size-independent
-identities (checksum of checksums) close the gap."""
+First line: the exact oracle on rows of EVERY 256-row M tile (at least 8 per
+tile, all residues mod 32; about 500 rows at 8192^3, which the OpenMP C oracle
+does in seconds).  Second line: every element against the independent
+one-thread-per-element device kernel (itself pinned against the oracle on the
+same rows), and size-independent identities (checksum of checksums)."""
 
 import numpy as np
 import pytest
@@ -21,13 +21,21 @@ from gpu_util import (BF16_ABS, BF16_REL, DEV, TILE_VARIANTS, assert_bf16_close,
 pytestmark = pytest.mark.gpu
 
 
-def sample_rows(m, count, seed, tile=256):
+def sample_rows(m, per_tile, seed, tile=256, lo=0):
+    """Rows of [lo, lo + m) for the exact oracle: in EVERY `tile`-row M tile (counted from `lo`, where a
+    group's tiles start) one row per 32-row block, at residue (4 * block + tile index) % 32, so that four
+    consecutive tiles cover every residue mod 32 (the MFMA's row-in-tile, lane and scale-block positions),
+    plus `per_tile - 8` random rows of the tile, plus the corners of the first and last tiles."""
     rng = np.random.default_rng(seed)
-    fixed = [0, 1, 31, 32, tile - 1, tile, m // 2, m - tile, m - 2, m - 1]
-    rows = {r for r in fixed if 0 <= r < m}
-    while len(rows) < min(count, m):
-        rows.add(int(rng.integers(0, m)))
-    return np.array(sorted(rows), dtype=np.int64)
+    rows = {r for r in (0, 1, 31, 32, tile - 1, tile, m // 2, m - tile, m - 2, m - 1) if 0 <= r < m}
+    for t in range((m + tile - 1) // tile):
+        base, height = t * tile, min(tile, m - t * tile)
+        for b in range((height + 31) // 32):
+            r = base + 32 * b + (4 * b + t) % 32
+            rows.add(min(r, m - 1))
+        for r in rng.integers(0, height, size=max(per_tile - 8, 0)):
+            rows.add(base + int(r))
+    return np.array(sorted(rows), dtype=np.int64) + lo
 
 
 def checksum_identities(c, x, xs, w_t, ws, rel_per_elem):
@@ -58,7 +66,9 @@ def test_config2_8192_cubed_bf16_seed1():
     m = n = k = 8192
     x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=1, scale_lo=124, scale_hi=130)
     gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
-    rows = sample_rows(m, 48, seed=1)
+    rows = sample_rows(m, 16, seed=1)      # about 500 rows, at least 8 in each of the 32 M tiles
+    assert len(rows) >= 8 * 32 and set(rows % 32) == set(range(32))
+    assert all(((rows >= t * 256) & (rows < (t + 1) * 256)).sum() >= 8 for t in range(32))
     ref_rows = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
 
     naive = torch.empty(m, n, dtype=torch.float32, device=DEV)
@@ -122,16 +132,20 @@ def test_config4_grouped_moe_bf16_seed3():
     e, n, k, rows = 8, 14336, 4096, 8192
     x, xs, w, ws, off = grouped_inputs(e, n, k, rows, seed=3)
     assert off[-1] == rows and len(set(np.diff(off))) > 1          # ragged
-    # sampled rows of every expert against the exact per-expert oracle
-    picks = []
+    # rows of every expert against the exact per-expert oracle: at least 8 in every 256-row tile of the
+    # expert's range (tiles start at the expert's first row), all residues mod 32 per expert
+    picks, ref = [], []
     for g in range(e):
         lo, hi = int(off[g]), int(off[g + 1])
-        picks += [r for r in (lo, lo + 1, (lo + hi) // 2, hi - 1) if lo <= r < hi]
-    picks = np.array(sorted(set(picks)))
-    ref = np.empty((len(picks), n))
-    for i, r in enumerate(picks):
-        g = int(np.searchsorted(off, r, side="right") - 1)
-        ref[i] = c_oracle.scaled_gemm_exact(x[r:r + 1], w[g], xs[r:r + 1], ws[g])[0]
+        if hi == lo:
+            continue
+        rows_g = sample_rows(hi - lo, 12, seed=30 + g, lo=lo)
+        assert rows_g.min() >= lo and rows_g.max() < hi
+        if hi - lo >= 1024:
+            assert set((rows_g - lo) % 32) == set(range(32))
+        ref.append(c_oracle.scaled_gemm_exact(x, w[g], xs, ws[g], rows=rows_g))
+        picks.append(rows_g)
+    picks, ref = np.concatenate(picks), np.concatenate(ref)
     naive = run_grouped(x, xs, w, ws, off, torch.float32, variant=_lib.VARIANT_NAIVE)
     assert_f32_close(naive[picks], ref, "naive grouped vs oracle rows")
     for vname in ("auto", "t256x256_w2x2", "t128x128_w2x2"):
@@ -175,7 +189,8 @@ def test_grouped_rows_past_last_offset_untouched_and_layouts():
 def test_config5_edge_shape_shuffled_scales_f32_seed4():
     m, n, k = 4093, 6144, 7168
     x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=4, scale_lo=100, scale_hi=154)
-    rows = sample_rows(m, 40, seed=4)
+    rows = sample_rows(m, 16, seed=4)      # at least 8 rows in each of the 16 M tiles (the last one 253 rows)
+    assert all(((rows >= t * 256) & (rows < (t + 1) * 256)).sum() >= 8 for t in range(16))
     ref_rows = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
     gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
 
@@ -210,3 +225,26 @@ def test_config5_edge_shape_shuffled_scales_f32_seed4():
                         b_scale_layout=_lib.SCALE_E8M0_SHUFFLE, b_layout=_lib.B_PRESHUFFLE)
     assert np.array_equal(out.cpu().numpy(), plain)
     checksum_identities(plain, x, xs, w_t, ws, rel_per_elem=2e-6)
+
+
+def test_grouped_many_expert_rows_with_scratch():
+    """E * N beyond 65535 blocks of 32 scale rows (E = 128, N = 16416: 2.1 M rows of B scales, 269 MB of B at
+    K = 256): the scale re-layout in front of the grouped GEMM must serve it, with and without the workspace."""
+    e, n, k, rows = 128, 16416, 256, 200
+    assert e * n > 65535 * 32
+    off = orc.make_group_offsets(e, rows, seed=40)
+    x, xs, _, _ = orc.make_inputs(rows, 1, k, 40, scale_lo=124, scale_hi=130)
+    gen = torch.Generator(device=DEV).manual_seed(40)
+    gw = torch.randint(0, 256, (e, n, k // 2), dtype=torch.uint8, device=DEV, generator=gen)
+    gws = torch.randint(124, 131, (e, n, k // 32), dtype=torch.uint8, device=DEV, generator=gen)
+    gx, gxs, goff = to_gpu(x, xs, off)
+    out = torch.full((rows, n), float("nan"), dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out)
+    c = out.cpu().numpy()
+    out.fill_(float("nan"))
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out, workspace=False)
+    assert np.array_equal(out.cpu().numpy(), c)
+    for g in sorted(set(np.searchsorted(off, np.arange(rows), side="right") - 1))[::9]:   # some of the used experts
+        lo, hi = int(off[g]), int(off[g + 1])
+        ref = c_oracle.scaled_gemm_exact(x[lo:hi], gw[g].cpu().numpy(), xs[lo:hi], gws[g].cpu().numpy())
+        assert_f32_close(c[lo:hi], ref, f"expert {g}")

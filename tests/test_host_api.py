@@ -115,3 +115,30 @@ def test_cpu_layout_helpers_match_oracle():
     assert np.array_equal(got, orc.e8m0_shuffle_padded(s)[:96])
     s = rng.integers(0, 256, size=(256, 32), dtype=np.uint8)
     assert np.array_equal(e8m0_shuffle(torch.from_numpy(s)).numpy(), orc.e8m0_shuffle(s))
+
+
+def test_superseded_scratch_buffers_stay_alive():
+    """A buffer that was handed out may sit in a captured HIP graph: growing the cache must not free it."""
+    import weakref
+
+    from wave_amd import mxfp4 as host
+
+    key = ("test-device", 12345)
+    made = []
+
+    def alloc(n):
+        t = torch.empty(n, dtype=torch.uint8)
+        made.append(weakref.ref(t))
+        return t
+
+    try:
+        small = host._grow_scratch(key, 100, alloc)
+        assert host._grow_scratch(key, 50, alloc) is small          # large enough: reused
+        ptr = small.data_ptr()
+        big = host._grow_scratch(key, 1000, alloc)
+        assert big is not small and big.numel() == 1000
+        del small
+        assert made[0]() is not None and made[0]().data_ptr() == ptr  # still referenced by the module
+        assert host._grow_scratch(key, 1000, alloc) is big
+    finally:
+        host._scratch.pop(key, None)

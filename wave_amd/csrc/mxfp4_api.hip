@@ -154,11 +154,14 @@ int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
 
 // Reference rule for an explicit split (tagged_mxfp4_gemm.py:636-645) with
 // BLOCK_K = 256: K per split = ceil(K / splits) must be >= 256 and a multiple
-// of 256.
+// of 256; and no split may be left without a K tile.
 bool split_ok(int64_t k, int splits, int *tiles_per_split) {
   const int64_t per = (k + splits - 1) / splits;
   if (per < kTileK || per % kTileK != 0) return false;
   *tiles_per_split = (int)(per / kTileK);
+  // every split must own at least one K tile: ceil() can leave the last ones empty (K = 299 * 256 in 300 splits),
+  // and an empty split writes no partial slice for the reduction to read
+  if ((int64_t)(splits - 1) * *tiles_per_split >= (k + kTileK - 1) / kTileK) return false;
   return true;
 }
 
@@ -484,7 +487,7 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
     if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
         (p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR || p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32) &&
         persist_gemm_applies(q, v, device_cus())) {
-      e = launch_grouped_tile_table(offsets, num_groups, 256, table, stream);
+      e = launch_grouped_tile_table(offsets, num_groups, 256, total_rows, table, stream);
       if (e != hipSuccess) return record_hip(e);
       const bool b_native = p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
       e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, total_rows, p.b_scale, ws_b, b_native ? 0 : (int64_t)num_groups * n,
@@ -498,9 +501,13 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
       // (the fast re-layout does not apply: fall through to the one-tile-per-workgroup kernel)
       e = hipSuccess;
     }
-    if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR) {
+    // both row-major: one launch re-lays both; where that launcher does not apply (it then launches nothing),
+    // or for any other pair of layouts, one general conversion per operand
+    e = hipErrorInvalidValue;
+    if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR)
       e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, total_rows, p.b_scale, ws_b, (int64_t)num_groups * n, p.ks, stream);
-    } else {
+    if (e == hipErrorInvalidValue) {
+      e = hipSuccess;
       if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32)
         e = launch_scale_convert(p.a_scale, p.a_scale_layout, ws_a, WAVE_MXFP4_SCALE_MFMA32, total_rows, p.ks, stream);
       else

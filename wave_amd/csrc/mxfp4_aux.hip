@@ -125,7 +125,7 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
   uint8_t *dst = blockIdx.z ? dst1 : dst0;
   int rows = blockIdx.z ? rows1 : rows0;
   const int k_tiles = (ks + 7) >> 3;  // ks % 4 == 0: the last K tile may hold 4 groups only (the rest is written as 0)
-  const int rt = blockIdx.y, kt0 = blockIdx.x * 32;
+  const int rt = blockIdx.x, kt0 = blockIdx.y * 32;  // row tiles along x: up to 2^31 - 1 of them
   int row_base = rt * 32;
   if (tiles0 != nullptr && blockIdx.z == 0) {
     const int tile = rt >> 3;
@@ -326,8 +326,8 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
   const int64_t n = rows_p * (ksp / 4);
   if (n == 0) return hipSuccess;
   if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 3) == 0 &&
-      ((uintptr_t)src & 3) == 0 && rows < ((int64_t)1 << 31) && ks < ((int64_t)1 << 31) && rows_p / 32 <= 65535) {
-    dim3 grid((unsigned)((ksp / 8 + 31) / 32), (unsigned)(rows_p / 32), 1);
+      ((uintptr_t)src & 3) == 0 && rows < ((int64_t)1 << 31) && (ksp / 8 + 31) / 32 <= 65535) {
+    dim3 grid((unsigned)(rows_p / 32), (unsigned)((ksp / 8 + 31) / 32), 1);
     scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks, nullptr);
     return hipGetLastError();
   }
@@ -363,9 +363,9 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
   const int64_t rows_max = a_rows_out > b_rows ? a_rows_out : b_rows;
   const int64_t rt = (rows_max + 31) / 32;
   if ((ks & 3) != 0 || ks == 0 || ((uintptr_t)a_src & 3) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 3) != 0) ||
-      rows_max >= ((int64_t)1 << 31) || ks >= ((int64_t)1 << 31) || rt > 65535 || a_rows <= 0 || b_rows < 0)
+      rows_max >= ((int64_t)1 << 31) || ((ks + 7) / 8 + 31) / 32 > 65535 || a_rows <= 0 || b_rows < 0)
     return hipErrorInvalidValue;
-  dim3 grid((unsigned)(((ks + 7) / 8 + 31) / 32), (unsigned)rt, b_rows > 0 ? 2 : 1);  // b_rows == 0: A alone
+  dim3 grid((unsigned)rt, (unsigned)(((ks + 7) / 8 + 31) / 32), b_rows > 0 ? 2 : 1);  // b_rows == 0: A alone
   scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks, a_tiles);
   return hipGetLastError();
 }

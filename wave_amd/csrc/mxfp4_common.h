@@ -164,7 +164,8 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
                                        const int32_t *a_tiles = nullptr, int64_t a_tile_cap = 0);
 hipError_t launch_scale_pair_shuffle_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
                                                uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream);
-hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int32_t *table, hipStream_t stream);
+hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int64_t total_rows, int32_t *table,
+                                     hipStream_t stream);
 hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t kp,
                                hipStream_t stream);
 

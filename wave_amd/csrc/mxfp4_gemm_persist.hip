@@ -136,7 +136,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       as_lim[which] = (int)min((int64_t)(m_blocks - (m0[which] >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
     }
     a_base[which] = p.a + (int64_t)m0[which] * kp;
-    a_lim[which] = (int)min((int64_t)(p.m - m0[which]) * kp, (int64_t)0x7FFFFFFF);
+    a_lim[which] = (int)min((int64_t)max(p.m - m0[which], 0) * kp, (int64_t)0x7FFFFFFF);
     if (SPLIT) {  // the item's K range starts at K tile kt_lo: move the bases there
       a_base[which] += kt_lo * kTileKBytes;
       a_lim[which] = max(a_lim[which] - kt_lo * kTileKBytes, 0);

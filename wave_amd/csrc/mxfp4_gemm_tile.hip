@@ -154,8 +154,9 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
     int e = 0, first = 0, lo = 0, hi = 0;
     bool found = false;
     for (; e < p.num_groups; ++e) {
-      lo = p.offsets[e];
-      hi = p.offsets[e + 1];
+      // (clamped, not validated: a group's range is cut to [0, M] with end >= begin)
+      lo = min(max(p.offsets[e], 0), p.m);
+      hi = min(max(p.offsets[e + 1], lo), p.m);
       const int t = (hi - lo + BM - 1) / BM;
       if (tm < first + t) {
         found = true;

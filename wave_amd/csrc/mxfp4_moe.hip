@@ -168,9 +168,13 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
 // band = 16 * (first tile of the tile's band) + (tiles in the band): a group's tiles form bands of at most 8
 // (as equal as possible), the unit inside which the GEMM walks column by column, so that the tiles running
 // together share one expert's B panels.
+// The offsets are clamped, not validated: each group's range is cut to [0, total_rows] with end >= begin, and
+// tiles beyond the table's capacity (total_rows / bm + num_groups entries, enough for any non-decreasing offsets)
+// are dropped, so a malformed offsets array cannot make this kernel or the GEMM leave their buffers.
 __global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const int32_t *__restrict__ offsets,
-                                                                           int num_groups, int bm,
+                                                                           int num_groups, int bm, int total_rows,
                                                                            int32_t *__restrict__ table) {
+  const int cap = total_rows / bm + num_groups;
   __shared__ int wave_sums[kAlignWaves];
   __shared__ int carry;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -180,7 +184,7 @@ __global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const
     const int e = e0 + t;
     int lo = 0, tiles = 0, hi = 0;
     if (e < num_groups) {
-      lo = offsets[e], hi = offsets[e + 1];
+      lo = min(max(offsets[e], 0), total_rows), hi = min(max(offsets[e + 1], lo), total_rows);
       tiles = hi > lo ? (hi - lo + bm - 1) / bm : 0;
     }
     const int base = carry;  // read before anyone moves it on
@@ -188,7 +192,7 @@ __global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const
     const int nb = (tiles + 7) >> 3;  // bands of the group: `rem` of height hb + 1, then the rest of height hb
     const int hb = nb ? tiles / nb : 0, rem = nb ? tiles - hb * nb : 0;
     const int first_tile = base + end - tiles;
-    for (int i = 0; i < tiles; ++i) {
+    for (int i = 0; i < tiles && first_tile + i < cap; ++i) {
       int32_t *ent = table + 4 * (1 + first_tile + i);
       ent[0] = lo + i * bm;
       ent[1] = min(bm, hi - lo - i * bm);
@@ -201,13 +205,14 @@ __global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const
     if (t == kAlignThreads - 1) carry = base + end;
     __syncthreads();
   }
-  if (t == 0) table[0] = carry;
+  if (t == 0) table[0] = min(carry, cap);
 }
 
 }  // namespace
 
-hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int32_t *table, hipStream_t stream) {
-  grouped_tile_table_kernel<<<1, kAlignThreads, 0, stream>>>(offsets, num_groups, bm, table);
+hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int64_t total_rows, int32_t *table,
+                                     hipStream_t stream) {
+  grouped_tile_table_kernel<<<1, kAlignThreads, 0, stream>>>(offsets, num_groups, bm, (int)total_rows, table);
   return hipGetLastError();
 }
 

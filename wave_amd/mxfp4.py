@@ -84,20 +84,32 @@ def workspace_bytes(m: int, n: int, k: int, split_k: int = 0, variant: int = _li
 # One scratch buffer per (device, stream), grown on demand: the split-K partial
 # sums and the re-laid-out scales of a call live there.  Calls on one stream are
 # ordered, so they can share it; different streams get different buffers.
+# A buffer that was handed out is never freed: a HIP graph captured while it was
+# current keeps its address, so a buffer that a larger call supersedes moves to
+# `_retired` and stays allocated until the process ends.
 _scratch: dict = {}
+_retired: list = []
 # signatures of mxfp4_gemm calls that passed every check: -> (m, n, k, out dtype code, a scale layout, scratch bytes)
 _checked: dict = {}
+
+
+def _grow_scratch(key, nbytes: int, alloc):
+    """The cached buffer of `key` if it holds `nbytes`, else a new one from
+    `alloc(nbytes)`; the superseded buffer is kept alive (see above)."""
+    buf = _scratch.get(key)
+    if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _retired.append(buf)
+        buf = alloc(nbytes)
+        _scratch[key] = buf
+    return buf
 
 
 def _workspace(device, nbytes: int):
     if nbytes == 0:
         return None
     key = (device, torch.cuda.current_stream(device).cuda_stream)
-    buf = _scratch.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _scratch[key] = buf
-    return buf
+    return _grow_scratch(key, nbytes, lambda n: torch.empty(n, dtype=torch.uint8, device=device))
 
 
 def mxfp4_gemm(x, x_scales, w_t, w_scales, out, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,

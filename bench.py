@@ -7,6 +7,12 @@ and the reference's CPU path (torch dequantise + f32 matmul) timed on a bounded
 sample on this box's host cores.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3_m16|...]
+
+Every timed leg is preceded by an untimed, time-based load of its own kernel
+(launches until 50 ms of GPU time have passed, reported as `settle_ms`): the
+GPU needs some tens of milliseconds of work to reach its steady clocks, so
+without it a short --steps/--warmup reads up to 18 % slow.  `steps` and `warmup`
+are then exactly what the caller passed.
 """
 
 import argparse
@@ -22,6 +28,8 @@ if ROOT not in sys.path:
 PEAK_MXFP4_TFLOPS = 10100.0   # MI355X dense FP4 MFMA
 PEAK_HBM_GBPS = 8000.0        # MI355X HBM3E
 PEAK_MXFP8_TFLOPS = 5000.0    # MI355X dense FP8 MFMA
+SETTLE = {"ms": 50.0}        # untimed load in front of every timed leg (GPU milliseconds)
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
 
 WORKLOADS = {
     # name: (m, n, k, out dtype, seed, scale range)
@@ -78,24 +86,104 @@ def make_gpu_inputs(torch, m, n, k, seed, scale_range, device, copies=1):
     return sets
 
 
-def time_gemm(torch, wave_amd, sets, out, steps, warmup, **kw):
-    """K launches back to back on the current stream; returns (wall seconds for
-    all K, average seconds per launch from HIP events on that stream)."""
-    for i in range(warmup):
-        x, xs, w, ws = sets[i % len(sets)]
-        wave_amd.mxfp4_gemm(x, xs, w, ws, out, **kw)
+def settle(torch, run, min_ms=None):
+    """Untimed clock-settle load: `run(n)` launches n of the leg's kernels; repeated until `min_ms` of GPU time have
+    passed.  Returns the GPU milliseconds spent."""
+    min_ms = SETTLE["ms"] if min_ms is None else min_ms
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    spent, n = 0.0, 4
+    while spent < min_ms:
+        e0.record()
+        run(n)
+        e1.record()
+        torch.cuda.synchronize()
+        dt = e0.elapsed_time(e1)
+        spent += dt
+        # aim each further chunk at about a fifth of the target
+        n = max(1, min(4096, int(n * (min_ms / 5.0) / max(dt, 1e-3))))
+    return spent
+
+
+def timed(torch, run, steps, warmup):
+    """settle, `warmup` untimed launches, then exactly `steps` launches between HIP events on the current stream
+    (the stream the kernels are launched on).  Returns (wall seconds for all steps, seconds per launch from the
+    events, settle milliseconds)."""
+    settle_ms = settle(torch, run)
+    run(warmup)
     torch.cuda.synchronize()
     ev0 = torch.cuda.Event(enable_timing=True)
     ev1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
-    for i in range(steps):
-        x, xs, w, ws = sets[i % len(sets)]
-        wave_amd.mxfp4_gemm(x, xs, w, ws, out, **kw)
+    run(steps)
     ev1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall, ev0.elapsed_time(ev1) * 1e-3 / steps
+    return wall, ev0.elapsed_time(ev1) * 1e-3 / steps, settle_ms
+
+
+def time_gemm(torch, wave_amd, sets, out, steps, warmup, **kw):
+    """K launches back to back on the current stream; returns (wall seconds for
+    all K, average seconds per launch from HIP events on that stream, settle ms)."""
+    state = {"i": 0}
+
+    def run(count):
+        i = state["i"]
+        for _ in range(count):
+            x, xs, w, ws = sets[i % len(sets)]
+            wave_amd.mxfp4_gemm(x, xs, w, ws, out, **kw)
+            i += 1
+        state["i"] = i
+
+    return timed(torch, run, steps, warmup)
+
+
+def read_traffic(workload):
+    """HBM bytes per launch of the workload's dominant kernel (fetched + written) from the committed summary of
+    the rocprofv3 FETCH_SIZE / WRITE_SIZE runs, or None when there is no line for it."""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            for line in fh:
+                f = line.split()
+                if len(f) >= 4 and not line.startswith("#") and f[0] == workload:
+                    return float(f[2]) + float(f[3])
+    except OSError:
+        pass
+    return None
+
+
+def write_traffic(workload, kernel_substr, fetch_csv, write_csv, fetch_factor, write_factor):
+    """Updates the workload's line of profiles/hbm_traffic.txt from two rocprofv3 --pmc counter CSVs (FETCH_SIZE
+    and WRITE_SIZE, KiB per dispatch) of the same bench command; the factors are bytes moved / bytes counted for
+    the same counters on a device copy of known size (bench.py --copy-calibration)."""
+    import csv
+
+    def mean_kib(path, counter):
+        vals = {}
+        with open(path) as fh:
+            for row in csv.DictReader(fh):
+                if row["Counter_Name"] == counter and kernel_substr in row["Kernel_Name"]:
+                    vals.setdefault(row.get("Dispatch_Id", len(vals)), 0.0)
+                    vals[row.get("Dispatch_Id", len(vals) - 1)] += float(row["Counter_Value"])
+        if not vals:
+            raise SystemExit(f"{path}: no {counter} rows for a kernel matching {kernel_substr!r}")
+        return sum(vals.values()) / len(vals)
+
+    fetch = mean_kib(fetch_csv, "FETCH_SIZE") * 1024 * fetch_factor
+    wrote = mean_kib(write_csv, "WRITE_SIZE") * 1024 * write_factor
+    lines = []
+    try:
+        lines = [ln for ln in open(TRAFFIC_FILE).read().splitlines() if ln.split()[:1] != [workload]]
+    except OSError:
+        lines = ["# HBM bytes per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE",
+                 "# (KiB per dispatch, mean over the dispatches of `python3 bench.py --no-cpu --no-legs --steps 3 --warmup 1",
+                 "# --workload <W>`), each scaled by the same counter on a 256 MiB device copy (--copy-calibration).",
+                 "# Written by `python bench.py --workload <W> --write-traffic KERNEL,FETCH.csv,WRITE.csv,FETCH_FACTOR,WRITE_FACTOR`;",
+                 "# read back into roofline.traffic.  Columns: workload kernel fetched_bytes written_bytes"]
+    lines.append(f"{workload} {kernel_substr} {fetch:.4e} {wrote:.4e}")
+    with open(TRAFFIC_FILE, "w") as fh:
+        fh.write("\n".join(lines) + "\n")
+    print(f"{TRAFFIC_FILE}: {lines[-1]}")
 
 
 def cpu_baseline(torch, m, n, k, seed, scale_range, sample_rows):
@@ -134,56 +222,186 @@ def cpu_baseline(torch, m, n, k, seed, scale_range, sample_rows):
 
 
 def time_quantize(torch, wave_amd, rows, k, steps, warmup, device, shuffle=True):
-    """(seconds per launch, algorithmic bytes) of the bf16 -> MXFP4 quantiser on a [rows, k] activation; three
-    inputs are rotated so that none is cache resident (402 MB together at 8192 x 8192)."""
+    """(seconds per launch, algorithmic bytes, settle ms) of the bf16 -> MXFP4 quantiser on a [rows, k] activation;
+    three inputs are rotated so that none is cache resident (402 MB together at 8192 x 8192)."""
     xs = [torch.randn(rows, k, device=device, dtype=torch.bfloat16) for _ in range(3)]
     lib = wave_amd._lib.load()
     q = torch.empty(rows, k // 2, dtype=torch.uint8, device=device)
     sc = torch.empty((rows + 31) // 32 * 32, (k // 32 + 7) // 8 * 8, dtype=torch.uint8, device=device)
     stream = torch.cuda.current_stream().cuda_stream
     layout = wave_amd._lib.SCALE_E8M0_SHUFFLE if shuffle else wave_amd._lib.SCALE_ROW_MAJOR
+    state = {"i": 0}
 
     def run(count):
-        for i in range(count):
-            st = lib.wave_mxfp4_quantize(xs[i % 3].data_ptr(), wave_amd._lib.IN_BF16, q.data_ptr(), sc.data_ptr(),
-                                         rows, k, layout, stream)
+        for _ in range(count):
+            st = lib.wave_mxfp4_quantize(xs[state["i"] % 3].data_ptr(), wave_amd._lib.IN_BF16, q.data_ptr(),
+                                         sc.data_ptr(), rows, k, layout, stream)
+            state["i"] += 1
             if st != 0:
                 raise RuntimeError(f"wave_mxfp4_quantize: status {st}")
 
-    run(warmup)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    run(steps)
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / steps, rows * k * 2 + rows * k // 2 + rows * k // 32
+    _, per, settle_ms = timed(torch, run, steps, warmup)
+    return per, rows * k * 2 + rows * k // 2 + rows * k // 32, settle_ms
+
+
+def leg_cfg4(torch, wave_amd, dev, steps, warmup, variant=0):
+    """The grouped (MoE) GEMM of cfg4: E = 8 experts, 4096 tokens x top-2 = 8192 rows dealt multinomially, rows
+    sorted by expert, N = 14336, K = 4096, bf16 out, seed 3."""
+    import numpy as np
+
+    from wave_amd import _lib as L
+
+    E, n, k, rows = 8, 14336, 4096, 8192
+    counts = np.random.default_rng(3).multinomial(rows, np.ones(E) / E)
+    offs = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).to(dev)
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, device=dev, generator=g)
+    xs = torch.randint(124, 131, (rows, k // 32), dtype=torch.uint8, device=dev, generator=g)
+    w = torch.randint(0, 256, (E, n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+    ws = torch.randint(124, 131, (E, n, k // 32), dtype=torch.uint8, device=dev, generator=g)
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device=dev)
+
+    def run(count):
+        for _ in range(count):
+            wave_amd.mxfp4_gemm_grouped(x, xs, w, ws, offs, out, variant=variant)
+
+    wall, per, settle_ms = timed(torch, run, steps, warmup)
+    # resident expert weights: their scales converted to the MFMA operand order once, outside the timed region
+    ws32 = torch.stack([wave_amd.scale_convert(ws[e], n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32) for e in range(E)])
+
+    def run32(count):
+        for _ in range(count):
+            wave_amd.mxfp4_gemm_grouped(x, xs, w, ws32, offs, out, b_scale_layout=L.SCALE_MFMA32, variant=variant)
+
+    _, per32, _ = timed(torch, run32, steps, warmup)
+    flops = 2.0 * rows * n * k
+    return {"workload": f"cfg4: E={E} N={n} K={k} rows={rows} (counts {counts.tolist()}) bf16 out seed 3",
+            "kernel": "persist_gemm_kernel (grouped)", "launch_us": round(per * 1e6, 2),
+            "tflops": round(flops / per / 1e12, 1), "frac_of_mxfp4_peak": round(flops / per / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+            "settle_ms": round(settle_ms, 1), "wall_s_per_step": wall / steps,
+            "resident_weight_scales": {"workload": "the same call with the experts' B scales already in MFMA operand order",
+                                       "launch_us": round(per32 * 1e6, 2), "tflops": round(flops / per32 / 1e12, 1),
+                                       "frac_of_mxfp4_peak": round(flops / per32 / 1e12 / PEAK_MXFP4_TFLOPS, 4)}}
+
+
+def leg_mxfp8(torch, wave_amd, dev, steps, warmup, variant=0):
+    """tests/kernel/wave_gemm_mxfp_test.py:416-501 at its larger shape: e5m2 operands, scales 124..127, f32 out."""
+    m = n = k = 8192
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn(m, k, device=dev, generator=g).to(torch.float8_e5m2)
+    w_t = torch.randn(n, k, device=dev, generator=g).to(torch.float8_e5m2)
+    xs = torch.randint(124, 128, (m, k // 32), dtype=torch.uint8, device=dev, generator=g)
+    ws = torch.randint(124, 128, (n, k // 32), dtype=torch.uint8, device=dev, generator=g)
+    out = torch.empty(m, n, dtype=torch.float32, device=dev)
+
+    def run(count):
+        for _ in range(count):
+            wave_amd.mxfp8_gemm(x, xs, w_t, ws, out, variant=variant)
+
+    wall, per, settle_ms = timed(torch, run, steps, warmup)
+    flops = 2.0 * m * n * k
+    return {"workload": f"mxfp8: M={m} N={n} K={k} e5m2 x e5m2, f32 out, seed 5", "kernel": "tile_gemm_kernel (8-bit operands)",
+            "launch_us": round(per * 1e6, 2), "tflops": round(flops / per / 1e12, 1),
+            "frac_of_mxfp8_peak": round(flops / per / 1e12 / PEAK_MXFP8_TFLOPS, 4), "settle_ms": round(settle_ms, 1),
+            "wall_s_per_step": wall / steps}
+
+
+def leg_dense(torch, wave_amd, dev, name, steps, warmup, variant=0):
+    """One of the dense WORKLOADS through the library's own kernel choice."""
+    m, n, k, od, seed, srange = WORKLOADS[name]
+    sets = make_gpu_inputs(torch, m, n, k, seed, srange, dev, copies=1)
+    out = torch.empty(m, n, dtype=torch.bfloat16 if od == "bf16" else torch.float32, device=dev)
+    _, per, settle_ms = time_gemm(torch, wave_amd, sets, out, steps, warmup, variant=variant)
+    flops = gemm_flops(m, n, k)
+    return {"workload": f"{name}: M={m} N={n} K={k} {od} out seed {seed}", "launch_us": round(per * 1e6, 2),
+            "tflops": round(flops / per / 1e12, 1), "frac_of_mxfp4_peak": round(flops / per / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+            "settle_ms": round(settle_ms, 1)}
+
+
+def mfma_ceiling(torch, dev, steps, warmup):
+    """What the matrix pipes sustain on the scaled FP4 MFMA alone (wave_amd/csrc/mfma_probe.hip): random operand
+    bytes against zeros, 4 and 8 waves per CU, one workgroup per CU."""
+    import ctypes
+
+    path = os.path.join(ROOT, "wave_amd", "csrc", "libwave_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `make -C wave_amd/csrc`")
+    probe = ctypes.CDLL(path)
+    vp, i32 = ctypes.c_void_p, ctypes.c_int
+    probe.wave_probe_mfma_fp4.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
+    probe.wave_probe_mfma_fp4.restype = i32
+    probe.wave_probe_operand_bytes.argtypes = [i32, i32]
+    probe.wave_probe_operand_bytes.restype = ctypes.c_size_t
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    stream = torch.cuda.current_stream().cuda_stream
+    iters = 8000   # x 32 MFMAs x 32 cycles per wave: about 4 ms per launch at one wave per SIMD
+    rows = []
+    for waves in (4, 8):
+        nbytes = probe.wave_probe_operand_bytes(cus, waves)
+        g = torch.Generator(device=dev).manual_seed(11)
+        operands = {"random": torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=dev, generator=g),
+                    "zeros": torch.zeros(nbytes, dtype=torch.uint8, device=dev)}
+        out = torch.empty(cus * waves * 64, dtype=torch.float32, device=dev)
+        ticks = torch.empty(cus, dtype=torch.int64, device=dev)
+        for data in ("random", "zeros"):
+            src = operands[data]
+
+            def run(count):
+                for _ in range(count):
+                    rc = probe.wave_probe_mfma_fp4(src.data_ptr(), out.data_ptr(), ticks.data_ptr(), iters, 110, cus,
+                                                   waves, stream)
+                    if rc != 0:
+                        raise RuntimeError(f"wave_probe_mfma_fp4: {rc}")
+
+            _, per, settle_ms = timed(torch, run, max(steps // 10, 10), max(warmup // 10, 2))
+            mfmas_per_wave = iters * 32
+            flops = cus * waves * mfmas_per_wave * 2.0 * 32 * 32 * 64
+            # MFMA cycles each SIMD has to issue (32 per instruction, waves / 4 waves per SIMD): the clock if the pipe
+            # never idles, a lower bound of it otherwise
+            clock_ghz = mfmas_per_wave * 32 * (waves / 4) / per / 1e9
+            rows.append({"operands": data, "waves_per_cu": waves, "launch_ms": round(per * 1e3, 3),
+                         "tflops": round(flops / per / 1e12, 1),
+                         "frac_of_mxfp4_peak": round(flops / per / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+                         "mfma_clock_ghz": round(clock_ghz, 3), "settle_ms": round(settle_ms, 1)})
+    best_random = max(r["tflops"] for r in rows if r["operands"] == "random")
+    return rows, best_random
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=300)
-    ap.add_argument("--warmup", type=int, default=100,
-                    help="untimed launches first; the GPU needs ~30 ms of load to reach its steady clocks")
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue", "ref_shapes"],
+    ap.add_argument("--warmup", type=int, default=100, help="untimed launches in front of the timed ones (after the "
+                    "time-based settle load every leg runs anyway)")
+    ap.add_argument("--workload", default="cfg2",
+                    choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue", "ref_shapes", "mfma_ceiling"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
                          "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out; "
                          "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096; moe_glue: the steps around "
-                         "it at the same sizes (token alignment, gathered quantiser, gated activation + quantiser)")
+                         "it at the same sizes (token alignment, gathered quantiser, gated activation + quantiser); "
+                         "ref_shapes: the reference's benchmark shape list; mfma_ceiling: the scaled FP4 MFMA alone, "
+                         "random operands against zeros (the power-limited ceiling of the matrix pipes)")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-decode", action="store_true", help="skip the M=16 decode-shape leg")
+    ap.add_argument("--no-legs", "--no-decode", dest="no_legs", action="store_true",
+                    help="cfg2 only: skip the legs beside the headline (decode shapes, quantiser, cfg4, cfg5, mxfp8)")
     ap.add_argument("--cpu-rows", type=int, default=8192,
                     help="rows of A in the CPU baseline leg (default: the whole workload)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of a GEMM, run device-to-device copies of 256 MiB (the known-size kernel "
                          "that hardware byte counters are scaled by) and print their size")
+    ap.add_argument("--write-traffic", metavar="KERNEL,FETCH_CSV,WRITE_CSV,FETCH_FACTOR,WRITE_FACTOR",
+                    help="no GPU work: update this workload's line of profiles/hbm_traffic.txt from two rocprofv3 "
+                         "--pmc counter CSVs of this command")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this operator runs on one GPU; --gpus N with N > 1 is not supported "
               "(the operator shards over GPUs by splitting N or M, with no exchange between them)", file=sys.stderr)
         sys.exit(2)
+    if args.write_traffic:
+        kernel, fetch_csv, write_csv, ff, wf = args.write_traffic.split(",")
+        write_traffic(args.workload, kernel, fetch_csv, write_csv, float(ff), float(wf))
+        return
 
     import torch
 
@@ -196,6 +414,8 @@ def main():
         sys.exit(3)
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+              "vs_baseline": None}
 
     if args.copy_calibration:
         nbytes = 256 << 20
@@ -208,20 +428,31 @@ def main():
                           "bytes_written_per_launch": nbytes, "launches": args.warmup + args.steps}))
         return
 
+    if args.workload == "mfma_ceiling":
+        rows, best = mfma_ceiling(torch, dev, args.steps, args.warmup)
+        print(json.dumps(dict(common, **{
+            "metric": "scaled FP4 MFMA alone (v_mfma_scale_f32_32x32x64_f8f6f4, no memory traffic), TFLOP/s on random operands",
+            "value": best, "unit": "TFLOP/s", "ms_per_step": min(r["launch_ms"] for r in rows if r["operands"] == "random"),
+            "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate", "data": "synthetic (uniform random bytes / zeros)",
+            "config": {"workload": "mfma_ceiling: one workgroup per CU, 4 or 8 waves, 8000 x 32 MFMAs per wave and launch"},
+            "roofline": {"bound": "mfma", "achieved": best, "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(best / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "mfma_probe_kernel"},
+            "runs": rows})))
+        return
+
     if args.workload == "quant_bf16":
         rows, k = 8192, 8192
-        qper, qbytes = time_quantize(torch, wave_amd, rows, k, args.steps, args.warmup, dev)
+        qper, qbytes, settle_ms = time_quantize(torch, wave_amd, rows, k, args.steps, args.warmup, dev)
         gbps = qbytes / qper / 1e9
-        print(json.dumps({
-            "metric": "activation quantiser, GB/s % HBM", "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1,
-            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(qper * 1e3, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in, e2m1 + e8m0 out",
-            "data": "synthetic (normal)",
+        print(json.dumps(dict(common, **{
+            "metric": "activation quantiser, GB/s % HBM", "value": round(gbps, 1), "unit": "GB/s",
+            "ms_per_step": round(qper * 1e3, 4), "dtype": "bf16 in, e2m1 + e8m0 out", "data": "synthetic (normal)",
+            "settle_ms": round(settle_ms, 1),
             "config": {"workload": f"quant_bf16: bf16 [{rows}, {k}] -> MXFP4, scales in e8m0_shuffle order, "
                                    "3 inputs rotated"},
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                         "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": 134.3e6 + 35.65e6, "kernel": "quantize_kernel",
-                         "launch_us": round(qper * 1e6, 2)}}))
+                         "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": read_traffic("quant_bf16"),
+                         "kernel": "quantize_kernel", "launch_us": round(qper * 1e6, 2)}})))
         return
 
     if args.workload == "ref_shapes":
@@ -230,27 +461,31 @@ def main():
 
         k = REF_SHAPES_K
         rows = []
+        first = True
         for m in sorted(REF_SHAPES_MN):
             for n in REF_SHAPES_MN[m]:
                 sets = make_gpu_inputs(torch, m, n, k, 1, (124, 130), dev, copies=1)
                 out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
                 flops = gemm_flops(m, n, k)
                 steps = max(10, min(args.steps, int(0.05 / (flops / 4.0e15))))
-                _, per = time_gemm(torch, wave_amd, sets, out, steps, max(5, steps // 3), variant=args.variant)
+                if not first:   # the clocks are up after the first shape: a short settle keeps them there
+                    SETTLE["ms"] = 10.0
+                first = False
+                _, per, _ = time_gemm(torch, wave_amd, sets, out, steps, max(5, steps // 3), variant=args.variant)
                 rows.append((m, n, per, flops / per / 1e12))
                 del sets, out
         geo = math.exp(sum(math.log(r[3]) for r in rows) / len(rows))
         big = [r for r in rows if r[0] * r[1] >= 4096 * 4096]
         geo_big = math.exp(sum(math.log(r[3]) for r in big) / len(big))
-        print(json.dumps({
+        print(json.dumps(dict(common, **{
             "metric": "MXFP4 GEMM TFLOPS over the reference's benchmark shapes (K = 16000), geometric mean",
-            "value": round(geo, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": round(sum(r[2] for r in rows) * 1e3, 3), "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out",
+            "value": round(geo, 1), "unit": "TFLOP/s",
+            "ms_per_step": round(sum(r[2] for r in rows) * 1e3, 3),
+            "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out",
             "data": "synthetic (seeded uniform nibbles and scales)",
             "config": {"workload": f"ref_shapes: {len(rows)} (M, N) pairs, K = {k}, bf16 out, seed 1"},
             "geomean_tflops_mn_ge_4096x4096": round(geo_big, 1),
-            "shapes": [{"m": r[0], "n": r[1], "us": round(r[2] * 1e6, 1), "tflops": round(r[3], 1)} for r in rows]}))
+            "shapes": [{"m": r[0], "n": r[1], "us": round(r[2] * 1e6, 1), "tflops": round(r[3], 1)} for r in rows]})))
         return
 
     if args.workload == "moe_glue":
@@ -266,17 +501,15 @@ def main():
         acts = [torch.randn(tokens, hidden, device=dev, generator=g).to(torch.bfloat16) for _ in range(3)]
         gemm1 = [torch.randn(n_ent, 2 * inter, device=dev, generator=g).to(torch.bfloat16) for _ in range(2)]
 
-        def timed(fn):
-            for i in range(args.warmup):
-                fn(i)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for i in range(args.steps):
-                fn(i)
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) * 1e-3 / args.steps
+        def timed_fn(fn):
+            state = {"i": 0}
+
+            def run(count):
+                for _ in range(count):
+                    fn(state["i"])
+                    state["i"] += 1
+
+            return timed(torch, run, args.steps, args.warmup)[1]
 
         # straight through the C ABI with outputs allocated once: the kernels are shorter than a Python wrapper call
         lib, st = _lib.load(), torch.cuda.current_stream().cuda_stream
@@ -284,23 +517,21 @@ def main():
         s1 = torch.empty(n_ent, hidden // 32, dtype=torch.uint8, device=dev)
         q2 = torch.empty(n_ent, inter // 2, dtype=torch.uint8, device=dev)
         s2 = torch.empty(n_ent, inter // 32, dtype=torch.uint8, device=dev)
-        t_align = timed(lambda i: lib.wave_mxfp4_moe_align_block_size(
+        t_align = timed_fn(lambda i: lib.wave_mxfp4_moe_align_block_size(
             ids.data_ptr(), 0, n_ent, E, 1, sorted_ids.data_ptr(), n_ent, expert_ids.data_ptr(), n_ent,
             total.data_ptr(), offs.data_ptr(), st))
-        t_gather = timed(lambda i: lib.wave_mxfp4_quantize_rows(
+        t_gather = timed_fn(lambda i: lib.wave_mxfp4_quantize_rows(
             acts[i % 3].data_ptr(), _lib.IN_BF16, tokens, sorted_ids.data_ptr(), topk, q1.data_ptr(), s1.data_ptr(),
             n_ent, hidden, _lib.SCALE_ROW_MAJOR, st))
-        t_act = timed(lambda i: lib.wave_mxfp4_silu_and_mul_quantize(
+        t_act = timed_fn(lambda i: lib.wave_mxfp4_silu_and_mul_quantize(
             gemm1[i % 2].data_ptr(), gemm1[i % 2].data_ptr() + 2 * inter, 2 * inter, 2 * inter, _lib.IN_BF16,
             q2.data_ptr(), s2.data_ptr(), n_ent, inter, _lib.SCALE_ROW_MAJOR, st))
         b_gather = n_ent * hidden * 2 + n_ent * hidden // 2 + n_ent * hidden // 32   # every source row is read top_k times
         b_act = n_ent * inter * 4 + n_ent * inter // 2 + n_ent * inter // 32
         gbps = b_act / t_act / 1e9
-        print(json.dumps({
+        print(json.dumps(dict(common, **{
             "metric": "MoE glue: gated activation + quantiser GB/s % HBM", "value": round(gbps, 1), "unit": "GB/s",
-            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(t_act * 1e3, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in, e2m1 + e8m0 out",
-            "data": "synthetic (normal)",
+            "ms_per_step": round(t_act * 1e3, 4), "dtype": "bf16 in, e2m1 + e8m0 out", "data": "synthetic (normal)",
             "config": {"workload": f"moe_glue: {tokens} tokens x top-{topk} of {E} experts, hidden {hidden}, "
                                    f"intermediate {inter}"},
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
@@ -308,98 +539,32 @@ def main():
                          "kernel": "quantize_kernel (gated)", "launch_us": round(t_act * 1e6, 2)},
             "moe_align_block_size_us": round(t_align * 1e6, 2),
             "gathered_quantiser": {"launch_us": round(t_gather * 1e6, 2), "gbps": round(b_gather / t_gather / 1e9, 1),
-                                   "bytes": b_gather}}))
+                                   "bytes": b_gather}})))
         return
 
     if args.workload == "cfg4":
-        # E = 8 experts, 4096 tokens x top-2 = 8192 rows dealt multinomially, rows sorted by expert, bf16 out, seed 3
-        import numpy as np
-
-        E, n, k, rows = 8, 14336, 4096, 8192
-        counts = np.random.default_rng(3).multinomial(rows, np.ones(E) / E)
-        offs = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).to(dev)
-        g = torch.Generator(device=dev).manual_seed(3)
-        x = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, device=dev, generator=g)
-        xs = torch.randint(124, 131, (rows, k // 32), dtype=torch.uint8, device=dev, generator=g)
-        w = torch.randint(0, 256, (E, n, k // 2), dtype=torch.uint8, device=dev, generator=g)
-        ws = torch.randint(124, 131, (E, n, k // 32), dtype=torch.uint8, device=dev, generator=g)
-        out = torch.empty(rows, n, dtype=torch.bfloat16, device=dev)
-
-        def run(count):
-            for _ in range(count):
-                wave_amd.mxfp4_gemm_grouped(x, xs, w, ws, offs, out, variant=args.variant)
-
-        run(args.warmup)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        run(args.steps)
-        e1.record()
-        torch.cuda.synchronize()
-        per = e0.elapsed_time(e1) * 1e-3 / args.steps
-        tflops = 2.0 * rows * n * k / per / 1e12
-        # resident expert weights: their scales converted to the MFMA operand order once, outside the timed region
-        from wave_amd import _lib as L
-        ws32 = torch.stack([wave_amd.scale_convert(ws[e], n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32) for e in range(E)])
-
-        def run32(count):
-            for _ in range(count):
-                wave_amd.mxfp4_gemm_grouped(x, xs, w, ws32, offs, out, b_scale_layout=L.SCALE_MFMA32, variant=args.variant)
-
-        run32(args.warmup)
-        torch.cuda.synchronize()
-        e0.record()
-        run32(args.steps)
-        e1.record()
-        torch.cuda.synchronize()
-        per32 = e0.elapsed_time(e1) * 1e-3 / args.steps
-        print(json.dumps({
-            "metric": "grouped (MoE) MXFP4 GEMM TFLOPS", "value": round(tflops, 2), "unit": "TFLOP/s",
-            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per * 1e3, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        leg = leg_cfg4(torch, wave_amd, dev, args.steps, args.warmup, args.variant)
+        print(json.dumps(dict(common, **{
+            "metric": "grouped (MoE) MXFP4 GEMM TFLOPS", "value": leg["tflops"], "unit": "TFLOP/s",
+            "ms_per_step": round(leg.pop("wall_s_per_step") * 1e3, 4),
             "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out", "data": "synthetic (seeded uniform)",
-            "config": {"workload": f"cfg4: E={E} N={n} K={k} rows={rows} (counts {counts.tolist()}) bf16 out seed 3",
-                       "variant": args.variant},
-            "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(tflops / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "persist_gemm_kernel (grouped)",
-                         "launch_us": round(per * 1e6, 2)},
-            "resident_weight_scales": {"workload": "the same call with the experts' B scales already in MFMA operand order",
-                                       "launch_us": round(per32 * 1e6, 2),
-                                       "tflops": round(2.0 * rows * n * k / per32 / 1e12, 1)}}))
+            "config": {"workload": leg["workload"], "variant": args.variant}, "settle_ms": leg["settle_ms"],
+            "roofline": {"bound": "mfma", "achieved": leg["tflops"], "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
+                         "frac": leg["frac_of_mxfp4_peak"], "traffic": read_traffic("cfg4"), "kernel": leg["kernel"],
+                         "launch_us": leg["launch_us"]},
+            "resident_weight_scales": leg["resident_weight_scales"]})))
         return
 
     if args.workload == "mxfp8":
-        # tests/kernel/wave_gemm_mxfp_test.py:416-501 at its larger shape: e5m2 operands, scales 124..127, f32 out
-        m = n = k = 8192
-        g = torch.Generator(device=dev).manual_seed(5)
-        x = torch.randn(m, k, device=dev, generator=g).to(torch.float8_e5m2)
-        w_t = torch.randn(n, k, device=dev, generator=g).to(torch.float8_e5m2)
-        xs = torch.randint(124, 128, (m, k // 32), dtype=torch.uint8, device=dev, generator=g)
-        ws = torch.randint(124, 128, (n, k // 32), dtype=torch.uint8, device=dev, generator=g)
-        out = torch.empty(m, n, dtype=torch.float32, device=dev)
-
-        def run(count):
-            for _ in range(count):
-                wave_amd.mxfp8_gemm(x, xs, w_t, ws, out, variant=args.variant)
-
-        run(args.warmup)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        run(args.steps)
-        e1.record()
-        torch.cuda.synchronize()
-        per = e0.elapsed_time(e1) * 1e-3 / args.steps
-        tflops = 2.0 * m * n * k / per / 1e12
-        print(json.dumps({
-            "metric": "MXFP8 GEMM TFLOPS + % of FP8 MFMA peak (8192^3)", "value": round(tflops, 2), "unit": "TFLOP/s",
-            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(per * 1e3, 4),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        leg = leg_mxfp8(torch, wave_amd, dev, args.steps, args.warmup, args.variant)
+        print(json.dumps(dict(common, **{
+            "metric": "MXFP8 GEMM TFLOPS + % of FP8 MFMA peak (8192^3)", "value": leg["tflops"], "unit": "TFLOP/s",
+            "ms_per_step": round(leg.pop("wall_s_per_step") * 1e3, 4),
             "dtype": "mxfp8 (e5m2 x e8m0) in, f32 accumulate, f32 out", "data": "synthetic (normal values, seeded)",
-            "config": {"workload": f"mxfp8: M={m} N={n} K={k} f32 out seed 5", "variant": args.variant},
-            "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_MXFP8_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(tflops / PEAK_MXFP8_TFLOPS, 4), "traffic": None, "kernel": "tile_gemm_kernel",
-                         "launch_us": round(per * 1e6, 2)}}))
+            "config": {"workload": leg["workload"], "variant": args.variant}, "settle_ms": leg["settle_ms"],
+            "roofline": {"bound": "mfma", "achieved": leg["tflops"], "peak": PEAK_MXFP8_TFLOPS, "unit": "TFLOP/s",
+                         "frac": leg["frac_of_mxfp8_peak"], "traffic": read_traffic("mxfp8"), "kernel": leg["kernel"],
+                         "launch_us": leg["launch_us"]}})))
         return
 
     m, n, k, od, seed, srange = WORKLOADS[args.workload]
@@ -410,12 +575,11 @@ def main():
     copies = 4 if memory_bound else 1
     sets = make_gpu_inputs(torch, m, n, k, seed, srange, dev, copies=copies)
     out = torch.empty(m, n, dtype=out_dtype, device=dev)
-    wall, per_launch = time_gemm(torch, wave_amd, sets, out, args.steps, args.warmup, variant=args.variant)
+    wall, per_launch, settle_ms = time_gemm(torch, wave_amd, sets, out, args.steps, args.warmup, variant=args.variant)
 
-    # HBM bytes per launch of the dominant kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this
-    # command, scaled by a device copy of known size (profiles/pmc_*.txt); not measurable from here
-    measured_traffic = {"cfg2": 435e6 + 134.2e6, "cfg3_m16": 125.6e6 + 0.92e6}.get(args.workload) \
-        if args.variant == 0 else None
+    # HBM bytes per launch of the dominant kernel: rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this command, scaled
+    # by a device copy of known size, kept in profiles/hbm_traffic.txt (not measurable from here); None without a line
+    measured_traffic = read_traffic(args.workload) if args.variant == 0 else None
     flops, nbytes = gemm_flops(m, n, k), gemm_bytes(m, n, k, out_bytes)
     ms_per_step = wall / args.steps * 1e3
     tflops = flops / (wall / args.steps) / 1e12
@@ -428,19 +592,15 @@ def main():
         achieved = flops / per_launch / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_MXFP4_TFLOPS,
                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_MXFP4_TFLOPS, 4), "traffic": measured_traffic,
-                    "kernel": "persist_gemm_kernel" if (m % 256 == 0 and n % 256 == 0 and (m // 256) * (n // 256) > 256) else "tile_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
+                    "kernel": "persist_gemm_kernel" if (n % 256 == 0 and ((m + 255) // 256) * (n // 256) > 256) else "tile_gemm_kernel",
+                    "launch_us": round(per_launch * 1e6, 2)}
 
-    result = {
+    result = dict(common, **{
         "metric": "MXFP4 GEMM TFLOPS + % of FP4 MFMA peak (8192^3); GB/s % HBM at M=16",
         "value": round(tflops, 2),
         "unit": "TFLOP/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
+        "settle_ms": round(settle_ms, 1),
         "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, " + od + " out",
         "data": "synthetic (seeded uniform nibbles and scales), random weights",
         "config": {"workload": f"{args.workload}: M={m} N={n} K={k} {od} out seed {seed}",
@@ -448,7 +608,7 @@ def main():
         "frac_of_mxfp4_peak": round(tflops / PEAK_MXFP4_TFLOPS, 4),
         "gbps": round(nbytes / (wall / args.steps) / 1e9, 1),
         "roofline": roofline,
-    }
+    })
 
     if not memory_bound and args.variant == 0:
         # The same launch with both scale tensors handed over in the MFMA operand order (the reference's headline
@@ -458,44 +618,53 @@ def main():
         x, xs, w, ws = sets[0]
         xs32 = wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
         ws32 = wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
-        _, pper = time_gemm(torch, wave_amd, [(x, xs32, w, ws32)], out, args.steps, args.warmup,
-                            a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32)
+        _, pper, _ = time_gemm(torch, wave_amd, [(x, xs32, w, ws32)], out, args.steps, args.warmup,
+                               a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32)
         result["preshuffled_scales"] = {
             "workload": "the same operands, scales already in MFMA operand order (no re-layout launch)",
             "launch_us": round(pper * 1e6, 2), "tflops": round(flops / pper / 1e12, 1),
             "frac_of_mxfp4_peak": round(flops / pper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
         }
         del xs32, ws32
+    del sets, out
 
-    if not args.no_decode and args.workload == "cfg2":
+    if not args.no_legs and args.workload == "cfg2":
         # the decode shapes of the metric's second half: M = 16 (its target), and M = 1 and 32 beside it
         for name in ("cfg3_m16", "cfg3_m1", "cfg3_m32"):
             dm, dn, dk, _, dseed, drange = WORKLOADS[name]
             dsets = make_gpu_inputs(torch, dm, dn, dk, dseed, drange, dev, copies=4)
             dout = torch.empty(dm, dn, dtype=torch.bfloat16, device=dev)
             dsteps = max(args.steps, 20) * (4 if name == "cfg3_m16" else 1)
-            dwall, dper = time_gemm(torch, wave_amd, dsets, dout, dsteps, args.warmup)
+            _, dper, dsettle = time_gemm(torch, wave_amd, dsets, dout, dsteps, args.warmup)
             dbytes = gemm_bytes(dm, dn, dk, 2)
             result["decode_m%d" % dm] = {
                 "workload": f"{name}: M={dm} N={dn} K={dk} bf16 out seed {dseed}, 4 operand sets rotated (HBM-cold B)",
                 "launch_us": round(dper * 1e6, 2),
                 "gbps": round(dbytes / dper / 1e9, 1),
                 "frac_of_hbm_peak": round(dbytes / dper / 1e9 / PEAK_HBM_GBPS, 4),
-                "bytes": dbytes,
+                "bytes": dbytes, "steps": dsteps, "settle_ms": round(dsettle, 1),
+                "traffic": read_traffic(name),
             }
             del dsets, dout
 
-    if not args.no_decode and args.workload == "cfg2":
         # the step in front of the GEMM: quantise the bf16 activation of this workload
-        qper, qbytes = time_quantize(torch, wave_amd, m, k, args.steps, args.warmup, dev)
+        qper, qbytes, qsettle = time_quantize(torch, wave_amd, m, k, args.steps, args.warmup, dev)
         result["quantize_a"] = {
             "workload": f"bf16 [{m}, {k}] -> e2m1 + e8m0 (e8m0_shuffle order), 3 inputs rotated",
             "kernel": "quantize_kernel",
             "launch_us": round(qper * 1e6, 2),
             "gbps": round(qbytes / qper / 1e9, 1),
             "frac_of_hbm_peak": round(qbytes / qper / 1e9 / PEAK_HBM_GBPS, 4),
-            "bytes": qbytes,
+            "bytes": qbytes, "settle_ms": round(qsettle, 1),
         }
+        # the other configurations and the 8-bit operands, each with its own settle load
+        leg = leg_cfg4(torch, wave_amd, dev, args.steps, args.warmup)
+        leg.pop("wall_s_per_step")
+        result["cfg4_grouped"] = leg
+        result["cfg5"] = leg_dense(torch, wave_amd, dev, "cfg5", args.steps, args.warmup)
+        leg = leg_mxfp8(torch, wave_amd, dev, args.steps, args.warmup)
+        leg.pop("wall_s_per_step")
+        result["mxfp8"] = leg
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, m, n, k, seed, srange, args.cpu_rows)

@@ -1,0 +1,94 @@
+// Measurement only, not part of the operator: what the matrix pipes of this GPU
+// sustain on the scaled FP4 MFMA alone, with no memory traffic at all.  Built as
+// its own small library (libwave_probe.so) so that the operator's C ABI stays what
+// include/wave_mxfp4.h declares; `bench.py --workload mfma_ceiling` is its caller.
+//
+// Every wave loads the operand fragments of its wave tile once (2 K steps x (4 + 4)
+// fragments of a 128 x 128 tile, or 4 K steps x (2 + 4) of a 64 x 128 tile) and then
+// issues, `iters` times, the 32 v_mfma_scale_f32_32x32x64_f8f6f4 they feed, in the
+// order the GEMM kernels use (K step outermost, every accumulator once per step).  With random operand bytes the
+// chip draws more power per instruction than with zeros and clocks lower: the two
+// rates bracket what any GEMM kernel on that data can reach.  The reference prices
+// its kernels against the instruction's issue cost the same way
+// (benchmark/wave_att_analyzer.py:35-36: 32 cycles for 32x32x64).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// NT = 256: 4 waves per workgroup, each a 128 x 128 wave tile (4 x 4 MFMA tiles, 16 accumulators).
+// NT = 512: 8 waves, each 64 x 128 (2 x 4 MFMA tiles), the shape of the 8-wave GEMM kernels: two waves per SIMD
+// have 256 registers each.
+template <int NT>
+__global__ void __launch_bounds__(NT) mfma_probe_kernel(const v4i *__restrict__ src, float *__restrict__ out,
+                                                        unsigned long long *__restrict__ ticks, int iters, int scale) {
+  constexpr int MI = NT == 256 ? 4 : 2, MJ = 4, KT = NT == 256 ? 2 : 4;  // 32 MFMAs per wave and iteration
+  v16f acc[MI * MJ];
+#pragma unroll
+  for (int i = 0; i < MI * MJ; ++i)
+#pragma unroll
+    for (int g = 0; g < 16; ++g) acc[i][g] = 0.f;
+  v4i fa[KT][MI], fb[KT][MJ];
+#pragma unroll
+  for (int t = 0; t < KT; ++t) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[t][i] = src[(((size_t)blockIdx.x * 4 + t) * 8 + i) * NT + threadIdx.x];
+#pragma unroll
+    for (int j = 0; j < MJ; ++j) fb[t][j] = src[(((size_t)blockIdx.x * 4 + t) * 8 + 4 + j) * NT + threadIdx.x];
+  }
+  const unsigned long long t0 = __builtin_amdgcn_s_memtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int t = 0; t < KT; ++t)
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < MJ; ++j) {
+          const v8i a = {fa[t][i].x, fa[t][i].y, fa[t][i].z, fa[t][i].w, 0, 0, 0, 0};
+          const v8i b = {fb[t][j].x, fb[t][j].y, fb[t][j].z, fb[t][j].w, 0, 0, 0, 0};
+          acc[i * MJ + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i * MJ + j], 4, 4, 0, scale, 0, scale);
+        }
+  }
+  const unsigned long long t1 = __builtin_amdgcn_s_memtime();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < MI * MJ; ++i)
+#pragma unroll
+    for (int g = 0; g < 16; ++g) s += acc[i][g];
+  out[(size_t)blockIdx.x * NT + threadIdx.x] = s;
+  if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Bytes of `operands` one launch reads: 32 fragments of 16 bytes per thread.
+size_t wave_probe_operand_bytes(int workgroups, int waves_per_workgroup) {
+  return (size_t)workgroups * 32 * (size_t)(waves_per_workgroup * 64) * 16;
+}
+
+// One launch: `workgroups` workgroups of 4 or 8 waves, each wave `iters` x 32 MFMAs of 2 * 32 * 32 * 64 flop.
+// out: workgroups * waves * 64 floats; ticks: workgroups 64-bit counts of the constant 100 MHz counter.
+// The sums are never rescaled (that would move all accumulators through the vector registers): pick scale_byte
+// so that iters * 32 products of at most 36 * 2^(2 * (scale_byte - 127)) stay finite, e.g. 110.
+// Returns 0, or -1 for a bad argument, or the hipError_t of the launch.
+int wave_probe_mfma_fp4(const void *operands, float *out, unsigned long long *ticks, int iters, int scale_byte,
+                        int workgroups, int waves_per_workgroup, void *hip_stream) {
+  if (!operands || !out || !ticks || iters < 1 || workgroups < 1 || scale_byte < 0 || scale_byte > 254) return -1;
+  hipStream_t stream = (hipStream_t)hip_stream;
+  const int s = scale_byte | (scale_byte << 8) | (scale_byte << 16) | (scale_byte << 24);
+  if (waves_per_workgroup == 4)
+    mfma_probe_kernel<256><<<workgroups, 256, 0, stream>>>((const v4i *)operands, out, ticks, iters, s);
+  else if (waves_per_workgroup == 8)
+    mfma_probe_kernel<512><<<workgroups, 512, 0, stream>>>((const v4i *)operands, out, ticks, iters, s);
+  else
+    return -1;
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

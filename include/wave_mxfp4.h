@@ -119,6 +119,26 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
 size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant);
 
 /*
+ * wave_mxfp4_gemm for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc); it has
+ * no counterpart in the reference.  Same arguments and results as
+ * wave_mxfp4_gemm without the workspace pair: the scratch (re-laid scales,
+ * split-K partial sums, the parts of a sparsely filled last round of tiles) is
+ * a fixed array of wave_mxfp4_static_scratch_bytes() = 16 MiB inside the
+ * library's device image, one per GPU, held until the process ends.  The call
+ * allocates and frees nothing.  A problem whose
+ * wave_mxfp4_workspace_bytes(m, n, k, split_k, variant) exceeds that size is
+ * rejected with WAVE_MXFP4_ERR_WORKSPACE (wave_mxfp4_last_hip_error() then
+ * holds the two sizes); 8192^3 needs 6.3 MB.  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (different streams, or threads
+ * without ordering) race on it; calls on one stream are ordered and safe.
+ */
+int wave_mxfp4_gemm_static(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
+                           int64_t m, int64_t n, int64_t k, int out_dtype, int a_scale_layout,
+                           int b_scale_layout, int b_layout, int split_k, int variant, void *hip_stream);
+size_t wave_mxfp4_static_scratch_bytes(void);
+
+/*
  * Grouped (MoE) GEMM: rows offsets[e] .. offsets[e+1]-1 of A (sorted by expert)
  * are multiplied by expert e's B[e] [N, K/2] with B_scale[e]; C is
  * [total_rows, N].  `offsets` is a DEVICE array of num_groups+1 int32,

@@ -1,0 +1,66 @@
+"""GPU: wave_mxfp4_gemm_static, the entry point that allocates nothing (its scratch is a fixed array inside the
+library's device image), through the C ABI against wave_mxfp4_gemm with a caller-provided workspace: the same
+kernels in the same order, so the same bits.  Two calls in a row share the array, the second on a smaller
+problem, so stale contents of the first must not leak into the second."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mxfp4_oracle as orc
+from wave_amd import _lib
+
+from gpu_util import DEV, assert_close, to_gpu
+
+pytestmark = pytest.mark.gpu
+
+
+def both(lib, m, n, k, out_dtype, seed, split_k=0, variant=0, asl=0, bsl=0):
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=seed, scale_lo=120, scale_hi=134)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    od = _lib.OUT_BF16 if out_dtype == torch.bfloat16 else _lib.OUT_F32
+    stream = torch.cuda.current_stream().cuda_stream
+    got = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    st = lib.wave_mxfp4_gemm_static(gx.data_ptr(), gxs.data_ptr(), gw.data_ptr(), gws.data_ptr(), got.data_ptr(),
+                                    m, n, k, od, asl, bsl, 0, split_k, variant, stream)
+    assert st == _lib.OK, (st, lib.wave_mxfp4_last_hip_error())
+    need = lib.wave_mxfp4_workspace_bytes(m, n, k, split_k, variant)
+    ws_buf = torch.empty(max(need, 256), dtype=torch.uint8, device=DEV)
+    want = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    st = lib.wave_mxfp4_gemm(gx.data_ptr(), gxs.data_ptr(), gw.data_ptr(), gws.data_ptr(), want.data_ptr(),
+                             m, n, k, od, asl, bsl, 0, split_k, ws_buf.data_ptr(), need, variant, stream)
+    assert st == _lib.OK
+    torch.cuda.synchronize()
+    return got, want, (x, xs, w_t, ws)
+
+
+@pytest.mark.parametrize("first,second", [
+    # (m, n, k, out dtype, split_k): a K split by the library itself (f32 parts in the scratch), then a smaller one
+    ((1024, 1024, 8192, torch.bfloat16, 0), (512, 768, 2048, torch.bfloat16, 0)),
+    # re-laid scales of a many-tile problem, then an explicit split of a small one
+    ((2304, 2048, 1024, torch.float32, 1), (200, 136, 1024, torch.float32, 4)),
+    # a decode shape whose K is split over workgroups, then a plain one
+    ((16, 2048, 16384, torch.bfloat16, 0), (16, 512, 1024, torch.bfloat16, 0)),
+])
+def test_static_scratch_matches_workspace_entry_point(first, second):
+    lib = _lib.load()
+    assert lib.wave_mxfp4_static_scratch_bytes() == 16 << 20
+    for i, (m, n, k, dt, split) in enumerate((first, second)):
+        got, want, (x, xs, w_t, ws) = both(lib, m, n, k, dt, seed=70 + i, split_k=split)
+        assert torch.equal(got.view(torch.uint8), want.view(torch.uint8)), (m, n, k)
+        assert_close(got.float().cpu().numpy(), orc.scaled_gemm_exact(x, w_t, xs, ws), dt, f"{m}x{n}x{k} vs oracle")
+
+
+def test_static_scratch_rejects_what_does_not_fit():
+    lib = _lib.load()
+    p = 0x1000
+    # 8 splits of 8192 x 8192 f32 parts: 2 GiB of partial sums
+    assert lib.wave_mxfp4_workspace_bytes(8192, 8192, 8192, 8, 0) > lib.wave_mxfp4_static_scratch_bytes()
+    st = lib.wave_mxfp4_gemm_static(p, p, p, p, p, 8192, 8192, 8192, 1, 0, 0, 0, 8, 0, None)
+    assert st == _lib.ERR_WORKSPACE
+    assert b"static" in lib.wave_mxfp4_last_hip_error()
+    # the headline shape fits
+    assert lib.wave_mxfp4_workspace_bytes(8192, 8192, 8192, 0, 0) <= lib.wave_mxfp4_static_scratch_bytes()
+    # argument errors come before the size test
+    assert lib.wave_mxfp4_gemm_static(None, p, p, p, p, 64, 64, 256, 0, 0, 0, 0, 1, 0, None) == _lib.ERR_NULL_POINTER
+    assert lib.wave_mxfp4_gemm_static(p, p, p, p, p, 64, 64, 48, 0, 0, 0, 0, 1, 0, None) == _lib.ERR_BAD_SHAPE

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # WAVE_MXFP4_LIB points at another build of the same ABI (e.g. an experiment)
 LIB_PATH = os.environ.get("WAVE_MXFP4_LIB") or os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 # status codes of include/wave_mxfp4.h
 OK = 0
@@ -42,6 +42,8 @@ VARIANT_T128x256_W2x2 = 6
 EXPORTS = (
     "wave_mxfp4_gemm",
     "wave_mxfp4_workspace_bytes",
+    "wave_mxfp4_gemm_static",
+    "wave_mxfp4_static_scratch_bytes",
     "wave_mxfp4_gemm_grouped",
     "wave_mxfp4_grouped_workspace_bytes",
     "wave_mxfp8_gemm",
@@ -81,6 +83,10 @@ def load():
     lib.wave_mxfp4_gemm.restype = i32
     lib.wave_mxfp4_workspace_bytes.argtypes = [i64, i64, i64, i32, i32]
     lib.wave_mxfp4_workspace_bytes.restype = sz
+    lib.wave_mxfp4_gemm_static.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, i32, i32, i32, p]
+    lib.wave_mxfp4_gemm_static.restype = i32
+    lib.wave_mxfp4_static_scratch_bytes.argtypes = []
+    lib.wave_mxfp4_static_scratch_bytes.restype = sz
     lib.wave_mxfp4_gemm_grouped.argtypes = [p, p, p, p, p, p, i32, i64, i64, i64, i32, i32, i32, i32, i32, p, sz, p]
     lib.wave_mxfp4_grouped_workspace_bytes.argtypes = [i64, i64, i64, i32]
     lib.wave_mxfp4_grouped_workspace_bytes.restype = sz

@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 7;
+constexpr int kAbiVersion = 8;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -163,6 +163,29 @@ bool split_ok(int64_t k, int splits, int *tiles_per_split) {
   // and an empty split writes no partial slice for the reduction to read
   if ((int64_t)(splits - 1) * *tiles_per_split >= (k + kTileK - 1) / kTileK) return false;
   return true;
+}
+
+// Scratch of wave_mxfp4_gemm_static: a fixed array in the library's device image, one copy per GPU, held until
+// the process ends.  On the host the array's name is only a handle for hipGetSymbolAddress: the address a
+// kernel can use is looked up once per device and kept here.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+void *g_static_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch_for_current_device(void **ptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return record_hip(e);
+  if (dev < 0 || dev >= kMaxDevices) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (g_static_scratch_ptr[dev] == nullptr) {
+    void *found = nullptr;
+    e = hipGetSymbolAddress(&found, HIP_SYMBOL(g_static_scratch));
+    if (e != hipSuccess) return record_hip(e);
+    if (found == nullptr) return WAVE_MXFP4_ERR_UNSUPPORTED;
+    g_static_scratch_ptr[dev] = found;  // two threads racing here store the same address
+  }
+  *ptr = g_static_scratch_ptr[dev];
+  return WAVE_MXFP4_OK;
 }
 
 }  // namespace
@@ -353,6 +376,32 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (e != hipSuccess) return record_hip(e);
   if (splits > 1) e = launch_splitk_reduce(p.partial, c, m * n, splits, p.out_bf16, stream);
   return record_hip(e);
+}
+
+size_t wave_mxfp4_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int wave_mxfp4_gemm_static(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c, int64_t m,
+                           int64_t n, int64_t k, int out_dtype, int a_scale_layout, int b_scale_layout, int b_layout,
+                           int split_k, int variant, void *hip_stream) {
+  // the same checks as wave_mxfp4_gemm, before the size test, so that a bad argument reports itself
+  const int rc = check_common(a, a_scale, b, b_scale, c, m, n, k, out_dtype, a_scale_layout, b_scale_layout, b_layout,
+                              variant);
+  if (rc <= 0) return rc;
+  if (split_k < 0) return WAVE_MXFP4_ERR_BAD_SPLIT;
+  if (wave_mxfp4_workspace_bytes(m, n, k, split_k, variant) > kStaticScratchBytes) {
+    snprintf(g_hip_error, sizeof(g_hip_error),
+             "wave_mxfp4_gemm_static: %lld x %lld x %lld with split_k %d needs %zu bytes of scratch, the static "
+             "buffer holds %zu", (long long)m, (long long)n, (long long)k, split_k,
+             wave_mxfp4_workspace_bytes(m, n, k, split_k, variant), kStaticScratchBytes);
+    return WAVE_MXFP4_ERR_WORKSPACE;
+  }
+  void *scratch = nullptr;
+  const int st = static_scratch_for_current_device(&scratch);
+  if (st != WAVE_MXFP4_OK) return st;
+  // Nothing in the scratch has to start from zero: every byte a kernel of this call reads from it (re-laid
+  // scales with their padding, split-K parts) is written earlier in the same call, on the same stream.
+  return wave_mxfp4_gemm(a, a_scale, b, b_scale, c, m, n, k, out_dtype, a_scale_layout, b_scale_layout, b_layout,
+                         split_k, scratch, kStaticScratchBytes, variant, hip_stream);
 }
 
 size_t wave_mxfp8_workspace_bytes(int64_t m, int64_t n, int64_t k) {

@@ -625,6 +625,19 @@ def main():
             "launch_us": round(pper * 1e6, 2), "tflops": round(flops / pper / 1e12, 1),
             "frac_of_mxfp4_peak": round(flops / pper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
         }
+        if n % 256 == 0 and k % 512 == 0 and k >= 1536:
+            # ... and B in b_preshuffle order on top (static weights, preshuffled once, as the reference's
+            # asymmetric kernels assume: templates/tagged_mxfp4_gemm.py:950-991): A through LDS, B straight from
+            # global memory into registers
+            wp = wave_amd.b_preshuffle(w)
+            _, bper, _ = time_gemm(torch, wave_amd, [(x, xs32, wp, ws32)], out, args.steps, args.warmup,
+                                   a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32, b_layout=L.B_PRESHUFFLE)
+            result["preshuffled_b"] = {
+                "workload": "the same operands, B in b_preshuffle order and scales in MFMA operand order",
+                "kernel": "asym_gemm_kernel", "launch_us": round(bper * 1e6, 2), "tflops": round(flops / bper / 1e12, 1),
+                "frac_of_mxfp4_peak": round(flops / bper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+            }
+            del wp
         del xs32, ws32
     del sets, out
 

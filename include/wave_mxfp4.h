@@ -88,6 +88,14 @@ typedef enum {
   WAVE_MXFP4_VARIANT_SKINNY = 4,        /* M <= 64 streaming kernel */
   WAVE_MXFP4_VARIANT_NAIVE = 5,         /* one thread per C element, for cross-checks */
   WAVE_MXFP4_VARIANT_T128x256_W2x2 = 6, /* 128x256x256 tile, 4 waves */
+  /* 256x256x256 tile, 4 waves side by side along N; A through LDS, preshuffled B
+   * straight from global memory into registers: the asymmetric kernels of the
+   * reference (tagged_mxfp4_gemm.py:950-991 with schedules/
+   * gemm_mxfp4_double_buffer.py:1781-2222).  Needs b_layout PRESHUFFLE,
+   * N % 256 == 0, K % 512 == 0, K >= 1536 and either MFMA32 scales or the
+   * workspace; WAVE_MXFP4_ERR_UNSUPPORTED otherwise.  AUTO takes it where it
+   * applies and the problem has more tiles than the GPU has CUs. */
+  WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT = 7,
   WAVE_MXFP4_VARIANT_COUNT_
 } wave_mxfp4_variant;
 

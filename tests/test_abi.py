@@ -162,3 +162,17 @@ def test_explicit_split_must_leave_no_split_empty():
     assert gemm(lib, m=128, k=k, split=300, variant=3, ws=P, wsb=1 << 40) == _lib.ERR_BAD_SPLIT
     assert gemm(lib, m=128, k=k, split=1000, variant=3, ws=P, wsb=1 << 40) == _lib.ERR_BAD_SPLIT
     assert gemm(lib, m=128, k=1024, split=8, variant=3, ws=P, wsb=1 << 40) == _lib.ERR_BAD_SPLIT   # 128 per split
+
+
+def test_b_direct_variant_rejects_what_it_does_not_take():
+    """Variant 7 (A through LDS, preshuffled B straight into registers) is refused, before anything is launched,
+    for row-major B, ragged N, an odd number of K tiles, a short K, a split, or row-major scales without scratch."""
+    lib = _lib.load()
+    v = _lib.VARIANT_T256x256_W1x4_BDIRECT
+    ok = dict(m=512, n=512, k=2048, bl=1, asl=2, bsl=2, variant=v)
+    assert gemm(lib, **dict(ok, bl=0)) == _lib.ERR_UNSUPPORTED
+    assert gemm(lib, **dict(ok, n=384)) == _lib.ERR_UNSUPPORTED
+    assert gemm(lib, **dict(ok, k=2304)) == _lib.ERR_UNSUPPORTED      # 9 K tiles
+    assert gemm(lib, **dict(ok, k=1024)) == _lib.ERR_UNSUPPORTED
+    assert gemm(lib, **dict(ok, split=2)) in (_lib.ERR_UNSUPPORTED, _lib.ERR_WORKSPACE)
+    assert gemm(lib, **dict(ok, asl=0)) == _lib.ERR_UNSUPPORTED       # row-major scales need the workspace

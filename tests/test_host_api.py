@@ -142,3 +142,21 @@ def test_superseded_scratch_buffers_stay_alive():
         assert host._grow_scratch(key, 1000, alloc) is big
     finally:
         host._scratch.pop(key, None)
+
+
+def test_asymmetric_schedule_selects_the_b_direct_kernel():
+    """wave_compile(options, preshuffle-B template, get_mxfp4_asymmetric_schedule()) names the kernel that keeps A in
+    LDS and reads preshuffled B straight into registers, where the shape allows; other schedules, shapes and
+    templates keep their (block_shape, wave_shape) choice."""
+    spec, options = get_tagged_mxfp4_gemm_preshuffle_b((1024, 1024, 8192), (256, 256, 256), wave_shape=(2, 2))
+    assert wave_compile(options, spec, get_mxfp4_asymmetric_schedule()).spec.variant == _lib.VARIANT_T256x256_W1x4_BDIRECT
+    assert wave_compile(options, spec, get_mxfp4_dbuf_schedule()).spec.variant == _lib.VARIANT_T256x256_W2x2
+    assert spec.variant == _lib.VARIANT_T256x256_W2x2                       # the template object is left as it was
+    for shape, block in [((1024, 1024, 1024), (256, 256, 256)),             # K too short
+                         ((1024, 3072, 8192), (256, 192, 256)),             # another tile
+                         ((512, 768, 2304), (256, 256, 256))]:              # an odd number of K tiles
+        spec, options = get_tagged_mxfp4_gemm_preshuffle_b(shape, block, wave_shape=(2, 2))
+        k = wave_compile(options, spec, get_mxfp4_asymmetric_schedule())
+        assert k.spec.variant != _lib.VARIANT_T256x256_W1x4_BDIRECT
+    spec, options = get_tagged_mxfp4_gemm((1024, 1024, 8192), (256, 256, 256), wave_shape=(2, 2))
+    assert wave_compile(options, spec, get_mxfp4_asymmetric_schedule()).spec.variant == _lib.VARIANT_T256x256_W2x2

@@ -37,6 +37,7 @@ VARIANT_T128x128_W2x2 = 3
 VARIANT_SKINNY = 4
 VARIANT_NAIVE = 5
 VARIANT_T128x256_W2x2 = 6
+VARIANT_T256x256_W1x4_BDIRECT = 7
 
 # every symbol include/wave_mxfp4.h declares
 EXPORTS = (

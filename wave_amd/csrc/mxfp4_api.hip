@@ -124,7 +124,7 @@ int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
   }
   int bm, bn;
   tile_variant_shape(variant, &bm, &bn);
-  if (bm == 0) return 1;
+  if (bm == 0 || variant == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT) return 1;  // (that kernel takes whole K ranges)
   const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
   const int64_t k_tiles = (k + kTileK - 1) / kTileK;  // a partial last K tile belongs to the last split
   if (tiles > 128 || k_tiles < 8) return 1;
@@ -255,6 +255,14 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   fill_params(p, a, a_scale, b, b_scale, c, m, n, k, out_dtype, a_scale_layout, b_scale_layout, b_layout);
   const int v = pick_variant(m, n, k, variant);
   if (v == WAVE_MXFP4_VARIANT_SKINNY && m > skinny_max_m()) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT) {
+    // what the B-direct kernel takes, checked before anything is launched: preshuffled B, whole 256-column tiles,
+    // an even number (at least 6) of K tiles, no split, scales in MFMA32 order or scratch to bring them there
+    const bool native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+    if (b_layout != WAVE_MXFP4_B_PRESHUFFLE || n % 256 != 0 || k % 512 != 0 || k < 1536 || split_k > 1 ||
+        (!native && !workspace))
+      return WAVE_MXFP4_ERR_UNSUPPORTED;
+  }
 
   if (k == 0) return record_hip(launch_naive_gemm(p, stream));  // empty reduction: C = 0
 
@@ -360,7 +368,12 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     tile_variant_shape(tv, &bm, &bn);
     p.tiles_m = (int)((m + bm - 1) / bm);
     p.tiles_n = (int)((n + bn - 1) / bn);
-    if (persist_gemm_applies(p, tv, device_cus())) {
+    const bool want_asym = v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT;
+    if (want_asym && !asym_gemm_applies(p, device_cus(), true)) return WAVE_MXFP4_ERR_UNSUPPORTED;
+    if (want_asym || (variant == WAVE_MXFP4_VARIANT_AUTO && tv == WAVE_MXFP4_VARIANT_T256x256_W4x2 &&
+                      asym_gemm_applies(p, device_cus(), false))) {
+      e = launch_asym_gemm(p, device_cus(), stream);
+    } else if (persist_gemm_applies(p, tv, device_cus())) {
       // a last round of tiles that would leave most workgroups idle is cut along K instead, if there is scratch
       size_t part_bytes = 0;
       const int parts = persist_tail_parts(p, tv, device_cus(), &part_bytes);
@@ -507,7 +520,8 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   // every expert's B and B_scale must keep the base alignment
   if (p.b_group_stride % 16 != 0 || p.b_scale_group_stride % 8 != 0) return WAVE_MXFP4_ERR_MISALIGNED;
 
-  if (variant == WAVE_MXFP4_VARIANT_SKINNY) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (variant == WAVE_MXFP4_VARIANT_SKINNY || variant == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT)
+    return WAVE_MXFP4_ERR_UNSUPPORTED;
   const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_variant(total_rows > 64 ? total_rows : 65, n, k, variant)
                                                    : pick_variant(total_rows, n, k, variant);
   if (v == WAVE_MXFP4_VARIANT_NAIVE) return record_hip(launch_naive_gemm(p, stream));

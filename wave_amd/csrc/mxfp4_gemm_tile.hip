@@ -753,6 +753,7 @@ typedef TileCfg<128, 256, 2, 2> Cfg128x256w4;
 void tile_variant_shape(int variant, int *bm, int *bn) {
   switch (variant) {
     case WAVE_MXFP4_VARIANT_T256x256_W2x2:
+    case WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT:
     case WAVE_MXFP4_VARIANT_T256x256_W4x2: *bm = 256; *bn = 256; break;
     case WAVE_MXFP4_VARIANT_T128x128_W2x2: *bm = 128; *bn = 128; break;
     case WAVE_MXFP4_VARIANT_T128x256_W2x2: *bm = 128; *bn = 256; break;

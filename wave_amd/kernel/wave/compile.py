@@ -9,6 +9,8 @@ selects one of them from the template's parameters."""
 
 from __future__ import annotations
 
+import dataclasses
+
 from dataclasses import dataclass, field
 from typing import Any
 
@@ -97,4 +99,12 @@ def wave_compile(options: WaveCompileOptions, kernel: KernelSpec, schedule=None)
     if not isinstance(kernel, KernelSpec):
         raise TypeError("wave_compile expects the kernel object returned by a template getter")
     _lib.load()  # fail here, not at first launch, if the HIP library is missing
+    # The asymmetric schedule of the reference (A through LDS, preshuffled B straight into registers,
+    # schedules/gemm_mxfp4_double_buffer.py:1781-2222) names a kernel of its own here: the B-direct variant, where
+    # the template's shape allows it (256 x 256 tiles, whole 256-column tiles, an even number of at least 6 K
+    # tiles); every other schedule is pipelining the hand-written kernels already fix.
+    if (getattr(schedule, "name", None) == "mxfp4_asymmetric" and kernel.b_layout == _lib.B_PRESHUFFLE
+            and kernel.num_splits <= 1 and tuple(kernel.block_shape[:2]) == (256, 256)
+            and kernel.shape[1] % 256 == 0 and kernel.shape[2] % 512 == 0 and kernel.shape[2] >= 1536):
+        kernel = dataclasses.replace(kernel, variant=_lib.VARIANT_T256x256_W1x4_BDIRECT)
     return WaveKernel(kernel, options, schedule)

@@ -38,6 +38,8 @@ WORKLOADS = {
     "cfg3_m1": (1, 28672, 8192, "bf16", 2, (120, 134)),
     "cfg3_m16": (16, 28672, 8192, "bf16", 2, (120, 134)),
     "cfg3_m32": (32, 28672, 8192, "bf16", 2, (120, 134)),
+    "cfg3_m64": (64, 28672, 8192, "bf16", 2, (120, 134)),
+    "cfg3_m128": (128, 28672, 8192, "bf16", 2, (120, 134)),
     "cfg5": (4093, 6144, 7168, "f32", 4, (100, 154)),
 }
 
@@ -570,7 +572,7 @@ def main():
     m, n, k, od, seed, srange = WORKLOADS[args.workload]
     out_dtype = torch.bfloat16 if od == "bf16" else torch.float32
     out_bytes = 2 if od == "bf16" else 4
-    memory_bound = m <= 64
+    memory_bound = m <= 128
     # memory-bound shapes rotate distinct operand sets so B is not cache resident
     copies = 4 if memory_bound else 1
     sets = make_gpu_inputs(torch, m, n, k, seed, srange, dev, copies=copies)
@@ -587,7 +589,8 @@ def main():
         achieved = nbytes / per_launch / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                     "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": measured_traffic,
-                    "kernel": "stream_gemm_kernel", "launch_us": round(per_launch * 1e6, 2)}
+                    "kernel": "stream_gemm_kernel" if m <= 48 else "mid_gemm_kernel",
+                    "launch_us": round(per_launch * 1e6, 2)}
     else:
         achieved = flops / per_launch / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_MXFP4_TFLOPS,
@@ -642,8 +645,8 @@ def main():
     del sets, out
 
     if not args.no_legs and args.workload == "cfg2":
-        # the decode shapes of the metric's second half: M = 16 (its target), and M = 1 and 32 beside it
-        for name in ("cfg3_m16", "cfg3_m1", "cfg3_m32"):
+        # the decode shapes of the metric's second half: M = 16 (its target), and M = 1, 32, 64 and 128 beside it
+        for name in ("cfg3_m16", "cfg3_m1", "cfg3_m32", "cfg3_m64", "cfg3_m128"):
             dm, dn, dk, _, dseed, drange = WORKLOADS[name]
             dsets = make_gpu_inputs(torch, dm, dn, dk, dseed, drange, dev, copies=4)
             dout = torch.empty(dm, dn, dtype=torch.bfloat16, device=dev)

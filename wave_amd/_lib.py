@@ -38,6 +38,7 @@ VARIANT_SKINNY = 4
 VARIANT_NAIVE = 5
 VARIANT_T128x256_W2x2 = 6
 VARIANT_T256x256_W1x4_BDIRECT = 7
+VARIANT_MID_M = 8
 
 # every symbol include/wave_mxfp4.h declares
 EXPORTS = (

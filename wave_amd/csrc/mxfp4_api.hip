@@ -97,12 +97,29 @@ bool is_tile_variant(int v) {
   return bm != 0;
 }
 
+// What the mid-M kernel takes (the part of it that the shape alone decides).
+bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
+  return m >= 1 && m <= mid_max_m() && k % kTileK == 0 && k >= 4 * kTileK && n % 4 == 0;
+}
+
 int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
   int v = variant;
-  if (v == WAVE_MXFP4_VARIANT_AUTO)
-    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
+  if (v == WAVE_MXFP4_VARIANT_AUTO) {
+    // 48 < M <= 256 and enough 128-column strips to put most CUs to work: reading B once from HBM bounds the
+    // problem, and the mid-M kernel gives B all of LDS.  Measured at K = 8192 against the streaming kernel
+    // (M <= 64) and the tile kernels: it wins from N = 14336 on for 64 < M <= 192 (128 x 28672: 46 -> 34 us,
+    // 128 x 12288 loses, 23 -> 26 us) and from about N = 24576 on at M = 64 (32 -> 30 us) and M = 256 (55 -> 51 us).
+    if (mid_shape_ok(m, n, k) && m > 48 && n >= ((m > 64 && m <= 192) ? 14336 : 24576)) return WAVE_MXFP4_VARIANT_MID_M;
+    if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;
+    v = pick_tile_variant(m, n);
+  }
   return v;
 }
+
+// Kernels that read both scale tensors in MFMA32 order (the library re-lays them out first when it has scratch).
+// The mid-M kernel also reads row-major scales as they are; only e8m0_shuffle order is re-laid out for it.
+bool wants_mfma32_scales(int v) { return is_tile_variant(v) || v == WAVE_MXFP4_VARIANT_MID_M; }
+bool mid_reads(int layout) { return layout == WAVE_MXFP4_SCALE_ROW_MAJOR || layout == WAVE_MXFP4_SCALE_MFMA32; }
 
 // A partial last K tile with scales that are not (or cannot be brought) in MFMA32 order is only built for the
 // 128x128 tile kernel.
@@ -226,7 +243,7 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
   int splits = split_k;
   if (splits == 0) splits = auto_split(m, n, k, v);
   if (splits > 1) bytes += round_up_256((size_t)splits * (size_t)m * (size_t)n * sizeof(float));
-  if (is_tile_variant(v)) bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
+  if (wants_mfma32_scales(v)) bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
   if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && n % 256 == 0 && splits <= 1) {
     // the parts of the tiles of a sparsely filled last round (persistent kernel)
     const int grid = device_cus() / 8 * 8;
@@ -253,8 +270,14 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
 
   GemmParams p;
   fill_params(p, a, a_scale, b, b_scale, c, m, n, k, out_dtype, a_scale_layout, b_scale_layout, b_layout);
-  const int v = pick_variant(m, n, k, variant);
+  int v = pick_variant(m, n, k, variant);
+  if (variant == WAVE_MXFP4_VARIANT_AUTO && v == WAVE_MXFP4_VARIANT_MID_M && split_k > 1)  // (it takes whole K ranges)
+    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
   if (v == WAVE_MXFP4_VARIANT_SKINNY && m > skinny_max_m()) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (variant == WAVE_MXFP4_VARIANT_MID_M) {
+    const bool native = (mid_reads(a_scale_layout) || a_scale_layout == WAVE_MXFP4_SCALE_PER_ROW) && mid_reads(b_scale_layout);
+    if (!mid_shape_ok(m, n, k) || split_k > 1 || (!native && !workspace)) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  }
   if (v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT) {
     // what the B-direct kernel takes, checked before anything is launched: preshuffled B, whole 256-column tiles,
     // an even number (at least 6) of K tiles, no split, scales in MFMA32 order or scratch to bring them there
@@ -314,10 +337,11 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   const bool small_short = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 && p.tiles_per_split <= (splits > 1 ? 12 : 16) &&
                            k % kTileK == 0 &&
                            p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
-  if (is_tile_variant(v) && workspace && !small_short) {
+  if (wants_mfma32_scales(v) && workspace && !small_short) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
-    const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? a_bytes : 0;
-    const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 ? b_bytes : 0;
+    const bool mid = v == WAVE_MXFP4_VARIANT_MID_M;
+    const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads(p.a_scale_layout)) ? a_bytes : 0;
+    const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads(p.b_scale_layout)) ? b_bytes : 0;
     if (ws_used + a_need + b_need <= workspace_bytes) {
       uint8_t *ws = (uint8_t *)workspace + ws_used;
       ws_scales_end = ws_used + a_need + b_need;
@@ -354,7 +378,15 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   }
 
   if (ws_scales_end < ws_used) ws_scales_end = ws_used;
-  if (v == WAVE_MXFP4_VARIANT_NAIVE) {
+  int vv = v;
+  if (vv == WAVE_MXFP4_VARIANT_MID_M && !mid_gemm_applies(p)) {
+    // (the library's own choice without scratch for the scales, or offsets beyond 32 bits: the tile kernels)
+    if (variant == WAVE_MXFP4_VARIANT_MID_M) return WAVE_MXFP4_ERR_UNSUPPORTED;
+    vv = pick_tile_variant(m, n);
+  }
+  if (vv == WAVE_MXFP4_VARIANT_MID_M) {
+    e = launch_mid_gemm(p, device_cus(), stream);
+  } else if (v == WAVE_MXFP4_VARIANT_NAIVE) {
     e = launch_naive_gemm(p, stream);
   } else if (v == WAVE_MXFP4_VARIANT_SKINNY) {
     // The streaming kernel keeps A in registers and serves up to 32 K tiles per
@@ -364,7 +396,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     if (e == hipErrorInvalidValue) e = launch_skinny_gemm(p, stream);
   } else {
     int bm, bn;
-    const int tv = needs_generic_k(p) ? WAVE_MXFP4_VARIANT_T128x128_W2x2 : v;
+    const int tv = needs_generic_k(p) ? WAVE_MXFP4_VARIANT_T128x128_W2x2 : vv;
     tile_variant_shape(tv, &bm, &bn);
     p.tiles_m = (int)((m + bm - 1) / bm);
     p.tiles_n = (int)((n + bn - 1) / bn);
@@ -520,9 +552,10 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   // every expert's B and B_scale must keep the base alignment
   if (p.b_group_stride % 16 != 0 || p.b_scale_group_stride % 8 != 0) return WAVE_MXFP4_ERR_MISALIGNED;
 
-  if (variant == WAVE_MXFP4_VARIANT_SKINNY || variant == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT)
+  if (variant == WAVE_MXFP4_VARIANT_SKINNY || variant == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT ||
+      variant == WAVE_MXFP4_VARIANT_MID_M)
     return WAVE_MXFP4_ERR_UNSUPPORTED;
-  const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_variant(total_rows > 64 ? total_rows : 65, n, k, variant)
+  const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_tile_variant(total_rows > 64 ? total_rows : 65, n)
                                                    : pick_variant(total_rows, n, k, variant);
   if (v == WAVE_MXFP4_VARIANT_NAIVE) return record_hip(launch_naive_gemm(p, stream));
   int bm, bn;

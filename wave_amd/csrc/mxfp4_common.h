@@ -133,6 +133,9 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus);
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream);
 bool asym_gemm_applies(const GemmParams &p, int num_cus, bool forced);
 hipError_t launch_asym_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
+bool mid_gemm_applies(const GemmParams &p);
+hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
+int mid_max_m();
 int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *partial_bytes);
 hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);
 hipError_t launch_scale_spread_rows(const uint8_t *src, uint8_t *dst, int64_t rows, int64_t ks, hipStream_t stream);

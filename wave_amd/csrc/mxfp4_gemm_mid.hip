@@ -1,0 +1,353 @@
+// Mid-M MXFP4 GEMM for gfx950 (MI355X): 16 < M <= 256 against a wide B that comes from HBM.
+//
+// Up to M of about 200 the operation is still bound by reading B once (2*M*N*K flops against N*K/2 bytes), but M
+// is too large for the streaming kernel's resident A (64 registers per 16 rows) and too small for the tile
+// kernels, whose ring gives B two K tiles of prefetch next to A's: one tile per CU then waits for memory latency
+// (128 x 28672 x 8192 ran at 2.9 TB/s there).  What this regime wants is all of LDS for B and a shallow, cheap
+// path for A, which comes from L2.  Vector memory operations of a wave retire in issue order, so a wave that
+// waits for a recent A tile also waits for every older B request: the two streams need different waves.
+//
+//   * One workgroup per 4 * WV columns of C: four compute waves side by side along N (WV <= 32 columns each, all
+//     BM = 64 .. 256 rows; v_mfma_scale_f32_32x32x64_f8f6f4, BM / 32 accumulator tiles) and a fifth, the
+//     producer wave, which does nothing but request A.  WV is chosen per problem so that the strips come out as
+//     a whole number of rounds over the CUs (N = 28672 on 256 CUs: 28 columns per wave, 256 workgroups, where
+//     strips of 128 columns would leave 32 CUs without work and the rest 14 % more): the rate at which one CU
+//     pulls from HBM is what bounds the kernel.  The rows of a wave's MFMA operand past WV are zero-filled by
+//     the buffer descriptor (no memory request) and their columns are not stored.
+//   * B is wave private: a compute wave fetches the 32 B rows it multiplies (4 DMA instructions of 8 rows x 128
+//     bytes per K tile, whole cache lines, non-temporal) into its own ring of DB K tiles and waits for its own
+//     requests only, with a counted vmcnt that leaves the younger DB - 2 K tiles in flight.  Its scales come in
+//     by one DMA instruction per FOUR K tiles: in MFMA32 order the blocks of consecutive K tiles are contiguous
+//     and a lane reads its dword; row-major scales are fetched as 32 rows x 32 bytes (two lanes per row) and a
+//     lane picks its four bytes of the row's eight with one v_perm, so neither order needs a pass of its own.
+//   * The producer wave fetches A (BM rows x 128 bytes per K tile) and its scales into a ring of DA K tiles,
+//     DA - 1 ahead, waits for its own requests, and meets the compute waves at one barrier per K tile: behind it
+//     A(j) is visible to all and the slot of A(j - 1) is free.
+//   * C leaves through the wave's own (by then idle) B ring, 64 or 128 bytes per row and store.
+//
+// Taken for K % 256 == 0 (at least 4 K tiles), N % 4 == 0, each scale tensor row-major or in MFMA32 order
+// (e8m0_shuffle order is re-laid out first when the library has scratch; B scales in MFMA32 order fix WV at 32,
+// the row block of that layout), B row-major or preshuffled.  The reference runs these shapes
+// through its generic tile kernel (tests/kernel/wave_gemm_mxfp_test.py:291-339); the result contract is the same.
+#include <type_traits>
+
+#include "mxfp4_tile_common.h"
+
+namespace wave_mxfp4 {
+
+namespace {
+
+constexpr int kMidBN = 128, kMidCW = 4, kMidNT = (kMidCW + 1) * 64;
+constexpr int kMidOnce = 2;  // the "nt" bit: B is read exactly once
+
+template <int BM_>
+struct MidCfg {
+  static constexpr int BM = BM_, MT_M = BM / 32;
+  static constexpr int A_SLOT = BM * kTileKBytes;
+  static constexpr int DA = BM <= 128 ? 3 : 2;                           // K tiles of A in LDS
+  static constexpr int DB = BM <= 64 ? 7 : BM <= 192 ? 5 : 4;            // K tiles of B in each wave's ring
+  static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
+  static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
+  static constexpr int A_RING = DA * A_SLOT, AS_RING = 2 * AS_SLOT;
+  static constexpr int B_WAVE = DB * 32 * kTileKBytes;                   // one wave's B ring (4 KB per K tile)
+  static constexpr int BS_WAVE = 4 * 1024;                               // one wave's scale ring: 4 groups of 4 K tiles
+  static constexpr int LDS = A_RING + AS_RING + kMidCW * (B_WAVE + BS_WAVE);
+  static constexpr int A_LD = BM / 8;                                    // A DMA instructions per K tile (producer)
+  static_assert(LDS <= 160 * 1024, "LDS");
+  static_assert(B_WAVE >= 32 * 32 * 4, "the C staging of a 32 x 32 f32 tile must fit the wave's ring");
+  static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
+};
+
+template <class Cfg>
+__device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
+  constexpr int MT_M = Cfg::MT_M, DA = Cfg::DA, DB = Cfg::DB, LB = Cfg::LB;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  uint8_t *const a_ring = smem;
+  uint8_t *const as_ring = smem + Cfg::A_RING;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kp = p.kp, nkt = p.k_tiles;
+  const int n0 = blockIdx.x * (kMidCW * wv);
+  const int k_tiles_blocks = nkt * 256;   // bytes of one 32-row block row of MFMA32 scales
+  const int groups = (nkt + 3) >> 2;      // scale groups of 4 K tiles
+  const bool a_rowmajor = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
+  const bool b_rowmajor = p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
+
+  if (wave == kMidCW) {
+    // ================= the producer wave: A and its scales =================
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(p.a, (int)min((int64_t)p.m * kp, (int64_t)0x7FFFFFFF));
+    const int64_t as_bytes = a_rowmajor ? (int64_t)p.m * p.ks : (int64_t)((p.m + 31) >> 5) * k_tiles_blocks;
+    const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc_n(p.a_scale, (int)min(as_bytes, (int64_t)0x7FFFFFFF));
+    const int row0 = lane >> 3;  // instruction d fills rows 8d .. 8d + 7
+    // chunk position lane % 8 of row r holds chunk (lane % 8) ^ ((r / 2) % 8); 8d is a multiple of 8, so the
+    // swizzle depends on the lane alone when d is even, and flips bit 2 of it when d is odd
+    const int goff_even = row0 * kp + (((lane & 7) ^ ((row0 >> 1) & 7)) << 4);
+    const int goff_odd = row0 * kp + (((lane & 7) ^ (((row0 + 8) >> 1) & 7)) << 4);
+    auto issue_a = [&](int kt, int slot) {
+      // past the last K tile: the same number of requests, from beyond the end of A (zeros into a slot nobody reads)
+      const int soff = kt < nkt ? kt * kTileKBytes : (int)0x80000000;
+#pragma unroll
+      for (int d = 0; d < Cfg::A_LD; ++d)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, WAVE_LDS_PTR(a_ring + slot * Cfg::A_SLOT + d * 1024), 16,
+                                                 (d & 1) ? goff_odd : goff_even, soff + d * 8 * kp, 0, 0);
+    };
+    // scales of K tiles 4g .. 4g + 3, 1 KB per 32 rows, MT_M instructions.  MFMA32 order: the four 256-byte blocks
+    // are contiguous (lane * 16).  Row-major: 32 bytes of each row; lane l fetches the half l / 32 of row l % 32
+    // and the image is half-major (half * 512 + row * 16).
+    const int as_goff = a_rowmajor ? (lane & 31) * p.ks + (lane >> 5) * 16 : lane * 16;
+    const int as_gstep = a_rowmajor ? 32 : 1024, as_istep = a_rowmajor ? 32 * p.ks : k_tiles_blocks;
+    auto issue_as = [&](int g) {
+      const int soff = g < groups ? g * as_gstep : (int)0x80000000;
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(as_rsrc, WAVE_LDS_PTR(as_ring + (g & 1) * Cfg::AS_SLOT + i * 1024), 16,
+                                                 as_goff, soff + i * as_istep, 0, 0);
+    };
+    // (a group's last K tiles may lie past K: those bytes belong to the next block or row, or lie past the
+    // buffer; nobody reads them)
+    // prologue: A(0 .. DA - 2), with the scale groups they belong to in front
+    issue_as(0);
+#pragma unroll
+    for (int j = 0; j < DA - 1; ++j) issue_a(j, j);
+    int slot_next = DA - 1;  // slot of the K tile requested next
+    for (int j = 0; j < nkt; ++j) {
+      // A(j) has landed: younger than it are A(j + 1 .. j + DA - 2) and at most one scale group
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((DA - 2) * Cfg::A_LD));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();  // A(j) visible to the compute waves; they are done with A(j - 1)
+      asm volatile("" ::: "memory");
+      const int jn = j + DA - 1;
+      if ((jn & 3) == 0) issue_as(jn >> 2);  // (group g's slot was last read in K tile 4g - 5 at the latest)
+      issue_a(jn, slot_next);
+      slot_next = slot_next + 1 == DA ? 0 : slot_next + 1;
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    return;
+  }
+
+  // ================= a compute wave =================
+  uint8_t *const b_ring = smem + Cfg::A_RING + Cfg::AS_RING + wave * (Cfg::B_WAVE + Cfg::BS_WAVE);
+  uint8_t *const bs_ring = b_ring + Cfg::B_WAVE;
+  const int nw0 = n0 + wave * wv;  // the wave's first column of C = first row of B
+  const int cols = max(0, min(wv, p.n - nw0));  // columns it owns
+  // B: the descriptor starts at the wave's first row (row-major) or at the 16-row block that holds it
+  // (preshuffled) and ends with B; rows past N read zeros, like the operand rows past the wave's own columns
+  const int b_blk = p.b_preshuffled ? (nw0 & ~15) : nw0, b_sub = nw0 - b_blk;
+  const int64_t b_bytes = (int64_t)p.n * kp - (int64_t)b_blk * kp;
+  const __amdgpu_buffer_rsrc_t b_rsrc =
+      make_rsrc_n(p.b + (int64_t)b_blk * kp, (int)min(max(b_bytes, (int64_t)0), (int64_t)0x7FFFFFFF));
+  // B scales: MFMA32 order from the wave's 32-row block on (there WV is 32), row-major from its first row on
+  const int64_t bs_skip = b_rowmajor ? (int64_t)nw0 * p.ks : (int64_t)(nw0 >> 5) * k_tiles_blocks;
+  const int64_t bs_bytes = (b_rowmajor ? (int64_t)p.n * p.ks : (int64_t)((p.n + 31) >> 5) * k_tiles_blocks) - bs_skip;
+  const __amdgpu_buffer_rsrc_t bs_rsrc =
+      make_rsrc_n(p.b_scale + bs_skip, (int)min(max(bs_bytes, (int64_t)0), (int64_t)0x7FFFFFFF));
+  // B DMA: instruction d fills rows 8d .. 8d + 7 of the wave's 32 (LDS: row * 128, swizzled chunks)
+  const int ld_row = lane >> 3;
+  int b_goff[4];
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const int r = d * 8 + ld_row, chunk = (lane & 7) ^ ((r >> 1) & 7), rb = r + b_sub;
+    const int off = p.b_preshuffled ? (rb >> 4) * 16 * kp + (rb & 15) * 16 + (chunk >> 1) * 512 + (chunk & 1) * 256
+                                    : r * kp + chunk * 16;
+    b_goff[d] = r < cols ? off : (int)0x80000000;  // past the wave's columns: out of range, zeros, no request
+  }
+  const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
+  auto issue_b = [&](int kt, int slot) {
+    const int soff = kt < nkt ? kt * b_kt_stride : (int)0x80000000;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(b_ring + slot * 4096 + d * 1024), 16, b_goff[d], soff,
+                                               0, kMidOnce);
+  };
+  const int bs_goff = b_rowmajor ? (lane & 31) * p.ks + (lane >> 5) * 16 : lane * 16;
+  const int bs_gstep = b_rowmajor ? 32 : 1024;
+  auto issue_bs = [&](int g) {
+    const int soff = g < groups ? g * bs_gstep : (int)0x80000000;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (g & 3) * 1024), 16, bs_goff, soff, 0, 0);
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  uint32_t foff[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) foff[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
+  // A lane's scale dword of a K tile holds the bytes of its K steps 0 .. 3: groups fg, 2 + fg, 4 + fg, 6 + fg of
+  // row fr.  MFMA32 order stores exactly that dword; from a row's eight bytes one v_perm picks it.
+  // (Branch-free on the layout: a branch in the K loop makes the compiler wait for every outstanding request at
+  // the join.)  The lane reads two dwords at c0 + (j % 2) * c1 + (j / 2 % 2) * 512 and permutes them by `pick`.
+  struct ScaleRead { int c0, c1, hi; uint32_t pick; };
+  auto scale_read = [&](bool rowmajor) -> ScaleRead {
+    if (rowmajor) return {fr * 16, 8, 4, fg ? 0x07050301u : 0x06040200u};
+    return {lane * 4, 256, 0, 0x03020100u};
+  };
+  const ScaleRead ra = scale_read(a_rowmajor), rb = scale_read(b_rowmajor);
+  auto lane_scales = [&](const uint8_t *img, const ScaleRead &r, int j) -> uint32_t {
+    const uint8_t *at = img + r.c0 + (j & 1) * r.c1 + ((j & 2) << 8);
+    return __builtin_amdgcn_perm(*(const uint32_t *)(at + r.hi), *(const uint32_t *)at, r.pick);
+  };
+
+  v16f acc[MT_M];
+#pragma unroll
+  for (int i = 0; i < MT_M; ++i)
+#pragma unroll
+    for (int g = 0; g < 16; ++g) acc[i][g] = 0.f;
+
+  // prologue: B(0 .. LB - 1) with the scale groups they belong to in front
+#pragma unroll
+  for (int j = 0; j < LB; ++j) {
+    if ((j & 3) == 0) issue_bs(j >> 2);
+    issue_b(j, j);
+  }
+  int slot = 0, slot_next = LB;  // slots of B(j) and of the K tile requested next
+  int a_slot = 0;
+  typedef std::integral_constant<int, 0> T0;
+  typedef std::integral_constant<int, 1> T1;
+  typedef std::integral_constant<int, 2> T2;
+  typedef std::integral_constant<int, 3> T3;
+  for (int j = 0; j < nkt; ++j) {
+    // B(j) and its scales have landed: younger are B(j + 1 .. j + LB - 1), 4 requests each (and up to two scale
+    // groups, which the count leaves out: it then waits for that much more than it must)
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(4 * (LB - 1)));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();  // A(j) is in LDS
+    asm volatile("" ::: "memory");
+    // the slot of B(j - 1) is free (its fragments were consumed before the wait above): request B(j + LB)
+    const int jn = j + LB;
+    if ((jn & 3) == 0) issue_bs(jn >> 2);
+    issue_b(jn, slot_next);
+    slot_next = slot_next + 1 == DB ? 0 : slot_next + 1;
+
+    const uint8_t *a_t = a_ring + a_slot * Cfg::A_SLOT, *b_t = b_ring + slot * 4096;
+    uint32_t sa[MT_M];
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) sa[i] = lane_scales(as_ring + ((j >> 2) & 1) * Cfg::AS_SLOT + i * 1024, ra, j);
+    const uint32_t sb = lane_scales(bs_ring + ((j >> 2) & 3) * 1024, rb, j);
+    auto step = [&](auto t_tag) {
+      constexpr int T = decltype(t_tag)::value;
+      const v4i fb = *(const v4i *)(b_t + foff[T]);
+      const v8i vb = {fb.x, fb.y, fb.z, fb.w, 0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) {
+        const v4i fa = *(const v4i *)(a_t + i * 32 * kTileKBytes + foff[T]);
+        const v8i va = {fa.x, fa.y, fa.z, fa.w, 0, 0, 0, 0};
+        acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i], 4, 4, T, (int)sb, T, (int)sa[i]);
+      }
+    };
+    step(T0{});
+    step(T1{});
+    step(T2{});
+    step(T3{});
+    slot = slot + 1 == DB ? 0 : slot + 1;
+    a_slot = a_slot + 1 == DA ? 0 : a_slot + 1;
+  }
+  // the trailing (empty) requests must have landed before the ring becomes the C staging area
+  __builtin_amdgcn_s_waitcnt(0);
+  asm volatile("" ::: "memory");
+
+  // ---------------- C: accumulators -> the wave's ring -> global ----------------
+  // acc[i][4q + e] is row lane % 32, column 8q + 4 * (lane / 32) + e of the wave's strip, row block i.  The strip
+  // is staged as 32 rows of eight 4-column pieces and stored 8 rows per instruction, a lane one piece (8 bytes of
+  // bf16, 16 of f32), the pieces past the wave's columns left out.
+  uint8_t *stage = b_ring;
+  const bool out_bf16 = p.out_bf16 != 0;
+  const int elt = out_bf16 ? 2 : 4;
+  const __amdgpu_buffer_rsrc_t c_rsrc =
+      make_rsrc_n(p.c, (int)min((int64_t)p.m * p.n * elt, (int64_t)0x7FFFFFFF));
+  if (cols <= 0) return;
+  const int lr = lane >> 3, lc = lane & 7;
+  const bool mine = lc * 4 < cols;
+  if (out_bf16) {
+    typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bf4 h = {(__bf16)acc[i][4 * q], (__bf16)acc[i][4 * q + 1], (__bf16)acc[i][4 * q + 2], (__bf16)acc[i][4 * q + 3]};
+        *(bf4 *)(stage + fr * 64 + (((q * 2 + fg) ^ ((fr >> 2) & 7)) << 3)) = h;
+      }
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int r0 = 0; r0 < 32; r0 += 8) {
+        const int r = r0 + lr, row = i * 32 + r;
+        const v2i v = *(const v2i *)(stage + r * 64 + ((lc ^ ((r >> 2) & 7)) << 3));
+        // rows past M lie past the end of C: dropped by the descriptor
+        if (mine) __builtin_amdgcn_raw_buffer_store_b64(v, c_rsrc, (int)(((int64_t)row * p.n + nw0 + lc * 4) * 2), 0, 0);
+      }
+      asm volatile("" ::: "memory");
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MT_M; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4f v = {acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
+        const int chunk = q * 2 + fg;
+        *(v4f *)(stage + fr * 128 + ((chunk ^ (fr & 7)) << 4)) = v;
+      }
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int r0 = 0; r0 < 32; r0 += 8) {
+        const int r = r0 + lr, row = i * 32 + r;
+        const v4f v = *(const v4f *)(stage + r * 128 + ((lc ^ (r & 7)) << 4));
+        if (mine)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc,
+                                                 (int)(((int64_t)row * p.n + nw0 + lc * 4) * 4), 0, 0);
+      }
+      asm volatile("" ::: "memory");
+    }
+  }
+}
+
+template <class Cfg>
+__global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p, const int wv) {
+  mid_body<Cfg>(p, wv);
+}
+
+template <class Cfg>
+hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg>, Cfg::LDS);
+  if (e != hipSuccess) return e;
+  const int bn = kMidCW * wv;
+  mid_gemm_kernel<Cfg><<<dim3((p.n + bn - 1) / bn, 1, 1), dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
+  return hipGetLastError();
+}
+
+// Columns per compute wave: the narrowest strips (a multiple of 4 columns, 16 to 32) that still fit the number of
+// rounds which strips of 128 columns would take on this many CUs.  B scales in MFMA32 order come in blocks of 32
+// rows, so there a wave's strip is a block.
+int mid_wave_cols(const GemmParams &p, int num_cus) {
+  if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR || num_cus <= 0) return 32;
+  const int64_t strips = (p.n + kMidBN - 1) / kMidBN;
+  const int64_t wgs = (strips + num_cus - 1) / num_cus * num_cus;
+  int64_t wv = (p.n + 4 * wgs - 1) / (4 * wgs);
+  wv = (wv + 3) / 4 * 4;
+  return (int)(wv < 16 ? 16 : wv > 32 ? 32 : wv);
+}
+
+}  // namespace
+
+int mid_max_m() { return 256; }
+
+// Whether the mid-M kernel serves this problem.
+bool mid_gemm_applies(const GemmParams &p) {
+  if (p.num_groups != 0 || p.splits != 1 || p.partial != nullptr || p.m < 1 || p.m > mid_max_m()) return false;
+  const auto layout_ok = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
+  if (!layout_ok(p.a_scale_layout) || !layout_ok(p.b_scale_layout)) return false;
+  if ((p.k & (kTileK - 1)) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
+  // 32-bit offsets: inside A, inside a wave's 48 rows of B, inside C, inside the scales of A and of a wave's rows
+  if ((int64_t)p.m * p.kp >= ((int64_t)1 << 31) || (int64_t)48 * p.kp >= ((int64_t)1 << 31) ||
+      (int64_t)p.m * p.n * 4 >= ((int64_t)1 << 31) || (int64_t)8 * p.k_tiles * 256 >= ((int64_t)1 << 31))
+    return false;
+  return true;
+}
+
+hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream) {
+  const int wv = mid_wave_cols(p, num_cus);
+  if (p.m <= 64) return launch_mid_cfg<MidCfg<64>>(p, wv, stream);
+  if (p.m <= 128) return launch_mid_cfg<MidCfg<128>>(p, wv, stream);
+  if (p.m <= 192) return launch_mid_cfg<MidCfg<192>>(p, wv, stream);
+  return launch_mid_cfg<MidCfg<256>>(p, wv, stream);
+}
+
+}  // namespace wave_mxfp4

@@ -102,6 +102,13 @@ typedef enum {
    * otherwise.  AUTO takes it for 48 < M <= 256 and a wide N.  The reference runs such shapes through its generic
    * tile kernel (tests/kernel/wave_gemm_mxfp_test.py:291-339). */
   WAVE_MXFP4_VARIANT_MID_M = 8,
+  /* 256x192x256 tile, 8 waves, persistent kernel only: for problems whose count of 256x256 tiles leaves the last
+   * round over the CUs partly empty while 256x192 tiles fill whole rounds (4093 x 6144: 384 tiles are 1.5 rounds
+   * of 256 CUs, 512 tiles of 256x192 are 2 rounds of three quarters the work each).  Needs N % 192 == 0, more
+   * tiles than CUs, K >= 768 and scales in MFMA32 order or the workspace; WAVE_MXFP4_ERR_UNSUPPORTED otherwise.
+   * AUTO takes it when its rounds cost less.  The reference fixes one block shape per compiled kernel
+   * (wave_lang/kernel/wave/templates/tagged_mxfp4_gemm.py:38-145); picking it per problem is the library's. */
+  WAVE_MXFP4_VARIANT_T256x192_W4x2 = 9,
   WAVE_MXFP4_VARIANT_COUNT_
 } wave_mxfp4_variant;
 

@@ -39,6 +39,7 @@ VARIANT_NAIVE = 5
 VARIANT_T128x256_W2x2 = 6
 VARIANT_T256x256_W1x4_BDIRECT = 7
 VARIANT_MID_M = 8
+VARIANT_T256x192_W4x2 = 9
 
 # every symbol include/wave_mxfp4.h declares
 EXPORTS = (

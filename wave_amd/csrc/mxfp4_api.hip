@@ -287,6 +287,14 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
       return WAVE_MXFP4_ERR_UNSUPPORTED;
   }
 
+  if (v == WAVE_MXFP4_VARIANT_T256x192_W4x2) {
+    // the 256x192 tiles exist in the persistent kernel only: whole tiles along N, more tiles than CUs, no split
+    const bool native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+    const int grid = device_cus() / 8 * 8;
+    if (n % 192 != 0 || k < 768 || split_k > 1 || (!native && !workspace) || ((m + 255) / 256) * (n / 192) <= grid)
+      return WAVE_MXFP4_ERR_UNSUPPORTED;
+  }
+
   if (k == 0) return record_hip(launch_naive_gemm(p, stream));  // empty reduction: C = 0
 
   int splits = 1;
@@ -408,12 +416,24 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     } else if (persist_gemm_applies(p, tv, device_cus())) {
       // a last round of tiles that would leave most workgroups idle is cut along K instead, if there is scratch
       size_t part_bytes = 0;
-      const int parts = persist_tail_parts(p, tv, device_cus(), &part_bytes);
-      if (parts > 1 && workspace && ws_scales_end + part_bytes <= workspace_bytes) {
-        p.tail_parts = parts;
-        p.tail_partial = (float *)((uint8_t *)workspace + ws_scales_end);
+      int parts = persist_tail_parts(p, tv, device_cus(), &part_bytes);
+      if (!(parts > 1 && workspace && ws_scales_end + part_bytes <= workspace_bytes)) parts = 1;
+      GemmParams p192 = p;
+      p192.tiles_n = (int)(n / 192);
+      if (variant == WAVE_MXFP4_VARIANT_AUTO && tv == WAVE_MXFP4_VARIANT_T256x256_W4x2 &&
+          persist_prefers_192(p, device_cus(), parts) &&
+          persist_gemm_applies(p192, WAVE_MXFP4_VARIANT_T256x192_W4x2, device_cus())) {
+        // narrower tiles that fill whole rounds over the CUs
+        e = launch_persist_gemm(p192, WAVE_MXFP4_VARIANT_T256x192_W4x2, device_cus(), stream);
+      } else {
+        if (parts > 1) {
+          p.tail_parts = parts;
+          p.tail_partial = (float *)((uint8_t *)workspace + ws_scales_end);
+        }
+        e = launch_persist_gemm(p, tv, device_cus(), stream);
       }
-      e = launch_persist_gemm(p, tv, device_cus(), stream);
+    } else if (tv == WAVE_MXFP4_VARIANT_T256x192_W4x2) {
+      return WAVE_MXFP4_ERR_UNSUPPORTED;  // (no one-tile-per-workgroup kernel of that shape)
     } else {
       e = launch_tile_gemm(p, tv, stream);
     }
@@ -553,7 +573,7 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   if (p.b_group_stride % 16 != 0 || p.b_scale_group_stride % 8 != 0) return WAVE_MXFP4_ERR_MISALIGNED;
 
   if (variant == WAVE_MXFP4_VARIANT_SKINNY || variant == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT ||
-      variant == WAVE_MXFP4_VARIANT_MID_M)
+      variant == WAVE_MXFP4_VARIANT_MID_M || variant == WAVE_MXFP4_VARIANT_T256x192_W4x2)
     return WAVE_MXFP4_ERR_UNSUPPORTED;
   const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_tile_variant(total_rows > 64 ? total_rows : 65, n)
                                                    : pick_variant(total_rows, n, k, variant);

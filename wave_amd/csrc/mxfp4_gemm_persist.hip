@@ -136,7 +136,10 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       as_lim[which] = (int)min((int64_t)(m_blocks - (m0[which] >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
     }
     a_base[which] = p.a + (int64_t)m0[which] * kp;
-    a_lim[which] = (int)min((int64_t)max(p.m - m0[which], 0) * kp, (int64_t)0x7FFFFFFF);
+    // (grouped: A ends with the tile's own rows.  The rows of the next group would do as padding, their results
+    // are dropped, but zeros cost the matrix pipes far less power than data does, and power is what bounds the
+    // kernel.)
+    a_lim[which] = (int)min((int64_t)max(GROUPED ? c_rows[which] : p.m - m0[which], 0) * kp, (int64_t)0x7FFFFFFF);
     if (SPLIT) {  // the item's K range starts at K tile kt_lo: move the bases there
       a_base[which] += kt_lo * kTileKBytes;
       a_lim[which] = max(a_lim[which] - kt_lo * kTileKBytes, 0);
@@ -243,7 +246,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   typedef std::integral_constant<int, 2> T2;
   typedef std::integral_constant<int, 3> T3;
 
-  constexpr int HALF_LD = (A_LD < B_LD ? A_LD : B_LD) / 2;
+  constexpr int HALF_LD = (A_LD > B_LD ? A_LD : B_LD) / 2;
   constexpr int NGROUP = HALF_LD < 1 ? 1 : HALF_LD;
   auto order_phase = [&]() {
     constexpr int R = MT_M + MT_N, Q = MT_M * MT_N;
@@ -350,6 +353,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const int wr0 = wave_m * Cfg::WM;  // the wave's first row inside the tile
     if (out_bf16) {
       constexpr int CP = RP / 2, JP = CP / 32;  // columns, 32-column tiles per pass
+      constexpr int REM = MT_N % JP;            // 32-column tiles left for a narrower last pass
+      static_assert(REM == 0 || (JP == 2 && REM == 1), "odd wave tiles: 8-wave configurations only");
       typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) {
@@ -371,6 +376,25 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
             const int r = r0 + lr;
             const v4i v = *(const v4i *)(stage + r * RP + ((lc ^ (r & (NCH - 1))) << 4));
             __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, ((wr0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 8) * 2,
+                                                       0, 0);
+          }
+          asm volatile("" ::: "memory");
+        }
+        if constexpr (REM != 0) {
+          // the last 32 columns: rows of 64 bytes, four lanes a row, 16 rows per store instruction
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const v16f &a = acc[i][MT_N - 1];
+            const bf4 h = {(__bf16)a[4 * q], (__bf16)a[4 * q + 1], (__bf16)a[4 * q + 2], (__bf16)a[4 * q + 3]};
+            *(bf4 *)(stage + fr * RP + ((q ^ (fr & (NCH - 1))) << 4) + fg * 8) = h;
+          }
+          asm volatile("" ::: "memory");
+          const int lr4 = lane_v >> 2, lc4 = lane_v & 3;
+#pragma unroll
+          for (int r0 = 0; r0 < 32; r0 += 16) {
+            const int r = r0 + lr4;
+            const v4i v = *(const v4i *)(stage + r * RP + ((lc4 ^ (r & (NCH - 1))) << 4));
+            __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, ((wr0 + i * 32 + r) * ldc + wn0 + (MT_N - 1) * 32 + lc4 * 8) * 2,
                                                        0, 0);
           }
           asm volatile("" ::: "memory");
@@ -537,7 +561,7 @@ static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_
 template <class Cfg, bool OUT_BF16>
 static hipError_t launch_persist_dense(const GemmParams &p, int grid_x, hipStream_t stream) {
   const bool tail = (p.k & (kTileK - 1)) != 0;
-  if constexpr (Cfg::NWAVES == 8) {  // (the 4-wave kernel has no registers to spare for the split bookkeeping)
+  if constexpr (Cfg::NWAVES == 8 && Cfg::BN == 256) {  // (the 4-wave kernel has no registers to spare for the split bookkeeping)
     if (p.tail_parts > 1)
       return tail ? launch_persist_out<Cfg, OUT_BF16, false, true, true>(p, grid_x, stream)
                   : launch_persist_out<Cfg, OUT_BF16, false, false, true>(p, grid_x, stream);
@@ -580,13 +604,36 @@ int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *pa
   return parts;
 }
 
+// Whether 256x192 tiles serve a dense problem better than 256x256 tiles.  The kernels are bound by power, not by
+// issue slots, so a partly filled last round costs less than a full one: measured on both tile shapes over the
+// reference's shape list (K = 16000), a last round that gives a fraction f of the workgroups a tile takes
+// 0.4 + 0.6 f of a full round's time (about 1 / parts + 0.2, at least 0.4, when its tiles are cut along K into
+// `parts256` parts instead), and a round of 256x192 tiles 0.785 of a round of 256x256 tiles.  With fewer than 8 tile rows the wider tiles kept
+// their lead (1024 x 24576: the XCDs' bands of the tile walk are 8 tile rows high).
+bool persist_prefers_192(const GemmParams &p, int num_cus, int parts256) {
+  if (p.num_groups != 0 || p.n % 192 != 0 || p.splits != 1) return false;
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  if (grid < kNumXcd) return false;
+  const int64_t tm = (p.m + 255) / 256, t256 = tm * ((p.n + 255) / 256), t192 = tm * (p.n / 192);
+  if (t192 <= grid || tm < 8) return false;
+  const auto rounds = [grid](int64_t tiles, int parts) {
+    const double f = (double)(tiles % grid) / grid;
+    const double cut = 1.0 / parts + 0.2;
+    return (double)(tiles / grid) + (f == 0.0 ? 0.0 : parts > 1 ? (cut > 0.4 ? cut : 0.4) : 0.4 + 0.6 * f);
+  };
+  return 0.785 * rounds(t192, 1) < 0.95 * rounds(t256, parts256);
+}
+
 // Whether the persistent kernel serves this problem with `num_cus` CUs.
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
-  if (variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 && variant != WAVE_MXFP4_VARIANT_T256x256_W4x2) return false;
+  if (variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 && variant != WAVE_MXFP4_VARIANT_T256x256_W4x2 &&
+      variant != WAVE_MXFP4_VARIANT_T256x192_W4x2)
+    return false;
+  const int bn = variant == WAVE_MXFP4_VARIANT_T256x192_W4x2 ? 192 : 256;
   // (a grouped problem comes with its M tile table and per-tile A scales, or not at all)
   if ((p.num_groups != 0) != (p.tile_table != nullptr) || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
-  if ((p.n & 255) != 0 || p.k_tiles < 3) return false;  // any M
+  if (p.n % bn != 0 || p.tiles_n != p.n / bn || p.k_tiles < 3) return false;  // any M
   // a partial last K tile: dense problems with at least four K tiles
   if ((p.k & (kTileK - 1)) != 0 && (p.num_groups != 0 || p.k_tiles < 4)) return false;
   if (p.out_bf16 ? (p.n & 7) != 0 : (p.n & 3) != 0) return false;
@@ -601,6 +648,7 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream) {
   const int grid = num_cus / kNumXcd * kNumXcd;
   if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_persist_cfg<TileCfg<256, 256, 2, 2>>(p, grid, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T256x192_W4x2) return launch_persist_cfg<TileCfg<256, 192, 4, 2>>(p, grid, stream);
   return launch_persist_cfg<TileCfg<256, 256, 4, 2>>(p, grid, stream);
 }
 

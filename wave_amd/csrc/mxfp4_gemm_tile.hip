@@ -757,6 +757,7 @@ void tile_variant_shape(int variant, int *bm, int *bn) {
     case WAVE_MXFP4_VARIANT_T256x256_W4x2: *bm = 256; *bn = 256; break;
     case WAVE_MXFP4_VARIANT_T128x128_W2x2: *bm = 128; *bn = 128; break;
     case WAVE_MXFP4_VARIANT_T128x256_W2x2: *bm = 128; *bn = 256; break;
+    case WAVE_MXFP4_VARIANT_T256x192_W4x2: *bm = 256; *bn = 192; break;  // (persistent kernel only)
     default: *bm = 0; *bn = 0; break;
   }
 }

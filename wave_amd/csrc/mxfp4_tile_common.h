@@ -20,7 +20,7 @@ struct TileCfg {
   static constexpr int LDS_BYTES = RING_SLOTS * SLOT_BYTES;
   // One DMA instruction of a wave fills 8 LDS rows (64 lanes x 16 B).
   static constexpr int A_LD = BM / 8 / NWAVES, B_LD = BN / 8 / NWAVES;
-  static_assert(BM % (16 * NWAVES) == 0 && BN % (16 * NWAVES) == 0, "half operand tiles must split over waves");
+  static_assert(BM % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0, "operand tiles must split over the waves' DMA instructions");
   static_assert(LDS_BYTES <= 160 * 1024, "ring does not fit LDS");
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be MFMA aligned");
 };

@@ -432,6 +432,27 @@ def main():
 
     if args.workload == "mfma_ceiling":
         rows, best = mfma_ceiling(torch, dev, args.steps, args.warmup)
+        # the GEMM kernels themselves at 8192^3 on the seeded random operands and on all-zero operands (scales in
+        # MFMA order, no pre-pass): the same instruction stream and memory traffic, only the power per instruction
+        # differs; and with B preshuffled, the B-direct kernel
+        from wave_amd import _lib as L
+        gm = gn = gk = 8192
+        (gx, gxs, gw, gws), = make_gpu_inputs(torch, gm, gn, gk, 1, (124, 130), dev)
+        gxs = wave_amd.scale_convert(gxs, gm, gk // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
+        gws = wave_amd.scale_convert(gws, gn, gk // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
+        gout = torch.empty(gm, gn, dtype=torch.bfloat16, device=dev)
+        gemm_rows = []
+        for kernel, b_layout, bmat in (("persist_gemm_kernel", L.B_ROW_MAJOR, gw),
+                                       ("asym_gemm_kernel", L.B_PRESHUFFLE, wave_amd.b_preshuffle(gw))):
+            for data, xa, wb in (("random", gx, bmat), ("zeros", torch.zeros_like(gx), torch.zeros_like(bmat))):
+                _, per, settle_ms = time_gemm(torch, wave_amd, [(xa, gxs, wb, gws)], gout, args.steps, args.warmup,
+                                              a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32,
+                                              b_layout=b_layout)
+                tf = gemm_flops(gm, gn, gk) / per / 1e12
+                gemm_rows.append({"kernel": kernel, "operands": data, "launch_us": round(per * 1e6, 2),
+                                  "tflops": round(tf, 1), "frac_of_mxfp4_peak": round(tf / PEAK_MXFP4_TFLOPS, 4),
+                                  "frac_of_mfma_alone": round(tf / max(r["tflops"] for r in rows if r["operands"] == data), 4),
+                                  "settle_ms": round(settle_ms, 1)})
         print(json.dumps(dict(common, **{
             "metric": "scaled FP4 MFMA alone (v_mfma_scale_f32_32x32x64_f8f6f4, no memory traffic), TFLOP/s on random operands",
             "value": best, "unit": "TFLOP/s", "ms_per_step": min(r["launch_ms"] for r in rows if r["operands"] == "random"),
@@ -439,7 +460,7 @@ def main():
             "config": {"workload": "mfma_ceiling: one workgroup per CU, 4 or 8 waves, 8000 x 32 MFMAs per wave and launch"},
             "roofline": {"bound": "mfma", "achieved": best, "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(best / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "mfma_probe_kernel"},
-            "runs": rows})))
+            "runs": rows, "gemm_8192": gemm_rows})))
         return
 
     if args.workload == "quant_bf16":

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # WAVE_MXFP4_LIB points at another build of the same ABI (e.g. an experiment)
 LIB_PATH = os.environ.get("WAVE_MXFP4_LIB") or os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 # status codes of include/wave_mxfp4.h
 OK = 0

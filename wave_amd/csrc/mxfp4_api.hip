@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 8;
+constexpr int kAbiVersion = 9;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.

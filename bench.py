@@ -302,7 +302,7 @@ def leg_mxfp8(torch, wave_amd, dev, steps, warmup, variant=0):
 
     wall, per, settle_ms = timed(torch, run, steps, warmup)
     flops = 2.0 * m * n * k
-    return {"workload": f"mxfp8: M={m} N={n} K={k} e5m2 x e5m2, f32 out, seed 5", "kernel": "tile_gemm_kernel (8-bit operands)",
+    return {"workload": f"mxfp8: M={m} N={n} K={k} e5m2 x e5m2, f32 out, seed 5", "kernel": "persist_gemm_fp8_kernel",
             "launch_us": round(per * 1e6, 2), "tflops": round(flops / per / 1e12, 1),
             "frac_of_mxfp8_peak": round(flops / per / 1e12 / PEAK_MXFP8_TFLOPS, 4), "settle_ms": round(settle_ms, 1),
             "wall_s_per_step": wall / steps}

@@ -66,6 +66,26 @@ def test_mxfp8_mixed_formats_against_oracle(m, n, k, vname, fmt):
     assert_f32_close(run(x, xs, w_t, ws, fmt, variant=VARIANTS[vname]), ref, f"{vname} {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fmt", [o8.E5M2, (o8.E4M3, o8.E5M2)], ids=["e5m2", "e4m3_x_e5m2"])
+@pytest.mark.parametrize("m,n,k", [(4352, 4096, 512), (4100, 4352, 1024)])
+def test_mxfp8_more_tiles_than_cus(m, n, k, fmt, out_dtype):
+    """272 and 289 tiles of 256x256 on 256 CUs: with the scratch buffer the persistent kernel walks two tiles per
+    workgroup and its request stream runs across the tile boundary; without it every tile has its own workgroup and
+    the scales are read as given.  Same products in the same order: the same bits (checked in run()); rows of every
+    M tile against the oracle."""
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=m + k, fmt=fmt, scale_lo=120, scale_hi=134)
+    c = run(x, xs, w_t, ws, fmt, out_dtype=out_dtype)
+    rows = np.unique(np.concatenate([np.arange(0, m, 31), [m - 1, 255, 256]]))
+    ref = o8.scaled_gemm_mxfp8(x[rows], w_t, xs[rows], ws, fmt)
+    if out_dtype == torch.bfloat16:
+        # one bf16 ulp on top of what the f32 sums are allowed (1e-4 * max|Cref| with scales spread this wide)
+        tol = 2.0 ** -7 * np.abs(ref) + 1e-4 * np.abs(ref).max()
+        assert (np.abs(c[rows] - ref) <= tol).all(), f"{m}x{n}x{k}: beyond one bf16 ulp + 1e-4 * max"
+    else:
+        assert_f32_close(c[rows], ref, f"{m}x{n}x{k}")
+
+
 def test_mxfp8_mixed_formats_from_torch_dtypes():
     """float8 tensors carry their own format: e4m3 activations against e5m2 weights, exact on one-hot rows."""
     m, n, k = 128, 96, 256

@@ -527,6 +527,9 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
     p.b_scale = (const uint8_t *)workspace + a_bytes;
     p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
   }
+  // large dense problems on the 8-wave tiles with re-laid scales: the persistent kernel
+  if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && persist_gemm_fp8_applies(p, device_cus()))
+    return record_hip(launch_persist_gemm_fp8(p, device_cus(), a_format == WAVE_MXFP8_E5M2, b_format == WAVE_MXFP8_E5M2, stream));
   return record_hip(launch_tile_gemm_fp8(p, v, a_format == WAVE_MXFP8_E5M2, b_format == WAVE_MXFP8_E5M2, stream));
 }
 

@@ -53,8 +53,14 @@ enum KtKind {
 // workgroup (its last item); the parts go to p.tail_partial as f32 tiles and a
 // small kernel adds them up.  A 288-tile problem on 256 CUs then takes 1 + 1/8
 // tile times instead of 2.
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
+// FMT_A / FMT_B: element format codes of the scaled MFMA, 4 = e2m1 (MXFP4); 0 = e4m3, 1 = e5m2 (MXFP8, both
+// operands 8-bit: a 128-byte K tile is then 128 elements = two 64-deep K steps of 32 bytes per lane, the MFMA
+// takes 64 cycles instead of 32, and one MFMA32 scale block serves two K tiles; dense, whole K tiles, no cut).
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, int FMT_A = 4, int FMT_B = 4>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
+  constexpr bool FP8 = FMT_A != 4;
+  static_assert((FMT_A == 4) == (FMT_B == 4), "MXFP4 x MXFP8 operands are not built");
+  static_assert(!FP8 || (!GROUPED && !TAIL && !SPLIT), "MXFP8: dense problems with whole K tiles");
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
   constexpr int SLOT = Cfg::SLOT_BYTES, RING = Cfg::RING_SLOTS;
@@ -183,61 +189,97 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
 
   // ---------------- fragments ----------------
   const int fr = lane & 31, fg = lane >> 5;
+  // (MXFP8: K step s takes 32 bytes per lane in two halves, chunks 4s + fg and 4s + 2 + fg; foff[2s + h] is half h)
   uint32_t foff[4];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) foff[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
+  for (int t = 0; t < 4; ++t) {
+    const int chunk = FP8 ? (t >> 1) * 4 + (t & 1) * 2 + fg : t * 2 + fg;
+    foff[t] = (uint32_t)(fr * kTileKBytes + ((chunk ^ ((fr >> 1) & 7)) << 4));
+  }
   const uint32_t a_fbase = (uint32_t)(wave_m * Cfg::WM * kTileKBytes);
   const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
-  auto read_frags = [&](int slot_a, int slot_b, int t, v4i(&fa)[MT_M], v4i(&fb)[MT_N]) {
-    const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
-    const uint8_t *bb = smem + slot_b * SLOT + b_fbase + foff[t];
+  typedef typename std::conditional<FP8, v8i, v4i>::type Frag;
+  auto read_frags = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], Frag(&fb)[MT_N]) {
+    if constexpr (FP8) {
+      const uint8_t *ta = smem + slot_a * SLOT + a_fbase, *tb = smem + slot_b * SLOT + b_fbase;
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(ba + i * 32 * kTileKBytes);
+      for (int i = 0; i < MT_M; ++i) {
+        const v4i lo = *(const v4i *)(ta + foff[2 * t] + i * 32 * kTileKBytes);
+        const v4i hi = *(const v4i *)(ta + foff[2 * t + 1] + i * 32 * kTileKBytes);
+        fa[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
 #pragma unroll
-    for (int j = 0; j < MT_N; ++j) fb[j] = *(const v4i *)(bb + j * 32 * kTileKBytes);
+      for (int j = 0; j < MT_N; ++j) {
+        const v4i lo = *(const v4i *)(tb + foff[2 * t] + j * 32 * kTileKBytes);
+        const v4i hi = *(const v4i *)(tb + foff[2 * t + 1] + j * 32 * kTileKBytes);
+        fb[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      }
+    } else {
+      const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
+      const uint8_t *bb = smem + slot_b * SLOT + b_fbase + foff[t];
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(ba + i * 32 * kTileKBytes);
+#pragma unroll
+      for (int j = 0; j < MT_N; ++j) fb[j] = *(const v4i *)(bb + j * 32 * kTileKBytes);
+    }
   };
 
   // ---------------- scales (MFMA-native order: one dword per lane, 32 rows and K tile) ----------------
   const int a_srow = ((wave_m * Cfg::WM) >> 5) * k_tiles_blocks, b_srow = ((wave_n * Cfg::WN) >> 5) * k_tiles_blocks;
   const int s_lane = lane * 4;
   uint32_t raw_a[MT_M], raw_b[MT_N], sc_a[MT_M], sc_b[MT_N];
+  auto sblk = [](int kt) { return FP8 ? kt >> 1 : kt; };  // MXFP8: one MFMA32 block serves two K tiles
   auto load_scales = [&](int which, int kt) {
     const __amdgpu_buffer_rsrc_t ra = make_rsrc_n(as_base[which], as_lim[which]), rb = make_rsrc(bs_base[which]);
 #pragma unroll
     for (int i = 0; i < MT_M; ++i)
-      raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, s_lane, a_srow + i * k_tiles_blocks + kt * 256, 0);
+      raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, s_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256, 0);
 #pragma unroll
     for (int j = 0; j < MT_N; ++j)
-      raw_b[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + kt * 256, 0);
+      raw_b[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + sblk(kt) * 256, 0);
   };
   // Real register moves, pinned here (a compiler copy would be folded into the
   // loop's phi and wait for the next scale load at the top of every iteration).
-  auto canon_scales = [&]() {
+  // (MXFP8, `kt` = the K tile the scales are for: its two K steps' bytes are bytes 0, 1 of the block's dword for
+  // the even K tile of a pair and bytes 2, 3 for the odd one)
+  auto canon_scales = [&](int kt) {
+    if constexpr (FP8) {
+      const int shift = (kt & 1) * 16;
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_a[i]) : "v"(raw_a[i]));
+      for (int i = 0; i < MT_M; ++i) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(sc_a[i]) : "s"(shift), "v"(raw_a[i]));
 #pragma unroll
-    for (int j = 0; j < MT_N; ++j) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_b[j]) : "v"(raw_b[j]));
+      for (int j = 0; j < MT_N; ++j) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(sc_b[j]) : "s"(shift), "v"(raw_b[j]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_a[i]) : "v"(raw_a[i]));
+#pragma unroll
+      for (int j = 0; j < MT_N; ++j) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_b[j]) : "v"(raw_b[j]));
+    }
   };
 
   // ---------------- accumulators and MFMA ----------------
   v16f acc[MT_M][MT_N];  // started from 0 by the first K step of every tile
 
   // ZERO: start the tile's sums from 0 (the first K step of a new output tile).
-  auto mfma_block = [&](const v4i(&fa)[MT_M], const v4i(&fb)[MT_N], auto t_tag, auto zero_tag) {
+  auto mfma_block = [&](const Frag(&fa)[MT_M], const Frag(&fb)[MT_N], auto t_tag, auto zero_tag) {
     constexpr int T = decltype(t_tag)::value;
     constexpr bool ZERO = decltype(zero_tag)::value;
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
-      const v8i va = {fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
+      v8i va;
+      if constexpr (FP8) va = fa[i];
+      else va = v8i{fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
-        const v8i vb = {fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
+        v8i vb;
+        if constexpr (FP8) vb = fb[j];
+        else vb = v8i{fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
         v16f c = acc[i][j];
         if (ZERO) {
 #pragma unroll
           for (int g = 0; g < 16; ++g) c[g] = 0.f;
         }
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, c, 4, 4, T, (int)sc_b[j], T, (int)sc_a[i]);
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, c, FMT_B, FMT_A, T, (int)sc_b[j], T, (int)sc_a[i]);
       }
     }
   };
@@ -269,7 +311,16 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // ---------------- one K tile (phases as in the one-tile kernel) ----------------
   //   P0: second half of B(j+1)      P1, P2: A(j+2)      P3: barrier, first half of B(j+2)
   // with (j+1), (j+2) running on into the next output tile at a boundary.
-  v4i fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  Frag fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  // MXFP8: one MFMA, two fragment halves each for its operands, and a DMA instruction while there are any
+  auto order_phase8 = [&]() {
+#pragma unroll
+    for (int g = 0; g < MT_M * MT_N; ++g) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+  };
   // PENDING: the C stores of the previous output tile are in the queue (every tile but the first).
   auto k_tile = [&](int j, int sa, int sb, auto kind_tag, auto pending_tag) {
     constexpr int KIND = decltype(kind_tag)::value;
@@ -284,6 +335,33 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const int sa1 = sa + 2 >= RING ? sa + 2 - RING : sa + 2;
     const int sb1 = sa + 3 >= RING ? sa + 3 - RING : sa + 3;
     const int sa2 = sa + 4 >= RING ? sa + 4 - RING : sa + 4;
+    if constexpr (FP8) {
+      // two K steps of 64-cycle MFMAs: the same request sequence folded into two phases
+      read_frags(sa, sb, 1, fa1, fb1);
+      mfma_block(fa0, fb0, T0{}, Zero{});
+      if (KIND != kFirst) issue_g2l(W1, 1, kt1, sb1, B_LD / 2, B_LD);
+      issue_g2l(W2, 0, kt2, sa2, 0, A_LD);
+      order_phase8();
+      __builtin_amdgcn_sched_barrier(0);
+      if (KIND == kFirst && PENDING) {
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(OUT_BF16 ? kWaitFirstBf16 : kWaitFirstF32));
+      } else {
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(A_LD));
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(sa1, sb1, 0, fa0, fb0);
+      mfma_block(fa1, fb1, T1{}, Keep{});
+      issue_g2l(W2, 1, kt2, sa, 0, B_LD / 2);
+      order_phase8();
+      __builtin_amdgcn_sched_barrier(0);
+      canon_scales(kt1);
+      load_scales(W2, kt2);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
     read_frags(sa, sb, 1, fa1, fb1);
     mfma_block(fa0, fb0, T0{}, Zero{});
     if (KIND != kFirst) issue_g2l(W1, 1, kt1, sb1, B_LD / 2, B_LD);
@@ -319,7 +397,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     issue_g2l(W2, 1, kt2, sa, 0, B_LD / 2);
     order_phase();
     __builtin_amdgcn_sched_barrier(0);
-    canon_scales();
+    canon_scales(kt1);
     load_scales(W2, kt2);
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -440,7 +518,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-  canon_scales();
+  canon_scales(0);
   load_scales(0, 1);
   read_frags(0, 1, 0, fa0, fb0);
   __builtin_amdgcn_sched_barrier(0);
@@ -513,6 +591,11 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
 template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
 __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_kernel(const GemmParams p) {
   persist_body<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>(p);
+}
+
+template <class Cfg, bool OUT_BF16, int FMT_A, int FMT_B>
+__global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_fp8_kernel(const GemmParams p) {
+  persist_body<Cfg, OUT_BF16, false, false, false, FMT_A, FMT_B>(p);
 }
 
 // Adds up the parts of the tiles of the last round (SPLIT) and writes them to C: one workgroup per 32 rows of a
@@ -643,6 +726,38 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
   // (grouped: tiles_m is an upper bound, the rows give the estimate)
   const int64_t tiles_m = p.num_groups != 0 ? p.m / 256 : p.tiles_m;
   return grid >= kNumXcd && tiles_m * p.tiles_n > grid;
+}
+
+// MXFP8 (`p` in byte geometry: kp = K bytes per row, k_tiles = K / 128): the 8-wave 256x256 configuration, dense.
+bool persist_gemm_fp8_applies(const GemmParams &p, int num_cus) {
+  if (p.num_groups != 0 || p.tile_table != nullptr || p.splits != 1 || p.partial != nullptr || p.b_preshuffled) return false;
+  if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  if ((p.n & 255) != 0 || p.tiles_n != p.n / 256 || (p.k & 255) != 0 || p.k_tiles < 4) return false;
+  if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31)) return false;
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  return grid >= kNumXcd && (int64_t)p.tiles_m * p.tiles_n > grid;
+}
+
+template <class Cfg, bool OUT_BF16, int FMT_A, int FMT_B>
+static hipError_t launch_persist_fp8_out(const GemmParams &p, int grid_x, hipStream_t stream) {
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, (const void *)persist_gemm_fp8_kernel<Cfg, OUT_BF16, FMT_A, FMT_B>, Cfg::LDS_BYTES);
+  if (e != hipSuccess) return e;
+  persist_gemm_fp8_kernel<Cfg, OUT_BF16, FMT_A, FMT_B><<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  return hipGetLastError();
+}
+
+template <int FMT_A, int FMT_B>
+static hipError_t launch_persist_fp8_fmt(const GemmParams &p, int grid_x, hipStream_t stream) {
+  typedef TileCfg<256, 256, 4, 2> Cfg;
+  return p.out_bf16 ? launch_persist_fp8_out<Cfg, true, FMT_A, FMT_B>(p, grid_x, stream)
+                    : launch_persist_fp8_out<Cfg, false, FMT_A, FMT_B>(p, grid_x, stream);
+}
+
+hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2, int b_e5m2, hipStream_t stream) {
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  if (a_e5m2) return b_e5m2 ? launch_persist_fp8_fmt<1, 1>(p, grid, stream) : launch_persist_fp8_fmt<1, 0>(p, grid, stream);
+  return b_e5m2 ? launch_persist_fp8_fmt<0, 1>(p, grid, stream) : launch_persist_fp8_fmt<0, 0>(p, grid, stream);
 }
 
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream) {

@@ -302,9 +302,21 @@ def leg_mxfp8(torch, wave_amd, dev, steps, warmup, variant=0):
 
     wall, per, settle_ms = timed(torch, run, steps, warmup)
     flops = 2.0 * m * n * k
+    # the same activations against packed MXFP4 weights (8-bit x 4-bit operands of the scaled MFMA)
+    from wave_amd import _lib as L
+    w4 = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+
+    def run_mixed(count):
+        for _ in range(count):
+            wave_amd.mxfp8_gemm(x, xs, w4, ws, out, elem_format=(L.MXFP8_E5M2, L.MXFP8_B_E2M1), variant=variant)
+
+    _, mper, _ = timed(torch, run_mixed, steps, warmup)
     return {"workload": f"mxfp8: M={m} N={n} K={k} e5m2 x e5m2, f32 out, seed 5", "kernel": "persist_gemm_fp8_kernel",
             "launch_us": round(per * 1e6, 2), "tflops": round(flops / per / 1e12, 1),
             "frac_of_mxfp8_peak": round(flops / per / 1e12 / PEAK_MXFP8_TFLOPS, 4), "settle_ms": round(settle_ms, 1),
+            "e5m2_x_e2m1": {"workload": "the same activations against MXFP4 weights [N, K/2]",
+                            "launch_us": round(mper * 1e6, 2), "tflops": round(flops / mper / 1e12, 1),
+                            "frac_of_mxfp8_peak": round(flops / mper / 1e12 / PEAK_MXFP8_TFLOPS, 4)},
             "wall_s_per_step": wall / steps}
 
 
@@ -585,6 +597,7 @@ def main():
             "ms_per_step": round(leg.pop("wall_s_per_step") * 1e3, 4),
             "dtype": "mxfp8 (e5m2 x e8m0) in, f32 accumulate, f32 out", "data": "synthetic (normal values, seeded)",
             "config": {"workload": leg["workload"], "variant": args.variant}, "settle_ms": leg["settle_ms"],
+            "e5m2_x_e2m1": leg["e5m2_x_e2m1"],
             "roofline": {"bound": "mfma", "achieved": leg["tflops"], "peak": PEAK_MXFP8_TFLOPS, "unit": "TFLOP/s",
                          "frac": leg["frac_of_mxfp8_peak"], "traffic": read_traffic("mxfp8"), "kernel": leg["kernel"],
                          "launch_us": leg["launch_us"]}})))

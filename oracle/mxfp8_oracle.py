@@ -17,9 +17,12 @@ from __future__ import annotations
 
 import numpy as np
 
-from .mxfp4_oracle import SCALE_GROUP_SIZE, e8m0_to_f32
+from .mxfp4_oracle import SCALE_GROUP_SIZE, e8m0_to_f32, mxfp4_to_f32
 
 E4M3, E5M2 = 0, 1
+E2M1 = 2   # second operand only: packed MXFP4 weights [N, K/2] against 8-bit activations (the mixed operand
+           # types of the scaled MMA, wave_lang/kernel/wave/constraints.py:425-431; the reference holds no test of
+           # it, the restatement is the composition of the two pinned decodes and the same f64 product)
 
 
 def _decode_table(exp_bits: int, man_bits: int, bias: int, ieee_specials: bool) -> np.ndarray:
@@ -57,7 +60,7 @@ def scaled_gemm_mxfp8(x, w_t, x_scales, w_scales, fmt) -> np.ndarray:
     xs = e8m0_to_f32(np.asarray(x_scales, dtype=np.uint8)).astype(np.float64).repeat(SCALE_GROUP_SIZE, axis=1)
     ws = e8m0_to_f32(np.asarray(w_scales, dtype=np.uint8)).astype(np.float64).repeat(SCALE_GROUP_SIZE, axis=1)
     a = fp8_to_f64(x, fmt_x) * xs
-    b = fp8_to_f64(w_t, fmt_w) * ws
+    b = (mxfp4_to_f32(np.asarray(w_t, dtype=np.uint8)).astype(np.float64) if fmt_w == E2M1 else fp8_to_f64(w_t, fmt_w)) * ws
     return a @ b.T
 
 
@@ -80,7 +83,10 @@ def make_inputs_mxfp8(m, n, k, seed, fmt, scale_lo=124, scale_hi=127):
         return codes[np.where(lower, idx - 1, idx)]
 
     x = quantise(rng.standard_normal((m, k)), fmt_x)
-    w_t = quantise(rng.standard_normal((n, k)), fmt_w)
+    if fmt_w == E2M1:   # uniform nibbles, as the MXFP4 generator draws them
+        w_t = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    else:
+        w_t = quantise(rng.standard_normal((n, k)), fmt_w)
     xs = rng.integers(scale_lo, scale_hi + 1, size=(m, k // 32), dtype=np.uint8)
     ws = rng.integers(scale_lo, scale_hi + 1, size=(n, k // 32), dtype=np.uint8)
     return x, xs, w_t, ws

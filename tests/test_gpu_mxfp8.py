@@ -86,6 +86,36 @@ def test_mxfp8_more_tiles_than_cus(m, n, k, fmt, out_dtype):
         assert_f32_close(c[rows], ref, f"{m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("fmt_x", [o8.E5M2, o8.E4M3], ids=["e5m2", "e4m3"])
+@pytest.mark.parametrize("vname", sorted(VARIANTS))
+@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (256, 256, 512), (300, 200, 384), (1, 40, 256), (257, 33, 1152),
+                                   (1024, 1024, 1024)])
+def test_mxfp8_activations_against_mxfp4_weights(m, n, k, vname, fmt_x):
+    """8-bit A against packed e2m1 B [N, K/2] (the mixed operand types of the scaled MMA,
+    wave_lang/kernel/wave/constraints.py:425-431; the reference holds no test of them)."""
+    fmt = (fmt_x, o8.E2M1)
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=m + n + k + 2, fmt=fmt, scale_lo=120, scale_hi=134)
+    ref = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, fmt)
+    assert_f32_close(run(x, xs, w_t, ws, fmt, variant=VARIANTS[vname]), ref, f"{vname} {m}x{n}x{k}")
+
+
+def test_mxfp8_against_mxfp4_one_hot_and_more_tiles_than_cus():
+    """One-hot rows of A (1.0 at one position, scale 1) read back columns of dequantised B exactly, on 272 tiles
+    (the persistent kernel with the scratch buffer, one tile per workgroup without: the same bits)."""
+    m, n, k = 4352, 4096, 512
+    fmt = (o8.E4M3, o8.E2M1)
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=3, fmt=fmt, scale_lo=118, scale_hi=136)
+    x[:] = 0
+    xs[:] = 127
+    one = int(np.nonzero(o8.E4M3_TABLE == 1.0)[0][0])
+    pos = (np.arange(m) * 37) % k
+    x[np.arange(m), pos] = one
+    c = run(x, xs, w_t, ws, fmt)
+    from oracle import mxfp4_oracle as o4
+    b = o4.mxfp4_to_f32(w_t).astype(np.float64) * o4.e8m0_to_f32(ws).astype(np.float64).repeat(32, axis=1)
+    assert np.array_equal(c, b[:, pos].T.astype(np.float32))
+
+
 def test_mxfp8_mixed_formats_from_torch_dtypes():
     """float8 tensors carry their own format: e4m3 activations against e5m2 weights, exact on one-hot rows."""
     m, n, k = 128, 96, 256

@@ -44,6 +44,32 @@ def test_gemm_equals_brute_force(fmt):
             assert abs(Fraction(float(got[i, j])) - acc) <= abs(acc) * Fraction(1, 2 ** 45)
 
 
+@pytest.mark.parametrize("fmt_x", [o8.E5M2, o8.E4M3])
+def test_mixed_gemm_equals_brute_force(fmt_x):
+    """8-bit activations against packed e2m1 weights: exact rationals, the nibble decoded here from its
+    sign / exponent / mantissa fields (low nibble = even element), not through the oracle's table."""
+    m, n, k = 3, 5, 64
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=2, fmt=(fmt_x, o8.E2M1), scale_lo=100, scale_hi=150)
+    assert w_t.shape == (n, k // 2)
+    got = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, (fmt_x, o8.E2M1))
+    table = o8.E5M2_TABLE if fmt_x == o8.E5M2 else o8.E4M3_TABLE
+
+    def e2m1(code):
+        e, mnt = (code >> 1) & 3, code & 1
+        mag = Fraction(mnt, 2) if e == 0 else Fraction(2) ** (e - 1) * (1 + Fraction(mnt, 2))
+        return -mag if code & 8 else mag
+
+    for i in range(m):
+        for j in range(n):
+            acc = Fraction(0)
+            for kk in range(k):
+                byte = int(w_t[j, kk // 2])
+                wv = e2m1((byte >> 4) if kk & 1 else (byte & 15))
+                acc += (Fraction(float(table[x[i, kk]])) * Fraction(2) ** (int(xs[i, kk // 32]) - 127)
+                        * wv * Fraction(2) ** (int(ws[j, kk // 32]) - 127))
+            assert abs(Fraction(float(got[i, j])) - acc) <= abs(acc) * Fraction(1, 2 ** 45) + Fraction(1, 2 ** 300)
+
+
 def test_generator_rounds_to_nearest_code():
     x, xs, w_t, ws = o8.make_inputs_mxfp8(8, 8, 128, seed=0, fmt=o8.E4M3)
     assert x.dtype == np.uint8 and xs.shape == (8, 4) and np.isfinite(o8.fp8_to_f64(x, o8.E4M3)).all()

@@ -479,7 +479,7 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
                     size_t workspace_bytes, int variant, void *hip_stream) {
   if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim || k % 128 != 0)
     return WAVE_MXFP4_ERR_BAD_SHAPE;
-  if (bad_enum(a_format, 2) || bad_enum(b_format, 2) || bad_enum(out_dtype, 2) ||
+  if (bad_enum(a_format, 2) || bad_enum(b_format, 3) || bad_enum(out_dtype, 2) ||
       bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
     return WAVE_MXFP4_ERR_BAD_ENUM;
   if (variant != WAVE_MXFP4_VARIANT_AUTO && variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 &&
@@ -529,8 +529,8 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   }
   // large dense problems on the 8-wave tiles with re-laid scales: the persistent kernel
   if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && persist_gemm_fp8_applies(p, device_cus()))
-    return record_hip(launch_persist_gemm_fp8(p, device_cus(), a_format == WAVE_MXFP8_E5M2, b_format == WAVE_MXFP8_E5M2, stream));
-  return record_hip(launch_tile_gemm_fp8(p, v, a_format == WAVE_MXFP8_E5M2, b_format == WAVE_MXFP8_E5M2, stream));
+    return record_hip(launch_persist_gemm_fp8(p, device_cus(), a_format == WAVE_MXFP8_E5M2, b_format, stream));
+  return record_hip(launch_tile_gemm_fp8(p, v, a_format == WAVE_MXFP8_E5M2, b_format, stream));
 }
 
 // Scratch of a grouped call: [M tile table | A scales, one 256-row slab per possible M tile | B scales].

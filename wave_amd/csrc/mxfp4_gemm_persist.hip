@@ -59,7 +59,8 @@ enum KtKind {
 template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, int FMT_A = 4, int FMT_B = 4>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
   constexpr bool FP8 = FMT_A != 4;
-  static_assert((FMT_A == 4) == (FMT_B == 4), "MXFP4 x MXFP8 operands are not built");
+  constexpr bool B4 = FP8 && FMT_B == 4;  // 8-bit A against 4-bit B [N, K/2]: the lower half of B's LDS rows
+  static_assert(FMT_A != 4 || FMT_B == 4, "an MXFP4 A against an MXFP8 B is not built");
   static_assert(!FP8 || (!GROUPED && !TAIL && !SPLIT), "MXFP8: dense problems with whole K tiles");
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
@@ -87,7 +88,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   int m0[2], n0[2], a_lim[2], as_lim[2], c_rows[2], nkt_of[2], part_of[2];
   bool tail_on[2];
   const int m_blocks = (p.m + 31) >> 5;
-  const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
+  const int b_kt_stride = p.b_preshuffled ? 2048 : B4 ? kTileKBytes / 2 : kTileKBytes;
   static_assert(!(GROUPED && SPLIT), "the K cut of the last round is for dense problems");
   // Grouped: the same XCD regrouping as map_tile, but the bands the sequence walks column by column are the
   // table's (at most 8 tiles of one expert), not fixed runs of 8 tile rows.
@@ -136,7 +137,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     } else {
       m0[which] = tm * BM;
       c_rows[which] = p.m - m0[which];
-      b_base[which] = p.b + (int64_t)n0[which] * kp;
+      b_base[which] = p.b + (int64_t)n0[which] * (B4 ? kp >> 1 : kp);
       bs_base[which] = p.b_scale + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
       as_base[which] = p.a_scale + (int64_t)(m0[which] >> 5) * k_tiles_blocks;
       as_lim[which] = (int)min((int64_t)(m_blocks - (m0[which] >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
@@ -164,11 +165,14 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   const int ld_chunk = (lane & 7) ^ ((ld_row0 >> 1) & 7);
   // DMA instruction d of a wave fills rows 8*NWAVES*d further down: one per-lane
   // offset per operand, the rest is scalar (registers are what this kernel is short of).
+  const int kpb = B4 ? kp >> 1 : kp;  // bytes of a row of B
   int a_goff = ld_row0 * kp + ld_chunk * 16;
   int b_goff = p.b_preshuffled ? (ld_row0 >> 4) * 16 * kp + (ld_row0 & 15) * 16 + (ld_chunk >> 1) * 512 +
                                            (ld_chunk & 1) * 256
-                                     : ld_row0 * kp + ld_chunk * 16;
+                                     : ld_row0 * kpb + ld_chunk * 16;
+  if (B4 && ld_chunk >= 4) b_goff = (int)0x80000000;  // the upper half of the LDS row: no request, zeros
   const int ld_step = NWAVES * 8 * kp;  // bytes between consecutive d, either layout (8*NWAVES is a multiple of 16)
+  const int ld_step_b = NWAVES * 8 * kpb;
   const bool tail_lane = TAIL && ld_chunk >= ((p.k & (kTileK - 1)) >> 5);
   auto flip_tail = [&](int &goff) { goff ^= tail_lane && (!SPLIT || tail_on[0]) ? (int)0x80000000 : 0; };
 
@@ -183,7 +187,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     for (int d = d0; d < d1; ++d) {
       uint8_t *dst = dst_tile + (d * NWAVES + wave) * 1024;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, WAVE_LDS_PTR(dst), 16, op == 0 ? a_goff : b_goff,
-                                               soff + d * ld_step, 0, 0);
+                                               soff + d * (op == 0 ? ld_step : ld_step_b), 0, 0);
     }
   };
 
@@ -199,7 +203,11 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   const uint32_t a_fbase = (uint32_t)(wave_m * Cfg::WM * kTileKBytes);
   const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
   typedef typename std::conditional<FP8, v8i, v4i>::type Frag;
-  auto read_frags = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], Frag(&fb)[MT_N]) {
+  typedef typename std::conditional<FP8 && !B4, v8i, v4i>::type FragB;
+  uint32_t foff_b4[2];  // 8-bit A against 4-bit B: K step s of B is the chunk 2s + fg of the row's lower half
+#pragma unroll
+  for (int t = 0; t < 2; ++t) foff_b4[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
+  auto read_frags = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], FragB(&fb)[MT_N]) {
     if constexpr (FP8) {
       const uint8_t *ta = smem + slot_a * SLOT + a_fbase, *tb = smem + slot_b * SLOT + b_fbase;
 #pragma unroll
@@ -210,9 +218,13 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       }
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
-        const v4i lo = *(const v4i *)(tb + foff[2 * t] + j * 32 * kTileKBytes);
-        const v4i hi = *(const v4i *)(tb + foff[2 * t + 1] + j * 32 * kTileKBytes);
-        fb[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        if constexpr (B4) {
+          fb[j] = *(const v4i *)(tb + foff_b4[t] + j * 32 * kTileKBytes);
+        } else {
+          const v4i lo = *(const v4i *)(tb + foff[2 * t] + j * 32 * kTileKBytes);
+          const v4i hi = *(const v4i *)(tb + foff[2 * t + 1] + j * 32 * kTileKBytes);
+          fb[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
       }
     } else {
       const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
@@ -261,7 +273,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   v16f acc[MT_M][MT_N];  // started from 0 by the first K step of every tile
 
   // ZERO: start the tile's sums from 0 (the first K step of a new output tile).
-  auto mfma_block = [&](const Frag(&fa)[MT_M], const Frag(&fb)[MT_N], auto t_tag, auto zero_tag) {
+  auto mfma_block = [&](const Frag(&fa)[MT_M], const FragB(&fb)[MT_N], auto t_tag, auto zero_tag) {
     constexpr int T = decltype(t_tag)::value;
     constexpr bool ZERO = decltype(zero_tag)::value;
 #pragma unroll
@@ -272,7 +284,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
         v8i vb;
-        if constexpr (FP8) vb = fb[j];
+        if constexpr (FP8 && !B4) vb = fb[j];
         else vb = v8i{fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
         v16f c = acc[i][j];
         if (ZERO) {
@@ -311,7 +323,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // ---------------- one K tile (phases as in the one-tile kernel) ----------------
   //   P0: second half of B(j+1)      P1, P2: A(j+2)      P3: barrier, first half of B(j+2)
   // with (j+1), (j+2) running on into the next output tile at a boundary.
-  Frag fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  Frag fa0[MT_M], fa1[MT_M];
+  FragB fb0[MT_N], fb1[MT_N];
   // MXFP8: one MFMA, two fragment halves each for its operands, and a DMA instruction while there are any
   auto order_phase8 = [&]() {
 #pragma unroll
@@ -754,10 +767,12 @@ static hipError_t launch_persist_fp8_fmt(const GemmParams &p, int grid_x, hipStr
                     : launch_persist_fp8_out<Cfg, false, FMT_A, FMT_B>(p, grid_x, stream);
 }
 
-hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2, int b_e5m2, hipStream_t stream) {
+// b_fmt: 0 = e4m3, 1 = e5m2, 2 = e2m1 (packed, two per byte)
+hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2, int b_fmt, hipStream_t stream) {
   const int grid = num_cus / kNumXcd * kNumXcd;
-  if (a_e5m2) return b_e5m2 ? launch_persist_fp8_fmt<1, 1>(p, grid, stream) : launch_persist_fp8_fmt<1, 0>(p, grid, stream);
-  return b_e5m2 ? launch_persist_fp8_fmt<0, 1>(p, grid, stream) : launch_persist_fp8_fmt<0, 0>(p, grid, stream);
+  if (b_fmt == 2) return a_e5m2 ? launch_persist_fp8_fmt<1, 4>(p, grid, stream) : launch_persist_fp8_fmt<0, 4>(p, grid, stream);
+  if (a_e5m2) return b_fmt ? launch_persist_fp8_fmt<1, 1>(p, grid, stream) : launch_persist_fp8_fmt<1, 0>(p, grid, stream);
+  return b_fmt ? launch_persist_fp8_fmt<0, 1>(p, grid, stream) : launch_persist_fp8_fmt<0, 0>(p, grid, stream);
 }
 
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream) {

@@ -121,14 +121,18 @@ constexpr int kSlabMaxPitch = (kSlabMaxKTiles + 2) * 8;  // bytes per row: the K
 // covers 8 groups = two MXFP8 K tiles, the odd one's bytes sit in the upper half
 // of the lane's dword).
 // FMT is A's format, FMT_B B's (MXFP8 operands may differ: e4m3 activations against e5m2 weights or the other
-// way round, cbsz / blgp 0 / 1 of the instruction).
+// way round, cbsz / blgp 0 / 1 of the instruction).  An 8-bit A may also meet a 4-bit B (FMT_B = 4: MXFP8
+// activations against MXFP4 weights, B [N, K/2] packed): the K tile is A's, 128 elements, of which a row of B
+// holds 64 bytes - the lower four chunks of its LDS row, the other four are neither fetched nor read - and a
+// K step takes one 16-byte chunk of B per lane, as in MXFP4.
 template <class Cfg, int MODE, int FMT = 4, int FMT_B = FMT>
 __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
-  static_assert((FMT == 4) == (FMT_B == 4), "MXFP4 x MXFP8 operands are not built");
+  static_assert(FMT != 4 || FMT_B == 4, "an MXFP4 A against an MXFP8 B is not built");
   constexpr bool GENERIC_K = MODE == kGenericK;
   constexpr bool NATIVE = MODE == kNative;
   constexpr bool SC_LDS = MODE == kDirectLds;
   constexpr bool FP8 = FMT != 4;
+  constexpr bool B4 = FP8 && FMT_B == 4;  // 8-bit A against 4-bit B
   static_assert(!SC_LDS || (!FP8 && Cfg::LDS_BYTES + (Cfg::BM + Cfg::BN) * kSlabMaxPitch <= 160 * 1024),
                 "scale rows in LDS: MXFP4 on a tile whose ring leaves room");
   static_assert(!FP8 || MODE != kGenericK, "MXFP8 needs whole K tiles");
@@ -186,8 +190,9 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   // hold logical chunk (t%8) ^ swz(row), swz(row) = (row/2) % 8.  Consecutive d
   // are 8*NWAVES rows apart (a multiple of 16), so the chunk does not depend on d.
   const int kp = p.kp;
+  const int kpb = B4 ? kp >> 1 : kp;  // bytes of a row of B
   const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(p.a + (int64_t)m0 * kp);
-  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_ptr + (int64_t)n0 * kp);  // preshuffle keeps 16-row blocks contiguous
+  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_ptr + (int64_t)n0 * kpb);  // preshuffle keeps 16-row blocks contiguous
   const int ld_row0 = wave * 8 + (lane >> 3);
   const int ld_chunk = (lane & 7) ^ ((ld_row0 >> 1) & 7);
   const int a_row_lim = p.m - 1 - m0, b_row_lim = p.n - 1 - n0;  // clamp to allocated rows
@@ -203,9 +208,10 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
     const int r = min(ld_row0 + d * NWAVES * 8, b_row_lim);
     b_goff[d] = p.b_preshuffled
                     ? (r >> 4) * 16 * kp + (r & 15) * 16 + (ld_chunk >> 1) * 512 + (ld_chunk & 1) * 256
-                    : r * kp + ld_chunk * 16;
+                    : r * kpb + ld_chunk * 16;
+    if (B4 && ld_chunk >= 4) b_goff[d] = (int)0x80000000;  // the upper half of the LDS row: no request, zeros
   }
-  const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
+  const int b_kt_stride = p.b_preshuffled ? 2048 : B4 ? kTileKBytes / 2 : kTileKBytes;
   const int tail_chunks = GENERIC_K ? ((p.k & (kTileK - 1)) >> 5) : 0;  // valid chunks of a partial last tile
   // kNative with a partial last K tile (MXFP4 only): the lanes whose chunk lies past the end of K fetch from
   // beyond the descriptor instead, which lands zeros in LDS: the same instructions as for a whole tile, so the
@@ -269,7 +275,12 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
 
   typedef typename std::conditional<FP8, v8i, v4i>::type Frag;
-  auto read_frags = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], Frag(&fb)[MT_N]) {
+  typedef typename std::conditional<FP8 && !B4, v8i, v4i>::type FragB;
+  // (8-bit A against 4-bit B: K step s of B is the chunk 2s + fg of the row's lower half)
+  uint32_t foff_b4[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) foff_b4[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
+  auto read_frags = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], FragB(&fb)[MT_N]) {
     if constexpr (FP8) {
       const uint8_t *ta = smem + slot_a * SLOT + a_fbase, *tb = smem + slot_b * SLOT + b_fbase;
 #pragma unroll
@@ -280,9 +291,13 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
       }
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
-        const v4i lo = *(const v4i *)(tb + foff[2 * t] + j * 32 * kTileKBytes);
-        const v4i hi = *(const v4i *)(tb + foff[2 * t + 1] + j * 32 * kTileKBytes);
-        fb[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        if constexpr (B4) {
+          fb[j] = *(const v4i *)(tb + foff_b4[t] + j * 32 * kTileKBytes);
+        } else {
+          const v4i lo = *(const v4i *)(tb + foff[2 * t] + j * 32 * kTileKBytes);
+          const v4i hi = *(const v4i *)(tb + foff[2 * t + 1] + j * 32 * kTileKBytes);
+          fb[j] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
       }
     } else {
       const uint8_t *ba = smem + slot_a * SLOT + a_fbase + foff[t];
@@ -456,7 +471,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
 #pragma unroll
       for (int g = 0; g < 16; ++g) acc[i][j][g] = 0.f;
 
-  auto mfma_block = [&](const Frag(&fa)[MT_M], const Frag(&fb)[MT_N], auto t_tag) {
+  auto mfma_block = [&](const Frag(&fa)[MT_M], const FragB(&fb)[MT_N], auto t_tag) {
     constexpr int T = decltype(t_tag)::value;
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
@@ -466,7 +481,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
         v8i vb;
-        if constexpr (FP8) vb = fb[j];
+        if constexpr (FP8 && !B4) vb = fb[j];
         else vb = v8i{fb[j].x, fb[j].y, fb[j].z, fb[j].w, 0, 0, 0, 0};
         // first port = B rows (N index), second port = A rows (M index)
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][j], FMT_B, FMT, T,
@@ -508,7 +523,8 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   // After it all waves have finished reading tile j, which frees the slots of
   // A(j) (-> B(j+2), issued from P3 on) and B(j) (-> A(j+3)).
   // Fragments are double-buffered in registers across the K steps.
-  Frag fa0[MT_M], fb0[MT_N], fa1[MT_M], fb1[MT_N];
+  Frag fa0[MT_M], fa1[MT_M];
+  FragB fb0[MT_N], fb1[MT_N];
   constexpr int kWaitSteady = GENERIC_K ? 0 : A_LD;
   constexpr int kWaitPrologue = GENERIC_K ? 0 : A_LD + B_LD / 2;
 
@@ -815,17 +831,19 @@ static hipError_t launch_fp8_by_scales(const GemmParams &p, hipStream_t stream) 
   return native ? launch_cfg<Cfg, kNative, FMT_A, FMT_B>(p, stream) : launch_cfg<Cfg, kDirect, FMT_A, FMT_B>(p, stream);
 }
 
+// b_fmt: 0 = e4m3, 1 = e5m2, 2 = e2m1 (packed, two per byte)
 template <class Cfg>
-static hipError_t launch_fp8_formats(const GemmParams &p, int a_e5m2, int b_e5m2, hipStream_t stream) {
-  if (a_e5m2) return b_e5m2 ? launch_fp8_by_scales<Cfg, 1, 1>(p, stream) : launch_fp8_by_scales<Cfg, 1, 0>(p, stream);
-  return b_e5m2 ? launch_fp8_by_scales<Cfg, 0, 1>(p, stream) : launch_fp8_by_scales<Cfg, 0, 0>(p, stream);
+static hipError_t launch_fp8_formats(const GemmParams &p, int a_e5m2, int b_fmt, hipStream_t stream) {
+  if (b_fmt == 2) return a_e5m2 ? launch_fp8_by_scales<Cfg, 1, 4>(p, stream) : launch_fp8_by_scales<Cfg, 0, 4>(p, stream);
+  if (a_e5m2) return b_fmt ? launch_fp8_by_scales<Cfg, 1, 1>(p, stream) : launch_fp8_by_scales<Cfg, 1, 0>(p, stream);
+  return b_fmt ? launch_fp8_by_scales<Cfg, 0, 1>(p, stream) : launch_fp8_by_scales<Cfg, 0, 0>(p, stream);
 }
 
 // MXFP8: `p` describes the byte geometry (kp = K bytes per row, ks = K/32, k_tiles = K/128).
-hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_e5m2, hipStream_t stream) {
-  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_fp8_formats<Cfg256x256w4>(p, a_e5m2, b_e5m2, stream);
-  if (variant == WAVE_MXFP4_VARIANT_T256x256_W4x2) return launch_fp8_formats<Cfg256x256w8>(p, a_e5m2, b_e5m2, stream);
-  if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2) return launch_fp8_formats<Cfg128x128w4>(p, a_e5m2, b_e5m2, stream);
+hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_fmt, hipStream_t stream) {
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_fp8_formats<Cfg256x256w4>(p, a_e5m2, b_fmt, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W4x2) return launch_fp8_formats<Cfg256x256w8>(p, a_e5m2, b_fmt, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2) return launch_fp8_formats<Cfg128x128w4>(p, a_e5m2, b_fmt, stream);
   return hipErrorInvalidValue;
 }
 

@@ -85,7 +85,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // c_rows: rows of the tile that are stored
   // nkt_of / part_of / tail_on: K tiles of the item, its slot in tail_partial (-1: a whole tile), and whether
   // its K range ends with the (partial) last K tile of the problem
-  int m0[2], n0[2], a_lim[2], as_lim[2], c_rows[2], nkt_of[2], part_of[2];
+  int m0[2], n0[2], a_lim[2], as_lim[2], b_lim[2], bs_lim[2], c_rows[2], nkt_of[2], part_of[2];
   bool tail_on[2];
   const int m_blocks = (p.m + 31) >> 5;
   const int b_kt_stride = p.b_preshuffled ? 2048 : B4 ? kTileKBytes / 2 : kTileKBytes;
@@ -142,6 +142,9 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       as_base[which] = p.a_scale + (int64_t)(m0[which] >> 5) * k_tiles_blocks;
       as_lim[which] = (int)min((int64_t)(m_blocks - (m0[which] >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
     }
+    // B and its scales end with the tensor (grouped: with the expert's)
+    b_lim[which] = rsrc_bytes(((int64_t)p.n - n0[which]) * (B4 ? kp >> 1 : kp));
+    bs_lim[which] = rsrc_bytes((int64_t)(((p.n + 31) >> 5) - (n0[which] >> 5)) * k_tiles_blocks);
     a_base[which] = p.a + (int64_t)m0[which] * kp;
     // (grouped: A ends with the tile's own rows.  The rows of the next group would do as padding, their results
     // are dropped, but zeros cost the matrix pipes far less power than data does, and power is what bounds the
@@ -154,6 +157,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       as_base[which] += kt_lo * 256;
       as_lim[which] = max(as_lim[which] - kt_lo * 256, 0);
       bs_base[which] += kt_lo * 256;
+      b_lim[which] = max(b_lim[which] - kt_lo * b_kt_stride, 0);
+      bs_lim[which] = max(bs_lim[which] - kt_lo * 256, 0);
     }
     return true;
   };
@@ -181,7 +186,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   auto issue_g2l = [&](int which, int op, int kt, int slot, int d0, int d1) {
     uint8_t *dst_tile = smem + slot * SLOT;
     const __amdgpu_buffer_rsrc_t rsrc =
-        op == 0 ? make_rsrc_n(a_base[which], a_lim[which]) : make_rsrc(b_base[which]);
+        op == 0 ? make_rsrc_n(a_base[which], a_lim[which]) : make_rsrc_n(b_base[which], b_lim[which]);
     const int soff = op == 0 ? kt * kTileKBytes : kt * b_kt_stride;
 #pragma unroll
     for (int d = d0; d < d1; ++d) {
@@ -242,7 +247,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   uint32_t raw_a[MT_M], raw_b[MT_N], sc_a[MT_M], sc_b[MT_N];
   auto sblk = [](int kt) { return FP8 ? kt >> 1 : kt; };  // MXFP8: one MFMA32 block serves two K tiles
   auto load_scales = [&](int which, int kt) {
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc_n(as_base[which], as_lim[which]), rb = make_rsrc(bs_base[which]);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc_n(as_base[which], as_lim[which]), rb = make_rsrc_n(bs_base[which], bs_lim[which]);
 #pragma unroll
     for (int i = 0; i < MT_M; ++i)
       raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, s_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256, 0);
@@ -550,6 +555,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const bool has_next = set_tile(1, npid);
     if (!has_next) {
       m0[1] = m0[0], n0[1] = n0[0], a_lim[1] = a_lim[0], as_lim[1] = as_lim[0], c_rows[1] = c_rows[0];
+      b_lim[1] = b_lim[0], bs_lim[1] = bs_lim[0];
       nkt_of[1] = nkt_of[0], part_of[1] = part_of[0], tail_on[1] = tail_on[0];
       a_base[1] = a_base[0], b_base[1] = b_base[0], as_base[1] = as_base[0], bs_base[1] = bs_base[0];
     }
@@ -588,6 +594,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     __builtin_amdgcn_sched_barrier(0);
     pid = npid;
     m0[0] = m0[1], n0[0] = n0[1], a_lim[0] = a_lim[1], as_lim[0] = as_lim[1], c_rows[0] = c_rows[1];
+    b_lim[0] = b_lim[1], bs_lim[0] = bs_lim[1];
     nkt_of[0] = nkt_of[1], part_of[0] = part_of[1], tail_on[0] = tail_on[1];
     a_base[0] = a_base[1], b_base[0] = b_base[1], as_base[0] = as_base[1], bs_base[0] = bs_base[1];
     return true;

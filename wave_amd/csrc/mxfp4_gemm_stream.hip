@@ -33,7 +33,7 @@
 // same C = dequant(A) . dequant(B)^T.
 #include <type_traits>
 
-#include "mxfp4_common.h"
+#include "mxfp4_tile_common.h"
 
 namespace wave_mxfp4 {
 
@@ -117,8 +117,9 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   //   preshuffled : K step i = 2*j + s of the 16-row block (already in MFMA order: lane l's
   //                 16 bytes at l*16), landing at i*1024 + l*16 and read back from there.
   const bool bpre = p.b_preshuffled != 0;
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<uint8_t *>(p.b + (int64_t)nt_begin * 16 * kp), 0, 0x7FFFFFFF, 0x00020000);
+  // (every descriptor ends with its tensor: an access past it reads zeros instead of a neighbour's memory)
+  const __amdgpu_buffer_rsrc_t b_rsrc =
+      make_rsrc_n(p.b + (int64_t)nt_begin * 16 * kp, rsrc_bytes(((int64_t)p.n - (int64_t)nt_begin * 16) * kp));
   const int b_voff = bpre ? lane * 16 : min(lane, ktw * 8 - 1) * 16;
   auto issue_rows = [&](int nt, int buf) {
     uint8_t *dst = lds.tile[wave][buf];
@@ -183,7 +184,7 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   const int sc_block_row_bytes = (p.ksp >> 3) * 256;  // one 32-row tile, all K tiles
   const bool sc_pieces = (p.ks & 15) == 0;
   const __amdgpu_buffer_rsrc_t bs_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.b_scale), 0, 0x7FFFFFFF, 0x00020000);
+      make_rsrc_n(p.b_scale, rsrc_bytes(scale_tensor_bytes(p.b_scale_layout, p.n, p.ks, p.ksp)));
   auto issue_scales = [&](int nt, int buf) {
     uint8_t *dst = lds.scales[wave][buf];
     const int n0 = nt * 16;
@@ -263,10 +264,9 @@ __device__ __forceinline__ void stream_body(const GemmParams &p) {
   v4i a_frag[MT_M][kStreamKtPerWave][2];
   uint32_t a_sc[MT_M][kStreamKtPerWave][2];
   constexpr int kOpselA1 = FULL ? 1 : 0;  // op_sel of the A scale for the second K step
-  const __amdgpu_buffer_rsrc_t a_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a), 0, 0x7FFFFFFF, 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(p.a, rsrc_bytes((int64_t)p.m * kp));
   const __amdgpu_buffer_rsrc_t as_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(p.a_scale), 0, 0x7FFFFFFF, 0x00020000);
+      make_rsrc_n(p.a_scale, rsrc_bytes(scale_tensor_bytes(p.a_scale_layout, p.m, p.ks, p.ksp)));
   auto load_b128 = [&](__amdgpu_buffer_rsrc_t r, int voff, int soff) -> v4i {
     typedef unsigned int u4 __attribute__((ext_vector_type(4)));
     const u4 v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);

@@ -191,8 +191,11 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   // are 8*NWAVES rows apart (a multiple of 16), so the chunk does not depend on d.
   const int kp = p.kp;
   const int kpb = B4 ? kp >> 1 : kp;  // bytes of a row of B
-  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(p.a + (int64_t)m0 * kp);
-  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(b_ptr + (int64_t)n0 * kpb);  // preshuffle keeps 16-row blocks contiguous
+  // (every descriptor ends with its tensor, or its expert's part of it: an access past it reads zeros instead of
+  // a neighbour's memory)
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(p.a + (int64_t)m0 * kp, rsrc_bytes(((int64_t)p.m - m0) * kp));
+  // preshuffle keeps 16-row blocks contiguous
+  const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc_n(b_ptr + (int64_t)n0 * kpb, rsrc_bytes(((int64_t)p.n - n0) * kpb));
   const int ld_row0 = wave * 8 + (lane >> 3);
   const int ld_chunk = (lane & 7) ^ ((ld_row0 >> 1) & 7);
   const int a_row_lim = p.m - 1 - m0, b_row_lim = p.n - 1 - n0;  // clamp to allocated rows
@@ -334,8 +337,10 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   const ScaleAddr b_sa = FP8 && !NATIVE ? ScaleAddr{4, 0} : scale_addr(p.b_scale_layout);
   const uint8_t *as_base = scale_tile_base(p.a_scale, p.a_scale_layout, m0, p.ks, p.ksp);
   const uint8_t *bs_base = scale_tile_base(bs_ptr, p.b_scale_layout, n0, p.ks, p.ksp);
-  const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc(as_base);
-  const __amdgpu_buffer_rsrc_t bs_rsrc = make_rsrc(bs_base);
+  const __amdgpu_buffer_rsrc_t as_rsrc =
+      make_rsrc_n(as_base, rsrc_bytes(scale_tensor_bytes(p.a_scale_layout, p.m, p.ks, p.ksp) - (as_base - p.a_scale)));
+  const __amdgpu_buffer_rsrc_t bs_rsrc =
+      make_rsrc_n(bs_base, rsrc_bytes(scale_tensor_bytes(p.b_scale_layout, p.n, p.ks, p.ksp) - (bs_base - bs_ptr)));
 
   // kDirectLds: rows 0..BM-1 of the slab are A's tile rows, BM..BM+BN-1 B's; row r holds the 8 bytes of each of
   // the workgroup's K tiles (rows past the tensor repeat its last row, like the clamped loads of kDirect).

@@ -62,6 +62,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc_n(const void *base, 
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
 }
 
+// Bytes of a scale tensor of `rows` rows in `layout` (row-major: rows * ks; the blocked layouts are padded to
+// whole 32-row blocks of ksp = ceil(ks / 8) * 8 groups), and a descriptor size clipped to what one holds.
+__device__ __forceinline__ int64_t scale_tensor_bytes(int layout, int64_t rows, int64_t ks, int64_t ksp) {
+  return layout == WAVE_MXFP4_SCALE_ROW_MAJOR ? rows * ks : ((rows + 31) >> 5) * 32 * ksp;
+}
+__device__ __forceinline__ int rsrc_bytes(int64_t bytes) {
+  return (int)(bytes < 0 ? 0 : bytes > 0x7FFFFFFF ? 0x7FFFFFFF : bytes);
+}
+
 // s_waitcnt immediate that waits for vmcnt <= n and lgkmcnt == 0 (gfx9
 // encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14).
 __host__ __device__ constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | (7 << 4) | ((n >> 4) << 14); }

@@ -248,3 +248,34 @@ def test_grouped_many_expert_rows_with_scratch():
         lo, hi = int(off[g]), int(off[g + 1])
         ref = c_oracle.scaled_gemm_exact(x[lo:hi], gw[g].cpu().numpy(), xs[lo:hi], gws[g].cpu().numpy())
         assert_f32_close(c[lo:hi], ref, f"expert {g}")
+
+
+def torch_seeded_inputs(m, n, k, seed, scale_lo, scale_hi):
+    """The configuration's operands drawn the way the reference draws its own (torch.manual_seed(seed), then the
+    draw order of wave_lang/kernel/wave/utils/mxfp_utils.py:37-57 through the host mirror's generator), on the CPU
+    so that the bytes do not depend on the GPU's random number generator."""
+    from wave_amd.kernel.wave.utils.mxfp_utils import generate_gemm_afp4wfp4_inputs
+
+    x, w, xs, ws = generate_gemm_afp4wfp4_inputs((m, n, k), device="cpu", seed=seed, scale_range=(scale_lo, scale_hi + 1))
+    return x.numpy(), xs.numpy(), w.T.contiguous().numpy(), ws.numpy()
+
+
+@pytest.mark.parametrize("name,m,n,k,dt,seed,lo,hi", [
+    ("cfg1", 1024, 1024, 1024, torch.float32, 0, 124, 130),
+    ("cfg2", 8192, 8192, 8192, torch.bfloat16, 1, 124, 130),
+    ("cfg3_m16", 16, 28672, 8192, torch.bfloat16, 2, 120, 134),
+    ("cfg3_m128", 128, 28672, 8192, torch.bfloat16, 2, 120, 134),
+    ("cfg5", 4093, 6144, 7168, torch.float32, 4, 100, 154),
+])
+def test_configs_with_torch_seeded_inputs(name, m, n, k, dt, seed, lo, hi):
+    """The same configurations on inputs seeded with torch.manual_seed(n) (the other tests of this file draw them
+    with numpy's generator): the library's own kernel choice against the exact oracle, whole C for the small ones,
+    at least 8 rows of every 256-row M tile for the large ones."""
+    x, xs, w_t, ws = torch_seeded_inputs(m, n, k, seed, lo, hi)
+    assert x.shape == (m, k // 2) and w_t.shape == (n, k // 2) and xs.min() >= lo and xs.max() <= hi
+    c = run_gemm(x, xs, w_t, ws, dt)
+    if m * n <= 1 << 22:
+        assert_close(c, c_oracle.scaled_gemm_exact(x, w_t, xs, ws), dt, name)
+    else:
+        rows = sample_rows(m, 8, seed=seed)
+        assert_close(c[rows], c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows), dt, name)

@@ -662,6 +662,12 @@ def main():
             "launch_us": round(pper * 1e6, 2), "tflops": round(flops / pper / 1e12, 1),
             "frac_of_mxfp4_peak": round(flops / pper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
         }
+        # roofline: the dominant kernel by itself, i.e. this leg's launches (a call with row-major scales is that
+        # kernel + the scale re-layout launch in front of it: `call_us`, the figure `value` is computed from)
+        roofline["call_us"] = roofline["launch_us"]
+        roofline["launch_us"] = round(pper * 1e6, 2)
+        roofline["achieved"] = round(flops / pper / 1e12, 1)
+        roofline["frac"] = round(flops / pper / 1e12 / PEAK_MXFP4_TFLOPS, 4)
         if n % 256 == 0 and k % 512 == 0 and k >= 1536:
             # ... and B in b_preshuffle order on top (static weights, preshuffled once, as the reference's
             # asymmetric kernels assume: templates/tagged_mxfp4_gemm.py:950-991): A through LDS, B straight from

@@ -58,7 +58,9 @@ struct MidCfg {
   static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
 };
 
-template <class Cfg>
+// A_RM / B_RM: the operand's scales are row-major (else MFMA32 order).  Template parameters, not run-time flags:
+// a branch on the layout inside the K loop makes the compiler wait for every outstanding request at the join.
+template <class Cfg, bool A_RM, bool B_RM>
 __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   constexpr int MT_M = Cfg::MT_M, DA = Cfg::DA, DB = Cfg::DB, LB = Cfg::LB;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -71,8 +73,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   const int n0 = blockIdx.x * (kMidCW * wv);
   const int k_tiles_blocks = nkt * 256;   // bytes of one 32-row block row of MFMA32 scales
   const int groups = (nkt + 3) >> 2;      // scale groups of 4 K tiles
-  const bool a_rowmajor = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
-  const bool b_rowmajor = p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
+  constexpr bool a_rowmajor = A_RM, b_rowmajor = B_RM;
 
   if (wave == kMidCW) {
     // ================= the producer wave: A and its scales =================
@@ -172,18 +173,19 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
 #pragma unroll
   for (int t = 0; t < 4; ++t) foff[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
   // A lane's scale dword of a K tile holds the bytes of its K steps 0 .. 3: groups fg, 2 + fg, 4 + fg, 6 + fg of
-  // row fr.  MFMA32 order stores exactly that dword; from a row's eight bytes one v_perm picks it.
-  // (Branch-free on the layout: a branch in the K loop makes the compiler wait for every outstanding request at
-  // the join.)  The lane reads two dwords at c0 + (j % 2) * c1 + (j / 2 % 2) * 512 and permutes them by `pick`.
-  struct ScaleRead { int c0, c1, hi; uint32_t pick; };
-  auto scale_read = [&](bool rowmajor) -> ScaleRead {
-    if (rowmajor) return {fr * 16, 8, 4, fg ? 0x07050301u : 0x06040200u};
-    return {lane * 4, 256, 0, 0x03020100u};
-  };
-  const ScaleRead ra = scale_read(a_rowmajor), rb = scale_read(b_rowmajor);
-  auto lane_scales = [&](const uint8_t *img, const ScaleRead &r, int j) -> uint32_t {
-    const uint8_t *at = img + r.c0 + (j & 1) * r.c1 + ((j & 2) << 8);
-    return __builtin_amdgcn_perm(*(const uint32_t *)(at + r.hi), *(const uint32_t *)at, r.pick);
+  // row fr.  MFMA32 order stores exactly that dword.  From a row-major image the lane reads the row's 16-byte
+  // piece (K tiles j & ~1 and j | 1; one ds_read_b128 of 32 contiguous pieces - 8-byte reads at a 16-byte pitch
+  // are bank conflicts, which made the scale reads 80 % of the kernel's LDS time on top of the fragment reads),
+  // takes the half of its K tile and picks its four bytes with one v_perm.
+  const uint32_t pick = fg ? 0x07050301u : 0x06040200u;
+  auto lane_scales = [&](const uint8_t *img, auto rm_tag, int j) -> uint32_t {
+    if constexpr (decltype(rm_tag)::value) {
+      const v4i q = *(const v4i *)(img + ((j & 2) << 8) + fr * 16);
+      const bool odd = (j & 1) != 0;
+      return __builtin_amdgcn_perm((uint32_t)(odd ? q.w : q.y), (uint32_t)(odd ? q.z : q.x), pick);
+    } else {
+      return *(const uint32_t *)(img + (j & 3) * 256 + lane * 4);
+    }
   };
 
   v16f acc[MT_M];
@@ -220,8 +222,8 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     const uint8_t *a_t = a_ring + a_slot * Cfg::A_SLOT, *b_t = b_ring + slot * 4096;
     uint32_t sa[MT_M];
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) sa[i] = lane_scales(as_ring + ((j >> 2) & 1) * Cfg::AS_SLOT + i * 1024, ra, j);
-    const uint32_t sb = lane_scales(bs_ring + ((j >> 2) & 3) * 1024, rb, j);
+    for (int i = 0; i < MT_M; ++i) sa[i] = lane_scales(as_ring + ((j >> 2) & 1) * Cfg::AS_SLOT + i * 1024, std::integral_constant<bool, A_RM>{}, j);
+    const uint32_t sb = lane_scales(bs_ring + ((j >> 2) & 3) * 1024, std::integral_constant<bool, B_RM>{}, j);
     auto step = [&](auto t_tag) {
       constexpr int T = decltype(t_tag)::value;
       const v4i fb = *(const v4i *)(b_t + foff[T]);
@@ -298,19 +300,26 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   }
 }
 
-template <class Cfg>
+template <class Cfg, bool A_RM, bool B_RM>
 __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p, const int wv) {
-  mid_body<Cfg>(p, wv);
+  mid_body<Cfg, A_RM, B_RM>(p, wv);
+}
+
+template <class Cfg, bool A_RM, bool B_RM>
+hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, B_RM>, Cfg::LDS);
+  if (e != hipSuccess) return e;
+  const int bn = kMidCW * wv;
+  mid_gemm_kernel<Cfg, A_RM, B_RM><<<dim3((p.n + bn - 1) / bn, 1, 1), dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
+  return hipGetLastError();
 }
 
 template <class Cfg>
 hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
-  static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg>, Cfg::LDS);
-  if (e != hipSuccess) return e;
-  const int bn = kMidCW * wv;
-  mid_gemm_kernel<Cfg><<<dim3((p.n + bn - 1) / bn, 1, 1), dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
-  return hipGetLastError();
+  const bool a_rm = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR, b_rm = p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
+  if (a_rm) return b_rm ? launch_mid_layouts<Cfg, true, true>(p, wv, stream) : launch_mid_layouts<Cfg, true, false>(p, wv, stream);
+  return b_rm ? launch_mid_layouts<Cfg, false, true>(p, wv, stream) : launch_mid_layouts<Cfg, false, false>(p, wv, stream);
 }
 
 // Columns per compute wave: the narrowest strips (a multiple of 4 columns, 16 to 32) that still fit the number of

@@ -701,6 +701,18 @@ def main():
                 "bytes": dbytes, "steps": dsteps, "settle_ms": round(dsettle, 1),
                 "traffic": read_traffic(name),
             }
+            if dm > 48:
+                # resident weights: B's scales converted once to the MFMA operand order (wave_mxfp4_scale_convert),
+                # as a serving stack would keep them; A's scales stay row-major
+                from wave_amd import _lib as L
+                rsets = [(x, xs, w, wave_amd.scale_convert(ws, dn, dk // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32))
+                         for (x, xs, w, ws) in dsets]
+                _, rper, _ = time_gemm(torch, wave_amd, rsets, dout, dsteps, args.warmup, b_scale_layout=L.SCALE_MFMA32)
+                result["decode_m%d" % dm]["resident_weight_scales"] = {
+                    "workload": "the same call with B's scales already in MFMA operand order",
+                    "launch_us": round(rper * 1e6, 2), "gbps": round(dbytes / rper / 1e9, 1),
+                    "frac_of_hbm_peak": round(dbytes / rper / 1e9 / PEAK_HBM_GBPS, 4)}
+                del rsets
             del dsets, dout
 
         # the step in front of the GEMM: quantise the bf16 activation of this workload

@@ -40,17 +40,20 @@ namespace {
 constexpr int kMidBN = 128, kMidCW = 4, kMidNT = (kMidCW + 1) * 64;
 constexpr int kMidOnce = 2;  // the "nt" bit: B is read exactly once
 
-template <int BM_>
+// B_RM: B's scales are row-major: their image is then two buffers of 32 rows x 128 bytes (16 K tiles) per wave
+// instead of four of 1 KB (4 K tiles), and B's ring a K tile shorter.
+template <int BM_, bool B_RM_>
 struct MidCfg {
   static constexpr int BM = BM_, MT_M = BM / 32;
+  static constexpr bool B_RM = B_RM_;
   static constexpr int A_SLOT = BM * kTileKBytes;
   static constexpr int DA = BM <= 128 ? 3 : 2;                           // K tiles of A in LDS
-  static constexpr int DB = BM <= 64 ? 7 : BM <= 192 ? 5 : 4;            // K tiles of B in each wave's ring
+  static constexpr int DB = (BM <= 64 ? 7 : BM <= 192 ? 5 : 4) - (B_RM ? 1 : 0);  // K tiles of B in each wave's ring
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
   static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
   static constexpr int A_RING = DA * A_SLOT, AS_RING = 2 * AS_SLOT;
   static constexpr int B_WAVE = DB * 32 * kTileKBytes;                   // one wave's B ring (4 KB per K tile)
-  static constexpr int BS_WAVE = 4 * 1024;                               // one wave's scale ring: 4 groups of 4 K tiles
+  static constexpr int BS_WAVE = B_RM ? 8 * 1024 : 4 * 1024;             // one wave's scale images
   static constexpr int LDS = A_RING + AS_RING + kMidCW * (B_WAVE + BS_WAVE);
   static constexpr int A_LD = BM / 8;                                    // A DMA instructions per K tile (producer)
   static_assert(LDS <= 160 * 1024, "LDS");
@@ -60,8 +63,9 @@ struct MidCfg {
 
 // A_RM / B_RM: the operand's scales are row-major (else MFMA32 order).  Template parameters, not run-time flags:
 // a branch on the layout inside the K loop makes the compiler wait for every outstanding request at the join.
-template <class Cfg, bool A_RM, bool B_RM>
+template <class Cfg, bool A_RM>
 __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
+  constexpr bool B_RM = Cfg::B_RM;
   constexpr int MT_M = Cfg::MT_M, DA = Cfg::DA, DB = Cfg::DB, LB = Cfg::LB;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   uint8_t *const a_ring = smem;
@@ -161,11 +165,25 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(b_ring + slot * 4096 + d * 1024), 16, b_goff[d], soff,
                                                0, kMidOnce);
   };
-  const int bs_goff = b_rowmajor ? (lane & 31) * p.ks + (lane >> 5) * 16 : lane * 16;
-  const int bs_gstep = b_rowmajor ? 32 : 1024;
+  // MFMA32 order: the four 256-byte blocks of K tiles 4g .. 4g + 3 are contiguous, one instruction per group.
   auto issue_bs = [&](int g) {
-    const int soff = g < groups ? g * bs_gstep : (int)0x80000000;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (g & 3) * 1024), 16, bs_goff, soff, 0, 0);
+    const int soff = g < groups ? g * 1024 : (int)0x80000000;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (g & 3) * 1024), 16, lane * 16, soff, 0, 0);
+  };
+  // Row-major: whole 128-byte lines of the rows (16 K tiles), 8 rows per instruction, swizzled like the operand
+  // tiles; instructions [d0, d1) of the image of K tiles 16 g16 .. 16 g16 + 15.  (Fetched as 32 bytes of each of
+  // 32 rows per 4 K tiles, every instruction touched 32 cache lines and every line was requested four times:
+  // 1.3 us of a 32 us call at M = 128.)
+  auto issue_bs16 = [&](int g16, int d0, auto count_tag) {
+    const int soff = g16 * 128 < p.ks ? g16 * 128 : (int)0x80000000;
+#pragma unroll
+    for (int dd = 0; dd < decltype(count_tag)::value; ++dd) {
+      const int d = d0 + dd;
+      const int r = d * 8 + ld_row;
+      const int goff = r * p.ks + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (g16 & 1) * 4096 + d * 1024), 16, goff, soff,
+                                               0, 0);
+    }
   };
 
   const int fr = lane & 31, fg = lane >> 5;
@@ -178,13 +196,24 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   // are bank conflicts, which made the scale reads 80 % of the kernel's LDS time on top of the fragment reads),
   // takes the half of its K tile and picks its four bytes with one v_perm.
   const uint32_t pick = fg ? 0x07050301u : 0x06040200u;
+  auto pick_scales = [&](const v4i q, int j) -> uint32_t {
+    const bool odd = (j & 1) != 0;
+    return __builtin_amdgcn_perm((uint32_t)(odd ? q.w : q.y), (uint32_t)(odd ? q.z : q.x), pick);
+  };
   auto lane_scales = [&](const uint8_t *img, auto rm_tag, int j) -> uint32_t {
     if constexpr (decltype(rm_tag)::value) {
-      const v4i q = *(const v4i *)(img + ((j & 2) << 8) + fr * 16);
-      const bool odd = (j & 1) != 0;
-      return __builtin_amdgcn_perm((uint32_t)(odd ? q.w : q.y), (uint32_t)(odd ? q.z : q.x), pick);
+      return pick_scales(*(const v4i *)(img + ((j & 2) << 8) + fr * 16), j);
     } else {
       return *(const uint32_t *)(img + (j & 3) * 256 + lane * 4);
+    }
+  };
+  // B, row-major: the piece (j / 2) % 8 of row fr in the swizzled 32 x 128-byte image of the K tile's group of 16
+  auto lane_scales_b = [&](int j) -> uint32_t {
+    if constexpr (B_RM) {
+      const int c = (j >> 1) & 7;
+      return pick_scales(*(const v4i *)(bs_ring + ((j >> 4) & 1) * 4096 + fr * 128 + ((c ^ ((fr >> 1) & 7)) << 4)), j);
+    } else {
+      return lane_scales(bs_ring + ((j >> 2) & 3) * 1024, std::false_type{}, j);
     }
   };
 
@@ -195,9 +224,10 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     for (int g = 0; g < 16; ++g) acc[i][g] = 0.f;
 
   // prologue: B(0 .. LB - 1) with the scale groups they belong to in front
+  if constexpr (B_RM) issue_bs16(0, 0, std::integral_constant<int, 4>{});
 #pragma unroll
   for (int j = 0; j < LB; ++j) {
-    if ((j & 3) == 0) issue_bs(j >> 2);
+    if (!B_RM && (j & 3) == 0) issue_bs(j >> 2);
     issue_b(j, j);
   }
   int slot = 0, slot_next = LB;  // slots of B(j) and of the K tile requested next
@@ -215,7 +245,13 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     asm volatile("" ::: "memory");
     // the slot of B(j - 1) is free (its fragments were consumed before the wait above): request B(j + LB)
     const int jn = j + LB;
-    if ((jn & 3) == 0) issue_bs(jn >> 2);
+    if constexpr (B_RM) {
+      // the image of the next 16 K tiles, in the first two of this group's four quarters: its buffer held the
+      // previous group's, last read in K tile j - 1 at the latest, and the requests are older than that group's B
+      if ((j & 11) == 0) issue_bs16((j >> 4) + 1, (j & 4) >> 1, std::integral_constant<int, 2>{});
+    } else {
+      if ((jn & 3) == 0) issue_bs(jn >> 2);
+    }
     issue_b(jn, slot_next);
     slot_next = slot_next + 1 == DB ? 0 : slot_next + 1;
 
@@ -223,7 +259,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     uint32_t sa[MT_M];
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) sa[i] = lane_scales(as_ring + ((j >> 2) & 1) * Cfg::AS_SLOT + i * 1024, std::integral_constant<bool, A_RM>{}, j);
-    const uint32_t sb = lane_scales(bs_ring + ((j >> 2) & 3) * 1024, std::integral_constant<bool, B_RM>{}, j);
+    const uint32_t sb = lane_scales_b(j);
     auto step = [&](auto t_tag) {
       constexpr int T = decltype(t_tag)::value;
       const v4i fb = *(const v4i *)(b_t + foff[T]);
@@ -300,26 +336,29 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   }
 }
 
-template <class Cfg, bool A_RM, bool B_RM>
+template <class Cfg, bool A_RM>
 __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p, const int wv) {
-  mid_body<Cfg, A_RM, B_RM>(p, wv);
+  mid_body<Cfg, A_RM>(p, wv);
 }
 
-template <class Cfg, bool A_RM, bool B_RM>
+template <class Cfg, bool A_RM>
 hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
   static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, B_RM>, Cfg::LDS);
+  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM>, Cfg::LDS);
   if (e != hipSuccess) return e;
   const int bn = kMidCW * wv;
-  mid_gemm_kernel<Cfg, A_RM, B_RM><<<dim3((p.n + bn - 1) / bn, 1, 1), dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
+  mid_gemm_kernel<Cfg, A_RM><<<dim3((p.n + bn - 1) / bn, 1, 1), dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
   return hipGetLastError();
 }
 
-template <class Cfg>
+template <int BM>
 hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
   const bool a_rm = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR, b_rm = p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
-  if (a_rm) return b_rm ? launch_mid_layouts<Cfg, true, true>(p, wv, stream) : launch_mid_layouts<Cfg, true, false>(p, wv, stream);
-  return b_rm ? launch_mid_layouts<Cfg, false, true>(p, wv, stream) : launch_mid_layouts<Cfg, false, false>(p, wv, stream);
+  if (a_rm)
+    return b_rm ? launch_mid_layouts<MidCfg<BM, true>, true>(p, wv, stream)
+                : launch_mid_layouts<MidCfg<BM, false>, true>(p, wv, stream);
+  return b_rm ? launch_mid_layouts<MidCfg<BM, true>, false>(p, wv, stream)
+              : launch_mid_layouts<MidCfg<BM, false>, false>(p, wv, stream);
 }
 
 // Columns per compute wave: the narrowest strips (a multiple of 4 columns, 16 to 32) that still fit the number of
@@ -353,10 +392,10 @@ bool mid_gemm_applies(const GemmParams &p) {
 
 hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream) {
   const int wv = mid_wave_cols(p, num_cus);
-  if (p.m <= 64) return launch_mid_cfg<MidCfg<64>>(p, wv, stream);
-  if (p.m <= 128) return launch_mid_cfg<MidCfg<128>>(p, wv, stream);
-  if (p.m <= 192) return launch_mid_cfg<MidCfg<192>>(p, wv, stream);
-  return launch_mid_cfg<MidCfg<256>>(p, wv, stream);
+  if (p.m <= 64) return launch_mid_cfg<64>(p, wv, stream);
+  if (p.m <= 128) return launch_mid_cfg<128>(p, wv, stream);
+  if (p.m <= 192) return launch_mid_cfg<192>(p, wv, stream);
+  return launch_mid_cfg<256>(p, wv, stream);
 }
 
 }  // namespace wave_mxfp4

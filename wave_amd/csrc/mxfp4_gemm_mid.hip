@@ -7,23 +7,24 @@
 // path for A, which comes from L2.  Vector memory operations of a wave retire in issue order, so a wave that
 // waits for a recent A tile also waits for every older B request: the two streams need different waves.
 //
-//   * One workgroup per 4 * WV columns of C: four compute waves side by side along N (WV <= 32 columns each, all
-//     BM = 64 .. 256 rows; v_mfma_scale_f32_32x32x64_f8f6f4, BM / 32 accumulator tiles) and a fifth, the
-//     producer wave, which does nothing but request A.  WV is chosen per problem so that the strips come out as
-//     a whole number of rounds over the CUs (N = 28672 on 256 CUs: 28 columns per wave, 256 workgroups, where
-//     strips of 128 columns would leave 32 CUs without work and the rest 14 % more): the rate at which one CU
-//     pulls from HBM is what bounds the kernel.  The rows of a wave's MFMA operand past WV are zero-filled by
-//     the buffer descriptor (no memory request) and their columns are not stored.
-//   * B is wave private: a compute wave fetches the 32 B rows it multiplies (4 DMA instructions of 8 rows x 128
-//     bytes per K tile, whole cache lines, non-temporal) into its own ring of DB K tiles and waits for its own
-//     requests only, with a counted vmcnt that leaves the younger DB - 2 K tiles in flight.  Its scales come in
-//     by one DMA instruction per FOUR K tiles: in MFMA32 order the blocks of consecutive K tiles are contiguous
-//     and a lane reads its dword; row-major scales are fetched as 32 rows x 32 bytes (two lanes per row) and a
-//     lane picks its four bytes of the row's eight with one v_perm, so neither order needs a pass of its own.
+//   * One workgroup per strip of 4 * WV columns of C: four compute waves, 2 x 2 on the strip (each BM / 2 rows
+//     and two of the strip's four groups of WV <= 32 columns; v_mfma_scale_f32_32x32x64_f8f6f4, BM / 32
+//     accumulator tiles, one A fragment per two MFMAs) and a fifth, the producer wave, which does nothing but
+//     request A.  WV is chosen per problem so that the strips come out as a whole number of rounds over the CUs
+//     (N = 28672 on 256 CUs: 28 columns per group, 256 workgroups).  The rows of a group's MFMA operand past WV
+//     are zero-filled by the buffer descriptor (no memory request) and their columns are not stored.
+//   * B goes into a ring of DB K tiles (four groups of 32 rows x 128 bytes each).  Compute wave w fetches group
+//     w (4 DMA instructions of 8 rows x 128 bytes per K tile, whole cache lines, non-temporal) and waits for its
+//     own requests only, with a counted vmcnt that leaves the younger DB - 2 K tiles in flight; the K tile's one
+//     barrier then makes all four groups visible to all.  The groups' scales travel the same way: in MFMA32
+//     order one DMA instruction per FOUR K tiles (the blocks of consecutive K tiles are contiguous) and a lane
+//     reads its dword; row-major scales as whole 128-byte lines of the 32 rows (16 K tiles per image, swizzled
+//     like the operand tiles) from which a lane reads its row's 16-byte piece and picks the four bytes of its K
+//     tile with one v_perm, so neither order needs a pass of its own.
 //   * The producer wave fetches A (BM rows x 128 bytes per K tile) and its scales into a ring of DA K tiles,
-//     DA - 1 ahead, waits for its own requests, and meets the compute waves at one barrier per K tile: behind it
-//     A(j) is visible to all and the slot of A(j - 1) is free.
-//   * C leaves through the wave's own (by then idle) B ring, 64 or 128 bytes per row and store.
+//     DA - 1 ahead, waits for its own requests, and meets the compute waves at the barrier: behind it A(j) is
+//     visible to all and the slots of A(j - 1) and B(j - 1) are free.
+//   * C leaves through the (by then idle) B ring, 4 KB per wave, 64 or 128 bytes per row and store.
 //
 // Taken for K % 256 == 0 (at least 4 K tiles), N % 4 == 0, each scale tensor row-major or in MFMA32 order
 // (e8m0_shuffle order is re-laid out first when the library has scratch; B scales in MFMA32 order fix WV at 32,
@@ -52,12 +53,12 @@ struct MidCfg {
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
   static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
   static constexpr int A_RING = DA * A_SLOT, AS_RING = 2 * AS_SLOT;
-  static constexpr int B_WAVE = DB * 32 * kTileKBytes;                   // one wave's B ring (4 KB per K tile)
+  static constexpr int B_RING = DB * kMidBN * kTileKBytes;               // B ring (16 KB per K tile: four 32-row groups)
   static constexpr int BS_WAVE = B_RM ? 8 * 1024 : 4 * 1024;             // one wave's scale images
-  static constexpr int LDS = A_RING + AS_RING + kMidCW * (B_WAVE + BS_WAVE);
+  static constexpr int LDS = A_RING + AS_RING + B_RING + kMidCW * BS_WAVE;
   static constexpr int A_LD = BM / 8;                                    // A DMA instructions per K tile (producer)
   static_assert(LDS <= 160 * 1024, "LDS");
-  static_assert(B_WAVE >= 32 * 32 * 4, "the C staging of a 32 x 32 f32 tile must fit the wave's ring");
+  static_assert(MT_M % 2 == 0 && B_RING >= kMidCW * 32 * 32 * 4, "two row halves; the waves' C staging fits the ring");
   static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
 };
 
@@ -127,13 +128,21 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
       issue_a(jn, slot_next);
       slot_next = slot_next + 1 == DA ? 0 : slot_next + 1;
     }
+    __builtin_amdgcn_s_barrier();  // (the compute waves' barrier in front of their C staging)
     __builtin_amdgcn_s_waitcnt(0);
     return;
   }
 
   // ================= a compute wave =================
-  uint8_t *const b_ring = smem + Cfg::A_RING + Cfg::AS_RING + wave * (Cfg::B_WAVE + Cfg::BS_WAVE);
-  uint8_t *const bs_ring = b_ring + Cfg::B_WAVE;
+  // The four compute waves sit 2 x 2 on the strip: wave (wm, wn) multiplies rows wm * BM / 2 .. and the strip's
+  // 32-row groups 2 wn and 2 wn + 1 of B (one A fragment per two MFMAs instead of one per MFMA: the kernel is
+  // bound by LDS bandwidth).  Each wave still requests, and waits for, the group `wave` of B and of its scales;
+  // the K tile's barrier makes all four groups visible to all.
+  constexpr int MI = MT_M / 2;
+  const int wm = wave >> 1, wn = wave & 1;
+  uint8_t *const b_ring = smem + Cfg::A_RING + Cfg::AS_RING;  // DB slots of 4 groups x 32 rows x 128 bytes
+  uint8_t *const bs_all = b_ring + Cfg::B_RING;               // the four groups' scale images
+  uint8_t *const bs_ring = bs_all + wave * Cfg::BS_WAVE;      // ... the one this wave fills
   const int nw0 = n0 + wave * wv;  // the wave's first column of C = first row of B
   const int cols = max(0, min(wv, p.n - nw0));  // columns it owns
   // B: the descriptor starts at the wave's first row (row-major) or at the 16-row block that holds it
@@ -162,8 +171,8 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     const int soff = kt < nkt ? kt * b_kt_stride : (int)0x80000000;
 #pragma unroll
     for (int d = 0; d < 4; ++d)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(b_ring + slot * 4096 + d * 1024), 16, b_goff[d], soff,
-                                               0, kMidOnce);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(b_ring + slot * 16384 + wave * 4096 + d * 1024), 16,
+                                               b_goff[d], soff, 0, kMidOnce);
   };
   // MFMA32 order: the four 256-byte blocks of K tiles 4g .. 4g + 3 are contiguous, one instruction per group.
   auto issue_bs = [&](int g) {
@@ -208,20 +217,23 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     }
   };
   // B, row-major: the piece (j / 2) % 8 of row fr in the swizzled 32 x 128-byte image of the K tile's group of 16
-  auto lane_scales_b = [&](int j) -> uint32_t {
+  auto lane_scales_b = [&](int g, int j) -> uint32_t {  // g: the 32-row group of the strip
+    const uint8_t *img = bs_all + g * Cfg::BS_WAVE;
     if constexpr (B_RM) {
       const int c = (j >> 1) & 7;
-      return pick_scales(*(const v4i *)(bs_ring + ((j >> 4) & 1) * 4096 + fr * 128 + ((c ^ ((fr >> 1) & 7)) << 4)), j);
+      return pick_scales(*(const v4i *)(img + ((j >> 4) & 1) * 4096 + fr * 128 + ((c ^ ((fr >> 1) & 7)) << 4)), j);
     } else {
-      return lane_scales(bs_ring + ((j >> 2) & 3) * 1024, std::false_type{}, j);
+      return lane_scales(img + ((j >> 2) & 3) * 1024, std::false_type{}, j);
     }
   };
 
-  v16f acc[MT_M];
+  v16f acc[MI][2];
 #pragma unroll
-  for (int i = 0; i < MT_M; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int g = 0; g < 16; ++g) acc[i][g] = 0.f;
+    for (int jn = 0; jn < 2; ++jn)
+#pragma unroll
+      for (int g = 0; g < 16; ++g) acc[i][jn][g] = 0.f;
 
   // prologue: B(0 .. LB - 1) with the scale groups they belong to in front
   if constexpr (B_RM) issue_bs16(0, 0, std::integral_constant<int, 4>{});
@@ -255,20 +267,30 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     issue_b(jn, slot_next);
     slot_next = slot_next + 1 == DB ? 0 : slot_next + 1;
 
-    const uint8_t *a_t = a_ring + a_slot * Cfg::A_SLOT, *b_t = b_ring + slot * 4096;
-    uint32_t sa[MT_M];
+    const uint8_t *a_t = a_ring + a_slot * Cfg::A_SLOT + wm * MI * 32 * kTileKBytes;
+    const uint8_t *b_t = b_ring + slot * 16384 + wn * 2 * 4096;
+    uint32_t sa[MI], sb[2];
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) sa[i] = lane_scales(as_ring + ((j >> 2) & 1) * Cfg::AS_SLOT + i * 1024, std::integral_constant<bool, A_RM>{}, j);
-    const uint32_t sb = lane_scales_b(j);
+    for (int i = 0; i < MI; ++i)
+      sa[i] = lane_scales(as_ring + ((j >> 2) & 1) * Cfg::AS_SLOT + (wm * MI + i) * 1024, std::integral_constant<bool, A_RM>{}, j);
+#pragma unroll
+    for (int jn = 0; jn < 2; ++jn) sb[jn] = lane_scales_b(wn * 2 + jn, j);
     auto step = [&](auto t_tag) {
       constexpr int T = decltype(t_tag)::value;
-      const v4i fb = *(const v4i *)(b_t + foff[T]);
-      const v8i vb = {fb.x, fb.y, fb.z, fb.w, 0, 0, 0, 0};
+      v8i vb[2];
 #pragma unroll
-      for (int i = 0; i < MT_M; ++i) {
+      for (int jn = 0; jn < 2; ++jn) {
+        const v4i fb = *(const v4i *)(b_t + jn * 4096 + foff[T]);
+        vb[jn] = v8i{fb.x, fb.y, fb.z, fb.w, 0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
         const v4i fa = *(const v4i *)(a_t + i * 32 * kTileKBytes + foff[T]);
         const v8i va = {fa.x, fa.y, fa.z, fa.w, 0, 0, 0, 0};
-        acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i], 4, 4, T, (int)sb, T, (int)sa[i]);
+#pragma unroll
+        for (int jn = 0; jn < 2; ++jn)
+          acc[i][jn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb[jn], va, acc[i][jn], 4, 4, T, (int)sb[jn], T,
+                                                                       (int)sa[i]);
       }
     };
     step(T0{});
@@ -278,60 +300,68 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     slot = slot + 1 == DB ? 0 : slot + 1;
     a_slot = a_slot + 1 == DA ? 0 : a_slot + 1;
   }
-  // the trailing (empty) requests must have landed before the ring becomes the C staging area
+  // the trailing (empty) requests must have landed, and every wave must be done reading the last K tile, before
+  // the ring becomes the C staging area
   __builtin_amdgcn_s_waitcnt(0);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 
   // ---------------- C: accumulators -> the wave's ring -> global ----------------
-  // acc[i][4q + e] is row lane % 32, column 8q + 4 * (lane / 32) + e of the wave's strip, row block i.  The strip
-  // is staged as 32 rows of eight 4-column pieces and stored 8 rows per instruction, a lane one piece (8 bytes of
-  // bf16, 16 of f32), the pieces past the wave's columns left out.
-  uint8_t *stage = b_ring;
+  // acc[i][jn][4q + e] is row lane % 32, column 8q + 4 * (lane / 32) + e of the 32 x 32 tile (row block
+  // wm * MI + i, group 2 wn + jn).  A tile is staged as 32 rows of eight 4-column pieces and stored 8 rows per
+  // instruction, a lane one piece (8 bytes of bf16, 16 of f32), the pieces past the group's columns left out.
+  uint8_t *stage = b_ring + wave * 4096;
   const bool out_bf16 = p.out_bf16 != 0;
   const int elt = out_bf16 ? 2 : 4;
   const __amdgpu_buffer_rsrc_t c_rsrc =
       make_rsrc_n(p.c, (int)min((int64_t)p.m * p.n * elt, (int64_t)0x7FFFFFFF));
-  if (cols <= 0) return;
   const int lr = lane >> 3, lc = lane & 7;
-  const bool mine = lc * 4 < cols;
-  if (out_bf16) {
-    typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i) {
+  for (int jn = 0; jn < 2; ++jn) {
+    const int gc0 = n0 + (wn * 2 + jn) * wv;                 // the group's first column of C
+    const bool mine = lc * 4 < min(wv, p.n - gc0);          // (negative past N: nothing stored)
+    if (out_bf16) {
+      typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const bf4 h = {(__bf16)acc[i][4 * q], (__bf16)acc[i][4 * q + 1], (__bf16)acc[i][4 * q + 2], (__bf16)acc[i][4 * q + 3]};
-        *(bf4 *)(stage + fr * 64 + (((q * 2 + fg) ^ ((fr >> 2) & 7)) << 3)) = h;
+      for (int i = 0; i < MI; ++i) {
+        const v16f &a = acc[i][jn];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const bf4 h = {(__bf16)a[4 * q], (__bf16)a[4 * q + 1], (__bf16)a[4 * q + 2], (__bf16)a[4 * q + 3]};
+          *(bf4 *)(stage + fr * 64 + (((q * 2 + fg) ^ ((fr >> 2) & 7)) << 3)) = h;
+        }
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += 8) {
+          const int r = r0 + lr, row = (wm * MI + i) * 32 + r;
+          const v2i v = *(const v2i *)(stage + r * 64 + ((lc ^ ((r >> 2) & 7)) << 3));
+          // rows past M lie past the end of C: dropped by the descriptor
+          if (mine) __builtin_amdgcn_raw_buffer_store_b64(v, c_rsrc, (int)(((int64_t)row * p.n + gc0 + lc * 4) * 2), 0, 0);
+        }
+        asm volatile("" ::: "memory");
       }
-      asm volatile("" ::: "memory");
+    } else {
 #pragma unroll
-      for (int r0 = 0; r0 < 32; r0 += 8) {
-        const int r = r0 + lr, row = i * 32 + r;
-        const v2i v = *(const v2i *)(stage + r * 64 + ((lc ^ ((r >> 2) & 7)) << 3));
-        // rows past M lie past the end of C: dropped by the descriptor
-        if (mine) __builtin_amdgcn_raw_buffer_store_b64(v, c_rsrc, (int)(((int64_t)row * p.n + nw0 + lc * 4) * 2), 0, 0);
+      for (int i = 0; i < MI; ++i) {
+        const v16f &a = acc[i][jn];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4f v = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+          const int chunk = q * 2 + fg;
+          *(v4f *)(stage + fr * 128 + ((chunk ^ (fr & 7)) << 4)) = v;
+        }
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += 8) {
+          const int r = r0 + lr, row = (wm * MI + i) * 32 + r;
+          const v4f v = *(const v4f *)(stage + r * 128 + ((lc ^ (r & 7)) << 4));
+          if (mine)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc,
+                                                   (int)(((int64_t)row * p.n + gc0 + lc * 4) * 4), 0, 0);
+        }
+        asm volatile("" ::: "memory");
       }
-      asm volatile("" ::: "memory");
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < MT_M; ++i) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const v4f v = {acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
-        const int chunk = q * 2 + fg;
-        *(v4f *)(stage + fr * 128 + ((chunk ^ (fr & 7)) << 4)) = v;
-      }
-      asm volatile("" ::: "memory");
-#pragma unroll
-      for (int r0 = 0; r0 < 32; r0 += 8) {
-        const int r = r0 + lr, row = i * 32 + r;
-        const v4f v = *(const v4f *)(stage + r * 128 + ((lc ^ (r & 7)) << 4));
-        if (mine)
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc,
-                                                 (int)(((int64_t)row * p.n + nw0 + lc * 4) * 4), 0, 0);
-      }
-      asm volatile("" ::: "memory");
     }
   }
 }

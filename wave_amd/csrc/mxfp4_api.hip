@@ -106,10 +106,11 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
   int v = variant;
   if (v == WAVE_MXFP4_VARIANT_AUTO) {
     // 48 < M <= 256 and enough 128-column strips to put most CUs to work: reading B once from HBM bounds the
-    // problem, and the mid-M kernel gives B all of LDS.  Measured at K = 8192 against the streaming kernel
-    // (M <= 64) and the tile kernels: it wins from N = 14336 on for 64 < M <= 192 (128 x 28672: 46 -> 34 us,
-    // 128 x 12288 loses, 23 -> 26 us) and from about N = 24576 on at M = 64 (32 -> 30 us) and M = 256 (55 -> 51 us).
-    if (mid_shape_ok(m, n, k) && m > 48 && n >= ((m > 64 && m <= 192) ? 14336 : 24576)) return WAVE_MXFP4_VARIANT_MID_M;
+    // problem, and the mid-M kernel gives B and A rings of their own.  Measured at K = 8192 against the streaming
+    // kernel (M <= 64) and the tile kernels: it wins from N = 12288 on for 64 < M <= 192 (128 x 28672: 46 -> 31 us,
+    // 128 x 12288: 23.4 -> 22.3 us, 96 x 8192 loses, 17 -> 21 us) and from about N = 24576 on at M = 64
+    // (32 -> 28 us) and M = 256 (55 -> 48 us; 256 x 16384 loses, 39 -> 42 us).
+    if (mid_shape_ok(m, n, k) && m > 48 && n >= ((m > 64 && m <= 192) ? 12288 : 24576)) return WAVE_MXFP4_VARIANT_MID_M;
     if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;
     v = pick_tile_variant(m, n);
   }

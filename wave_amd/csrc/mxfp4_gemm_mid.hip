@@ -18,9 +18,9 @@
 //     own requests only, with a counted vmcnt that leaves the younger DB - 2 K tiles in flight; the K tile's one
 //     barrier then makes all four groups visible to all.  The groups' scales travel the same way: in MFMA32
 //     order one DMA instruction per FOUR K tiles (the blocks of consecutive K tiles are contiguous) and a lane
-//     reads its dword; row-major scales as whole 128-byte lines of the 32 rows (16 K tiles per image, swizzled
-//     like the operand tiles) from which a lane reads its row's 16-byte piece and picks the four bytes of its K
-//     tile with one v_perm, so neither order needs a pass of its own.
+//     reads its dword; row-major scales as 64 bytes of each of the 32 rows (8 K tiles per image, the 16-byte
+//     pieces swizzled for conflict-free reads) from which a lane reads its row's piece of two K tiles and picks
+//     the four bytes of its K tile with one v_perm, so neither order needs a pass of its own.
 //   * The producer wave fetches A (BM rows x 128 bytes per K tile) and its scales into a ring of DA K tiles,
 //     DA - 1 ahead, waits for its own requests, and meets the compute waves at the barrier: behind it A(j) is
 //     visible to all and the slots of A(j - 1) and B(j - 1) are free.
@@ -41,20 +41,28 @@ namespace {
 constexpr int kMidBN = 128, kMidCW = 4, kMidNT = (kMidCW + 1) * 64;
 constexpr int kMidOnce = 2;  // the "nt" bit: B is read exactly once
 
-// B_RM: B's scales are row-major: their image is then two buffers of 32 rows x 128 bytes (16 K tiles) per wave
-// instead of four of 1 KB (4 K tiles), and B's ring a K tile shorter.
+// B_RM: B's scales are row-major: a group's image is then two buffers of 32 rows x 64 bytes (8 K tiles) instead
+// of four buffers of 1 KB (4 K tiles).
 template <int BM_, bool B_RM_>
 struct MidCfg {
   static constexpr int BM = BM_, MT_M = BM / 32;
   static constexpr bool B_RM = B_RM_;
   static constexpr int A_SLOT = BM * kTileKBytes;
-  static constexpr int DA = BM <= 128 ? 3 : 2;                           // K tiles of A in LDS
-  static constexpr int DB = (BM <= 64 ? 7 : BM <= 192 ? 5 : 4) - (B_RM ? 1 : 0);  // K tiles of B in each wave's ring
+  // Ring depths, measured at N = 28672, K = 8192 (us at M = 64 / 128 / 192): A, which every workgroup re-reads
+  // from L2 at the same moment as all the others, needs the deeper ring.  With no B traffic at all the kernel
+  // took 17 / 22 us at two K tiles of A ahead: its latency, not B's, set the pace.
+  //   (DA, DB) = (3, 7) / (3, 5) / (2, 5): 29.9 / 33.1 / 43.5     (6, 5) / (5, 3) / (3, 3): 27.9 / 31.4 / 39.0
+  static constexpr int DA = BM <= 64 ? 6 : BM <= 128 ? 5 : BM <= 192 ? 3 : 2;  // K tiles of A in LDS
+  static constexpr int DB = BM <= 64 ? 5 : BM <= 192 ? 3 : 4;            // K tiles of B in the ring
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
   static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
-  static constexpr int A_RING = DA * A_SLOT, AS_RING = 2 * AS_SLOT;
+  // Scale groups of A in LDS: the one being read, (j / 4), up to the one requested with A(j + DA - 1); a group's
+  // slot may be overwritten only when the group before it in that slot is no longer read: more than
+  // ceil((DA - 1) / 4) slots (a power of two, for the slot index).
+  static constexpr int AS_SLOTS = (DA - 1 + 3) / 4 + 1 <= 2 ? 2 : 4;
+  static constexpr int A_RING = DA * A_SLOT, AS_RING = AS_SLOTS * AS_SLOT;
   static constexpr int B_RING = DB * kMidBN * kTileKBytes;               // B ring (16 KB per K tile: four 32-row groups)
-  static constexpr int BS_WAVE = B_RM ? 8 * 1024 : 4 * 1024;             // one wave's scale images
+  static constexpr int BS_WAVE = 4 * 1024;                               // one group's scale images
   static constexpr int LDS = A_RING + AS_RING + B_RING + kMidCW * BS_WAVE;
   static constexpr int A_LD = BM / 8;                                    // A DMA instructions per K tile (producer)
   static_assert(LDS <= 160 * 1024, "LDS");
@@ -107,13 +115,14 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
       const int soff = g < groups ? g * as_gstep : (int)0x80000000;
 #pragma unroll
       for (int i = 0; i < MT_M; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(as_rsrc, WAVE_LDS_PTR(as_ring + (g & 1) * Cfg::AS_SLOT + i * 1024), 16,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(as_rsrc, WAVE_LDS_PTR(as_ring + (g & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + i * 1024), 16,
                                                  as_goff, soff + i * as_istep, 0, 0);
     };
     // (a group's last K tiles may lie past K: those bytes belong to the next block or row, or lie past the
     // buffer; nobody reads them)
     // prologue: A(0 .. DA - 2), with the scale groups they belong to in front
-    issue_as(0);
+#pragma unroll
+    for (int g = 0; g <= (DA - 2) / 4; ++g) issue_as(g);  // the groups of A(0 .. DA - 2)
 #pragma unroll
     for (int j = 0; j < DA - 1; ++j) issue_a(j, j);
     int slot_next = DA - 1;  // slot of the K tile requested next
@@ -124,7 +133,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
       __builtin_amdgcn_s_barrier();  // A(j) visible to the compute waves; they are done with A(j - 1)
       asm volatile("" ::: "memory");
       const int jn = j + DA - 1;
-      if ((jn & 3) == 0) issue_as(jn >> 2);  // (group g's slot was last read in K tile 4g - 5 at the latest)
+      if ((jn & 3) == 0) issue_as(jn >> 2);  // (its slot's previous group is no longer read: AS_SLOTS)
       issue_a(jn, slot_next);
       slot_next = slot_next + 1 == DA ? 0 : slot_next + 1;
     }
@@ -179,19 +188,19 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     const int soff = g < groups ? g * 1024 : (int)0x80000000;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (g & 3) * 1024), 16, lane * 16, soff, 0, 0);
   };
-  // Row-major: whole 128-byte lines of the rows (16 K tiles), 8 rows per instruction, swizzled like the operand
-  // tiles; instructions [d0, d1) of the image of K tiles 16 g16 .. 16 g16 + 15.  (Fetched as 32 bytes of each of
-  // 32 rows per 4 K tiles, every instruction touched 32 cache lines and every line was requested four times:
-  // 1.3 us of a 32 us call at M = 128.)
-  auto issue_bs16 = [&](int g16, int d0, auto count_tag) {
-    const int soff = g16 * 128 < p.ks ? g16 * 128 : (int)0x80000000;
+  // Row-major: 64 bytes of each of the group's rows (8 K tiles), 16 rows per instruction, two instructions per
+  // image, the 16-byte pieces swizzled so that the lanes' reads of one piece per row are conflict-free (piece c
+  // of row r at position c ^ (r / 4) % 4 of the row's 64 bytes).  Image h holds K tiles 8 h .. 8 h + 7.
+  // (Fetched as 32 bytes of each of 32 rows per 4 K tiles, every instruction touched 32 cache lines and every
+  // line was requested four times.)
+  auto issue_bs8 = [&](int h) {
+    const int soff = h * 64 < p.ks ? h * 64 : (int)0x80000000;
 #pragma unroll
-    for (int dd = 0; dd < decltype(count_tag)::value; ++dd) {
-      const int d = d0 + dd;
-      const int r = d * 8 + ld_row;
-      const int goff = r * p.ks + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (g16 & 1) * 4096 + d * 1024), 16, goff, soff,
-                                               0, 0);
+    for (int dd = 0; dd < 2; ++dd) {
+      const int r = dd * 16 + (lane >> 2);
+      const int goff = r * p.ks + (((lane & 3) ^ ((r >> 2) & 3)) << 4);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (h & 1) * 2048 + dd * 1024), 16, goff, soff, 0,
+                                               0);
     }
   };
 
@@ -216,12 +225,12 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
       return *(const uint32_t *)(img + (j & 3) * 256 + lane * 4);
     }
   };
-  // B, row-major: the piece (j / 2) % 8 of row fr in the swizzled 32 x 128-byte image of the K tile's group of 16
+  // B, row-major: the piece (j / 2) % 4 of row fr in the swizzled 32 x 64-byte image of the K tile's group of 8
   auto lane_scales_b = [&](int g, int j) -> uint32_t {  // g: the 32-row group of the strip
     const uint8_t *img = bs_all + g * Cfg::BS_WAVE;
     if constexpr (B_RM) {
-      const int c = (j >> 1) & 7;
-      return pick_scales(*(const v4i *)(img + ((j >> 4) & 1) * 4096 + fr * 128 + ((c ^ ((fr >> 1) & 7)) << 4)), j);
+      const int c = (j >> 1) & 3;
+      return pick_scales(*(const v4i *)(img + ((j >> 3) & 1) * 2048 + fr * 64 + ((c ^ ((fr >> 2) & 3)) << 4)), j);
     } else {
       return lane_scales(img + ((j >> 2) & 3) * 1024, std::false_type{}, j);
     }
@@ -236,7 +245,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
       for (int g = 0; g < 16; ++g) acc[i][jn][g] = 0.f;
 
   // prologue: B(0 .. LB - 1) with the scale groups they belong to in front
-  if constexpr (B_RM) issue_bs16(0, 0, std::integral_constant<int, 4>{});
+  if constexpr (B_RM) issue_bs8(0);
 #pragma unroll
   for (int j = 0; j < LB; ++j) {
     if (!B_RM && (j & 3) == 0) issue_bs(j >> 2);
@@ -258,9 +267,9 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     // the slot of B(j - 1) is free (its fragments were consumed before the wait above): request B(j + LB)
     const int jn = j + LB;
     if constexpr (B_RM) {
-      // the image of the next 16 K tiles, in the first two of this group's four quarters: its buffer held the
-      // previous group's, last read in K tile j - 1 at the latest, and the requests are older than that group's B
-      if ((j & 11) == 0) issue_bs16((j >> 4) + 1, (j & 4) >> 1, std::integral_constant<int, 2>{});
+      // the image of the next 8 K tiles: its buffer held the previous image, last read in K tile j - 1, and the
+      // requests are older than those K tiles' B
+      if ((j & 7) == 0) issue_bs8((j >> 3) + 1);
     } else {
       if ((jn & 3) == 0) issue_bs(jn >> 2);
     }
@@ -272,7 +281,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     uint32_t sa[MI], sb[2];
 #pragma unroll
     for (int i = 0; i < MI; ++i)
-      sa[i] = lane_scales(as_ring + ((j >> 2) & 1) * Cfg::AS_SLOT + (wm * MI + i) * 1024, std::integral_constant<bool, A_RM>{}, j);
+      sa[i] = lane_scales(as_ring + ((j >> 2) & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + (wm * MI + i) * 1024, std::integral_constant<bool, A_RM>{}, j);
 #pragma unroll
     for (int jn = 0; jn < 2; ++jn) sb[jn] = lane_scales_b(wn * 2 + jn, j);
     auto step = [&](auto t_tag) {

@@ -53,3 +53,27 @@ def test_random_shape_against_oracle(case):
     got = run_gemm(x, conv[layouts[a_layout]](xs), w_in, conv[layouts[b_layout]](ws), out_dtype, **kw)
     assert not np.isnan(got).any()
     assert_close(got[rows], ref, out_dtype, f"case {case}")
+
+
+def _wide_cases(count, seed):
+    """Shapes the newer kernels take under the library's own choice: 49..256 rows against a wide N (mid-M kernel,
+    every strip width), more than 256 tiles with N a multiple of 192 (256x192 tiles) or with preshuffled B
+    (B-direct kernel), K a multiple of 256 so that they qualify, and ragged M."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        kind = rng.integers(0, 3)
+        if kind == 0:    # mid-M
+            m, n, k = int(rng.integers(49, 257)), 4 * int(rng.integers(3072, 9000)), 256 * int(rng.integers(4, 12))
+        elif kind == 1:  # 256x192 tiles
+            m, n, k = int(rng.integers(2100, 5000)), 192 * int(rng.integers(20, 40)), 256 * int(rng.integers(3, 8))
+        else:            # more tiles than CUs, N % 256 == 0 (B-direct when preshuffled)
+            m, n, k = int(rng.integers(2100, 5000)), 256 * int(rng.integers(14, 24)), 512 * int(rng.integers(3, 6))
+        out.append((i, m, n, k, int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2)),
+                    bool(rng.integers(0, 2)), bool(rng.integers(0, 4) > 0)))
+    return out
+
+
+@pytest.mark.parametrize("case", _wide_cases(18, seed=21), ids=lambda c: f"w{c[0]}-{c[1]}x{c[2]}x{c[3]}")
+def test_random_wide_shape_against_oracle(case):
+    test_random_shape_against_oracle(case)

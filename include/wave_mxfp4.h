@@ -99,8 +99,9 @@ typedef enum {
   /* M <= 256 against a wide B from HBM: one workgroup per strip of 64 to 128 columns, B through deep
    * wave-private LDS rings, A fed by a producer wave.  Needs K % 256 == 0, K >= 1024, N % 4 == 0, no split, and
    * each scale tensor row-major or MFMA32 (e8m0_shuffle order needs the workspace); WAVE_MXFP4_ERR_UNSUPPORTED
-   * otherwise.  AUTO takes it for 48 < M <= 256 and a wide N.  The reference runs such shapes through its generic
-   * tile kernel (tests/kernel/wave_gemm_mxfp_test.py:291-339). */
+   * otherwise.  AUTO takes it for 48 < M <= 256 and a wide N, and for a grouped problem of few rows per expert
+   * (see wave_mxfp4_gemm_grouped).  The reference runs such shapes through its generic tile kernel
+   * (tests/kernel/wave_gemm_mxfp_test.py:291-339). */
   WAVE_MXFP4_VARIANT_MID_M = 8,
   /* 256x192x256 tile, 8 waves, persistent kernel only: for problems whose count of 256x256 tiles leaves the last
    * round over the CUs partly empty while 256x192 tiles fill whole rounds (4093 x 6144: 384 tiles are 1.5 rounds
@@ -175,6 +176,14 @@ size_t wave_mxfp4_static_scratch_bytes(void);
  * wave_mxfp4_grouped_workspace_bytes(...) bytes: with it the scales of both
  * operands are first re-laid out for one-dword-per-lane reads, as in
  * wave_mxfp4_gemm (N % 32 == 0 and K % 256 == 0; otherwise it is not used).
+ * A small batch (AUTO: at most 128 rows per expert on average, and enough
+ * experts x 128-column strips to occupy half the CUs) runs on the mid-M kernel,
+ * one workgroup per (expert, strip), with no table and no scale re-layout: the
+ * call is then bound by reading every expert's B once.  It needs K % 256 == 0,
+ * K >= 1024, N % 4 == 0, A's scales row-major and B's row-major or MFMA32;
+ * WAVE_MXFP4_VARIANT_MID_M asks for it by name (WAVE_MXFP4_ERR_UNSUPPORTED
+ * where it does not apply).  The other variants accepted here are AUTO, NAIVE
+ * and the square tile shapes.
  */
 int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,
                             void *c, const int32_t *offsets, int num_groups, int64_t total_rows,

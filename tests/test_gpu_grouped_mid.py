@@ -1,0 +1,110 @@
+"""GPU: the grouped GEMM at a small batch (a few rows per expert: the decode step of a mixture of experts, the
+per-expert loop of tests/kernel/moe_test.py:175-246 at serving sizes) through the mid-M kernel, one workgroup per
+(expert, strip of columns), against the exact oracle applied per group: ragged and empty groups, groups of more rows
+than one block, N that ends inside a strip, row-major and MFMA32 expert scales, preshuffled expert weights, both
+output types, rows past the last offset left alone, and the library's own choice of it."""
+
+import numpy as np
+import pytest
+import torch
+
+import wave_amd
+from oracle import c_oracle
+from oracle import mxfp4_oracle as orc
+from wave_amd import _lib
+
+from gpu_util import DEV, assert_close, to_gpu
+
+pytestmark = pytest.mark.gpu
+V = _lib.VARIANT_MID_M
+RM, M32 = _lib.SCALE_ROW_MAJOR, _lib.SCALE_MFMA32
+
+
+def inputs(e, n, k, rows, seed, force_empty=(), lo=118, hi=136):
+    off = orc.make_group_offsets(e, rows, seed, force_empty=force_empty)
+    x, xs, _, _ = orc.make_inputs(rows, 1, k, seed, scale_lo=lo, scale_hi=hi)
+    rng = np.random.default_rng(seed + 100)
+    w = rng.integers(0, 256, size=(e, n, k // 2), dtype=np.uint8)
+    ws = rng.integers(lo, hi + 1, size=(e, n, k // 32), dtype=np.uint8)
+    return x, xs, w, ws, off
+
+
+def reference(x, xs, w, ws, off):
+    out = np.full((x.shape[0], w.shape[1]), np.nan)
+    for g in range(len(off) - 1):
+        a, b = int(off[g]), int(off[g + 1])
+        if b > a:
+            out[a:b] = c_oracle.scaled_gemm_exact(x[a:b], w[g], xs[a:b], ws[g])
+    return out
+
+
+def run(x, xs, w, ws, off, dt, lb=RM, pre=False, **kw):
+    e, n, k = w.shape[0], w.shape[1], x.shape[1] * 2
+    gx, gxs, gw, gws, goff = to_gpu(x, xs, w, ws, off)
+    if pre:
+        gw = torch.stack([wave_amd.b_preshuffle(gw[g]) for g in range(e)])
+    if lb != RM:
+        gws = torch.stack([wave_amd.scale_convert(gws[g], n, k // 32, RM, lb) for g in range(e)])
+    out = torch.full((x.shape[0], n), float("nan"), dtype=dt, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out, b_scale_layout=lb,
+                                b_layout=_lib.B_PRESHUFFLE if pre else _lib.B_ROW_MAJOR, **kw)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+def check(c, ref, dt, what):
+    done = ~np.isnan(ref)
+    assert np.isnan(c[~done]).all(), f"{what}: rows of no group were written"
+    assert_close(c[done.all(axis=1)], ref[done.all(axis=1)], dt, what)
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("lb,pre", [(RM, False), (M32, False), (RM, True), (M32, True)])
+@pytest.mark.parametrize("e,n,k,rows", [(8, 160, 1024, 40), (5, 1008, 1280, 333), (16, 96, 2048, 16), (3, 4096, 1024, 700)])
+def test_grouped_mid_ragged_groups(e, n, k, rows, lb, pre, dt):
+    """Uneven groups (333 rows over 5 experts and 700 over 3: groups of more rows than a block, taken block by
+    block; 16 rows over 16 experts: groups of one row and none)."""
+    x, xs, w, ws, off = inputs(e, n, k, rows, seed=e + rows)
+    c = run(x, xs, w, ws, off, dt, lb=lb, pre=pre, variant=V)
+    check(c, reference(x, xs, w, ws, off), dt, f"E={e} {rows}x{n}x{k}")
+
+
+@pytest.mark.parametrize("force_empty", [(0,), (3, 4), (7,), (0, 1, 2, 3, 4, 5, 6)])
+def test_grouped_mid_empty_groups_and_rows_past_the_last_offset(force_empty):
+    e, n, k = 8, 640, 1536
+    x, xs, w, ws, off = inputs(e, n, k, 90, seed=21, force_empty=force_empty)
+    for g in force_empty:
+        assert off[g] == off[g + 1]
+    x = np.concatenate([x, np.zeros((10, k // 2), np.uint8)])
+    xs = np.concatenate([xs, np.full((10, k // 32), 127, np.uint8)])
+    ref = reference(x, xs, w, ws, off)
+    assert np.isnan(ref[90:]).all()
+    check(run(x, xs, w, ws, off, torch.float32, variant=V), ref, torch.float32, str(force_empty))
+
+
+@pytest.mark.parametrize("per_expert", [1, 8, 48, 96])
+def test_grouped_mid_is_the_librarys_choice_at_a_small_batch(per_expert):
+    """8 experts of config 4's N and K, a few rows per expert: AUTO must give the bits of the kernel asked for by
+    name, which is checked against the oracle (all rows up to 8 per expert, sampled rows beyond) and, element for
+    element, against the table-driven tile kernels."""
+    e, n, k = 8, 14336, 4096
+    rows = e * per_expert
+    x, xs, w, ws, off = inputs(e, n, k, rows, seed=3, lo=122, hi=132)
+    c = run(x, xs, w, ws, off, torch.bfloat16, variant=V)
+    assert np.array_equal(run(x, xs, w, ws, off, torch.bfloat16), c)
+    for g in range(e):
+        a, b = int(off[g]), int(off[g + 1])
+        if b == a:
+            continue
+        pick = np.unique(np.concatenate([np.arange(a, b, max(1, (b - a) // 6)), [b - 1]]))
+        ref = c_oracle.scaled_gemm_exact(x, w[g], xs, ws[g], rows=pick)
+        assert_close(c[pick], ref, torch.bfloat16, f"expert {g}")
+    tiles = run(x, xs, w, ws, off, torch.float32, variant=_lib.VARIANT_T128x128_W2x2)
+    assert_close(c, tiles.astype(np.float64), torch.bfloat16, "all elements vs the tile kernel")
+
+
+def test_grouped_mid_unsupported_cases_are_refused():
+    e, n, k, rows = 4, 128, 512, 32           # fewer than four K tiles
+    x, xs, w, ws, off = inputs(e, n, k, rows, seed=9)
+    with pytest.raises((ValueError, RuntimeError)):
+        run(x, xs, w, ws, off, torch.float32, variant=V)

@@ -97,6 +97,9 @@ bool is_tile_variant(int v) {
   return bm != 0;
 }
 
+// Grouped problems of at most this many rows per expert on average go to the mid-M kernel.
+constexpr int64_t kGroupedMidMaxAvgRows = 128;
+
 // What the mid-M kernel takes (the part of it that the shape alone decides).
 bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
   return m >= 1 && m <= mid_max_m() && k % kTileK == 0 && k >= 4 * kTileK && n % 4 == 0;
@@ -577,8 +580,24 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   if (p.b_group_stride % 16 != 0 || p.b_scale_group_stride % 8 != 0) return WAVE_MXFP4_ERR_MISALIGNED;
 
   if (variant == WAVE_MXFP4_VARIANT_SKINNY || variant == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT ||
-      variant == WAVE_MXFP4_VARIANT_MID_M || variant == WAVE_MXFP4_VARIANT_T256x192_W4x2)
+      variant == WAVE_MXFP4_VARIANT_T256x192_W4x2)
     return WAVE_MXFP4_ERR_UNSUPPORTED;
+  // A small batch routed over the experts: every expert's B is read once for a handful of rows, so the call is
+  // bound by streaming B, like the dense mid-M problem.  One workgroup per (expert, strip of columns), no table, no
+  // re-layout of the scales.  AUTO takes it up to 128 rows per expert on average (measured at 8 experts, N = 14336,
+  // K = 4096 against the table-driven tile kernels), when there are enough strips to put most CUs to work.
+  if (variant == WAVE_MXFP4_VARIANT_MID_M || variant == WAVE_MXFP4_VARIANT_AUTO) {
+    const bool fits = mid_grouped_applies(p);
+    if (variant == WAVE_MXFP4_VARIANT_MID_M && !fits) return WAVE_MXFP4_ERR_UNSUPPORTED;
+    const int64_t avg = (total_rows + num_groups - 1) / num_groups;
+    const bool pays = avg <= kGroupedMidMaxAvgRows && (int64_t)num_groups * ((n + 127) / 128) >= device_cus() / 2;
+    if (fits && (variant == WAVE_MXFP4_VARIANT_MID_M || pays)) {
+      // rows per block: twice the average group (the routing is uneven), in steps of 64, at most the whole batch
+      int64_t bm = 2 * avg < total_rows ? 2 * avg : total_rows;
+      bm = bm > 256 ? 256 : (bm + 63) / 64 * 64;
+      return record_hip(launch_mid_gemm(p, device_cus(), stream, (int)bm));
+    }
+  }
   const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_tile_variant(total_rows > 64 ? total_rows : 65, n)
                                                    : pick_variant(total_rows, n, k, variant);
   if (v == WAVE_MXFP4_VARIANT_NAIVE) return record_hip(launch_naive_gemm(p, stream));

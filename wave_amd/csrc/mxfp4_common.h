@@ -137,7 +137,8 @@ bool persist_prefers_192(const GemmParams &p, int num_cus, int parts256);
 bool asym_gemm_applies(const GemmParams &p, int num_cus, bool forced);
 hipError_t launch_asym_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
 bool mid_gemm_applies(const GemmParams &p);
-hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
+hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream, int bm = 0);
+bool mid_grouped_applies(const GemmParams &p);
 int mid_max_m();
 int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *partial_bytes);
 hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);

@@ -72,8 +72,11 @@ struct MidCfg {
 
 // A_RM / B_RM: the operand's scales are row-major (else MFMA32 order).  Template parameters, not run-time flags:
 // a branch on the layout inside the K loop makes the compiler wait for every outstanding request at the join.
+// One strip of one block of `m_rows` <= BM rows: A [m_rows, kp] at `a_base` with its scales at `as_base`, B [N, kp]
+// at `b_base` (one expert's, for a grouped problem) with its scales at `bs_base`, C rows at `c_base`.
 template <class Cfg, bool A_RM>
-__device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
+__device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, const uint8_t *a_base, const uint8_t *as_base,
+                                         const uint8_t *b_base, const uint8_t *bs_base, uint8_t *c_base, const int m_rows) {
   constexpr bool B_RM = Cfg::B_RM;
   constexpr int MT_M = Cfg::MT_M, DA = Cfg::DA, DB = Cfg::DB, LB = Cfg::LB;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -90,9 +93,9 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
 
   if (wave == kMidCW) {
     // ================= the producer wave: A and its scales =================
-    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(p.a, (int)min((int64_t)p.m * kp, (int64_t)0x7FFFFFFF));
-    const int64_t as_bytes = a_rowmajor ? (int64_t)p.m * p.ks : (int64_t)((p.m + 31) >> 5) * k_tiles_blocks;
-    const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc_n(p.a_scale, (int)min(as_bytes, (int64_t)0x7FFFFFFF));
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(a_base, (int)min((int64_t)m_rows * kp, (int64_t)0x7FFFFFFF));
+    const int64_t as_bytes = a_rowmajor ? (int64_t)m_rows * p.ks : (int64_t)((m_rows + 31) >> 5) * k_tiles_blocks;
+    const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc_n(as_base, (int)min(as_bytes, (int64_t)0x7FFFFFFF));
     const int row0 = lane >> 3;  // instruction d fills rows 8d .. 8d + 7
     // chunk position lane % 8 of row r holds chunk (lane % 8) ^ ((r / 2) % 8); 8d is a multiple of 8, so the
     // swizzle depends on the lane alone when d is even, and flips bit 2 of it when d is odd
@@ -159,12 +162,12 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   const int b_blk = p.b_preshuffled ? (nw0 & ~15) : nw0, b_sub = nw0 - b_blk;
   const int64_t b_bytes = (int64_t)p.n * kp - (int64_t)b_blk * kp;
   const __amdgpu_buffer_rsrc_t b_rsrc =
-      make_rsrc_n(p.b + (int64_t)b_blk * kp, (int)min(max(b_bytes, (int64_t)0), (int64_t)0x7FFFFFFF));
+      make_rsrc_n(b_base + (int64_t)b_blk * kp, (int)min(max(b_bytes, (int64_t)0), (int64_t)0x7FFFFFFF));
   // B scales: MFMA32 order from the wave's 32-row block on (there WV is 32), row-major from its first row on
   const int64_t bs_skip = b_rowmajor ? (int64_t)nw0 * p.ks : (int64_t)(nw0 >> 5) * k_tiles_blocks;
   const int64_t bs_bytes = (b_rowmajor ? (int64_t)p.n * p.ks : (int64_t)((p.n + 31) >> 5) * k_tiles_blocks) - bs_skip;
   const __amdgpu_buffer_rsrc_t bs_rsrc =
-      make_rsrc_n(p.b_scale + bs_skip, (int)min(max(bs_bytes, (int64_t)0), (int64_t)0x7FFFFFFF));
+      make_rsrc_n(bs_base + bs_skip, (int)min(max(bs_bytes, (int64_t)0), (int64_t)0x7FFFFFFF));
   // B DMA: instruction d fills rows 8d .. 8d + 7 of the wave's 32 (LDS: row * 128, swizzled chunks)
   const int ld_row = lane >> 3;
   int b_goff[4];
@@ -257,6 +260,12 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   typedef std::integral_constant<int, 1> T1;
   typedef std::integral_constant<int, 2> T2;
   typedef std::integral_constant<int, 3> T3;
+  // Row block i of this wave is block 2 i + wm of the tile, so that a block of fewer rows than BM (a small group
+  // of a grouped problem) leaves both halves of the workgroup the same share; the blocks past the rows take no
+  // fragment reads and no MFMAs: the K loop exists once per count of live blocks, with no branch inside it.
+  const int live = min(max((m_rows - 32 * wm + 63) >> 6, 0), MI);
+  auto k_loop = [&](auto live_tag) {
+  constexpr int LIVE = decltype(live_tag)::value;
   for (int j = 0; j < nkt; ++j) {
     // B(j) and its scales have landed: younger are B(j + 1 .. j + LB - 1), 4 requests each (and up to two scale
     // groups, which the count leaves out: it then waits for that much more than it must)
@@ -276,12 +285,12 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     issue_b(jn, slot_next);
     slot_next = slot_next + 1 == DB ? 0 : slot_next + 1;
 
-    const uint8_t *a_t = a_ring + a_slot * Cfg::A_SLOT + wm * MI * 32 * kTileKBytes;
+    const uint8_t *a_t = a_ring + a_slot * Cfg::A_SLOT + wm * 32 * kTileKBytes;
     const uint8_t *b_t = b_ring + slot * 16384 + wn * 2 * 4096;
     uint32_t sa[MI], sb[2];
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
-      sa[i] = lane_scales(as_ring + ((j >> 2) & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + (wm * MI + i) * 1024, std::integral_constant<bool, A_RM>{}, j);
+    for (int i = 0; i < LIVE; ++i)
+      sa[i] = lane_scales(as_ring + ((j >> 2) & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + (2 * i + wm) * 1024, std::integral_constant<bool, A_RM>{}, j);
 #pragma unroll
     for (int jn = 0; jn < 2; ++jn) sb[jn] = lane_scales_b(wn * 2 + jn, j);
     auto step = [&](auto t_tag) {
@@ -293,8 +302,8 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
         vb[jn] = v8i{fb.x, fb.y, fb.z, fb.w, 0, 0, 0, 0};
       }
 #pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        const v4i fa = *(const v4i *)(a_t + i * 32 * kTileKBytes + foff[T]);
+      for (int i = 0; i < LIVE; ++i) {
+        const v4i fa = *(const v4i *)(a_t + i * 64 * kTileKBytes + foff[T]);
         const v8i va = {fa.x, fa.y, fa.z, fa.w, 0, 0, 0, 0};
 #pragma unroll
         for (int jn = 0; jn < 2; ++jn)
@@ -309,6 +318,19 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     slot = slot + 1 == DB ? 0 : slot + 1;
     a_slot = a_slot + 1 == DA ? 0 : a_slot + 1;
   }
+  };
+  auto with_live = [&](auto self, auto tag) -> void {
+    constexpr int L = decltype(tag)::value;
+    if constexpr (L == 0) {
+      k_loop(tag);
+    } else {
+      if (live >= L)
+        k_loop(tag);
+      else
+        self(self, std::integral_constant<int, L - 1>{});
+    }
+  };
+  with_live(with_live, std::integral_constant<int, MI>{});
   // the trailing (empty) requests must have landed, and every wave must be done reading the last K tile, before
   // the ring becomes the C staging area
   __builtin_amdgcn_s_waitcnt(0);
@@ -318,13 +340,13 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
 
   // ---------------- C: accumulators -> the wave's ring -> global ----------------
   // acc[i][jn][4q + e] is row lane % 32, column 8q + 4 * (lane / 32) + e of the 32 x 32 tile (row block
-  // wm * MI + i, group 2 wn + jn).  A tile is staged as 32 rows of eight 4-column pieces and stored 8 rows per
+  // 2 i + wm, group 2 wn + jn).  A tile is staged as 32 rows of eight 4-column pieces and stored 8 rows per
   // instruction, a lane one piece (8 bytes of bf16, 16 of f32), the pieces past the group's columns left out.
   uint8_t *stage = b_ring + wave * 4096;
   const bool out_bf16 = p.out_bf16 != 0;
   const int elt = out_bf16 ? 2 : 4;
   const __amdgpu_buffer_rsrc_t c_rsrc =
-      make_rsrc_n(p.c, (int)min((int64_t)p.m * p.n * elt, (int64_t)0x7FFFFFFF));
+      make_rsrc_n(c_base, (int)min((int64_t)m_rows * p.n * elt, (int64_t)0x7FFFFFFF));
   const int lr = lane >> 3, lc = lane & 7;
 #pragma unroll
   for (int jn = 0; jn < 2; ++jn) {
@@ -334,6 +356,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
       typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
+        if (i >= live) break;
         const v16f &a = acc[i][jn];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -343,7 +366,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int r0 = 0; r0 < 32; r0 += 8) {
-          const int r = r0 + lr, row = (wm * MI + i) * 32 + r;
+          const int r = r0 + lr, row = (2 * i + wm) * 32 + r;
           const v2i v = *(const v2i *)(stage + r * 64 + ((lc ^ ((r >> 2) & 7)) << 3));
           // rows past M lie past the end of C: dropped by the descriptor
           if (mine) __builtin_amdgcn_raw_buffer_store_b64(v, c_rsrc, (int)(((int64_t)row * p.n + gc0 + lc * 4) * 2), 0, 0);
@@ -353,6 +376,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
     } else {
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
+        if (i >= live) break;
         const v16f &a = acc[i][jn];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -363,7 +387,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int r0 = 0; r0 < 32; r0 += 8) {
-          const int r = r0 + lr, row = (wm * MI + i) * 32 + r;
+          const int r = r0 + lr, row = (2 * i + wm) * 32 + r;
           const v4f v = *(const v4f *)(stage + r * 128 + ((lc ^ (r & 7)) << 4));
           if (mine)
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc,
@@ -375,29 +399,54 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv) {
   }
 }
 
-template <class Cfg, bool A_RM>
+// GROUPED: blockIdx.y is the expert; its rows offsets[e] .. offsets[e + 1] (clamped to [0, M], not validated) are
+// taken BM at a time - a group of more rows than BM streams its expert's B once per block of rows, which is what
+// the table-driven persistent kernel is for; this one is for the few rows per expert of a small batch.
+template <class Cfg, bool A_RM, bool GROUPED>
 __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p, const int wv) {
-  mid_body<Cfg, A_RM>(p, wv);
+  if constexpr (!GROUPED) {
+    mid_body<Cfg, A_RM>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
+  } else {
+    static_assert(A_RM, "a group may start at any row: A's scales row-major");
+    const int e = blockIdx.y;
+    const int lo = __builtin_amdgcn_readfirstlane(min(max(p.offsets[e], 0), p.m));
+    const int hi = __builtin_amdgcn_readfirstlane(min(max(p.offsets[e + 1], lo), p.m));
+    const uint8_t *b = p.b + (int64_t)e * p.b_group_stride, *bs = p.b_scale + (int64_t)e * p.b_scale_group_stride;
+    const int elt = p.out_bf16 ? 2 : 4;
+    for (int m0 = lo; m0 < hi; m0 += Cfg::BM) {
+      mid_body<Cfg, A_RM>(p, wv, p.a + (int64_t)m0 * p.kp, p.a_scale + (int64_t)m0 * p.ks, b, bs,
+                          (uint8_t *)p.c + (int64_t)m0 * p.n * elt, min(Cfg::BM, hi - m0));
+      // every wave is done with the rings (the C staging's reads included) before the next block's requests
+      __builtin_amdgcn_s_waitcnt(0);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    }
+  }
 }
 
-template <class Cfg, bool A_RM>
+template <class Cfg, bool A_RM, bool GROUPED>
 hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
   static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM>, Cfg::LDS);
+  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, GROUPED>, Cfg::LDS);
   if (e != hipSuccess) return e;
   const int bn = kMidCW * wv;
-  mid_gemm_kernel<Cfg, A_RM><<<dim3((p.n + bn - 1) / bn, 1, 1), dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
+  const dim3 grid((p.n + bn - 1) / bn, GROUPED ? p.num_groups : 1, 1);
+  mid_gemm_kernel<Cfg, A_RM, GROUPED><<<grid, dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
   return hipGetLastError();
 }
 
 template <int BM>
 hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
   const bool a_rm = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR, b_rm = p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
+  if (p.num_groups != 0)  // (row-major A scales: checked by mid_grouped_applies)
+    return b_rm ? launch_mid_layouts<MidCfg<BM, true>, true, true>(p, wv, stream)
+                : launch_mid_layouts<MidCfg<BM, false>, true, true>(p, wv, stream);
   if (a_rm)
-    return b_rm ? launch_mid_layouts<MidCfg<BM, true>, true>(p, wv, stream)
-                : launch_mid_layouts<MidCfg<BM, false>, true>(p, wv, stream);
-  return b_rm ? launch_mid_layouts<MidCfg<BM, true>, false>(p, wv, stream)
-              : launch_mid_layouts<MidCfg<BM, false>, false>(p, wv, stream);
+    return b_rm ? launch_mid_layouts<MidCfg<BM, true>, true, false>(p, wv, stream)
+                : launch_mid_layouts<MidCfg<BM, false>, true, false>(p, wv, stream);
+  return b_rm ? launch_mid_layouts<MidCfg<BM, true>, false, false>(p, wv, stream)
+              : launch_mid_layouts<MidCfg<BM, false>, false, false>(p, wv, stream);
 }
 
 // Columns per compute wave: the narrowest strips (a multiple of 4 columns, 16 to 32) that still fit the number of
@@ -405,9 +454,11 @@ hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
 // rows, so there a wave's strip is a block.
 int mid_wave_cols(const GemmParams &p, int num_cus) {
   if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR || num_cus <= 0) return 32;
-  const int64_t strips = (p.n + kMidBN - 1) / kMidBN;
-  const int64_t wgs = (strips + num_cus - 1) / num_cus * num_cus;
-  int64_t wv = (p.n + 4 * wgs - 1) / (4 * wgs);
+  const int64_t experts = p.num_groups != 0 ? p.num_groups : 1;
+  const int64_t strips = (p.n + kMidBN - 1) / kMidBN * experts;
+  const int64_t wgs = (strips + num_cus - 1) / num_cus * num_cus;   // whole rounds of the CUs
+  const int64_t per_expert = wgs / experts > 0 ? wgs / experts : 1;  // strips of one expert
+  int64_t wv = (p.n + 4 * per_expert - 1) / (4 * per_expert);
   wv = (wv + 3) / 4 * 4;
   return (int)(wv < 16 ? 16 : wv > 32 ? 32 : wv);
 }
@@ -429,11 +480,28 @@ bool mid_gemm_applies(const GemmParams &p) {
   return true;
 }
 
-hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream) {
+// Whether the mid-M kernel serves this grouped problem: row-major A scales (a group starts at any row), each
+// expert's B scales row-major or MFMA32, whole K tiles.  Any group sizes are computed correctly; it pays for few rows
+// per expert.
+bool mid_grouped_applies(const GemmParams &p) {
+  if (p.num_groups <= 0 || p.num_groups > 65535 || p.offsets == nullptr || p.splits != 1 || p.partial != nullptr) return false;
+  if (p.a_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR) return false;
+  if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  if ((p.k & (kTileK - 1)) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
+  if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)48 * p.kp >= ((int64_t)1 << 31) ||
+      (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31) || (int64_t)8 * p.k_tiles * 256 >= ((int64_t)1 << 31))
+    return false;
+  return true;
+}
+
+// `bm`: rows per block of a group (dense: M; grouped: the library's guess from the average group, a group of more
+// rows takes several blocks).
+hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream, int bm) {
   const int wv = mid_wave_cols(p, num_cus);
-  if (p.m <= 64) return launch_mid_cfg<64>(p, wv, stream);
-  if (p.m <= 128) return launch_mid_cfg<128>(p, wv, stream);
-  if (p.m <= 192) return launch_mid_cfg<192>(p, wv, stream);
+  if (bm <= 0) bm = p.m;
+  if (bm <= 64) return launch_mid_cfg<64>(p, wv, stream);
+  if (bm <= 128) return launch_mid_cfg<128>(p, wv, stream);
+  if (bm <= 192) return launch_mid_cfg<192>(p, wv, stream);
   return launch_mid_cfg<256>(p, wv, stream);
 }
 

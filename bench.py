@@ -277,13 +277,35 @@ def leg_cfg4(torch, wave_amd, dev, steps, warmup, variant=0):
 
     _, per32, _ = timed(torch, run32, steps, warmup)
     flops = 2.0 * rows * n * k
+    # the same experts at a serving batch: 64 tokens x top-2 = 128 rows dealt multinomially; every expert's B is
+    # read once for a handful of rows, so the call is bound by HBM (two copies of the weights rotated: 500 MB)
+    srows = 128
+    scounts = np.random.default_rng(3).multinomial(srows, np.ones(E) / E)
+    soffs = torch.from_numpy(np.concatenate([[0], np.cumsum(scounts)]).astype(np.int32)).to(dev)
+    wsets = [(w, ws), (w.clone(), ws.clone())]
+    sout = torch.empty(srows, n, dtype=torch.bfloat16, device=dev)
+    state = {"i": 0}
+
+    def run_serving(count):
+        for _ in range(count):
+            wi, wsi = wsets[state["i"] & 1]
+            state["i"] += 1
+            wave_amd.mxfp4_gemm_grouped(x[:srows], xs[:srows], wi, wsi, soffs, sout, variant=variant)
+
+    _, pers, _ = timed(torch, run_serving, steps, warmup)
+    sbytes = srows * (k // 2 + k // 32) + E * n * (k // 2 + k // 32) + srows * n * 2
+    del wsets
     return {"workload": f"cfg4: E={E} N={n} K={k} rows={rows} (counts {counts.tolist()}) bf16 out seed 3",
             "kernel": "persist_gemm_kernel (grouped)", "launch_us": round(per * 1e6, 2),
             "tflops": round(flops / per / 1e12, 1), "frac_of_mxfp4_peak": round(flops / per / 1e12 / PEAK_MXFP4_TFLOPS, 4),
             "settle_ms": round(settle_ms, 1), "wall_s_per_step": wall / steps,
             "resident_weight_scales": {"workload": "the same call with the experts' B scales already in MFMA operand order",
                                        "launch_us": round(per32 * 1e6, 2), "tflops": round(flops / per32 / 1e12, 1),
-                                       "frac_of_mxfp4_peak": round(flops / per32 / 1e12 / PEAK_MXFP4_TFLOPS, 4)}}
+                                       "frac_of_mxfp4_peak": round(flops / per32 / 1e12 / PEAK_MXFP4_TFLOPS, 4)},
+            "serving_batch": {"workload": f"the same experts, {srows} rows (counts {scounts.tolist()}), weights from HBM",
+                              "kernel": "mid_gemm_kernel (grouped)", "launch_us": round(pers * 1e6, 2),
+                              "algorithmic_bytes": sbytes, "gb_per_s": round(sbytes / pers / 1e9, 1),
+                              "frac_of_hbm_peak": round(sbytes / pers / 1e9 / PEAK_HBM_GBPS, 4)}}
 
 
 def leg_mxfp8(torch, wave_amd, dev, steps, warmup, variant=0):

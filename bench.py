@@ -645,7 +645,7 @@ def main():
         achieved = nbytes / per_launch / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                     "frac": round(achieved / PEAK_HBM_GBPS, 4), "traffic": measured_traffic,
-                    "kernel": "stream_gemm_kernel" if m <= 48 else "mid_gemm_kernel",
+                    "kernel": "stream_gemm_kernel" if m <= 16 else "mid_gemm_kernel",
                     "launch_us": round(per_launch * 1e6, 2)}
     else:
         achieved = flops / per_launch / 1e12
@@ -721,9 +721,10 @@ def main():
                 "gbps": round(dbytes / dper / 1e9, 1),
                 "frac_of_hbm_peak": round(dbytes / dper / 1e9 / PEAK_HBM_GBPS, 4),
                 "bytes": dbytes, "steps": dsteps, "settle_ms": round(dsettle, 1),
+                "kernel": "stream_gemm_kernel" if dm <= 16 else "mid_gemm_kernel",
                 "traffic": read_traffic(name),
             }
-            if dm > 48:
+            if dm > 16:
                 # resident weights: B's scales converted once to the MFMA operand order (wave_mxfp4_scale_convert),
                 # as a serving stack would keep them; A's scales stay row-major
                 from wave_amd import _lib as L

@@ -59,6 +59,17 @@ def test_mid_wide_n_strip_widths_and_scale_layouts(m, n, k, la, lb):
         assert np.array_equal(c, run(x, xs, w, ws, torch.float32, variant=V, split_k=1))
 
 
+@pytest.mark.parametrize("la,lb", [(RM, RM), (M32, M32), (RM, M32), (M32, RM)])
+@pytest.mark.parametrize("m,n,k", [(20, 2048, 2048), (32, 4100, 4096), (100, 3000, 2048), (256, 1500, 4096), (64, 5120, 6144)])
+def test_mid_rotated_start_in_k(m, n, k, la, lb):
+    """K in whole groups of 8 K tiles: the workgroups start at different K tiles (workgroup 8 i + x at tile i) and
+    walk around the end of K, each through the scale groups of 4 and 8 K tiles from the middle of one on; enough
+    strips that starts 0 .. 7 and beyond occur, every scale layout pair, the 32-row block shape (M <= 32) too."""
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=m + n, scale_lo=104, scale_hi=150)
+    c = run(x, xs, w, ws, torch.float32, la=la, lb=lb, pre=(n % 16 == 0 and lb == RM), variant=V, split_k=1)
+    assert_close(c, c_oracle.scaled_gemm_exact(x, w, xs, ws), torch.float32, f"{m}x{n}x{k} {la}/{lb}")
+
+
 @pytest.mark.parametrize("m", [48, 64, 128, 256])
 def test_mid_decode_shapes_and_auto_choice(m):
     """cfg3's N and K at M = 48 .. 256, bf16 out: sampled rows against the oracle (all rows up to 64), all elements

@@ -108,12 +108,25 @@ bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
 int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
   int v = variant;
   if (v == WAVE_MXFP4_VARIANT_AUTO) {
-    // 48 < M <= 256 and enough 128-column strips to put most CUs to work: reading B once from HBM bounds the
-    // problem, and the mid-M kernel gives B and A rings of their own.  Measured at K = 8192 against the streaming
-    // kernel (M <= 64) and the tile kernels: it wins from N = 12288 on for 64 < M <= 192 (128 x 28672: 46 -> 31 us,
-    // 128 x 12288: 23.4 -> 22.3 us, 96 x 8192 loses, 17 -> 21 us) and from about N = 24576 on at M = 64
-    // (32 -> 28 us) and M = 256 (55 -> 48 us; 256 x 16384 loses, 39 -> 42 us).
-    if (mid_shape_ok(m, n, k) && m > 48 && n >= ((m > 64 && m <= 192) ? 12288 : 24576)) return WAVE_MXFP4_VARIANT_MID_M;
+    // Reading B once from HBM bounds these problems, and the mid-M kernel gives B and A rings of their own.
+    // Measured at K = 2048 .. 8192 (us, other kernel -> mid-M):
+    //   64 < M <= 192 against the tile kernels: from N = 12288 on (128 x 12288 x 8192: 29.7 -> 23.3,
+    //     128 x 24576: 43.4 -> 27.6; 128 x 8192 loses, 19.3 -> 22.8); M = 256 from N = 24576 on (51.5 -> 43.9;
+    //     256 x 16384 loses, 38.3 -> 39.9)
+    //   32 < M <= 64 against the streaming kernel: from N = 12288 on (48 x 28672 x 8192: 28.0 -> 22.5), and from
+    //     N = 4096 on at K <= 4096 (64 x 8192 x 4096: 14.5 -> 10.7; 48 x 8192 x 8192 loses, 14.4 -> 17.3)
+    //   16 < M <= 32: where the strips are one round of the CUs, N = 12288 .. 128 CUs (32 x 28672 x 8192:
+    //     24.8 -> 22.2; 32 x 57344 loses, 43.3 -> 45.2: the streaming kernel's contiguous ranges have no rounds)
+    //   M <= 16: the same range of N at K <= 4096 (16 x 28672 x 4096: 13.6 -> 13.0; a tie at K = 8192)
+    if (mid_shape_ok(m, n, k)) {
+      const int64_t one_round = (int64_t)128 * device_cus();
+      const bool mid = m > 192  ? n >= 24576
+                       : m > 64 ? n >= 12288
+                       : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096)
+                       : m > 16 ? n >= 12288 && n <= one_round
+                                : n >= 12288 && n <= one_round && k <= 4096;
+      if (mid) return WAVE_MXFP4_VARIANT_MID_M;
+    }
     if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;
     v = pick_tile_variant(m, n);
   }
@@ -390,12 +403,13 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   }
 
   if (ws_scales_end < ws_used) ws_scales_end = ws_used;
-  int vv = v;
-  if (vv == WAVE_MXFP4_VARIANT_MID_M && !mid_gemm_applies(p)) {
-    // (the library's own choice without scratch for the scales, or offsets beyond 32 bits: the tile kernels)
+  if (v == WAVE_MXFP4_VARIANT_MID_M && !mid_gemm_applies(p)) {
+    // (the library's own choice without scratch for the scales, or offsets beyond 32 bits: the kernels that
+    // served these shapes before)
     if (variant == WAVE_MXFP4_VARIANT_MID_M) return WAVE_MXFP4_ERR_UNSUPPORTED;
-    vv = pick_tile_variant(m, n);
+    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
   }
+  const int vv = v;
   if (vv == WAVE_MXFP4_VARIANT_MID_M) {
     e = launch_mid_gemm(p, device_cus(), stream);
   } else if (v == WAVE_MXFP4_VARIANT_NAIVE) {
@@ -592,9 +606,10 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
     const int64_t avg = (total_rows + num_groups - 1) / num_groups;
     const bool pays = avg <= kGroupedMidMaxAvgRows && (int64_t)num_groups * ((n + 127) / 128) >= device_cus() / 2;
     if (fits && (variant == WAVE_MXFP4_VARIANT_MID_M || pays)) {
-      // rows per block: twice the average group (the routing is uneven), in steps of 64, at most the whole batch
+      // rows per block: twice the average group (the routing is uneven), 32 or in steps of 64, at most the whole
+      // batch
       int64_t bm = 2 * avg < total_rows ? 2 * avg : total_rows;
-      bm = bm > 256 ? 256 : (bm + 63) / 64 * 64;
+      bm = bm > 256 ? 256 : bm <= 32 ? 32 : (bm + 63) / 64 * 64;
       return record_hip(launch_mid_gemm(p, device_cus(), stream, (int)bm));
     }
   }

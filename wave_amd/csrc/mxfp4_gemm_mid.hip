@@ -47,13 +47,16 @@ template <int BM_, bool B_RM_>
 struct MidCfg {
   static constexpr int BM = BM_, MT_M = BM / 32;
   static constexpr bool B_RM = B_RM_;
+  // The four compute waves sit WM x (4 / WM) on the strip: two row halves times two pairs of column groups from
+  // BM = 64 on (one A fragment per two MFMAs), side by side on one row block at BM = 32.
+  static constexpr int WM = BM >= 64 ? 2 : 1;
   static constexpr int A_SLOT = BM * kTileKBytes;
   // Ring depths, measured at N = 28672, K = 8192 (us at M = 64 / 128 / 192): A, which every workgroup re-reads
   // from L2 at the same moment as all the others, needs the deeper ring.  With no B traffic at all the kernel
   // took 17 / 22 us at two K tiles of A ahead: its latency, not B's, set the pace.
   //   (DA, DB) = (3, 7) / (3, 5) / (2, 5): 29.9 / 33.1 / 43.5     (6, 5) / (5, 3) / (3, 3): 27.9 / 31.4 / 39.0
   static constexpr int DA = BM <= 64 ? 6 : BM <= 128 ? 5 : BM <= 192 ? 3 : 2;  // K tiles of A in LDS
-  static constexpr int DB = BM <= 64 ? 5 : BM <= 192 ? 3 : 4;            // K tiles of B in the ring
+  static constexpr int DB = BM <= 32 ? 7 : BM <= 64 ? 5 : BM <= 192 ? 3 : 4;   // K tiles of B in the ring
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
   static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
   // Scale groups of A in LDS: the one being read, (j / 4), up to the one requested with A(j + DA - 1); a group's
@@ -66,7 +69,7 @@ struct MidCfg {
   static constexpr int LDS = A_RING + AS_RING + B_RING + kMidCW * BS_WAVE;
   static constexpr int A_LD = BM / 8;                                    // A DMA instructions per K tile (producer)
   static_assert(LDS <= 160 * 1024, "LDS");
-  static_assert(MT_M % 2 == 0 && B_RING >= kMidCW * 32 * 32 * 4, "two row halves; the waves' C staging fits the ring");
+  static_assert(MT_M % WM == 0 && B_RING >= kMidCW * 32 * 32 * 4, "whole row blocks per wave; the waves' C staging fits the ring");
   static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
 };
 
@@ -88,7 +91,20 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
   const int kp = p.kp, nkt = p.k_tiles;
   const int n0 = blockIdx.x * (kMidCW * wv);
   const int k_tiles_blocks = nkt * 256;   // bytes of one 32-row block row of MFMA32 scales
-  const int groups = (nkt + 3) >> 2;      // scale groups of 4 K tiles
+  // Where this workgroup starts in K.  Workgroups that all walk K from tile 0 ask, at any moment, for the same
+  // 128 bytes of every row of A and of B: a few L2 and memory channels take all requests of the chip (a bare
+  // stream of B in this shape: 22.3 us; the same requests with the start rotated per workgroup: 18.0 us).  With
+  // whole groups of 8 K tiles, the workgroups of an XCD (ids x, x + 8, ..) therefore start one K tile apart and
+  // walk around the end of K; the sums are the same terms in another order.  The loops count a virtual K tile v
+  // from v0 = start % 8, so that v and the K tile it stands for agree mod 8 and the scale groups (4 and 8 K
+  // tiles) keep their places in the images.
+  const bool rotate = (nkt & 7) == 0;
+  const int k_start = rotate ? (int)(((blockIdx.y * gridDim.x + blockIdx.x) >> 3) % (uint32_t)nkt) : 0;
+  const int v0 = k_start & 7, vend = v0 + nkt, k_base = k_start - v0;
+  const int g_end = (vend + 3) >> 2, h_end = (vend + 7) >> 3;  // ends of the virtual groups of 4 and of 8
+  auto tile_of = [&](int v) { const int t = v + k_base; return t >= nkt ? t - nkt : t; };
+  auto group4_of = [&](int g) { const int t = g + (k_base >> 2); return rotate && t >= (nkt >> 2) ? t - (nkt >> 2) : t; };
+  auto group8_of = [&](int h) { const int t = h + (k_base >> 3); return rotate && t >= (nkt >> 3) ? t - (nkt >> 3) : t; };
   constexpr bool a_rowmajor = A_RM, b_rowmajor = B_RM;
 
   if (wave == kMidCW) {
@@ -101,9 +117,9 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     // swizzle depends on the lane alone when d is even, and flips bit 2 of it when d is odd
     const int goff_even = row0 * kp + (((lane & 7) ^ ((row0 >> 1) & 7)) << 4);
     const int goff_odd = row0 * kp + (((lane & 7) ^ (((row0 + 8) >> 1) & 7)) << 4);
-    auto issue_a = [&](int kt, int slot) {
+    auto issue_a = [&](int v, int slot) {
       // past the last K tile: the same number of requests, from beyond the end of A (zeros into a slot nobody reads)
-      const int soff = kt < nkt ? kt * kTileKBytes : (int)0x80000000;
+      const int soff = v < vend ? tile_of(v) * kTileKBytes : (int)0x80000000;
 #pragma unroll
       for (int d = 0; d < Cfg::A_LD; ++d)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, WAVE_LDS_PTR(a_ring + slot * Cfg::A_SLOT + d * 1024), 16,
@@ -115,7 +131,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     const int as_goff = a_rowmajor ? (lane & 31) * p.ks + (lane >> 5) * 16 : lane * 16;
     const int as_gstep = a_rowmajor ? 32 : 1024, as_istep = a_rowmajor ? 32 * p.ks : k_tiles_blocks;
     auto issue_as = [&](int g) {
-      const int soff = g < groups ? g * as_gstep : (int)0x80000000;
+      const int soff = g < g_end ? group4_of(g) * as_gstep : (int)0x80000000;
 #pragma unroll
       for (int i = 0; i < MT_M; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(as_rsrc, WAVE_LDS_PTR(as_ring + (g & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + i * 1024), 16,
@@ -123,13 +139,12 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     };
     // (a group's last K tiles may lie past K: those bytes belong to the next block or row, or lie past the
     // buffer; nobody reads them)
-    // prologue: A(0 .. DA - 2), with the scale groups they belong to in front
+    // prologue: A(v0 .. v0 + DA - 2), with the scale groups they belong to in front
+    for (int g = v0 >> 2; g <= (v0 + DA - 2) >> 2; ++g) issue_as(g);
 #pragma unroll
-    for (int g = 0; g <= (DA - 2) / 4; ++g) issue_as(g);  // the groups of A(0 .. DA - 2)
-#pragma unroll
-    for (int j = 0; j < DA - 1; ++j) issue_a(j, j);
+    for (int j = 0; j < DA - 1; ++j) issue_a(v0 + j, j);
     int slot_next = DA - 1;  // slot of the K tile requested next
-    for (int j = 0; j < nkt; ++j) {
+    for (int j = v0; j < vend; ++j) {
       // A(j) has landed: younger than it are A(j + 1 .. j + DA - 2) and at most one scale group
       __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((DA - 2) * Cfg::A_LD));
       asm volatile("" ::: "memory");
@@ -146,12 +161,12 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
   }
 
   // ================= a compute wave =================
-  // The four compute waves sit 2 x 2 on the strip: wave (wm, wn) multiplies rows wm * BM / 2 .. and the strip's
-  // 32-row groups 2 wn and 2 wn + 1 of B (one A fragment per two MFMAs instead of one per MFMA: the kernel is
-  // bound by LDS bandwidth).  Each wave still requests, and waits for, the group `wave` of B and of its scales;
-  // the K tile's barrier makes all four groups visible to all.
-  constexpr int MI = MT_M / 2;
-  const int wm = wave >> 1, wn = wave & 1;
+  // From BM = 64 on the four compute waves sit 2 x 2 on the strip: wave (wm, wn) multiplies every second row block
+  // from block wm on and the strip's 32-row groups 2 wn and 2 wn + 1 of B (one A fragment per two MFMAs instead of
+  // one per MFMA).  At BM = 32 they sit side by side, wave w on group w.  Either way each wave requests, and
+  // waits for, the group `wave` of B and of its scales; the K tile's barrier makes all four groups visible to all.
+  constexpr int WM = Cfg::WM, NJ = WM == 2 ? 2 : 1, MI = MT_M / WM;  // row blocks and column groups per wave
+  const int wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave;
   uint8_t *const b_ring = smem + Cfg::A_RING + Cfg::AS_RING;  // DB slots of 4 groups x 32 rows x 128 bytes
   uint8_t *const bs_all = b_ring + Cfg::B_RING;               // the four groups' scale images
   uint8_t *const bs_ring = bs_all + wave * Cfg::BS_WAVE;      // ... the one this wave fills
@@ -179,8 +194,8 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     b_goff[d] = r < cols ? off : (int)0x80000000;  // past the wave's columns: out of range, zeros, no request
   }
   const int b_kt_stride = p.b_preshuffled ? 2048 : kTileKBytes;
-  auto issue_b = [&](int kt, int slot) {
-    const int soff = kt < nkt ? kt * b_kt_stride : (int)0x80000000;
+  auto issue_b = [&](int v, int slot) {
+    const int soff = v < vend ? tile_of(v) * b_kt_stride : (int)0x80000000;
 #pragma unroll
     for (int d = 0; d < 4; ++d)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, WAVE_LDS_PTR(b_ring + slot * 16384 + wave * 4096 + d * 1024), 16,
@@ -188,7 +203,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
   };
   // MFMA32 order: the four 256-byte blocks of K tiles 4g .. 4g + 3 are contiguous, one instruction per group.
   auto issue_bs = [&](int g) {
-    const int soff = g < groups ? g * 1024 : (int)0x80000000;
+    const int soff = g < g_end ? group4_of(g) * 1024 : (int)0x80000000;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(bs_rsrc, WAVE_LDS_PTR(bs_ring + (g & 3) * 1024), 16, lane * 16, soff, 0, 0);
   };
   // Row-major: 64 bytes of each of the group's rows (8 K tiles), 16 rows per instruction, two instructions per
@@ -197,7 +212,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
   // (Fetched as 32 bytes of each of 32 rows per 4 K tiles, every instruction touched 32 cache lines and every
   // line was requested four times.)
   auto issue_bs8 = [&](int h) {
-    const int soff = h * 64 < p.ks ? h * 64 : (int)0x80000000;
+    const int soff = h < h_end ? group8_of(h) * 64 : (int)0x80000000;
 #pragma unroll
     for (int dd = 0; dd < 2; ++dd) {
       const int r = dd * 16 + (lane >> 2);
@@ -239,20 +254,24 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     }
   };
 
-  v16f acc[MI][2];
+  v16f acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int jn = 0; jn < 2; ++jn)
+    for (int jn = 0; jn < NJ; ++jn)
 #pragma unroll
       for (int g = 0; g < 16; ++g) acc[i][jn][g] = 0.f;
 
-  // prologue: B(0 .. LB - 1) with the scale groups they belong to in front
-  if constexpr (B_RM) issue_bs8(0);
+  // prologue: B(v0 .. v0 + LB - 1) with the scale groups they belong to in front (row-major: the second image
+  // too when the walk starts inside the first, because the K loop requests an image at the start of the one before)
+  if constexpr (B_RM) {
+    issue_bs8(0);
+    if (v0 != 0) issue_bs8(1);
+  }
 #pragma unroll
   for (int j = 0; j < LB; ++j) {
-    if (!B_RM && (j & 3) == 0) issue_bs(j >> 2);
-    issue_b(j, j);
+    if (!B_RM && (j == 0 || ((v0 + j) & 3) == 0)) issue_bs((v0 + j) >> 2);
+    issue_b(v0 + j, j);
   }
   int slot = 0, slot_next = LB;  // slots of B(j) and of the K tile requested next
   int a_slot = 0;
@@ -260,13 +279,13 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
   typedef std::integral_constant<int, 1> T1;
   typedef std::integral_constant<int, 2> T2;
   typedef std::integral_constant<int, 3> T3;
-  // Row block i of this wave is block 2 i + wm of the tile, so that a block of fewer rows than BM (a small group
+  // Row block i of this wave is block WM i + wm of the tile, so that a block of fewer rows than BM (a small group
   // of a grouped problem) leaves both halves of the workgroup the same share; the blocks past the rows take no
   // fragment reads and no MFMAs: the K loop exists once per count of live blocks, with no branch inside it.
-  const int live = min(max((m_rows - 32 * wm + 63) >> 6, 0), MI);
+  const int live = min(max((m_rows - 32 * wm + 32 * WM - 1) / (32 * WM), 0), MI);
   auto k_loop = [&](auto live_tag) {
   constexpr int LIVE = decltype(live_tag)::value;
-  for (int j = 0; j < nkt; ++j) {
+  for (int j = v0; j < vend; ++j) {
     // B(j) and its scales have landed: younger are B(j + 1 .. j + LB - 1), 4 requests each (and up to two scale
     // groups, which the count leaves out: it then waits for that much more than it must)
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(4 * (LB - 1)));
@@ -286,27 +305,27 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     slot_next = slot_next + 1 == DB ? 0 : slot_next + 1;
 
     const uint8_t *a_t = a_ring + a_slot * Cfg::A_SLOT + wm * 32 * kTileKBytes;
-    const uint8_t *b_t = b_ring + slot * 16384 + wn * 2 * 4096;
-    uint32_t sa[MI], sb[2];
+    const uint8_t *b_t = b_ring + slot * 16384 + wn * NJ * 4096;
+    uint32_t sa[MI], sb[NJ];
 #pragma unroll
     for (int i = 0; i < LIVE; ++i)
-      sa[i] = lane_scales(as_ring + ((j >> 2) & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + (2 * i + wm) * 1024, std::integral_constant<bool, A_RM>{}, j);
+      sa[i] = lane_scales(as_ring + ((j >> 2) & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + (WM * i + wm) * 1024, std::integral_constant<bool, A_RM>{}, j);
 #pragma unroll
-    for (int jn = 0; jn < 2; ++jn) sb[jn] = lane_scales_b(wn * 2 + jn, j);
+    for (int jn = 0; jn < NJ; ++jn) sb[jn] = lane_scales_b(wn * NJ + jn, j);
     auto step = [&](auto t_tag) {
       constexpr int T = decltype(t_tag)::value;
-      v8i vb[2];
+      v8i vb[NJ];
 #pragma unroll
-      for (int jn = 0; jn < 2; ++jn) {
+      for (int jn = 0; jn < NJ; ++jn) {
         const v4i fb = *(const v4i *)(b_t + jn * 4096 + foff[T]);
         vb[jn] = v8i{fb.x, fb.y, fb.z, fb.w, 0, 0, 0, 0};
       }
 #pragma unroll
       for (int i = 0; i < LIVE; ++i) {
-        const v4i fa = *(const v4i *)(a_t + i * 64 * kTileKBytes + foff[T]);
+        const v4i fa = *(const v4i *)(a_t + i * WM * 32 * kTileKBytes + foff[T]);
         const v8i va = {fa.x, fa.y, fa.z, fa.w, 0, 0, 0, 0};
 #pragma unroll
-        for (int jn = 0; jn < 2; ++jn)
+        for (int jn = 0; jn < NJ; ++jn)
           acc[i][jn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb[jn], va, acc[i][jn], 4, 4, T, (int)sb[jn], T,
                                                                        (int)sa[i]);
       }
@@ -340,7 +359,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
 
   // ---------------- C: accumulators -> the wave's ring -> global ----------------
   // acc[i][jn][4q + e] is row lane % 32, column 8q + 4 * (lane / 32) + e of the 32 x 32 tile (row block
-  // 2 i + wm, group 2 wn + jn).  A tile is staged as 32 rows of eight 4-column pieces and stored 8 rows per
+  // WM i + wm, group NJ wn + jn).  A tile is staged as 32 rows of eight 4-column pieces and stored 8 rows per
   // instruction, a lane one piece (8 bytes of bf16, 16 of f32), the pieces past the group's columns left out.
   uint8_t *stage = b_ring + wave * 4096;
   const bool out_bf16 = p.out_bf16 != 0;
@@ -349,8 +368,8 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
       make_rsrc_n(c_base, (int)min((int64_t)m_rows * p.n * elt, (int64_t)0x7FFFFFFF));
   const int lr = lane >> 3, lc = lane & 7;
 #pragma unroll
-  for (int jn = 0; jn < 2; ++jn) {
-    const int gc0 = n0 + (wn * 2 + jn) * wv;                 // the group's first column of C
+  for (int jn = 0; jn < NJ; ++jn) {
+    const int gc0 = n0 + (wn * NJ + jn) * wv;                // the group's first column of C
     const bool mine = lc * 4 < min(wv, p.n - gc0);          // (negative past N: nothing stored)
     if (out_bf16) {
       typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
@@ -366,7 +385,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int r0 = 0; r0 < 32; r0 += 8) {
-          const int r = r0 + lr, row = (2 * i + wm) * 32 + r;
+          const int r = r0 + lr, row = (WM * i + wm) * 32 + r;
           const v2i v = *(const v2i *)(stage + r * 64 + ((lc ^ ((r >> 2) & 7)) << 3));
           // rows past M lie past the end of C: dropped by the descriptor
           if (mine) __builtin_amdgcn_raw_buffer_store_b64(v, c_rsrc, (int)(((int64_t)row * p.n + gc0 + lc * 4) * 2), 0, 0);
@@ -387,7 +406,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int r0 = 0; r0 < 32; r0 += 8) {
-          const int r = r0 + lr, row = (2 * i + wm) * 32 + r;
+          const int r = r0 + lr, row = (WM * i + wm) * 32 + r;
           const v4f v = *(const v4f *)(stage + r * 128 + ((lc ^ (r & 7)) << 4));
           if (mine)
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc,
@@ -499,6 +518,7 @@ bool mid_grouped_applies(const GemmParams &p) {
 hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream, int bm) {
   const int wv = mid_wave_cols(p, num_cus);
   if (bm <= 0) bm = p.m;
+  if (bm <= 32) return launch_mid_cfg<32>(p, wv, stream);
   if (bm <= 64) return launch_mid_cfg<64>(p, wv, stream);
   if (bm <= 128) return launch_mid_cfg<128>(p, wv, stream);
   if (bm <= 192) return launch_mid_cfg<192>(p, wv, stream);

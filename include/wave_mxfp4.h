@@ -99,7 +99,7 @@ typedef enum {
   /* M <= 256 against a wide B from HBM: one workgroup per strip of 64 to 128 columns, B through deep
    * wave-private LDS rings, A fed by a producer wave.  Needs K % 256 == 0, K >= 1024, N % 4 == 0, no split, and
    * each scale tensor row-major or MFMA32 (e8m0_shuffle order needs the workspace); WAVE_MXFP4_ERR_UNSUPPORTED
-   * otherwise.  AUTO takes it for 48 < M <= 256 and a wide N, and for a grouped problem of few rows per expert
+   * otherwise.  AUTO takes it for 16 < M <= 256 and a wide N (M <= 16 too at K <= 4096), and for a grouped problem of few rows per expert
    * (see wave_mxfp4_gemm_grouped).  The reference runs such shapes through its generic tile kernel
    * (tests/kernel/wave_gemm_mxfp_test.py:291-339). */
   WAVE_MXFP4_VARIANT_MID_M = 8,

@@ -7,10 +7,10 @@
 // path for A, which comes from L2.  Vector memory operations of a wave retire in issue order, so a wave that
 // waits for a recent A tile also waits for every older B request: the two streams need different waves.
 //
-//   * One workgroup per strip of 4 * WV columns of C: four compute waves, 2 x 2 on the strip (each BM / 2 rows
-//     and two of the strip's four groups of WV <= 32 columns; v_mfma_scale_f32_32x32x64_f8f6f4, BM / 32
-//     accumulator tiles, one A fragment per two MFMAs) and a fifth, the producer wave, which does nothing but
-//     request A.  WV is chosen per problem so that the strips come out as a whole number of rounds over the CUs
+//   * One workgroup per strip of 4 * WV columns of C: four compute waves, 2 x 2 on the strip (each every second
+//     32-row block and two of the strip's four groups of WV <= 32 columns; v_mfma_scale_f32_32x32x64_f8f6f4,
+//     BM / 32 accumulator tiles, one A fragment per two MFMAs; side by side on one row block at BM = 32) and a
+//     fifth, the producer wave, which does nothing but request A.  WV is chosen per problem so that the strips come out as a whole number of rounds over the CUs
 //     (N = 28672 on 256 CUs: 28 columns per group, 256 workgroups).  The rows of a group's MFMA operand past WV
 //     are zero-filled by the buffer descriptor (no memory request) and their columns are not stored.
 //   * B goes into a ring of DB K tiles (four groups of 32 rows x 128 bytes each).  Compute wave w fetches group
@@ -25,6 +25,10 @@
 //     DA - 1 ahead, waits for its own requests, and meets the compute waves at the barrier: behind it A(j) is
 //     visible to all and the slots of A(j - 1) and B(j - 1) are free.
 //   * C leaves through the (by then idle) B ring, 4 KB per wave, 64 or 128 bytes per row and store.
+//   * Workgroups start at different K tiles and walk around the end of K, so that the chip's requests of a
+//     moment spread over the memory channels instead of all naming the same 128 bytes of every 4 KB row.
+//   * A grouped (mixture of experts) problem of few rows per expert runs the same body with one workgroup per
+//     (expert, strip); a wave skips the row blocks past its group's rows.
 //
 // Taken for K % 256 == 0 (at least 4 K tiles), N % 4 == 0, each scale tensor row-major or in MFMA32 order
 // (e8m0_shuffle order is re-laid out first when the library has scratch; B scales in MFMA32 order fix WV at 32,

@@ -56,15 +56,15 @@ def test_random_shape_against_oracle(case):
 
 
 def _wide_cases(count, seed):
-    """Shapes the newer kernels take under the library's own choice: 49..256 rows against a wide N (mid-M kernel,
-    every strip width), more than 256 tiles with N a multiple of 192 (256x192 tiles) or with preshuffled B
+    """Shapes the newer kernels take under the library's own choice: up to 256 rows against a wide N (mid-M kernel,
+    every strip width and block shape, K with and without the rotated start), more than 256 tiles with N a multiple of 192 (256x192 tiles) or with preshuffled B
     (B-direct kernel), K a multiple of 256 so that they qualify, and ragged M."""
     rng = np.random.default_rng(seed)
     out = []
     for i in range(count):
         kind = rng.integers(0, 3)
         if kind == 0:    # mid-M
-            m, n, k = int(rng.integers(49, 257)), 4 * int(rng.integers(3072, 9000)), 256 * int(rng.integers(4, 12))
+            m, n, k = int(rng.integers(1, 257)), 4 * int(rng.integers(3072, 9000)), 256 * int(rng.integers(4, 17))
         elif kind == 1:  # 256x192 tiles
             m, n, k = int(rng.integers(2100, 5000)), 192 * int(rng.integers(20, 40)), 256 * int(rng.integers(3, 8))
         else:            # more tiles than CUs, N % 256 == 0 (B-direct when preshuffled)

@@ -354,10 +354,11 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     const int sb1 = sa + 3 >= RING ? sa + 3 - RING : sa + 3;
     const int sa2 = sa + 4 >= RING ? sa + 4 - RING : sa + 4;
     if constexpr (FP8) {
-      // two K steps of 64-cycle MFMAs: the same request sequence folded into two phases
+      // two K steps of 64-cycle MFMAs, two phases: A(j+2) in the first, the barrier, all of B(j+2) in the second,
+      // so that every request has a whole K tile to land in (with B's second half requested in the first phase,
+      // as the four-phase MXFP4 sequence does, it had half a K tile, and the waves waited for it)
       read_frags(sa, sb, 1, fa1, fb1);
       mfma_block(fa0, fb0, T0{}, Zero{});
-      if (KIND != kFirst) issue_g2l(W1, 1, kt1, sb1, B_LD / 2, B_LD);
       issue_g2l(W2, 0, kt2, sa2, 0, A_LD);
       order_phase8();
       __builtin_amdgcn_sched_barrier(0);
@@ -372,7 +373,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       __builtin_amdgcn_sched_barrier(0);
       read_frags(sa1, sb1, 0, fa0, fb0);
       mfma_block(fa1, fb1, T1{}, Keep{});
-      issue_g2l(W2, 1, kt2, sa, 0, B_LD / 2);
+      issue_g2l(W2, 1, kt2, sa, 0, B_LD);
       order_phase8();
       __builtin_amdgcn_sched_barrier(0);
       canon_scales(kt1);
@@ -576,7 +577,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     k_tile(nk - 1, sa, stage_slot, std::integral_constant<int, kBound2>{}, pending_tag);
     // second half of B(1) of the next tile, ahead of the C stores (its first
     // half went into slot `sa` in the last phase above)
-    issue_g2l(1, 1, 1, sa, B_LD / 2, B_LD);
+    if constexpr (!FP8) issue_g2l(1, 1, 1, sa, B_LD / 2, B_LD);
     sa = next_slot(sa);
     __builtin_amdgcn_sched_barrier(0);
     if (SPLIT && part_of[0] >= 0) {  // a part of a tile of the last round: always the workgroup's last item,

@@ -371,9 +371,10 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
+      issue_g2l(W2, 1, kt2, sa, 0, B_LD);  // (ahead of the phase's MFMAs: spread between them it cost 10 %)
+      __builtin_amdgcn_sched_barrier(0);
       read_frags(sa1, sb1, 0, fa0, fb0);
       mfma_block(fa1, fb1, T1{}, Keep{});
-      issue_g2l(W2, 1, kt2, sa, 0, B_LD);
       order_phase8();
       __builtin_amdgcn_sched_barrier(0);
       canon_scales(kt1);

@@ -70,6 +70,20 @@ def test_mid_rotated_start_in_k(m, n, k, la, lb):
     assert_close(c, c_oracle.scaled_gemm_exact(x, w, xs, ws), torch.float32, f"{m}x{n}x{k} {la}/{lb}")
 
 
+@pytest.mark.parametrize("lb", [RM, M32])
+@pytest.mark.parametrize("m,n,k", [(24, 36864, 2048), (1, 40004, 1024), (32, 33000, 1280)])
+def test_mid_more_strips_than_cus(m, n, k, lb):
+    """Up to 32 rows against more 128-column strips than the GPU has CUs: the shallow rings with two workgroups per
+    CU; sampled columns of every strip region against the oracle, AUTO the same bits."""
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=n, scale_lo=110, scale_hi=144)
+    c = run(x, xs, w, ws, torch.float32, lb=lb, variant=V, split_k=1)
+    cols = np.unique(np.concatenate([np.arange(0, n, 97), np.arange(n - 130, n)]))
+    ref = c_oracle.scaled_gemm_exact(x, w[cols], xs, ws[cols])
+    assert_close(c[:, cols], ref, torch.float32, f"{m}x{n}x{k} {lb}")
+    assert not np.isnan(c).any()
+    assert np.array_equal(run(x, xs, w, ws, torch.float32, lb=lb), c)
+
+
 @pytest.mark.parametrize("m", [48, 64, 128, 256])
 def test_mid_decode_shapes_and_auto_choice(m):
     """cfg3's N and K at M = 48 .. 256, bf16 out: sampled rows against the oracle (all rows up to 64), all elements

@@ -115,16 +115,18 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
     //     256 x 16384 loses, 38.3 -> 39.9)
     //   32 < M <= 64 against the streaming kernel: from N = 12288 on (48 x 28672 x 8192: 28.0 -> 22.5), and from
     //     N = 4096 on at K <= 4096 (64 x 8192 x 4096: 14.5 -> 10.7; 48 x 8192 x 8192 loses, 14.4 -> 17.3)
-    //   16 < M <= 32: where the strips are one round of the CUs, N = 12288 .. 128 CUs (32 x 28672 x 8192:
-    //     24.8 -> 22.2; 32 x 57344 loses, 43.3 -> 45.2: the streaming kernel's contiguous ranges have no rounds)
-    //   M <= 16: the same range of N at K <= 4096 (16 x 28672 x 4096: 13.6 -> 13.0; a tie at K = 8192)
+    //   16 < M <= 32: N from 12288 up to 320 columns per CU (32 x 28672 x 8192: 24.8 -> 22.2; past one round of
+    //     128-column strips two workgroups share a CU, 32 x 57344 x 8192: 44.6 -> 38.6; 32 x 114688 x 4096 loses,
+    //     43.0 -> 44.5)
+    //   M <= 16: the same range of N; up to 192 columns per CU only at K <= 4096 (16 x 28672 x 4096: 13.6 -> 13.0;
+    //     a tie or 2 % lost at K = 8192: 16 x 40960 29.8 -> 30.3), beyond at any K (16 x 57344 x 8192: 41.4 -> 38.3)
     if (mid_shape_ok(m, n, k)) {
-      const int64_t one_round = (int64_t)128 * device_cus();
+      const int64_t cus = device_cus();
       const bool mid = m > 192  ? n >= 24576
                        : m > 64 ? n >= 12288
                        : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096)
-                       : m > 16 ? n >= 12288 && n <= one_round
-                                : n >= 12288 && n <= one_round && k <= 4096;
+                       : m > 16 ? n >= 12288 && n <= 320 * cus
+                                : n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus);
       if (mid) return WAVE_MXFP4_VARIANT_MID_M;
     }
     if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;

@@ -47,10 +47,15 @@ constexpr int kMidOnce = 2;  // the "nt" bit: B is read exactly once
 
 // B_RM: B's scales are row-major: a group's image is then two buffers of 32 rows x 64 bytes (8 K tiles) instead
 // of four buffers of 1 KB (4 K tiles).
-template <int BM_, bool B_RM_>
+// TWO_PER_CU (BM = 32 only): rings of three K tiles each, 78 KB of LDS, so that two workgroups share a CU and the
+// one's prologue and C write run under the other's stream.  For problems of more workgroups than CUs (measured, 8
+// experts x 14336 x 4096 at one row per expert: 47.0 -> 40.2 us, 6.2 TB/s; 64 experts x 2048 x 7168: 80.8 -> 74.1 us,
+// 6.75 TB/s); with one workgroup per CU or fewer the deep rings are the better use of the LDS.
+template <int BM_, bool B_RM_, bool TWO_PER_CU_ = false>
 struct MidCfg {
   static constexpr int BM = BM_, MT_M = BM / 32;
-  static constexpr bool B_RM = B_RM_;
+  static constexpr bool B_RM = B_RM_, TWO_PER_CU = TWO_PER_CU_;
+  static_assert(!TWO_PER_CU || BM == 32, "only the 32-row block leaves room for two workgroups");
   // The four compute waves sit WM x (4 / WM) on the strip: two row halves times two pairs of column groups from
   // BM = 64 on (one A fragment per two MFMAs), side by side on one row block at BM = 32.
   static constexpr int WM = BM >= 64 ? 2 : 1;
@@ -59,8 +64,8 @@ struct MidCfg {
   // from L2 at the same moment as all the others, needs the deeper ring.  With no B traffic at all the kernel
   // took 17 / 22 us at two K tiles of A ahead: its latency, not B's, set the pace.
   //   (DA, DB) = (3, 7) / (3, 5) / (2, 5): 29.9 / 33.1 / 43.5     (6, 5) / (5, 3) / (3, 3): 27.9 / 31.4 / 39.0
-  static constexpr int DA = BM <= 64 ? 6 : BM <= 128 ? 5 : BM <= 192 ? 3 : 2;  // K tiles of A in LDS
-  static constexpr int DB = BM <= 32 ? 7 : BM <= 64 ? 5 : BM <= 192 ? 3 : 4;   // K tiles of B in the ring
+  static constexpr int DA = TWO_PER_CU ? 3 : BM <= 64 ? 6 : BM <= 128 ? 5 : BM <= 192 ? 3 : 2;  // K tiles of A in LDS
+  static constexpr int DB = TWO_PER_CU ? 3 : BM <= 32 ? 7 : BM <= 64 ? 5 : BM <= 192 ? 3 : 4;   // K tiles of B in the ring
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
   static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
   // Scale groups of A in LDS: the one being read, (j / 4), up to the one requested with A(j + DA - 1); a group's
@@ -72,7 +77,7 @@ struct MidCfg {
   static constexpr int BS_WAVE = 4 * 1024;                               // one group's scale images
   static constexpr int LDS = A_RING + AS_RING + B_RING + kMidCW * BS_WAVE;
   static constexpr int A_LD = BM / 8;                                    // A DMA instructions per K tile (producer)
-  static_assert(LDS <= 160 * 1024, "LDS");
+  static_assert(LDS <= (TWO_PER_CU ? 80 : 160) * 1024, "LDS");
   static_assert(MT_M % WM == 0 && B_RING >= kMidCW * 32 * 32 * 4, "whole row blocks per wave; the waves' C staging fits the ring");
   static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
 };
@@ -459,17 +464,17 @@ hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int BM>
+template <int BM, bool TWO = false>
 hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
   const bool a_rm = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR, b_rm = p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
   if (p.num_groups != 0)  // (row-major A scales: checked by mid_grouped_applies)
-    return b_rm ? launch_mid_layouts<MidCfg<BM, true>, true, true>(p, wv, stream)
-                : launch_mid_layouts<MidCfg<BM, false>, true, true>(p, wv, stream);
+    return b_rm ? launch_mid_layouts<MidCfg<BM, true, TWO>, true, true>(p, wv, stream)
+                : launch_mid_layouts<MidCfg<BM, false, TWO>, true, true>(p, wv, stream);
   if (a_rm)
-    return b_rm ? launch_mid_layouts<MidCfg<BM, true>, true, false>(p, wv, stream)
-                : launch_mid_layouts<MidCfg<BM, false>, true, false>(p, wv, stream);
-  return b_rm ? launch_mid_layouts<MidCfg<BM, true>, false, false>(p, wv, stream)
-              : launch_mid_layouts<MidCfg<BM, false>, false, false>(p, wv, stream);
+    return b_rm ? launch_mid_layouts<MidCfg<BM, true, TWO>, true, false>(p, wv, stream)
+                : launch_mid_layouts<MidCfg<BM, false, TWO>, true, false>(p, wv, stream);
+  return b_rm ? launch_mid_layouts<MidCfg<BM, true, TWO>, false, false>(p, wv, stream)
+              : launch_mid_layouts<MidCfg<BM, false, TWO>, false, false>(p, wv, stream);
 }
 
 // Columns per compute wave: the narrowest strips (a multiple of 4 columns, 16 to 32) that still fit the number of
@@ -520,8 +525,12 @@ bool mid_grouped_applies(const GemmParams &p) {
 // `bm`: rows per block of a group (dense: M; grouped: the library's guess from the average group, a group of more
 // rows takes several blocks).
 hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream, int bm) {
-  const int wv = mid_wave_cols(p, num_cus);
   if (bm <= 0) bm = p.m;
+  // more strips than CUs at the 32-row block: two workgroups per CU
+  const int64_t strips = (int64_t)((p.n + kMidBN - 1) / kMidBN) * (p.num_groups != 0 ? p.num_groups : 1);
+  const bool two = bm <= 32 && strips > num_cus;
+  const int wv = mid_wave_cols(p, two ? 2 * num_cus : num_cus);
+  if (two) return launch_mid_cfg<32, true>(p, wv, stream);
   if (bm <= 32) return launch_mid_cfg<32>(p, wv, stream);
   if (bm <= 64) return launch_mid_cfg<64>(p, wv, stream);
   if (bm <= 128) return launch_mid_cfg<128>(p, wv, stream);

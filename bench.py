@@ -609,7 +609,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": leg["tflops"], "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
                          "frac": leg["frac_of_mxfp4_peak"], "traffic": read_traffic("cfg4"), "kernel": leg["kernel"],
                          "launch_us": leg["launch_us"]},
-            "resident_weight_scales": leg["resident_weight_scales"]})))
+            "resident_weight_scales": leg["resident_weight_scales"], "serving_batch": leg["serving_batch"]})))
         return
 
     if args.workload == "mxfp8":

@@ -84,9 +84,9 @@ def test_mid_more_strips_than_cus(m, n, k, lb):
     assert np.array_equal(run(x, xs, w, ws, torch.float32, lb=lb), c)
 
 
-@pytest.mark.parametrize("m", [48, 64, 128, 256])
+@pytest.mark.parametrize("m", [17, 32, 48, 64, 128, 256])
 def test_mid_decode_shapes_and_auto_choice(m):
-    """cfg3's N and K at M = 48 .. 256, bf16 out: sampled rows against the oracle (all rows up to 64), all elements
+    """cfg3's N and K at M = 17 .. 256, bf16 out: sampled rows against the oracle (all rows up to 64), all elements
     against the tile kernel; for M the library takes the kernel by itself, AUTO gives the same bits."""
     n, k = 28672, 8192
     x, xs, w, ws = orc.make_inputs(m, n, k, seed=2, scale_lo=120, scale_hi=134)
@@ -95,8 +95,7 @@ def test_mid_decode_shapes_and_auto_choice(m):
     assert_close(c[rows], c_oracle.scaled_gemm_exact(x, w, xs, ws, rows=rows), torch.bfloat16, "rows vs oracle")
     other = run(x, xs, w, ws, torch.float32, variant=_lib.VARIANT_T128x128_W2x2, split_k=1)
     assert_close(c, other.astype(np.float64), torch.bfloat16, "all elements vs the tile kernel")
-    if m > 48:
-        assert np.array_equal(run(x, xs, w, ws, torch.bfloat16), c)
+    assert np.array_equal(run(x, xs, w, ws, torch.bfloat16), c)
 
 
 def test_mid_nan_scale_poisons_its_row_and_column():

@@ -176,7 +176,7 @@ size_t wave_mxfp4_static_scratch_bytes(void);
  * wave_mxfp4_grouped_workspace_bytes(...) bytes: with it the scales of both
  * operands are first re-laid out for one-dword-per-lane reads, as in
  * wave_mxfp4_gemm (N % 32 == 0 and K % 256 == 0; otherwise it is not used).
- * A small batch (AUTO: at most 128 rows per expert on average, and enough
+ * A small batch (AUTO: at most 152 rows per expert on average, and enough
  * experts x 128-column strips to occupy half the CUs) runs on the mid-M kernel,
  * one workgroup per (expert, strip), with no table and no scale re-layout: the
  * call is then bound by reading every expert's B once.  It needs K % 256 == 0,

@@ -82,7 +82,7 @@ def test_grouped_mid_empty_groups_and_rows_past_the_last_offset(force_empty):
     check(run(x, xs, w, ws, off, torch.float32, variant=V), ref, torch.float32, str(force_empty))
 
 
-@pytest.mark.parametrize("per_expert", [1, 8, 48, 96])
+@pytest.mark.parametrize("per_expert", [1, 8, 24, 48, 96, 150])
 def test_grouped_mid_is_the_librarys_choice_at_a_small_batch(per_expert):
     """8 experts of config 4's N and K, a few rows per expert: AUTO must give the bits of the kernel asked for by
     name, which is checked against the oracle (all rows up to 8 per expert, sampled rows beyond) and, element for

@@ -98,7 +98,7 @@ bool is_tile_variant(int v) {
 }
 
 // Grouped problems of at most this many rows per expert on average go to the mid-M kernel.
-constexpr int64_t kGroupedMidMaxAvgRows = 128;
+constexpr int64_t kGroupedMidMaxAvgRows = 152;  // (rows per block up to 192: the 256-row block loses to the tile kernels)
 
 // What the mid-M kernel takes (the part of it that the shape alone decides).
 bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
@@ -600,7 +600,7 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
     return WAVE_MXFP4_ERR_UNSUPPORTED;
   // A small batch routed over the experts: every expert's B is read once for a handful of rows, so the call is
   // bound by streaming B, like the dense mid-M problem.  One workgroup per (expert, strip of columns), no table, no
-  // re-layout of the scales.  AUTO takes it up to 128 rows per expert on average (measured at 8 experts, N = 14336,
+  // re-layout of the scales.  AUTO takes it up to 152 rows per expert on average (measured at 8 experts, N = 14336,
   // K = 4096 against the table-driven tile kernels), when there are enough strips to put most CUs to work.
   if (variant == WAVE_MXFP4_VARIANT_MID_M || variant == WAVE_MXFP4_VARIANT_AUTO) {
     const bool fits = mid_grouped_applies(p);

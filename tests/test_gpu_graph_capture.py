@@ -16,7 +16,10 @@ pytestmark = pytest.mark.gpu
 
 
 def test_captured_gemm_sequence_replays_with_eager_results():
-    shapes = [(1024, 1024, 8192), (16, 4096, 4096), (512, 768, 16384), (300, 200, 1248), (2304, 2304, 1024)]
+    # (the last three: the mid-M kernel's 32-row block on one round of strips, with two workgroups per CU, and its
+    # 128-row block)
+    shapes = [(1024, 1024, 8192), (16, 4096, 4096), (512, 768, 16384), (300, 200, 1248), (2304, 2304, 1024),
+              (32, 16384, 2048), (24, 36864, 1024), (100, 12288, 1024)]
     ops = []
     for i, (m, n, k) in enumerate(shapes):
         x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=40 + i, scale_lo=120, scale_hi=134)

@@ -60,10 +60,12 @@ def check(c, ref, dt, what):
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("lb,pre", [(RM, False), (M32, False), (RM, True), (M32, True)])
-@pytest.mark.parametrize("e,n,k,rows", [(8, 160, 1024, 40), (5, 1008, 1280, 333), (16, 96, 2048, 16), (3, 4096, 1024, 700)])
+@pytest.mark.parametrize("e,n,k,rows", [(8, 160, 1024, 40), (5, 1008, 1280, 333), (16, 96, 2048, 16), (3, 4096, 1024, 700),
+                                        (40, 1024, 2048, 300)])
 def test_grouped_mid_ragged_groups(e, n, k, rows, lb, pre, dt):
     """Uneven groups (333 rows over 5 experts and 700 over 3: groups of more rows than a block, taken block by
-    block; 16 rows over 16 experts: groups of one row and none)."""
+    block; 16 rows over 16 experts: groups of one row and none; 40 experts x 8 strips: more strips than CUs, the
+    shallow rings with two workgroups per CU, K walked from a rotated start)."""
     x, xs, w, ws, off = inputs(e, n, k, rows, seed=e + rows)
     c = run(x, xs, w, ws, off, dt, lb=lb, pre=pre, variant=V)
     check(c, reference(x, xs, w, ws, off), dt, f"E={e} {rows}x{n}x{k}")

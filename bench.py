@@ -410,13 +410,17 @@ def main():
     ap.add_argument("--warmup", type=int, default=100, help="untimed launches in front of the timed ones (after the "
                     "time-based settle load every leg runs anyway)")
     ap.add_argument("--workload", default="cfg2",
-                    choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue", "ref_shapes", "mfma_ceiling"],
+                    choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue", "ref_shapes", "mfma_ceiling",
+                                                 "decode_sweep", "moe_serving"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
                          "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out; "
                          "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096; moe_glue: the steps around "
                          "it at the same sizes (token alignment, gathered quantiser, gated activation + quantiser); "
                          "ref_shapes: the reference's benchmark shape list; mfma_ceiling: the scaled FP4 MFMA alone, "
-                         "random operands against zeros (the power-limited ceiling of the matrix pipes)")
+                         "random operands against zeros (the power-limited ceiling of the matrix pipes); decode_sweep: "
+                         "M = 1 .. 256 against wide weights from HBM, every kernel that serves the shape beside the "
+                         "library's own choice; moe_serving: the grouped GEMM at serving batches, experts x rows per "
+                         "expert, the mid-M kernel beside the tile kernels")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-legs", "--no-decode", dest="no_legs", action="store_true",
@@ -510,6 +514,99 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": read_traffic("quant_bf16"),
                          "kernel": "quantize_kernel", "launch_us": round(qper * 1e6, 2)}})))
+        return
+
+    if args.workload == "decode_sweep":
+        # M x N x K against weights that come from HBM (operand sets rotated), bf16 out: the library's own choice
+        # beside the streaming kernel (M <= 64), the mid-M kernel and the best tile kernel, each asked for by name
+        from wave_amd import _lib as L
+
+        SETTLE["ms"] = 20.0
+        rows = []
+        for k in (8192, 4096):
+            for n in (8192, 14336, 28672, 57344):
+                for m in (1, 16, 32, 64, 128, 256):
+                    copies = max(2, min(6, int(600e6 / (n * k / 2))))
+                    sets = make_gpu_inputs(torch, m, n, k, 2, (120, 134), dev, copies=copies)
+                    out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+                    us = {}
+                    names = [("mid", L.VARIANT_MID_M, 1)]
+                    if m <= 64:
+                        names.append(("stream", L.VARIANT_SKINNY, 1))
+                    else:
+                        names += [("t128x128", L.VARIANT_T128x128_W2x2, 0), ("t128x256", L.VARIANT_T128x256_W2x2, 0),
+                                  ("t256x256", L.VARIANT_T256x256_W4x2, 0)]
+                    names.append(("auto", L.VARIANT_AUTO, 0))
+                    for name, v, split in names:
+                        _, per, _ = time_gemm(torch, wave_amd, sets, out, min(args.steps, 100), 20, variant=v, split_k=split)
+                        us[name] = round(per * 1e6, 2)
+                    nbytes = gemm_bytes(m, n, k, 2)
+                    rows.append({"m": m, "n": n, "k": k, "us": us, "bytes": nbytes,
+                                 "auto_frac_of_hbm_peak": round(nbytes / (us["auto"] * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4)})
+                    del sets, out
+        worst = max(r["us"]["auto"] / min(r["us"].values()) for r in rows)
+        print(json.dumps(dict(common, **{
+            "metric": "MXFP4 GEMM at decode shapes: worst ratio of the library's choice to the best kernel",
+            "value": round(worst, 3), "unit": "x", "higher_is_better": False,
+            "ms_per_step": round(sum(r["us"]["auto"] for r in rows) * 1e-3, 3),
+            "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out",
+            "data": "synthetic (seeded uniform nibbles and scales), weights from HBM",
+            "config": {"workload": f"decode_sweep: {len(rows)} shapes M x N x K, bf16 out, seed 2"}, "shapes": rows})))
+        return
+
+    if args.workload == "moe_serving":
+        # the grouped GEMM at serving batches: E experts x rows per expert (even groups and multinomially dealt ones),
+        # weights from HBM (three copies rotated), bf16 out; the library's choice beside the mid-M kernel and the
+        # table-driven tile kernels asked for by name
+        import numpy as np
+        from wave_amd import _lib as L
+
+        SETTLE["ms"] = 20.0
+        g = torch.Generator(device="cpu").manual_seed(3)
+        rows = []
+        for E, n, k in ((8, 14336, 4096), (32, 4096, 4096), (64, 2048, 7168), (128, 1536, 4096)):
+            W = [torch.randint(0, 256, (E, n, k // 2), dtype=torch.uint8, generator=g).to(dev) for _ in range(3)]
+            WS = [torch.randint(120, 135, (E, n, k // 32), dtype=torch.uint8, generator=g).to(dev) for _ in range(3)]
+            for per_e in (1, 16, 32, 64, 128, 192):
+                if E * per_e > 8192:
+                    continue
+                total = E * per_e
+                x = torch.randint(0, 256, (total, k // 2), dtype=torch.uint8, generator=g).to(dev)
+                xs = torch.randint(120, 135, (total, k // 32), dtype=torch.uint8, generator=g).to(dev)
+                out = torch.empty(total, n, dtype=torch.bfloat16, device=dev)
+                for ragged in (False, True):
+                    cnt = (np.random.default_rng(per_e).multinomial(total, np.ones(E) / E) if ragged
+                           else np.full(E, per_e))
+                    off = torch.tensor(np.concatenate([[0], np.cumsum(cnt)]), dtype=torch.int32, device=dev)
+                    us = {}
+                    for name, v in (("auto", L.VARIANT_AUTO), ("mid", L.VARIANT_MID_M),
+                                    ("t128x128", L.VARIANT_T128x128_W2x2), ("t256x256", L.VARIANT_T256x256_W4x2)):
+                        state = {"i": 0}
+
+                        def run(count):
+                            for _ in range(count):
+                                i = state["i"] % 3
+                                state["i"] += 1
+                                wave_amd.mxfp4_gemm_grouped(x, xs, W[i], WS[i], off, out, variant=v)
+
+                        _, per, _ = timed(torch, run, min(args.steps, 60), 10)
+                        us[name] = round(per * 1e6, 1)
+                    used = int((cnt > 0).sum())  # an expert without rows is not read
+                    nbytes = used * n * (k // 2 + k // 32) + total * (k // 2 + k // 32) + total * n * 2
+                    rows.append({"experts": E, "n": n, "k": k, "rows_per_expert": per_e,
+                                 "groups": "multinomial" if ragged else "even", "us": us, "bytes": nbytes,
+                                 "auto_frac_of_hbm_peak": round(nbytes / (us["auto"] * 1e-6) / 1e9 / PEAK_HBM_GBPS, 4)})
+                del x, xs, out
+            del W, WS
+        worst = max(r["us"]["auto"] / min(r["us"].values()) for r in rows)
+        print(json.dumps(dict(common, **{
+            "metric": "grouped MXFP4 GEMM at serving batches: worst ratio of the library's choice to the best kernel",
+            "value": round(worst, 3), "unit": "x", "higher_is_better": False,
+            "ms_per_step": round(sum(r["us"]["auto"] for r in rows) * 1e-3, 3),
+            "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out",
+            "data": "synthetic (seeded uniform), weights from HBM",
+            "config": {"workload": f"moe_serving: {len(rows)} (experts, N, K, rows per expert, even or multinomial groups)"},
+            "shapes": rows})))
         return
 
     if args.workload == "ref_shapes":

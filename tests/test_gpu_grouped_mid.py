@@ -17,7 +17,7 @@ from gpu_util import DEV, assert_close, to_gpu
 
 pytestmark = pytest.mark.gpu
 V = _lib.VARIANT_MID_M
-RM, M32 = _lib.SCALE_ROW_MAJOR, _lib.SCALE_MFMA32
+RM, M32, SH = _lib.SCALE_ROW_MAJOR, _lib.SCALE_MFMA32, _lib.SCALE_E8M0_SHUFFLE
 
 
 def inputs(e, n, k, rows, seed, force_empty=(), lo=118, hi=136):
@@ -59,7 +59,7 @@ def check(c, ref, dt, what):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("lb,pre", [(RM, False), (M32, False), (RM, True), (M32, True)])
+@pytest.mark.parametrize("lb,pre", [(RM, False), (M32, False), (RM, True), (M32, True), (SH, False), (SH, True)])
 @pytest.mark.parametrize("e,n,k,rows", [(8, 160, 1024, 40), (5, 1008, 1280, 333), (16, 96, 2048, 16), (3, 4096, 1024, 700),
                                         (40, 1024, 2048, 300)])
 def test_grouped_mid_ragged_groups(e, n, k, rows, lb, pre, dt):

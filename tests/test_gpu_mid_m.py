@@ -70,7 +70,19 @@ def test_mid_rotated_start_in_k(m, n, k, la, lb):
     assert_close(c, c_oracle.scaled_gemm_exact(x, w, xs, ws), torch.float32, f"{m}x{n}x{k} {la}/{lb}")
 
 
-@pytest.mark.parametrize("lb", [RM, M32])
+@pytest.mark.parametrize("m,n,k", [(20, 2048, 2048), (100, 3000, 2048), (256, 1504, 4096), (64, 28676, 1024), (33, 160, 1280)])
+@pytest.mark.parametrize("la", [RM, M32])
+def test_mid_reads_shuffled_b_scales_in_place(m, n, k, la):
+    """B's scales in e8m0_shuffle order (the reference's format for static weights, mxfp_utils.py:113-128) without
+    scratch, so that no pass can re-lay them out: the kernel reads the blocks as they are; the bits of the MFMA32
+    path (the same strips, the same order of the sums)."""
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=m * 7 + n, scale_lo=100, scale_hi=154)
+    c = run(x, xs, w, ws, torch.float32, la=la, lb=SH, variant=V, split_k=1, workspace=False)
+    assert_close(c, c_oracle.scaled_gemm_exact(x, w, xs, ws), torch.float32, f"{m}x{n}x{k} {la}/shuffle")
+    assert np.array_equal(c, run(x, xs, w, ws, torch.float32, la=la, lb=M32, variant=V, split_k=1, workspace=False))
+
+
+@pytest.mark.parametrize("lb", [RM, M32, SH])
 @pytest.mark.parametrize("m,n,k", [(24, 36864, 2048), (1, 40004, 1024), (32, 33000, 1280)])
 def test_mid_more_strips_than_cus(m, n, k, lb):
     """Up to 32 rows against more 128-column strips than the GPU has CUs: the shallow rings with two workgroups per

@@ -30,9 +30,10 @@
 //   * A grouped (mixture of experts) problem of few rows per expert runs the same body with one workgroup per
 //     (expert, strip); a wave skips the row blocks past its group's rows.
 //
-// Taken for K % 256 == 0 (at least 4 K tiles), N % 4 == 0, each scale tensor row-major or in MFMA32 order
-// (e8m0_shuffle order is re-laid out first when the library has scratch; B scales in MFMA32 order fix WV at 32,
-// the row block of that layout), B row-major or preshuffled.  The reference runs these shapes
+// Taken for K % 256 == 0 (at least 4 K tiles), N % 4 == 0, each scale tensor row-major or in MFMA32 order, B's
+// also in e8m0_shuffle order, the reference's format for static weights (A's in that order are re-laid out first
+// when the library has scratch; B scales in a blocked order fix WV at 32, the row block of those layouts), B
+// row-major or preshuffled.  The reference runs these shapes
 // through its generic tile kernel (tests/kernel/wave_gemm_mxfp_test.py:291-339); the result contract is the same.
 #include <type_traits>
 
@@ -82,11 +83,13 @@ struct MidCfg {
   static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
 };
 
-// A_RM / B_RM: the operand's scales are row-major (else MFMA32 order).  Template parameters, not run-time flags:
+// A_RM / B_RM: the operand's scales are row-major (else MFMA32 order, or for B, with B_SH, e8m0_shuffle order: the
+// same 256-byte blocks per 32 rows and K tile, fetched the same way; only the lane's read differs).  Template
+// parameters, not run-time flags:
 // a branch on the layout inside the K loop makes the compiler wait for every outstanding request at the join.
 // One strip of one block of `m_rows` <= BM rows: A [m_rows, kp] at `a_base` with its scales at `as_base`, B [N, kp]
 // at `b_base` (one expert's, for a grouped problem) with its scales at `bs_base`, C rows at `c_base`.
-template <class Cfg, bool A_RM>
+template <class Cfg, bool A_RM, bool B_SH>
 __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, const uint8_t *a_base, const uint8_t *as_base,
                                          const uint8_t *b_base, const uint8_t *bs_base, uint8_t *c_base, const int m_rows) {
   constexpr bool B_RM = Cfg::B_RM;
@@ -259,7 +262,19 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
       const int c = (j >> 1) & 3;
       return pick_scales(*(const v4i *)(img + ((j >> 3) & 1) * 2048 + fr * 64 + ((c ^ ((fr >> 2) & 3)) << 4)), j);
     } else {
-      return lane_scales(img + ((j >> 2) & 3) * 1024, std::false_type{}, j);
+      const uint8_t *blk = img + ((j >> 2) & 3) * 1024 + (j & 3) * 256;  // the K tile's block
+      if constexpr (B_SH) {
+        // e8m0_shuffle order (wave_lang/kernel/wave/utils/mxfp_utils.py:113-128): group k of row r sits at byte
+        // (k % 4) * 64 + (r % 16) * 4 + (k % 8) / 4 * 2 + r / 16 of the block.  The lane's K steps s = 0 .. 3 want
+        // groups 2 s + fg: steps 0 and 2 are bytes r / 16 and 2 + r / 16 of the dword at fg * 64 + (r % 16) * 4,
+        // steps 1 and 3 the same bytes of the dword 128 bytes further on.
+        static_assert(!Cfg::B_RM, "blocked layouts");
+        const uint32_t d0 = *(const uint32_t *)(blk + fg * 64 + (fr & 15) * 4);
+        const uint32_t d1 = *(const uint32_t *)(blk + 128 + fg * 64 + (fr & 15) * 4);
+        return __builtin_amdgcn_perm(d1, d0, 0x06020400u + (uint32_t)(fr >> 4) * 0x01010101u);
+      } else {
+        return *(const uint32_t *)(blk + lane * 4);
+      }
     }
   };
 
@@ -430,10 +445,10 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
 // GROUPED: blockIdx.y is the expert; its rows offsets[e] .. offsets[e + 1] (clamped to [0, M], not validated) are
 // taken BM at a time - a group of more rows than BM streams its expert's B once per block of rows, which is what
 // the table-driven persistent kernel is for; this one is for the few rows per expert of a small batch.
-template <class Cfg, bool A_RM, bool GROUPED>
+template <class Cfg, bool A_RM, bool GROUPED, bool B_SH>
 __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p, const int wv) {
   if constexpr (!GROUPED) {
-    mid_body<Cfg, A_RM>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
+    mid_body<Cfg, A_RM, B_SH>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
   } else {
     static_assert(A_RM, "a group may start at any row: A's scales row-major");
     const int e = blockIdx.y;
@@ -442,7 +457,7 @@ __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p,
     const uint8_t *b = p.b + (int64_t)e * p.b_group_stride, *bs = p.b_scale + (int64_t)e * p.b_scale_group_stride;
     const int elt = p.out_bf16 ? 2 : 4;
     for (int m0 = lo; m0 < hi; m0 += Cfg::BM) {
-      mid_body<Cfg, A_RM>(p, wv, p.a + (int64_t)m0 * p.kp, p.a_scale + (int64_t)m0 * p.ks, b, bs,
+      mid_body<Cfg, A_RM, B_SH>(p, wv, p.a + (int64_t)m0 * p.kp, p.a_scale + (int64_t)m0 * p.ks, b, bs,
                           (uint8_t *)p.c + (int64_t)m0 * p.n * elt, min(Cfg::BM, hi - m0));
       // every wave is done with the rings (the C staging's reads included) before the next block's requests
       __builtin_amdgcn_s_waitcnt(0);
@@ -453,15 +468,23 @@ __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p,
   }
 }
 
-template <class Cfg, bool A_RM, bool GROUPED>
-hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
+template <class Cfg, bool A_RM, bool GROUPED, bool B_SH>
+hipError_t launch_mid_kernel(const GemmParams &p, int wv, hipStream_t stream) {
   static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, GROUPED>, Cfg::LDS);
+  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH>, Cfg::LDS);
   if (e != hipSuccess) return e;
   const int bn = kMidCW * wv;
   const dim3 grid((p.n + bn - 1) / bn, GROUPED ? p.num_groups : 1, 1);
-  mid_gemm_kernel<Cfg, A_RM, GROUPED><<<grid, dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
+  mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH><<<grid, dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
   return hipGetLastError();
+}
+
+template <class Cfg, bool A_RM, bool GROUPED>
+hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
+  if constexpr (!Cfg::B_RM) {
+    if (p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) return launch_mid_kernel<Cfg, A_RM, GROUPED, true>(p, wv, stream);
+  }
+  return launch_mid_kernel<Cfg, A_RM, GROUPED, false>(p, wv, stream);
 }
 
 template <int BM, bool TWO = false>
@@ -499,7 +522,9 @@ int mid_max_m() { return 256; }
 bool mid_gemm_applies(const GemmParams &p) {
   if (p.num_groups != 0 || p.splits != 1 || p.partial != nullptr || p.m < 1 || p.m > mid_max_m()) return false;
   const auto layout_ok = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
-  if (!layout_ok(p.a_scale_layout) || !layout_ok(p.b_scale_layout)) return false;
+  // (B's scales also in e8m0_shuffle order, the reference's format for static weights)
+  if (!layout_ok(p.a_scale_layout) || !(layout_ok(p.b_scale_layout) || p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE))
+    return false;
   if ((p.k & (kTileK - 1)) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
   // 32-bit offsets: inside A, inside a wave's 48 rows of B, inside C, inside the scales of A and of a wave's rows
   if ((int64_t)p.m * p.kp >= ((int64_t)1 << 31) || (int64_t)48 * p.kp >= ((int64_t)1 << 31) ||
@@ -514,7 +539,9 @@ bool mid_gemm_applies(const GemmParams &p) {
 bool mid_grouped_applies(const GemmParams &p) {
   if (p.num_groups <= 0 || p.num_groups > 65535 || p.offsets == nullptr || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR) return false;
-  if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 &&
+      p.b_scale_layout != WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
+    return false;
   if ((p.k & (kTileK - 1)) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
   if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)48 * p.kp >= ((int64_t)1 << 31) ||
       (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31) || (int64_t)8 * p.k_tiles * 256 >= ((int64_t)1 << 31))

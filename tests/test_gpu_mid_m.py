@@ -2,7 +2,7 @@
 through its generic tile kernel, tests/kernel/wave_gemm_mxfp_test.py:291-339) against the exact oracle: every row
 block count, ragged M, N that is no multiple of the strip width (strips of 16 to 32 columns per wave), K with a
 partial group of four K tiles, both output types, both B layouts, row-major and MFMA32 scales per operand,
-e8m0_shuffle scales through the re-layout, NaN scales, and the library's own choice of it at the decode shapes."""
+e8m0_shuffle scales read in place, NaN scales, and the library's own choice of it at the decode shapes."""
 
 import numpy as np
 import pytest
@@ -71,15 +71,27 @@ def test_mid_rotated_start_in_k(m, n, k, la, lb):
 
 
 @pytest.mark.parametrize("m,n,k", [(20, 2048, 2048), (100, 3000, 2048), (256, 1504, 4096), (64, 28676, 1024), (33, 160, 1280)])
-@pytest.mark.parametrize("la", [RM, M32])
+@pytest.mark.parametrize("la", [RM, M32, SH])
 def test_mid_reads_shuffled_b_scales_in_place(m, n, k, la):
-    """B's scales in e8m0_shuffle order (the reference's format for static weights, mxfp_utils.py:113-128) without
-    scratch, so that no pass can re-lay them out: the kernel reads the blocks as they are; the bits of the MFMA32
-    path (the same strips, the same order of the sums)."""
+    """B's scales in e8m0_shuffle order (the reference's format for static weights, mxfp_utils.py:113-128), A's in
+    any of the three, without scratch, so that no pass can re-lay them out: the kernel reads the blocks as they
+    are; the bits of the MFMA32 path (the same strips, the same order of the sums)."""
     x, xs, w, ws = orc.make_inputs(m, n, k, seed=m * 7 + n, scale_lo=100, scale_hi=154)
     c = run(x, xs, w, ws, torch.float32, la=la, lb=SH, variant=V, split_k=1, workspace=False)
     assert_close(c, c_oracle.scaled_gemm_exact(x, w, xs, ws), torch.float32, f"{m}x{n}x{k} {la}/shuffle")
-    assert np.array_equal(c, run(x, xs, w, ws, torch.float32, la=la, lb=M32, variant=V, split_k=1, workspace=False))
+    assert np.array_equal(c, run(x, xs, w, ws, torch.float32, la=M32, lb=M32, variant=V, split_k=1, workspace=False))
+
+
+@pytest.mark.parametrize("lb", [RM, M32])
+@pytest.mark.parametrize("m,n,k", [(1, 1024, 1024), (31, 640, 2304), (130, 2048, 1536), (200, 700, 2048), (256, 28672, 1024)])
+def test_mid_reads_shuffled_a_scales_in_place(m, n, k, lb):
+    """A's scales in e8m0_shuffle order (what the quantiser writes for the reference's preshuffled-scale kernels)
+    against B's row-major and MFMA32 ones, without scratch; M that ends inside a 32-row block of the layout."""
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=m * 5 + k, scale_lo=100, scale_hi=154)
+    c = run(x, xs, w, ws, torch.float32, la=SH, lb=lb, variant=V, split_k=1, workspace=False)
+    cols = np.unique(np.concatenate([np.arange(0, n, max(1, n // 600)), [n - 1]]))
+    assert_close(c[:, cols], c_oracle.scaled_gemm_exact(x, w[cols], xs, ws[cols]), torch.float32, f"{m}x{n}x{k} shuffle/{lb}")
+    assert np.array_equal(c, run(x, xs, w, ws, torch.float32, la=M32, lb=lb, variant=V, split_k=1, workspace=False))
 
 
 @pytest.mark.parametrize("lb", [RM, M32, SH])

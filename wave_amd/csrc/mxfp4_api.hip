@@ -138,11 +138,12 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
 }
 
 // Kernels that read both scale tensors in MFMA32 order (the library re-lays them out first when it has scratch).
-// The mid-M kernel also reads row-major scales as they are, and B's in e8m0_shuffle order too; only A's in that order are re-laid out for it.
+// The mid-M kernel also reads row-major scales and scales in e8m0_shuffle order (the reference's format for
+// preshuffled scales) as they are: no pass per call for them.
 bool wants_mfma32_scales(int v) { return is_tile_variant(v) || v == WAVE_MXFP4_VARIANT_MID_M; }
-bool mid_reads(int layout) { return layout == WAVE_MXFP4_SCALE_ROW_MAJOR || layout == WAVE_MXFP4_SCALE_MFMA32; }
-// (B's scales also in e8m0_shuffle order: static weights in the reference's own format need no pass per call)
-bool mid_reads_b(int layout) { return mid_reads(layout) || layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE; }
+bool mid_reads(int layout) {
+  return layout == WAVE_MXFP4_SCALE_ROW_MAJOR || layout == WAVE_MXFP4_SCALE_MFMA32 || layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
+}
 
 // A partial last K tile with scales that are not (or cannot be brought) in MFMA32 order is only built for the
 // 128x128 tile kernel.
@@ -298,7 +299,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
   if (v == WAVE_MXFP4_VARIANT_SKINNY && m > skinny_max_m()) return WAVE_MXFP4_ERR_UNSUPPORTED;
   if (variant == WAVE_MXFP4_VARIANT_MID_M) {
-    const bool native = (mid_reads(a_scale_layout) || a_scale_layout == WAVE_MXFP4_SCALE_PER_ROW) && mid_reads_b(b_scale_layout);
+    const bool native = (mid_reads(a_scale_layout) || a_scale_layout == WAVE_MXFP4_SCALE_PER_ROW) && mid_reads(b_scale_layout);
     if (!mid_shape_ok(m, n, k) || split_k > 1 || (!native && !workspace)) return WAVE_MXFP4_ERR_UNSUPPORTED;
   }
   if (v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT) {
@@ -372,7 +373,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
     const bool mid = v == WAVE_MXFP4_VARIANT_MID_M;
     const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads(p.a_scale_layout)) ? a_bytes : 0;
-    const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads_b(p.b_scale_layout)) ? b_bytes : 0;
+    const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads(p.b_scale_layout)) ? b_bytes : 0;
     if (ws_used + a_need + b_need <= workspace_bytes) {
       uint8_t *ws = (uint8_t *)workspace + ws_used;
       ws_scales_end = ws_used + a_need + b_need;

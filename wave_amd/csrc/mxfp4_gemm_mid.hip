@@ -30,10 +30,10 @@
 //   * A grouped (mixture of experts) problem of few rows per expert runs the same body with one workgroup per
 //     (expert, strip); a wave skips the row blocks past its group's rows.
 //
-// Taken for K % 256 == 0 (at least 4 K tiles), N % 4 == 0, each scale tensor row-major or in MFMA32 order, B's
-// also in e8m0_shuffle order, the reference's format for static weights (A's in that order are re-laid out first
-// when the library has scratch; B scales in a blocked order fix WV at 32, the row block of those layouts), B
-// row-major or preshuffled.  The reference runs these shapes
+// Taken for K % 256 == 0 (at least 4 K tiles), N % 4 == 0, each scale tensor row-major, in MFMA32 order or in
+// e8m0_shuffle order, the reference's format for preshuffled scales (all read as they are; B scales in a blocked
+// order fix WV at 32, the row block of those layouts; a grouped problem takes A's row-major only), B row-major or
+// preshuffled.  The reference runs these shapes
 // through its generic tile kernel (tests/kernel/wave_gemm_mxfp_test.py:291-339); the result contract is the same.
 #include <type_traits>
 
@@ -83,13 +83,13 @@ struct MidCfg {
   static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
 };
 
-// A_RM / B_RM: the operand's scales are row-major (else MFMA32 order, or for B, with B_SH, e8m0_shuffle order: the
+// A_RM / B_RM: the operand's scales are row-major (else MFMA32 order, or with A_SH / B_SH e8m0_shuffle order: the
 // same 256-byte blocks per 32 rows and K tile, fetched the same way; only the lane's read differs).  Template
 // parameters, not run-time flags:
 // a branch on the layout inside the K loop makes the compiler wait for every outstanding request at the join.
 // One strip of one block of `m_rows` <= BM rows: A [m_rows, kp] at `a_base` with its scales at `as_base`, B [N, kp]
 // at `b_base` (one expert's, for a grouped problem) with its scales at `bs_base`, C rows at `c_base`.
-template <class Cfg, bool A_RM, bool B_SH>
+template <class Cfg, bool A_RM, bool B_SH, bool A_SH>
 __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, const uint8_t *a_base, const uint8_t *as_base,
                                          const uint8_t *b_base, const uint8_t *bs_base, uint8_t *c_base, const int m_rows) {
   constexpr bool B_RM = Cfg::B_RM;
@@ -248,9 +248,21 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     const bool odd = (j & 1) != 0;
     return __builtin_amdgcn_perm((uint32_t)(odd ? q.w : q.y), (uint32_t)(odd ? q.z : q.x), pick);
   };
+  // A lane's dword of a K tile's 256-byte block in e8m0_shuffle order
+  // (wave_lang/kernel/wave/utils/mxfp_utils.py:113-128): group k of row r sits at byte
+  // (k % 4) * 64 + (r % 16) * 4 + (k % 8) / 4 * 2 + r / 16 of the block.  The lane's K steps s = 0 .. 3 want groups
+  // 2 s + fg: steps 0 and 2 are bytes r / 16 and 2 + r / 16 of the dword at fg * 64 + (r % 16) * 4, steps 1 and 3
+  // the same bytes of the dword 128 bytes further on.
+  auto shuffled_scales = [&](const uint8_t *blk) -> uint32_t {
+    const uint32_t d0 = *(const uint32_t *)(blk + fg * 64 + (fr & 15) * 4);
+    const uint32_t d1 = *(const uint32_t *)(blk + 128 + fg * 64 + (fr & 15) * 4);
+    return __builtin_amdgcn_perm(d1, d0, 0x06020400u + (uint32_t)(fr >> 4) * 0x01010101u);
+  };
   auto lane_scales = [&](const uint8_t *img, auto rm_tag, int j) -> uint32_t {
     if constexpr (decltype(rm_tag)::value) {
       return pick_scales(*(const v4i *)(img + ((j & 2) << 8) + fr * 16), j);
+    } else if constexpr (A_SH) {
+      return shuffled_scales(img + (j & 3) * 256);
     } else {
       return *(const uint32_t *)(img + (j & 3) * 256 + lane * 4);
     }
@@ -264,14 +276,8 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     } else {
       const uint8_t *blk = img + ((j >> 2) & 3) * 1024 + (j & 3) * 256;  // the K tile's block
       if constexpr (B_SH) {
-        // e8m0_shuffle order (wave_lang/kernel/wave/utils/mxfp_utils.py:113-128): group k of row r sits at byte
-        // (k % 4) * 64 + (r % 16) * 4 + (k % 8) / 4 * 2 + r / 16 of the block.  The lane's K steps s = 0 .. 3 want
-        // groups 2 s + fg: steps 0 and 2 are bytes r / 16 and 2 + r / 16 of the dword at fg * 64 + (r % 16) * 4,
-        // steps 1 and 3 the same bytes of the dword 128 bytes further on.
         static_assert(!Cfg::B_RM, "blocked layouts");
-        const uint32_t d0 = *(const uint32_t *)(blk + fg * 64 + (fr & 15) * 4);
-        const uint32_t d1 = *(const uint32_t *)(blk + 128 + fg * 64 + (fr & 15) * 4);
-        return __builtin_amdgcn_perm(d1, d0, 0x06020400u + (uint32_t)(fr >> 4) * 0x01010101u);
+        return shuffled_scales(blk);
       } else {
         return *(const uint32_t *)(blk + lane * 4);
       }
@@ -445,10 +451,11 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
 // GROUPED: blockIdx.y is the expert; its rows offsets[e] .. offsets[e + 1] (clamped to [0, M], not validated) are
 // taken BM at a time - a group of more rows than BM streams its expert's B once per block of rows, which is what
 // the table-driven persistent kernel is for; this one is for the few rows per expert of a small batch.
-template <class Cfg, bool A_RM, bool GROUPED, bool B_SH>
+template <class Cfg, bool A_RM, bool GROUPED, bool B_SH, bool A_SH>
 __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p, const int wv) {
+  static_assert(!(A_RM && A_SH), "one layout");
   if constexpr (!GROUPED) {
-    mid_body<Cfg, A_RM, B_SH>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
+    mid_body<Cfg, A_RM, B_SH, A_SH>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
   } else {
     static_assert(A_RM, "a group may start at any row: A's scales row-major");
     const int e = blockIdx.y;
@@ -457,7 +464,7 @@ __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p,
     const uint8_t *b = p.b + (int64_t)e * p.b_group_stride, *bs = p.b_scale + (int64_t)e * p.b_scale_group_stride;
     const int elt = p.out_bf16 ? 2 : 4;
     for (int m0 = lo; m0 < hi; m0 += Cfg::BM) {
-      mid_body<Cfg, A_RM, B_SH>(p, wv, p.a + (int64_t)m0 * p.kp, p.a_scale + (int64_t)m0 * p.ks, b, bs,
+      mid_body<Cfg, A_RM, B_SH, A_SH>(p, wv, p.a + (int64_t)m0 * p.kp, p.a_scale + (int64_t)m0 * p.ks, b, bs,
                           (uint8_t *)p.c + (int64_t)m0 * p.n * elt, min(Cfg::BM, hi - m0));
       // every wave is done with the rings (the C staging's reads included) before the next block's requests
       __builtin_amdgcn_s_waitcnt(0);
@@ -468,21 +475,30 @@ __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p,
   }
 }
 
-template <class Cfg, bool A_RM, bool GROUPED, bool B_SH>
+template <class Cfg, bool A_RM, bool GROUPED, bool B_SH, bool A_SH = false>
 hipError_t launch_mid_kernel(const GemmParams &p, int wv, hipStream_t stream) {
   static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH>, Cfg::LDS);
+  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH, A_SH>, Cfg::LDS);
   if (e != hipSuccess) return e;
   const int bn = kMidCW * wv;
   const dim3 grid((p.n + bn - 1) / bn, GROUPED ? p.num_groups : 1, 1);
-  mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH><<<grid, dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
+  mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH, A_SH><<<grid, dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
   return hipGetLastError();
 }
 
 template <class Cfg, bool A_RM, bool GROUPED>
 hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
+  const bool b_sh = p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
+  if constexpr (!A_RM && !GROUPED) {
+    if (p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {
+      if constexpr (!Cfg::B_RM) {
+        if (b_sh) return launch_mid_kernel<Cfg, false, false, true, true>(p, wv, stream);
+      }
+      return launch_mid_kernel<Cfg, false, false, false, true>(p, wv, stream);
+    }
+  }
   if constexpr (!Cfg::B_RM) {
-    if (p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) return launch_mid_kernel<Cfg, A_RM, GROUPED, true>(p, wv, stream);
+    if (b_sh) return launch_mid_kernel<Cfg, A_RM, GROUPED, true>(p, wv, stream);
   }
   return launch_mid_kernel<Cfg, A_RM, GROUPED, false>(p, wv, stream);
 }
@@ -521,10 +537,11 @@ int mid_max_m() { return 256; }
 // Whether the mid-M kernel serves this problem.
 bool mid_gemm_applies(const GemmParams &p) {
   if (p.num_groups != 0 || p.splits != 1 || p.partial != nullptr || p.m < 1 || p.m > mid_max_m()) return false;
-  const auto layout_ok = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
-  // (B's scales also in e8m0_shuffle order, the reference's format for static weights)
-  if (!layout_ok(p.a_scale_layout) || !(layout_ok(p.b_scale_layout) || p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE))
-    return false;
+  // (row-major, MFMA32, or e8m0_shuffle order, the reference's format for preshuffled scales)
+  const auto layout_ok = [](int l) {
+    return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32 || l == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
+  };
+  if (!layout_ok(p.a_scale_layout) || !layout_ok(p.b_scale_layout)) return false;
   if ((p.k & (kTileK - 1)) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
   // 32-bit offsets: inside A, inside a wave's 48 rows of B, inside C, inside the scales of A and of a wave's rows
   if ((int64_t)p.m * p.kp >= ((int64_t)1 << 31) || (int64_t)48 * p.kp >= ((int64_t)1 << 31) ||

@@ -447,6 +447,12 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     // C goes out through a descriptor that ends with the tile's last valid row: rows past M (or past the
     // tile's group) are dropped
     constexpr int ELT = out_bf16 ? 2 : 4;
+    // Grouped: non-temporal stores (the nt bit).  Every expert's B streams from HBM once, and a round's C tiles,
+    // as many bytes as the XCD's L2 holds, written back lazily from there, got in the way of it: 8 experts x 1024
+    // rows x 14336 x 4096 236 -> 221 us, multinomial groups 258 -> 244 us.  A dense problem, whose B the XCDs
+    // share through the Infinity Cache, loses 1-2 % with them (8192^3: 237 -> 241 us) and keeps the default.
+    // MXFP8 (twice the operand bytes, f32 C: more than the Infinity Cache holds at 8192^3) gains 2 %.
+    constexpr int kStorePolicy = (GROUPED || FP8) ? 2 : 0;
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc_n(cbase, (int)min((int64_t)rows * ldc * ELT, (int64_t)0x7FFFFFFF));
     const int wr0 = wave_m * Cfg::WM;  // the wave's first row inside the tile
     if (out_bf16) {
@@ -474,7 +480,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
             const int r = r0 + lr;
             const v4i v = *(const v4i *)(stage + r * RP + ((lc ^ (r & (NCH - 1))) << 4));
             __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, ((wr0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 8) * 2,
-                                                       0, 0);
+                                                       0, kStorePolicy);
           }
           asm volatile("" ::: "memory");
         }
@@ -493,7 +499,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
             const int r = r0 + lr4;
             const v4i v = *(const v4i *)(stage + r * RP + ((lc4 ^ (r & (NCH - 1))) << 4));
             __builtin_amdgcn_raw_buffer_store_b128(v, c_rsrc, ((wr0 + i * 32 + r) * ldc + wn0 + (MT_N - 1) * 32 + lc4 * 8) * 2,
-                                                       0, 0);
+                                                       0, kStorePolicy);
           }
           asm volatile("" ::: "memory");
         }
@@ -520,7 +526,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
             const int r = r0 + lr;
             const v4f v = *(const v4f *)(stage + r * RP + ((lc ^ (r & (NCH - 1))) << 4));
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc,
-                                                       ((wr0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 4) * 4, 0, 0);
+                                                       ((wr0 + i * 32 + r) * ldc + wn0 + jg * CP + lc * 4) * 4, 0, kStorePolicy);
           }
           asm volatile("" ::: "memory");
         }

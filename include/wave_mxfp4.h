@@ -175,7 +175,10 @@ size_t wave_mxfp4_static_scratch_bytes(void);
  * `workspace` is optional scratch (256-byte aligned) of
  * wave_mxfp4_grouped_workspace_bytes(...) bytes: with it the scales of both
  * operands are first re-laid out for one-dword-per-lane reads, as in
- * wave_mxfp4_gemm (N % 32 == 0 and K % 256 == 0; otherwise it is not used).
+ * wave_mxfp4_gemm (N % 32 == 0 and K % 256 == 0; otherwise it is not used),
+ * and large problems run the persistent kernel over a table of M tiles built
+ * there; a scale tensor handed over in WAVE_MXFP4_SCALE_MFMA32 order (resident
+ * weights, activations from wave_mxfp4_quantize) is read where it is.
  * A small batch (AUTO: at most 152 rows per expert on average, and enough
  * experts x 128-column strips to occupy half the CUs) runs on the mid-M kernel,
  * one workgroup per (expert, strip), with no table and no scale re-layout: the

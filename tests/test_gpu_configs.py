@@ -250,6 +250,39 @@ def test_grouped_many_expert_rows_with_scratch():
         assert_f32_close(c[lo:hi], ref, f"expert {g}")
 
 
+@pytest.mark.parametrize("la,lb", [("rm", "rm"), ("m32", "rm"), ("rm", "m32"), ("m32", "m32")])
+def test_grouped_persistent_path_scale_layouts_and_ragged_starts(la, lb):
+    """The table-driven persistent kernel (more 256x256 tiles than CUs) with each scale tensor row-major or already
+    in MFMA32 order: groups start at rows that are no multiples of 32, so a tile's lanes find their scales in two
+    neighbouring blocks of A's scale tensor; a NaN scale in a group's last row must poison that row only (the rows
+    of the next group that share its tile's padding are not written by it).  Rows of every tile against the oracle."""
+    e, n, k, rows = 5, 4096, 1024, 4700
+    x, xs, w, ws, off = grouped_inputs(e, n, k, rows, seed=77)
+    assert any(int(o) % 32 for o in off[1:-1])
+    last = int(off[2]) - 1                      # last row of group 1
+    xs[last, 5] = 255
+    gx, gxs, gw, gws, goff = to_gpu(x, xs, w, ws, off)
+    m32 = _lib.SCALE_MFMA32
+    if la == "m32":
+        gxs = wave_amd.scale_convert(gxs, rows, k // 32, _lib.SCALE_ROW_MAJOR, m32)
+    if lb == "m32":
+        gws = torch.stack([wave_amd.scale_convert(gws[g], n, k // 32, _lib.SCALE_ROW_MAJOR, m32) for g in range(e)])
+    out = torch.full((rows + 3, n), float("nan"), dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out[:rows], variant=_lib.VARIANT_T256x256_W4x2,
+                                a_scale_layout=m32 if la == "m32" else _lib.SCALE_ROW_MAJOR,
+                                b_scale_layout=m32 if lb == "m32" else _lib.SCALE_ROW_MAJOR)
+    torch.cuda.synchronize()
+    c = out.cpu().numpy()
+    assert np.isnan(c[rows:]).all() and np.isnan(c[last]).all()
+    assert not np.isnan(np.delete(c[:rows], last, 0)).any()
+    for g in range(e):
+        lo, hi = int(off[g]), int(off[g + 1])
+        pick = np.unique(np.concatenate([np.arange(lo, hi, 37), np.arange(max(lo, hi - 3), hi)]))
+        pick = pick[pick != last]
+        ref = c_oracle.scaled_gemm_exact(x, w[g], xs, ws[g], rows=pick)
+        assert_f32_close(c[pick], ref, f"expert {g} {la}/{lb}")
+
+
 def torch_seeded_inputs(m, n, k, seed, scale_lo, scale_hi):
     """The configuration's operands drawn the way the reference draws its own (torch.manual_seed(seed), then the
     draw order of wave_lang/kernel/wave/utils/mxfp_utils.py:37-57 through the host mirror's generator), on the CPU

@@ -558,17 +558,15 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   return record_hip(launch_tile_gemm_fp8(p, v, a_format == WAVE_MXFP8_E5M2, b_format, stream));
 }
 
-// Scratch of a grouped call: [M tile table | A scales, one 256-row slab per possible M tile | B scales].
+// Scratch of a grouped call: [M tile table | A scales | B scales].
 static size_t grouped_table_bytes(int64_t total_rows, int num_groups) {
   return round_up_256((size_t)(1 + total_rows / 256 + num_groups) * 16);
 }
-static size_t grouped_a_scale_bytes(int64_t total_rows, int64_t k, int num_groups) {
-  return round_up_256(scale_buffer_bytes((total_rows / 256 + num_groups) * 256, k));
-}
+static size_t grouped_a_scale_bytes(int64_t total_rows, int64_t k) { return round_up_256(scale_buffer_bytes(total_rows, k)); }
 
 size_t wave_mxfp4_grouped_workspace_bytes(int64_t total_rows, int64_t n, int64_t k, int num_groups) {
   if (total_rows <= 0 || n <= 0 || k <= 0 || num_groups <= 0 || k % kTileK != 0 || n % 32 != 0) return 0;
-  return grouped_table_bytes(total_rows, num_groups) + grouped_a_scale_bytes(total_rows, k, num_groups) +
+  return grouped_table_bytes(total_rows, num_groups) + grouped_a_scale_bytes(total_rows, k) +
          round_up_256((size_t)num_groups * scale_buffer_bytes(n, k));
 }
 
@@ -641,28 +639,30 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   if (workspace && ws_need != 0 && workspace_bytes >= ws_need && (int64_t)num_groups * n <= 0x7FFFFFFF) {
     int32_t *table = (int32_t *)workspace;
     uint8_t *ws_a = (uint8_t *)workspace + grouped_table_bytes(total_rows, num_groups);
-    uint8_t *ws_b = ws_a + grouped_a_scale_bytes(total_rows, k, num_groups);
+    uint8_t *ws_b = ws_a + grouped_a_scale_bytes(total_rows, k);
     hipError_t e = hipSuccess;
-    // Large problems on the 256x256 tiles: the persistent kernel over a device-built table of M tiles, with
-    // A's scales laid out per tile (a group may start at any row).
+    // Large problems on the 256x256 tiles: the persistent kernel over a device-built table of M tiles.  The
+    // table is built by the launch that re-lays the row-major scales out (by one of its own when both tensors
+    // come in MFMA32 order already: activations from the quantiser, resident weights).
     GemmParams q = p;
     q.tile_table = table;
     q.a_scale_layout = q.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
-    if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR &&
-        (p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR || p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32) &&
-        persist_gemm_applies(q, v, device_cus())) {
-      e = launch_grouped_tile_table(offsets, num_groups, 256, total_rows, table, stream);
-      if (e != hipSuccess) return record_hip(e);
-      const bool b_native = p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
-      e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, total_rows, p.b_scale, ws_b, b_native ? 0 : (int64_t)num_groups * n,
-                                      p.ks, stream, table, total_rows / 256 + num_groups);
+    const auto rm_or_native = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
+    if (rm_or_native(p.a_scale_layout) && rm_or_native(p.b_scale_layout) && persist_gemm_applies(q, v, device_cus())) {
+      const bool a_native = p.a_scale_layout == WAVE_MXFP4_SCALE_MFMA32, b_native = p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+      const GroupTableArgs gt{offsets, num_groups, 256, (int)total_rows, table};
+      if (a_native && b_native)
+        e = launch_grouped_tile_table(offsets, num_groups, 256, total_rows, table, stream);
+      else
+        e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, a_native ? 0 : total_rows, p.b_scale, ws_b,
+                                        b_native ? 0 : (int64_t)num_groups * n, p.ks, stream, &gt);
       if (e == hipSuccess) {
-        q.a_scale = ws_a;
+        if (!a_native) q.a_scale = ws_a;
         if (!b_native) q.b_scale = ws_b;
         q.b_scale_group_stride = n * (int64_t)p.ksp;
         return record_hip(launch_persist_gemm(q, v, device_cus(), stream));
       }
-      // (the fast re-layout does not apply: fall through to the one-tile-per-workgroup kernel)
+      // (the fast re-layout does not apply and has launched nothing: on to the one-tile-per-workgroup kernel)
       e = hipSuccess;
     }
     // both row-major: one launch re-lays both; where that launcher does not apply (it then launches nothing),

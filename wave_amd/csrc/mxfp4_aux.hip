@@ -4,6 +4,7 @@
 // (mxfp_utils.py:98-128), the split-K reduction and a one-thread-per-element
 // GEMM used to cross-check the MFMA kernels on the device.
 #include "mxfp4_common.h"
+#include "mxfp4_group_table.h"
 
 namespace wave_mxfp4 {
 
@@ -110,32 +111,28 @@ __global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_la
 // a pass through LDS (block stride 65 dwords: conflict-free both ways), and
 // dword writes that walk the destination contiguously.
 // blockIdx.z picks one of two tensors with the same ks (the A and B scales of a
-// GEMM go through one launch; rows1 = 0 for a single tensor).
-// With `tiles0` (the M tile table of a grouped GEMM: entry 0 = {count}, entry
-// 1 + t = {first row, rows, expert}) tensor 0 is written tile by tile instead:
-// the 8 blocks of tile t hold rows first .. first + 255 (zeros past the tile's
-// rows), so that a tile's scales are block aligned wherever its group starts.
+// GEMM go through one launch; rows of one of them 0 for a single tensor).
+// With gt.table the launch's first workgroup builds the M tile table of a grouped
+// GEMM before its share of the scales (mxfp4_group_table.h): the table only needs
+// the offsets, so it costs the call no launch of its own.
 __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__restrict__ src0,
                                                               uint8_t *__restrict__ dst0, int rows0,
                                                               const uint8_t *__restrict__ src1,
                                                               uint8_t *__restrict__ dst1, int rows1, int ks,
-                                                              const int32_t *__restrict__ tiles0) {
+                                                              const GroupTableArgs gt) {
   __shared__ uint32_t stage[32 * 65];
+  if (gt.table != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
+    __shared__ int wave_sums[4];
+    __shared__ int carry;
+    build_group_tile_table<256>(gt, wave_sums, &carry);
+  }
   const uint8_t *src = blockIdx.z ? src1 : src0;
   uint8_t *dst = blockIdx.z ? dst1 : dst0;
-  int rows = blockIdx.z ? rows1 : rows0;
+  const int rows = blockIdx.z ? rows1 : rows0;
   const int k_tiles = (ks + 7) >> 3;  // ks % 4 == 0: the last K tile may hold 4 groups only (the rest is written as 0)
   const int rt = blockIdx.x, kt0 = blockIdx.y * 32;  // row tiles along x: up to 2^31 - 1 of them
-  int row_base = rt * 32;
-  if (tiles0 != nullptr && blockIdx.z == 0) {
-    const int tile = rt >> 3;
-    if (tile >= tiles0[0]) return;
-    const int first = tiles0[4 * (1 + tile)], count = tiles0[4 * (1 + tile) + 1];
-    row_base = first + (rt & 7) * 32;
-    rows = first + count;
-  } else if (rt * 32 >= rows) {
-    return;  // the grid is sized for the taller tensor
-  }
+  const int row_base = rt * 32;
+  if (rt * 32 >= rows) return;  // the grid is sized for the taller tensor
   const int t = threadIdx.x;
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
@@ -328,7 +325,7 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
   if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 3) == 0 &&
       ((uintptr_t)src & 3) == 0 && rows < ((int64_t)1 << 31) && (ksp / 8 + 31) / 32 <= 65535) {
     dim3 grid((unsigned)(rows_p / 32), (unsigned)((ksp / 8 + 31) / 32), 1);
-    scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks, nullptr);
+    scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks, GroupTableArgs{});
     return hipGetLastError();
   }
   if (src_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && ((uintptr_t)src & 3) == 0) {
@@ -354,19 +351,23 @@ hipError_t launch_scale_pair_shuffle_to_mfma32(const uint8_t *a_src, uint8_t *a_
 
 // Row-major -> MFMA32 for the scales of both GEMM operands in one launch.
 // Returns hipErrorInvalidValue (nothing launched) when the fast kernel does not apply.
-// With `a_tiles` (and room for a_tile_cap tiles of 256 rows in a_dst) A's scales are written per M tile of a
-// grouped GEMM, see the kernel.
+// With `table` the launch's first workgroup also builds the M tile table of a grouped GEMM, see the kernel.
+// One of a_rows, b_rows may be 0: the other tensor alone.
 hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
                                        uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream,
-                                       const int32_t *a_tiles, int64_t a_tile_cap) {
-  const int64_t a_rows_out = a_tiles ? a_tile_cap * 256 : a_rows;
-  const int64_t rows_max = a_rows_out > b_rows ? a_rows_out : b_rows;
+                                       const GroupTableArgs *table) {
+  if (a_rows == 0 && b_rows > 0) {  // B alone: as the launch's first tensor
+    a_src = b_src, a_dst = b_dst, a_rows = b_rows;
+    b_rows = 0;
+  }
+  const int64_t rows_max = a_rows > b_rows ? a_rows : b_rows;
   const int64_t rt = (rows_max + 31) / 32;
   if ((ks & 3) != 0 || ks == 0 || ((uintptr_t)a_src & 3) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 3) != 0) ||
       rows_max >= ((int64_t)1 << 31) || ((ks + 7) / 8 + 31) / 32 > 65535 || a_rows <= 0 || b_rows < 0)
     return hipErrorInvalidValue;
-  dim3 grid((unsigned)rt, (unsigned)(((ks + 7) / 8 + 31) / 32), b_rows > 0 ? 2 : 1);  // b_rows == 0: A alone
-  scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks, a_tiles);
+  dim3 grid((unsigned)rt, (unsigned)(((ks + 7) / 8 + 31) / 32), b_rows > 0 ? 2 : 1);
+  scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks,
+                                                   table ? *table : GroupTableArgs{});
   return hipGetLastError();
 }
 

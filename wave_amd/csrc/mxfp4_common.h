@@ -168,9 +168,16 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
                                 int64_t ks, hipStream_t stream);
 hipError_t launch_e8m0_shuffle(const uint8_t *scale, uint8_t *out, int64_t rows, int64_t ks,
                                hipStream_t stream);
+// What the builder of a grouped GEMM's M tile table takes (mxfp4_group_table.h); table == nullptr: none to build.
+struct GroupTableArgs {
+  const int32_t *offsets;
+  int num_groups, bm, total_rows;
+  int32_t *table;
+};
+// (with `table`, the launch's first workgroup also builds the M tile table of a grouped GEMM; a_rows == 0: B alone)
 hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
                                        uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream,
-                                       const int32_t *a_tiles = nullptr, int64_t a_tile_cap = 0);
+                                       const GroupTableArgs *table = nullptr);
 hipError_t launch_scale_pair_shuffle_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
                                                uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream);
 hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int64_t total_rows, int32_t *table,

@@ -42,7 +42,10 @@ enum KtKind {
 // store-free path and waits for the stores long before it must.
 // GROUPED: the M tiles come from a table (first row, rows, expert) built on the
 // device from the group offsets; a tile's rows past its group are computed and
-// dropped like rows past M, and A's scales are laid out per tile (8 blocks each).
+// dropped like rows past M.  A tile starts at any row, so a lane finds its row's
+// scales in block (first % 32 + row in tile) / 32 from the tile's first block, at
+// lane (first % 32 + row) % 32 of it: one dword per lane as before, from two
+// neighbouring blocks per wave instruction instead of one.
 // TAIL: K % 256 != 0.  The lanes whose 16-byte chunk lies past the end of K fetch
 // the last K tile from beyond the buffer descriptor (zeros land in LDS): their
 // offset gets its top bit flipped just before that tile's DMA is issued and
@@ -86,6 +89,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // nkt_of / part_of / tail_on: K tiles of the item, its slot in tail_partial (-1: a whole tile), and whether
   // its K range ends with the (partial) last K tile of the problem
   int m0[2], n0[2], a_lim[2], as_lim[2], b_lim[2], bs_lim[2], c_rows[2], nkt_of[2], part_of[2];
+  int a_row32[2] = {0, 0};  // grouped: the tile's first row inside its 32-row scale block
   bool tail_on[2];
   const int m_blocks = (p.m + 31) >> 5;
   const int b_kt_stride = p.b_preshuffled ? 2048 : B4 ? kTileKBytes / 2 : kTileKBytes;
@@ -132,8 +136,9 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       c_rows[which] = rows;
       b_base[which] = p.b + (int64_t)expert * p.b_group_stride + (int64_t)n0[which] * kp;
       bs_base[which] = p.b_scale + (int64_t)expert * p.b_scale_group_stride + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
-      as_base[which] = p.a_scale + (int64_t)tm * (BM / 32) * k_tiles_blocks;
-      as_lim[which] = (BM / 32) * k_tiles_blocks;
+      a_row32[which] = first & 31;
+      as_base[which] = p.a_scale + (int64_t)(first >> 5) * k_tiles_blocks;
+      as_lim[which] = (int)min((int64_t)(m_blocks - (first >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
     } else {
       m0[which] = tm * BM;
       c_rows[which] = p.m - m0[which];
@@ -248,9 +253,14 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   auto sblk = [](int kt) { return FP8 ? kt >> 1 : kt; };  // MXFP8: one MFMA32 block serves two K tiles
   auto load_scales = [&](int which, int kt) {
     const __amdgpu_buffer_rsrc_t ra = make_rsrc_n(as_base[which], as_lim[which]), rb = make_rsrc_n(bs_base[which], bs_lim[which]);
+    int a_lane = s_lane;
+    if constexpr (GROUPED) {
+      const int t = a_row32[which] + (lane & 31);
+      a_lane = ((t & 31) + (lane & 32)) * 4 + (t >> 5) * k_tiles_blocks;
+    }
 #pragma unroll
     for (int i = 0; i < MT_M; ++i)
-      raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, s_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256, 0);
+      raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256, 0);
 #pragma unroll
     for (int j = 0; j < MT_N; ++j)
       raw_b[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + sblk(kt) * 256, 0);
@@ -564,7 +574,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     if (!has_next) {
       m0[1] = m0[0], n0[1] = n0[0], a_lim[1] = a_lim[0], as_lim[1] = as_lim[0], c_rows[1] = c_rows[0];
       b_lim[1] = b_lim[0], bs_lim[1] = bs_lim[0];
-      nkt_of[1] = nkt_of[0], part_of[1] = part_of[0], tail_on[1] = tail_on[0];
+      nkt_of[1] = nkt_of[0], part_of[1] = part_of[0], tail_on[1] = tail_on[0], a_row32[1] = a_row32[0];
       a_base[1] = a_base[0], b_base[1] = b_base[0], as_base[1] = as_base[0], bs_base[1] = bs_base[0];
     }
     const int nk = SPLIT ? nkt_of[0] : nkt;  // K tiles of this item
@@ -603,7 +613,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     pid = npid;
     m0[0] = m0[1], n0[0] = n0[1], a_lim[0] = a_lim[1], as_lim[0] = as_lim[1], c_rows[0] = c_rows[1];
     b_lim[0] = b_lim[1], bs_lim[0] = bs_lim[1];
-    nkt_of[0] = nkt_of[1], part_of[0] = part_of[1], tail_on[0] = tail_on[1];
+    nkt_of[0] = nkt_of[1], part_of[0] = part_of[1], tail_on[0] = tail_on[1], a_row32[0] = a_row32[1];
     a_base[0] = a_base[1], b_base[0] = b_base[1], as_base[0] = as_base[1], bs_base[0] = bs_base[1];
     return true;
   };

@@ -5,6 +5,7 @@
 // sixteen waves does it in one launch (count, scan, place), everything but the
 // ids themselves in LDS.
 #include "mxfp4_common.h"
+#include "mxfp4_group_table.h"
 
 namespace wave_mxfp4 {
 
@@ -13,21 +14,6 @@ namespace {
 constexpr int kAlignWaves = 16;
 constexpr int kAlignThreads = kAlignWaves * 64;
 constexpr int kFewExperts = 16;
-
-// Inclusive sum over the workgroup's 1024 threads (one value each).
-__device__ __forceinline__ int block_inclusive_scan(int v, int *wave_sums, int lane, int wave) {
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int o = __shfl_up(v, d, 64);
-    if (lane >= d) v += o;
-  }
-  if (lane == 63) wave_sums[wave] = v;
-  __syncthreads();
-  int before = 0;
-  for (int w = 0; w < wave; ++w) before += wave_sums[w];
-  __syncthreads();
-  return v + before;
-}
 
 template <typename IdT>
 __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__restrict__ topk_ids, int n, int num_experts,
@@ -163,56 +149,18 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
   }
 }
 
-// M tile table of a grouped GEMM: group e's rows offsets[e] .. offsets[e+1]-1 cut into tiles of bm rows.
-// Entry 0 = {number of tiles}; entry 1 + t = {first row, rows, group, band}, in group order.
-// band = 16 * (first tile of the tile's band) + (tiles in the band): a group's tiles form bands of at most 8
-// (as equal as possible), the unit inside which the GEMM walks column by column, so that the tiles running
-// together share one expert's B panels.
-// The offsets are clamped, not validated: each group's range is cut to [0, total_rows] with end >= begin, and
-// tiles beyond the table's capacity (total_rows / bm + num_groups entries, enough for any non-decreasing offsets)
-// are dropped, so a malformed offsets array cannot make this kernel or the GEMM leave their buffers.
-__global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const int32_t *__restrict__ offsets,
-                                                                           int num_groups, int bm, int total_rows,
-                                                                           int32_t *__restrict__ table) {
-  const int cap = total_rows / bm + num_groups;
+// The M tile table of a grouped GEMM (mxfp4_group_table.h) by a launch of its own.
+__global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const GroupTableArgs g) {
   __shared__ int wave_sums[kAlignWaves];
   __shared__ int carry;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  if (t == 0) carry = 0;
-  __syncthreads();
-  for (int e0 = 0; e0 < num_groups; e0 += kAlignThreads) {
-    const int e = e0 + t;
-    int lo = 0, tiles = 0, hi = 0;
-    if (e < num_groups) {
-      lo = min(max(offsets[e], 0), total_rows), hi = min(max(offsets[e + 1], lo), total_rows);
-      tiles = hi > lo ? (hi - lo + bm - 1) / bm : 0;
-    }
-    const int base = carry;  // read before anyone moves it on
-    const int end = block_inclusive_scan(tiles, wave_sums, lane, wave);
-    const int nb = (tiles + 7) >> 3;  // bands of the group: `rem` of height hb + 1, then the rest of height hb
-    const int hb = nb ? tiles / nb : 0, rem = nb ? tiles - hb * nb : 0;
-    const int first_tile = base + end - tiles;
-    for (int i = 0; i < tiles && first_tile + i < cap; ++i) {
-      int32_t *ent = table + 4 * (1 + first_tile + i);
-      ent[0] = lo + i * bm;
-      ent[1] = min(bm, hi - lo - i * bm);
-      ent[2] = e;
-      const int tall = rem * (hb + 1);
-      const int start = i < tall ? i / (hb + 1) * (hb + 1) : tall + (i - tall) / hb * hb;
-      ent[3] = 16 * (first_tile + start) + (i < tall ? hb + 1 : hb);
-    }
-    __syncthreads();
-    if (t == kAlignThreads - 1) carry = base + end;
-    __syncthreads();
-  }
-  if (t == 0) table[0] = min(carry, cap);
+  build_group_tile_table<kAlignThreads>(g, wave_sums, &carry);
 }
 
 }  // namespace
 
 hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int64_t total_rows, int32_t *table,
                                      hipStream_t stream) {
-  grouped_tile_table_kernel<<<1, kAlignThreads, 0, stream>>>(offsets, num_groups, bm, (int)total_rows, table);
+  grouped_tile_table_kernel<<<1, kAlignThreads, 0, stream>>>(GroupTableArgs{offsets, num_groups, bm, (int)total_rows, table});
   return hipGetLastError();
 }
 

@@ -518,9 +518,12 @@ hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
 
 // Columns per compute wave: the narrowest strips (a multiple of 4 columns, 16 to 32) that still fit the number of
 // rounds which strips of 128 columns would take on this many CUs.  B scales in MFMA32 order come in blocks of 32
-// rows, so there a wave's strip is a block.
+// rows, so there a wave's strip is a block.  From 97 rows on a workgroup's time is mostly its copy of A (every
+// workgroup reads all of it), so fewer, wider strips win even where they leave CUs idle (128 x 28672 x 8192 with
+// row-major scales: 31.4 -> 29.8 us, 192 rows 39.9 -> 38.3 us; at 96 rows the narrow strips are still as good).
 int mid_wave_cols(const GemmParams &p, int num_cus) {
   if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR || num_cus <= 0) return 32;
+  if (p.num_groups == 0 && p.m > 96) return 32;
   const int64_t experts = p.num_groups != 0 ? p.num_groups : 1;
   const int64_t strips = (p.n + kMidBN - 1) / kMidBN * experts;
   const int64_t wgs = (strips + num_cus - 1) / num_cus * num_cus;   // whole rounds of the CUs

@@ -96,6 +96,29 @@ def test_quantize_feeds_the_gemm_and_shuffle_flag():
     assert np.abs(got - dense).max() <= 0.2 * np.abs(dense).max()
 
 
+@pytest.mark.parametrize("layout", [_lib.SCALE_ROW_MAJOR, _lib.SCALE_E8M0_SHUFFLE, _lib.SCALE_MFMA32])
+@pytest.mark.parametrize("m", [24, 100])
+def test_quantize_feeds_the_decode_kernel_without_a_pass_between(m, layout):
+    """A decode step: activations quantised on the device in each scale order, weights with resident scales in the
+    same order, and the mid-M kernel with no scratch (so nothing can re-lay the scales out in between): the oracle's
+    GEMM of the oracle's quantised operands."""
+    n, k = 4096, 2048
+    a, af = make_x(m, k, 3, "bf16", spread=2.0)
+    b, bf = make_x(n, k, 4, "bf16", spread=2.0)
+    aq, asc = wave_amd.quantize_mxfp4(a, scale_layout=layout)
+    bq, bsc = wave_amd.quantize_mxfp4(b, scale_layout=layout)
+    out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm(aq, asc, bq, bsc, out, a_scale_layout=layout, b_scale_layout=layout,
+                        variant=_lib.VARIANT_MID_M, split_k=1, workspace=False)
+    torch.cuda.synchronize()
+    oa, osa = qo.quantize_mxfp4(af)
+    ob, osb = qo.quantize_mxfp4(bf)
+    cols = np.arange(0, n, 7)
+    ref = orc.scaled_gemm_exact(oa, ob[cols], osa, osb[cols])
+    got = out.cpu().numpy().astype(np.float64)[:, cols]
+    assert np.abs(got - ref).max() <= 2e-6 * np.abs(ref).max()
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_quantize_full_size_properties(dtype):
     """8192 x 8192 (the benchmark's activation): no oracle pass over 64M

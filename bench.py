@@ -411,7 +411,7 @@ def main():
                     "time-based settle load every leg runs anyway)")
     ap.add_argument("--workload", default="cfg2",
                     choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue", "ref_shapes", "mfma_ceiling",
-                                                 "decode_sweep", "moe_serving"],
+                                                 "decode_sweep", "moe_serving", "moe_layer"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
                          "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out; "
                          "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096; moe_glue: the steps around "
@@ -420,7 +420,8 @@ def main():
                          "random operands against zeros (the power-limited ceiling of the matrix pipes); decode_sweep: "
                          "M = 1 .. 256 against wide weights from HBM, every kernel that serves the shape beside the "
                          "library's own choice; moe_serving: the grouped GEMM at serving batches, experts x rows per "
-                         "expert, the mid-M kernel beside the tile kernels")
+                         "expert, the mid-M kernel beside the tile kernels; moe_layer: one mixture-of-experts MLP end to end "
+                         "(alignment, gathered quantiser, grouped GEMM, gated quantiser, grouped GEMM), step by step and whole")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-legs", "--no-decode", dest="no_legs", action="store_true",
@@ -698,6 +699,80 @@ def main():
             "moe_align_block_size_us": round(t_align * 1e6, 2),
             "gathered_quantiser": {"launch_us": round(t_gather * 1e6, 2), "gbps": round(b_gather / t_gather / 1e9, 1),
                                    "bytes": b_gather}})))
+        return
+
+    if args.workload == "moe_layer":
+        # One mixture-of-experts MLP, the path of tests/kernel/moe_test.py:113-246 without its final weighted sum:
+        # routing table -> token alignment -> gathered quantiser -> grouped GEMM (gate and up projections) ->
+        # gated activation fused into the quantiser -> grouped GEMM (down projection).  Every scale tensor is
+        # written or kept in MFMA32 order, so no re-layout launch sits between the steps.
+        from wave_amd import _lib as L
+
+        tokens, topk, E, hidden, inter = 4096, 2, 8, 4096, 14336
+        M32 = L.SCALE_MFMA32
+        g = torch.Generator(device=dev).manual_seed(3)
+        ids = torch.stack([torch.randperm(E, device=dev, generator=g)[:topk] for _ in range(tokens)]).to(torch.int32)
+        n_ent = tokens * topk
+        sorted_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
+        expert_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
+        total = torch.empty(1, dtype=torch.int32, device=dev)
+        offs = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        act = torch.randn(tokens, hidden, device=dev, generator=g).to(torch.bfloat16)
+
+        def weights(n, k):
+            w = torch.randint(0, 256, (E, n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+            ws = torch.randint(120, 131, (E, n, k // 32), dtype=torch.uint8, device=dev, generator=g)
+            return w, torch.stack([wave_amd.scale_convert(ws[e], n, k // 32, L.SCALE_ROW_MAJOR, M32) for e in range(E)])
+
+        w1, w1s = weights(2 * inter, hidden)
+        w2, w2s = weights(hidden, inter)
+        h1 = torch.empty(n_ent, 2 * inter, dtype=torch.bfloat16, device=dev)
+        out = torch.empty(n_ent, hidden, dtype=torch.bfloat16, device=dev)
+        state = {}
+
+        def step_align():
+            wave_amd.moe_align_block_size(ids, E, 1, sorted_ids, expert_ids, total, offs)
+
+        def step_gather():
+            state["q1"], state["s1"] = wave_amd.quantize_mxfp4_rows(act, sorted_ids, topk, scale_layout=M32)
+
+        def step_gemm1():
+            wave_amd.mxfp4_gemm_grouped(state["q1"], state["s1"], w1, w1s, offs, h1, a_scale_layout=M32, b_scale_layout=M32)
+
+        def step_act():
+            state["q2"], state["s2"] = wave_amd.silu_and_mul_quantize(h1[:, :inter], h1[:, inter:], scale_layout=M32)
+
+        def step_gemm2():
+            wave_amd.mxfp4_gemm_grouped(state["q2"], state["s2"], w2, w2s, offs, out, a_scale_layout=M32, b_scale_layout=M32)
+
+        steps = [("moe_align_block_size", step_align), ("gathered_quantiser", step_gather), ("grouped_gemm_gate_up", step_gemm1),
+                 ("gated_activation_quantiser", step_act), ("grouped_gemm_down", step_gemm2)]
+
+        def layer(count):
+            for _ in range(count):
+                for _, fn in steps:
+                    fn()
+
+        layer(1)
+        torch.cuda.synchronize()
+        _, per_layer, _ = timed(torch, layer, args.steps, args.warmup)
+        each = {}
+        for name, fn in steps:
+            def run(count, fn=fn):
+                for _ in range(count):
+                    fn()
+            each[name] = round(timed(torch, run, args.steps, args.warmup)[1] * 1e6, 2)
+        flops = 2.0 * n_ent * (2 * inter) * hidden + 2.0 * n_ent * hidden * inter
+        tfl = flops / per_layer / 1e12
+        print(json.dumps(dict(common, **{
+            "metric": "MoE expert MLP (align, gather + quantise, grouped GEMM, gated quantiser, grouped GEMM) TFLOPS",
+            "value": round(tfl, 1), "unit": "TFLOP/s", "ms_per_step": round(per_layer * 1e3, 4),
+            "dtype": "bf16 activations, mxfp4 operands, f32 accumulate, bf16 out", "data": "synthetic (normal activations, uniform weights)",
+            "config": {"workload": f"moe_layer: {tokens} tokens x top-{topk} of {E} experts, hidden {hidden}, intermediate {inter}"},
+            "roofline": {"bound": "mfma", "achieved": round(tfl, 1), "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tfl / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "persist_gemm_kernel (grouped)",
+                         "launch_us": round(per_layer * 1e6, 2)},
+            "steps_us": each, "sum_of_steps_us": round(sum(each.values()), 2)})))
         return
 
     if args.workload == "cfg4":

@@ -127,6 +127,77 @@ def test_gathered_quantiser_and_grouped_gemm_pipeline(dtype):
     assert np.abs(got - ref).max() <= 2e-6 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("size", ["serving", "prefill"])
+def test_expert_mlp_chain_with_resident_scale_layouts(size):
+    """One mixture-of-experts MLP (the path of tests/kernel/moe_test.py:113-246 up to its weighted sum): alignment
+    -> gathered quantiser -> grouped GEMM (gate and up) -> gated activation fused into the quantiser -> grouped
+    GEMM (down), every scale tensor written or kept in MFMA32 order so that no re-layout launch sits between the
+    steps.  Each step against the oracle applied to the device's output of the step before: bytes exact for the
+    quantisers, the GEMMs within the bf16 bound.  "serving": a few rows per expert (mid-M kernel); "prefill": more
+    256x256 tiles than CUs (table-driven persistent kernel, groups starting at rows that are no multiples of 32)."""
+    tokens, topk, experts, hidden, inter = (40, 2, 8, 1024, 2048) if size == "serving" else (2600, 2, 4, 1024, 2048)
+    m32 = _lib.SCALE_MFMA32
+    rng = np.random.default_rng(31)
+    ids = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)])
+    act = torch.from_numpy(rng.standard_normal((tokens, hidden)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    sorted_ids, _, total, offsets = run_align(torch.from_numpy(ids).to(DEV), experts, 1, extra=0)
+    rows = tokens * topk
+    assert int(total[0]) == rows and any(int(o) % 32 for o in offsets[1:-1])
+    g_sorted, g_off = torch.from_numpy(sorted_ids).to(DEV), torch.from_numpy(offsets).to(DEV)
+
+    def weights(n, k, seed):
+        r = np.random.default_rng(seed)
+        w = r.integers(0, 256, size=(experts, n, k // 2), dtype=np.uint8)
+        ws = r.integers(118, 130, size=(experts, n, k // 32), dtype=np.uint8)
+        gws = torch.stack([wave_amd.scale_convert(torch.from_numpy(ws[e]).to(DEV), n, k // 32, _lib.SCALE_ROW_MAJOR, m32)
+                           for e in range(experts)])
+        return w, ws, torch.from_numpy(w).to(DEV), gws
+
+    w1, w1s, gw1, gw1s = weights(2 * inter, hidden, 1)
+    w2, w2s, gw2, gw2s = weights(hidden, inter, 2)
+    # gathered quantiser, scales straight into MFMA32 order
+    q1, s1 = wave_amd.quantize_mxfp4_rows(act, g_sorted, topk, scale_layout=m32)
+    want_q1, want_s1 = qo.quantize_mxfp4(act.float().cpu().numpy()[sorted_ids // topk])
+    assert np.array_equal(q1.cpu().numpy(), want_q1)
+    s1_rm = wave_amd.scale_convert(s1, rows, hidden // 32, m32, _lib.SCALE_ROW_MAJOR).cpu().numpy()
+    assert np.array_equal(s1_rm, want_s1)
+    # gate and up projections
+    h1 = torch.full((rows, 2 * inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(q1, s1, gw1, gw1s, g_off, h1, a_scale_layout=m32, b_scale_layout=m32)
+    torch.cuda.synchronize()
+    pick = np.unique(np.concatenate([np.arange(0, rows, max(1, rows // 40)), offsets[1:-1] - 1, offsets[1:-1] % rows, [rows - 1]]))
+    h1_host = h1.float().cpu().numpy()
+    for e in range(experts):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        sel = pick[(pick >= lo) & (pick < hi)]
+        if len(sel):
+            ref = c_oracle.scaled_gemm_exact(want_q1, w1[e], want_s1, w1s[e], rows=sel)
+            tol = 2.0 ** -7 * np.abs(ref).max()
+            assert np.abs(h1_host[sel] - ref).max() <= tol, f"gate/up, expert {e}"
+    assert not np.isnan(h1_host).any()
+    # gated activation + quantiser on the device's own h1
+    q2, s2 = wave_amd.silu_and_mul_quantize(h1[:, :inter], h1[:, inter:], scale_layout=m32)
+    stored = wave_amd.silu_and_mul(h1[:, :inter], h1[:, inter:])
+    want_q2, want_s2 = qo.quantize_mxfp4(stored.float().cpu().numpy())
+    assert np.array_equal(q2.cpu().numpy(), want_q2)
+    assert np.array_equal(wave_amd.scale_convert(s2, rows, inter // 32, m32, _lib.SCALE_ROW_MAJOR).cpu().numpy(), want_s2)
+    ref_act = mo.silu_and_mul(h1_host[:, :inter], h1_host[:, inter:])
+    got_act = stored.float().cpu().numpy().astype(np.float64)
+    assert np.abs(got_act - ref_act).max() <= 2.0 ** -7 * max(1.0, np.abs(ref_act).max())
+    # down projection
+    out = torch.full((rows, hidden), float("nan"), dtype=torch.bfloat16, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(q2, s2, gw2, gw2s, g_off, out, a_scale_layout=m32, b_scale_layout=m32)
+    torch.cuda.synchronize()
+    out_host = out.float().cpu().numpy()
+    for e in range(experts):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        sel = pick[(pick >= lo) & (pick < hi)]
+        if len(sel):
+            ref = c_oracle.scaled_gemm_exact(want_q2, w2[e], want_s2, w2s[e], rows=sel)
+            assert np.abs(out_host[sel] - ref).max() <= 2.0 ** -7 * np.abs(ref).max(), f"down, expert {e}"
+    assert not np.isnan(out_host).any()
+
+
 def test_moe_glue_argument_errors():
     lib = _lib.load()
     P = 0x1000

@@ -283,6 +283,35 @@ def test_grouped_persistent_path_scale_layouts_and_ragged_starts(la, lb):
         assert_f32_close(c[pick], ref, f"expert {g} {la}/{lb}")
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("e,n,k,rows", [(4, 2048, 14336, 9300), (8, 4096, 2048, 4200), (3, 1024, 8192, 16600)])
+def test_grouped_persistent_path_sparse_last_round_cut_along_k(e, n, k, rows, dt):
+    """A few rounds of tiles of which the last gives less than half of the workgroups one (296-320 tiles of 256x256
+    on 256 CUs and the like): its tiles are cut along K over the idle workgroups, the f32 parts summed by a second
+    launch; whether and how is decided on the device, where the tile count is known (56 and 32 K tiles: 3 and 8
+    parts; 8 K tiles: too short to pay, the tiles stay whole).  Rows of every tile against the oracle, every element against the one-tile-per-workgroup kernel, rows past the last offset untouched."""
+    x, xs, w, ws, off = grouped_inputs(e, n, k, rows, seed=e * 5 + 1)
+    tiles = int(sum((int(off[g + 1]) - int(off[g]) + 255) // 256 for g in range(e))) * (n // 256)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert tiles > cus and 0 < tiles % cus <= cus // 2, "the case is meant to leave a sparse last round"
+    gx, gxs, gw, gws, goff = to_gpu(x, xs, w, ws, off)
+    out = torch.full((rows + 2, n), float("nan"), dtype=dt, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out[:rows], variant=_lib.VARIANT_T256x256_W4x2)
+    torch.cuda.synchronize()
+    c = out.float().cpu().numpy()
+    assert np.isnan(c[rows:]).all() and not np.isnan(c[:rows]).any()
+    for g in range(e):
+        lo, hi = int(off[g]), int(off[g + 1])
+        pick = np.unique(np.concatenate([np.arange(lo, hi, 97), np.arange(lo, hi, 256), np.arange(lo + 255, hi, 256), [hi - 1]]))
+        ref = c_oracle.scaled_gemm_exact(x, w[g], xs, ws[g], rows=pick)
+        assert_close(c[pick], ref, dt, f"expert {g}")
+    other = torch.full((rows, n), float("nan"), dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, other, variant=_lib.VARIANT_T128x128_W2x2, workspace=False)
+    torch.cuda.synchronize()
+    o = other.cpu().numpy()
+    assert np.abs(c[:rows] - o).max() <= (4e-6 if dt == torch.float32 else 2.0 ** -7) * np.abs(o).max()
+
+
 def torch_seeded_inputs(m, n, k, seed, scale_lo, scale_hi):
     """The configuration's operands drawn the way the reference draws its own (torch.manual_seed(seed), then the
     draw order of wave_lang/kernel/wave/utils/mxfp_utils.py:37-57 through the host mirror's generator), on the CPU

@@ -563,11 +563,21 @@ static size_t grouped_table_bytes(int64_t total_rows, int num_groups) {
   return round_up_256((size_t)(1 + total_rows / 256 + num_groups) * 16);
 }
 static size_t grouped_a_scale_bytes(int64_t total_rows, int64_t k) { return round_up_256(scale_buffer_bytes(total_rows, k)); }
+// f32 parts of the tiles of a sparsely filled last round, cut along K (persistent kernel).  Only problems of at
+// most four rounds of 256x256 tiles get the room: there the round is a tenth of the call or more, and beyond, the
+// launch that sums the parts (which a grouped call cannot know to skip: the tile count is on the device) costs
+// more often than the cut pays.  One part per workgroup at most: a 256x256 f32 tile each.
+static size_t grouped_tail_bytes(int64_t total_rows, int64_t n, int64_t k, int num_groups) {
+  const int64_t grid = device_cus() / 8 * 8;
+  const int64_t tiles = (total_rows / 256 + num_groups) * (n / 256);
+  if (n % 256 != 0 || k / kTileK < 8 || grid <= 0 || tiles > 4 * grid) return 0;
+  return (size_t)grid * 256 * 256 * sizeof(float);
+}
 
 size_t wave_mxfp4_grouped_workspace_bytes(int64_t total_rows, int64_t n, int64_t k, int num_groups) {
   if (total_rows <= 0 || n <= 0 || k <= 0 || num_groups <= 0 || k % kTileK != 0 || n % 32 != 0) return 0;
   return grouped_table_bytes(total_rows, num_groups) + grouped_a_scale_bytes(total_rows, k) +
-         round_up_256((size_t)num_groups * scale_buffer_bytes(n, k));
+         round_up_256((size_t)num_groups * scale_buffer_bytes(n, k)) + grouped_tail_bytes(total_rows, n, k, num_groups);
 }
 
 int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, const void *b_scale,
@@ -660,6 +670,8 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
         if (!a_native) q.a_scale = ws_a;
         if (!b_native) q.b_scale = ws_b;
         q.b_scale_group_stride = n * (int64_t)p.ksp;
+        if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && grouped_tail_bytes(total_rows, n, k, num_groups) != 0)
+          q.tail_partial = (float *)(ws_b + round_up_256((size_t)num_groups * scale_buffer_bytes(n, k)));
         return record_hip(launch_persist_gemm(q, v, device_cus(), stream));
       }
       // (the fast re-layout does not apply and has launched nothing: on to the one-tile-per-workgroup kernel)

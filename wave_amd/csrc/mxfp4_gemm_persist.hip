@@ -29,6 +29,37 @@
 
 namespace wave_mxfp4 {
 
+// Into how many parts along K the tiles of a sparsely filled last round are cut (1 = left whole): `rest` tile ids
+// in that round on `grid` workgroups, tiles of `k_tiles` K tiles.  Cost of the last round in us: a tile's K tiles
+// at the measured 1.85 us each, divided among the parts, plus writing and re-reading the f32 parts (about 4 TB/s)
+// and the launch of the kernel that sums them.  Host code for dense problems; a grouped problem's tile count is
+// only known on the device, where the GEMM and the summing kernel both evaluate this.
+__host__ __device__ inline int tail_parts_rule(int rest, int grid, int k_tiles) {
+  if (rest <= 0 || rest * 2 > grid) return 1;
+  const float tile_us = 1.85f * (float)k_tiles;
+  int parts = 1;
+  float best = tile_us;
+  for (int c = 2; c <= 8 && c * rest <= grid && k_tiles / c >= 4; ++c) {
+    const float us = tile_us / (float)c + 2.0f * (float)rest * (float)c * (256.0f * 256.0f * 4.0f) / 4.0e6f + 6.0f;
+    if (us < best * 0.9f) best = us, parts = c;
+  }
+  return parts;
+}
+
+// Tile id -> (M tile, N tile) of a grouped problem: the same XCD regrouping as map_tile, but the bands the sequence
+// walks column by column are the table's (at most 8 tiles of one expert), not fixed runs of 8 tile rows.
+__device__ __forceinline__ bool map_grouped_tile(const int32_t *table, int total, int tiles_n, int id, int &tm, int &tn) {
+  const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
+  const int seq = (id % kNumXcd) * per_xcd + id / kNumXcd;
+  if (seq >= total) return false;
+  const int band = __builtin_amdgcn_readfirstlane(table[4 * (1 + seq / tiles_n) + 3]);
+  const int start = band >> 4, height = band & 15;
+  const int in_band = seq - start * tiles_n;
+  tn = in_band / height;
+  tm = start + in_band - tn * height;
+  return true;
+}
+
 enum KtKind {
   kSteadyTail = 4,  // kSteady whose K tile j+2 is a partial last K tile (TAIL kernels: j = nkt - 3)
   kSteady = 0,  // K tiles j+1, j+2 belong to this output tile
@@ -55,7 +86,9 @@ enum KtKind {
 // get one of, are cut along K into p.tail_parts parts instead, one part per
 // workgroup (its last item); the parts go to p.tail_partial as f32 tiles and a
 // small kernel adds them up.  A 288-tile problem on 256 CUs then takes 1 + 1/8
-// tile times instead of 2.
+// tile times instead of 2.  For a grouped problem the number of parts is worked
+// out on the device (tail_parts_rule on the table's tile count), by this kernel
+// and by the one that sums, and may come out as 1: then the tiles stay whole.
 // FMT_A / FMT_B: element format codes of the scaled MFMA, 4 = e2m1 (MXFP4); 0 = e4m3, 1 = e5m2 (MXFP8, both
 // operands 8-bit: a 128-byte K tile is then 128 elements = two 64-deep K steps of 32 bytes per lane, the MFMA
 // takes 64 cycles instead of 32, and one MFMA32 scale block serves two K tiles; dense, whole K tiles, no cut).
@@ -93,36 +126,29 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   bool tail_on[2];
   const int m_blocks = (p.m + 31) >> 5;
   const int b_kt_stride = p.b_preshuffled ? 2048 : B4 ? kTileKBytes / 2 : kTileKBytes;
-  static_assert(!(GROUPED && SPLIT), "the K cut of the last round is for dense problems");
-  // Grouped: the same XCD regrouping as map_tile, but the bands the sequence walks column by column are the
-  // table's (at most 8 tiles of one expert), not fixed runs of 8 tile rows.
   auto map_grouped = [&](int id, int &tm, int &tn) -> bool {
-    const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
-    const int seq = (id % kNumXcd) * per_xcd + id / kNumXcd;
-    if (seq >= total) return false;
-    const int band = __builtin_amdgcn_readfirstlane(p.tile_table[4 * (1 + seq / p.tiles_n) + 3]);
-    const int start = band >> 4, height = band & 15;
-    const int in_band = seq - start * p.tiles_n;
-    tn = in_band / height;
-    tm = start + in_band - tn * height;
-    return true;
+    return map_grouped_tile(p.tile_table, total, p.tiles_n, id, tm, tn);
   };
+  // (grouped: the tile count, and with it whether the last round is cut, is only known here)
+  const int tail_parts = !SPLIT ? 1
+                         : GROUPED ? tail_parts_rule(padded - total / (int)gridDim.x * (int)gridDim.x, (int)gridDim.x, nkt)
+                                   : p.tail_parts;
   auto set_tile = [&](int which, int pid) -> bool {
     int tm, tn, kt_lo = 0;
     nkt_of[which] = nkt;
     part_of[which] = -1;
-    if (SPLIT && pid >= total / (int)gridDim.x * (int)gridDim.x) {
+    if (SPLIT && tail_parts > 1 && pid >= total / (int)gridDim.x * (int)gridDim.x) {
       // the last round: workgroup w takes part w % parts of tile (whole rounds) + w / parts
       const int whole = total / (int)gridDim.x * (int)gridDim.x, w = pid - whole;
       if (w >= (int)gridDim.x) return false;
-      const int r = w / p.tail_parts, i = w - r * p.tail_parts;
+      const int r = w / tail_parts, i = w - r * tail_parts;
       if (whole + r >= padded) return false;  // (ids up to `padded`: map_tile skips the padding ids among them)
       pid = whole + r;
-      const int base = nkt / p.tail_parts, rem = nkt - base * p.tail_parts;
+      const int base = nkt / tail_parts, rem = nkt - base * tail_parts;
       nkt_of[which] = base + (i < rem ? 1 : 0);
       kt_lo = i * base + min(i, rem);
-      part_of[which] = r * p.tail_parts + i;
-      if (!map_tile(pid, tiles_m, p.tiles_n, tm, tn)) return false;
+      part_of[which] = r * tail_parts + i;
+      if (!(GROUPED ? map_grouped(pid, tm, tn) : map_tile(pid, tiles_m, p.tiles_n, tm, tn))) return false;
     } else if (pid >= padded || !(GROUPED ? map_grouped(pid, tm, tn) : map_tile(pid, tiles_m, p.tiles_n, tm, tn))) {
       return false;
     }
@@ -637,21 +663,33 @@ __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_fp8_kernel(const Gemm
 }
 
 // Adds up the parts of the tiles of the last round (SPLIT) and writes them to C: one workgroup per 32 rows of a
-// tile, a thread per 4 columns and row.
-template <class Cfg>
+// tile, a thread per 4 columns and row.  Grouped: launched for the most tile ids a cut round can have; how many
+// there are, and whether the round was cut at all, follows from the table's tile count as in the GEMM.
+template <class Cfg, bool GROUPED>
 __global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams p, int grid_main) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
-  const int total = p.tiles_m * p.tiles_n, whole = total / grid_main * grid_main;
+  const int tiles_m = GROUPED ? p.tile_table[0] : p.tiles_m;
+  const int total = tiles_m * p.tiles_n, whole = total / grid_main * grid_main;
+  const int padded = (total + kNumXcd - 1) / kNumXcd * kNumXcd;
+  const int parts = GROUPED ? tail_parts_rule(padded - whole, grid_main, p.k_tiles) : p.tail_parts;
   const int r = blockIdx.x / (BM / 32), band = blockIdx.x % (BM / 32);
+  if (GROUPED && (parts <= 1 || whole + r >= padded)) return;
   int tm, tn;
-  if (!map_tile(whole + r, p.tiles_m, p.tiles_n, tm, tn)) return;  // a padding id
-  const float *part = p.tail_partial + (int64_t)r * p.tail_parts * BM * BN;
+  if (!(GROUPED ? map_grouped_tile(p.tile_table, total, p.tiles_n, whole + r, tm, tn)
+                : map_tile(whole + r, p.tiles_m, p.tiles_n, tm, tn)))
+    return;  // a padding id
+  int m_first = tm * BM, m_end = p.m;
+  if (GROUPED) {  // the tile's rows: its group's, from the table
+    m_first = p.tile_table[4 * (1 + tm)];
+    m_end = m_first + p.tile_table[4 * (1 + tm) + 1];
+  }
+  const float *part = p.tail_partial + (int64_t)r * parts * BM * BN;
   for (int e = threadIdx.x; e < 32 * BN / 4; e += 256) {
     const int row = band * 32 + e / (BN / 4), col = (e % (BN / 4)) * 4;
-    const int m = tm * BM + row, n = tn * BN + col;
-    if (m >= p.m) continue;
+    const int m = m_first + row, n = tn * BN + col;
+    if (m >= m_end) continue;
     v4f sum = *(const v4f *)(part + (int64_t)row * BN + col);
-    for (int i = 1; i < p.tail_parts; ++i) sum += *(const v4f *)(part + ((int64_t)i * BM + row) * BN + col);
+    for (int i = 1; i < parts; ++i) sum += *(const v4f *)(part + ((int64_t)i * BM + row) * BN + col);
     if (p.out_bf16) {
       typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
       *(bf4 *)((__bf16 *)p.c + (int64_t)m * p.n + n) = bf4{(__bf16)sum.x, (__bf16)sum.y, (__bf16)sum.z, (__bf16)sum.w};
@@ -672,8 +710,9 @@ static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_
   e = hipGetLastError();
   if (SPLIT && e == hipSuccess) {
     const int total = p.tiles_m * p.tiles_n;
-    const int ids = (total + kNumXcd - 1) / kNumXcd * kNumXcd - total / grid_x * grid_x;  // tile ids of the last round
-    persist_tail_sum_kernel<Cfg><<<dim3(ids * (Cfg::BM / 32)), 256, 0, stream>>>(p, grid_x);
+    // tile ids of the last round (grouped: the most a round that is cut can have, the kernel knows how many there are)
+    const int ids = GROUPED ? grid_x / 2 : (total + kNumXcd - 1) / kNumXcd * kNumXcd - total / grid_x * grid_x;
+    persist_tail_sum_kernel<Cfg, GROUPED><<<dim3(ids * (Cfg::BM / 32)), 256, 0, stream>>>(p, grid_x);
     e = hipGetLastError();
   }
   return e;
@@ -693,9 +732,15 @@ static hipError_t launch_persist_dense(const GemmParams &p, int grid_x, hipStrea
 
 template <class Cfg>
 static hipError_t launch_persist_cfg(const GemmParams &p, int grid_x, hipStream_t stream) {
-  if (p.tile_table != nullptr)
+  if (p.tile_table != nullptr) {
+    if constexpr (Cfg::NWAVES == 8 && Cfg::BN == 256) {
+      if (p.tail_partial != nullptr)  // few rounds: a sparsely filled last one is cut along K (decided on the device)
+        return p.out_bf16 ? launch_persist_out<Cfg, true, true, false, true>(p, grid_x, stream)
+                          : launch_persist_out<Cfg, false, true, false, true>(p, grid_x, stream);
+    }
     return p.out_bf16 ? launch_persist_out<Cfg, true, true, false, false>(p, grid_x, stream)
                       : launch_persist_out<Cfg, false, true, false, false>(p, grid_x, stream);
+  }
   return p.out_bf16 ? launch_persist_dense<Cfg, true>(p, grid_x, stream) : launch_persist_dense<Cfg, false>(p, grid_x, stream);
 }
 
@@ -712,15 +757,7 @@ int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *pa
   // tile ids of the last round, the XCD padding ids among them included (they get a slot and stay unused)
   const int rest = (int)((total + kNumXcd - 1) / kNumXcd * kNumXcd - total / grid * grid);
   if (rest * 2 > grid) return 1;
-  // Cost of the last round in us: a tile's K tiles at the measured 1.85 us each, divided among the parts, plus
-  // writing and re-reading the f32 parts (about 4 TB/s) and the launch of the kernel that sums them.
-  const double tile_us = 1.85 * p.k_tiles;
-  int parts = 1;
-  double best = tile_us;
-  for (int c = 2; c <= 8 && c * rest <= grid && p.k_tiles / c >= 4; ++c) {
-    const double us = tile_us / c + 2.0 * rest * c * (256 * 256 * 4) / 4.0e6 + 6.0;
-    if (us < best * 0.9) best = us, parts = c;
-  }
+  const int parts = tail_parts_rule(rest, grid, p.k_tiles);
   if (parts > 1) *partial_bytes = (size_t)rest * parts * 256 * 256 * sizeof(float);
   return parts;
 }

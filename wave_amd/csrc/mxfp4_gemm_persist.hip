@@ -662,9 +662,11 @@ __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_fp8_kernel(const Gemm
   persist_body<Cfg, OUT_BF16, false, false, false, FMT_A, FMT_B>(p);
 }
 
-// Adds up the parts of the tiles of the last round (SPLIT) and writes them to C: one workgroup per 32 rows of a
-// tile, a thread per 4 columns and row.  Grouped: launched for the most tile ids a cut round can have; how many
+// Adds up the parts of the tiles of the last round (SPLIT) and writes them to C: one workgroup per 8 rows of a
+// tile, a thread per 4 columns and row (two of them: with 32 rows per workgroup the loads of a thread's eight
+// turns came one after the other, 11.5 us for 64 tiles of 3 parts).  Grouped: launched for the most tile ids a cut round can have; how many
 // there are, and whether the round was cut at all, follows from the table's tile count as in the GEMM.
+constexpr int kSumRows = 8;
 template <class Cfg, bool GROUPED>
 __global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams p, int grid_main) {
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
@@ -672,7 +674,7 @@ __global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams 
   const int total = tiles_m * p.tiles_n, whole = total / grid_main * grid_main;
   const int padded = (total + kNumXcd - 1) / kNumXcd * kNumXcd;
   const int parts = GROUPED ? tail_parts_rule(padded - whole, grid_main, p.k_tiles) : p.tail_parts;
-  const int r = blockIdx.x / (BM / 32), band = blockIdx.x % (BM / 32);
+  const int r = blockIdx.x / (BM / kSumRows), band = blockIdx.x % (BM / kSumRows);
   if (GROUPED && (parts <= 1 || whole + r >= padded)) return;
   int tm, tn;
   if (!(GROUPED ? map_grouped_tile(p.tile_table, total, p.tiles_n, whole + r, tm, tn)
@@ -684,8 +686,8 @@ __global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams 
     m_end = m_first + p.tile_table[4 * (1 + tm) + 1];
   }
   const float *part = p.tail_partial + (int64_t)r * parts * BM * BN;
-  for (int e = threadIdx.x; e < 32 * BN / 4; e += 256) {
-    const int row = band * 32 + e / (BN / 4), col = (e % (BN / 4)) * 4;
+  for (int e = threadIdx.x; e < kSumRows * BN / 4; e += 256) {
+    const int row = band * kSumRows + e / (BN / 4), col = (e % (BN / 4)) * 4;
     const int m = m_first + row, n = tn * BN + col;
     if (m >= m_end) continue;
     v4f sum = *(const v4f *)(part + (int64_t)row * BN + col);
@@ -712,7 +714,7 @@ static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_
     const int total = p.tiles_m * p.tiles_n;
     // tile ids of the last round (grouped: the most a round that is cut can have, the kernel knows how many there are)
     const int ids = GROUPED ? grid_x / 2 : (total + kNumXcd - 1) / kNumXcd * kNumXcd - total / grid_x * grid_x;
-    persist_tail_sum_kernel<Cfg, GROUPED><<<dim3(ids * (Cfg::BM / 32)), 256, 0, stream>>>(p, grid_x);
+    persist_tail_sum_kernel<Cfg, GROUPED><<<dim3(ids * (Cfg::BM / kSumRows)), 256, 0, stream>>>(p, grid_x);
     e = hipGetLastError();
   }
   return e;

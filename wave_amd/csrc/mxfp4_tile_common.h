@@ -48,16 +48,12 @@ __device__ __forceinline__ bool map_tile(int pid, int tiles_m, int tiles_n, int 
   return true;
 }
 
-// Raw (stride 0) buffer descriptor over [base, base + 2 GiB): loads take a
-// 32-bit per-lane offset plus a scalar offset, so no 64-bit address math is
-// issued between the MFMAs.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7FFFFFFF, 0x00020000);
-}
-
-// The same over [base, base + bytes): accesses past the end read zeros and drop
-// their stores, which is how the persistent kernel handles a last tile row that
-// runs past M without per-lane clamps or guards.
+// Raw (stride 0) buffer descriptor over [base, base + bytes): loads take a 32-bit
+// per-lane offset plus a scalar offset, so no 64-bit address math is issued
+// between the MFMAs; accesses past the end read zeros and drop their stores,
+// which is how the kernels handle a last tile row that runs past M (and a slip
+// in an index) without per-lane clamps or guards.  Every descriptor in the
+// library ends with its tensor.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc_n(const void *base, int bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
 }

@@ -178,7 +178,10 @@ size_t wave_mxfp4_static_scratch_bytes(void);
  * wave_mxfp4_gemm (N % 32 == 0 and K % 256 == 0; otherwise it is not used),
  * and large problems run the persistent kernel over a table of M tiles built
  * there; a scale tensor handed over in WAVE_MXFP4_SCALE_MFMA32 order (resident
- * weights, activations from wave_mxfp4_quantize) is read where it is.
+ * weights, activations from wave_mxfp4_quantize) is read where it is.  For
+ * problems of at most four rounds of 256x256 tiles over the CUs the size
+ * includes 256 KB per CU for the f32 parts of a sparsely filled last round,
+ * whose tiles are then cut along K and summed by a second launch.
  * A small batch (AUTO: at most 152 rows per expert on average, and enough
  * experts x 128-column strips to occupy half the CUs) runs on the mid-M kernel,
  * one workgroup per (expert, strip), with no table and no scale re-layout: the

@@ -57,3 +57,43 @@ def test_captured_gemm_sequence_replays_with_eager_results():
         for want, o in zip(eager, ops):
             assert torch.equal(want, o[4]), f"replay {replay}: {tuple(want.shape)}"
         assert torch.equal(q_graph, q_eager) and torch.equal(s_graph, s_eager)
+
+
+def test_captured_grouped_sequence_replays_with_eager_results():
+    """The grouped call under capture: the table-driven persistent kernel (scale re-layout launch that also builds
+    the M tile table; a sparsely filled last round cut along K and summed by a second launch, decided on the device)
+    and the serving-batch path (one launch of the mid-M kernel)."""
+    cases = []
+    for i, (e, n, k, rows) in enumerate([(4, 2048, 8192, 9300), (6, 4096, 1024, 3000), (8, 4096, 2048, 64)]):
+        off = orc.make_group_offsets(e, rows, seed=70 + i)
+        x, xs, _, _ = orc.make_inputs(rows, 1, k, 70 + i, scale_lo=122, scale_hi=132)
+        rng = np.random.default_rng(170 + i)
+        w = rng.integers(0, 256, size=(e, n, k // 2), dtype=np.uint8)
+        ws = rng.integers(122, 133, size=(e, n, k // 32), dtype=np.uint8)
+        cases.append(to_gpu(x, xs, w, ws, off) + (torch.empty(rows, n, dtype=torch.bfloat16 if i % 2 else torch.float32, device=DEV),))
+
+    def sequence():
+        for gx, gxs, gw, gws, goff, out in cases:
+            wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out)
+
+    sequence()
+    torch.cuda.synchronize()
+    eager = [c[5].clone() for c in cases]
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        sequence()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            sequence()
+    torch.cuda.current_stream().wait_stream(stream)
+    for replay in range(3):
+        for c in cases:
+            c[5].fill_(float("nan"))
+        wave_amd.mxfp4_gemm_grouped(*cases[replay % len(cases)][:5], torch.empty_like(cases[replay % len(cases)][5]))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for want, c in zip(eager, cases):
+            assert torch.equal(want, c[5]), f"replay {replay}: {tuple(want.shape)}"

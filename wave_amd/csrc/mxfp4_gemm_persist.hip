@@ -790,7 +790,7 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
       variant != WAVE_MXFP4_VARIANT_T256x192_W4x2)
     return false;
   const int bn = variant == WAVE_MXFP4_VARIANT_T256x192_W4x2 ? 192 : 256;
-  // (a grouped problem comes with its M tile table and per-tile A scales, or not at all)
+  // (a grouped problem comes with its M tile table, or not at all)
   if ((p.num_groups != 0) != (p.tile_table != nullptr) || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
   if (p.n % bn != 0 || p.tiles_n != p.n / bn || p.k_tiles < 3) return false;  // any M

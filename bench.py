@@ -246,6 +246,74 @@ def time_quantize(torch, wave_amd, rows, k, steps, warmup, device, shuffle=True)
     return per, rows * k * 2 + rows * k // 2 + rows * k // 32, settle_ms
 
 
+def leg_moe_layer(torch, wave_amd, dev, steps_, warmup_):
+    """One mixture-of-experts MLP, the path of tests/kernel/moe_test.py:113-246 without its final weighted sum:
+    routing table -> token alignment -> gathered quantiser -> grouped GEMM (gate and up projections) -> gated
+    activation fused into the quantiser -> grouped GEMM (down projection).  Every scale tensor is written or kept in
+    MFMA32 order, so no re-layout launch sits between the steps.  Returns the layer's time and that of each step."""
+    from wave_amd import _lib as L
+
+    tokens, topk, E, hidden, inter = 4096, 2, 8, 4096, 14336
+    M32 = L.SCALE_MFMA32
+    g = torch.Generator(device=dev).manual_seed(3)
+    ids = torch.stack([torch.randperm(E, device=dev, generator=g)[:topk] for _ in range(tokens)]).to(torch.int32)
+    n_ent = tokens * topk
+    sorted_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
+    total = torch.empty(1, dtype=torch.int32, device=dev)
+    offs = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    act = torch.randn(tokens, hidden, device=dev, generator=g).to(torch.bfloat16)
+
+    def weights(n, k):
+        w = torch.randint(0, 256, (E, n, k // 2), dtype=torch.uint8, device=dev, generator=g)
+        ws = torch.randint(120, 131, (E, n, k // 32), dtype=torch.uint8, device=dev, generator=g)
+        return w, torch.stack([wave_amd.scale_convert(ws[e], n, k // 32, L.SCALE_ROW_MAJOR, M32) for e in range(E)])
+
+    w1, w1s = weights(2 * inter, hidden)
+    w2, w2s = weights(hidden, inter)
+    h1 = torch.empty(n_ent, 2 * inter, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(n_ent, hidden, dtype=torch.bfloat16, device=dev)
+    state = {}
+
+    def step_align():
+        wave_amd.moe_align_block_size(ids, E, 1, sorted_ids, expert_ids, total, offs)
+
+    def step_gather():
+        state["q1"], state["s1"] = wave_amd.quantize_mxfp4_rows(act, sorted_ids, topk, scale_layout=M32)
+
+    def step_gemm1():
+        wave_amd.mxfp4_gemm_grouped(state["q1"], state["s1"], w1, w1s, offs, h1, a_scale_layout=M32, b_scale_layout=M32)
+
+    def step_act():
+        state["q2"], state["s2"] = wave_amd.silu_and_mul_quantize(h1[:, :inter], h1[:, inter:], scale_layout=M32)
+
+    def step_gemm2():
+        wave_amd.mxfp4_gemm_grouped(state["q2"], state["s2"], w2, w2s, offs, out, a_scale_layout=M32, b_scale_layout=M32)
+
+    steps = [("moe_align_block_size", step_align), ("gathered_quantiser", step_gather), ("grouped_gemm_gate_up", step_gemm1),
+             ("gated_activation_quantiser", step_act), ("grouped_gemm_down", step_gemm2)]
+
+    def layer(count):
+        for _ in range(count):
+            for _, fn in steps:
+                fn()
+
+    layer(1)
+    torch.cuda.synchronize()
+    _, per_layer, _ = timed(torch, layer, steps_, warmup_)
+    each = {}
+    for name, fn in steps:
+        def run(count, fn=fn):
+            for _ in range(count):
+                fn()
+        each[name] = round(timed(torch, run, steps_, warmup_)[1] * 1e6, 2)
+    flops = 2.0 * n_ent * (2 * inter) * hidden + 2.0 * n_ent * hidden * inter
+    return {"workload": f"moe_layer: {tokens} tokens x top-{topk} of {E} experts, hidden {hidden}, intermediate {inter}",
+            "layer_us": round(per_layer * 1e6, 2), "tflops": round(flops / per_layer / 1e12, 1),
+            "frac_of_mxfp4_peak": round(flops / per_layer / 1e12 / PEAK_MXFP4_TFLOPS, 4), "steps_us": each,
+            "sum_of_steps_us": round(sum(each.values()), 2)}
+
+
 def leg_cfg4(torch, wave_amd, dev, steps, warmup, variant=0):
     """The grouped (MoE) GEMM of cfg4: E = 8 experts, 4096 tokens x top-2 = 8192 rows dealt multinomially, rows
     sorted by expert, N = 14336, K = 4096, bf16 out, seed 3."""
@@ -702,77 +770,16 @@ def main():
         return
 
     if args.workload == "moe_layer":
-        # One mixture-of-experts MLP, the path of tests/kernel/moe_test.py:113-246 without its final weighted sum:
-        # routing table -> token alignment -> gathered quantiser -> grouped GEMM (gate and up projections) ->
-        # gated activation fused into the quantiser -> grouped GEMM (down projection).  Every scale tensor is
-        # written or kept in MFMA32 order, so no re-layout launch sits between the steps.
-        from wave_amd import _lib as L
-
-        tokens, topk, E, hidden, inter = 4096, 2, 8, 4096, 14336
-        M32 = L.SCALE_MFMA32
-        g = torch.Generator(device=dev).manual_seed(3)
-        ids = torch.stack([torch.randperm(E, device=dev, generator=g)[:topk] for _ in range(tokens)]).to(torch.int32)
-        n_ent = tokens * topk
-        sorted_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
-        expert_ids = torch.empty(n_ent, dtype=torch.int32, device=dev)
-        total = torch.empty(1, dtype=torch.int32, device=dev)
-        offs = torch.empty(E + 1, dtype=torch.int32, device=dev)
-        act = torch.randn(tokens, hidden, device=dev, generator=g).to(torch.bfloat16)
-
-        def weights(n, k):
-            w = torch.randint(0, 256, (E, n, k // 2), dtype=torch.uint8, device=dev, generator=g)
-            ws = torch.randint(120, 131, (E, n, k // 32), dtype=torch.uint8, device=dev, generator=g)
-            return w, torch.stack([wave_amd.scale_convert(ws[e], n, k // 32, L.SCALE_ROW_MAJOR, M32) for e in range(E)])
-
-        w1, w1s = weights(2 * inter, hidden)
-        w2, w2s = weights(hidden, inter)
-        h1 = torch.empty(n_ent, 2 * inter, dtype=torch.bfloat16, device=dev)
-        out = torch.empty(n_ent, hidden, dtype=torch.bfloat16, device=dev)
-        state = {}
-
-        def step_align():
-            wave_amd.moe_align_block_size(ids, E, 1, sorted_ids, expert_ids, total, offs)
-
-        def step_gather():
-            state["q1"], state["s1"] = wave_amd.quantize_mxfp4_rows(act, sorted_ids, topk, scale_layout=M32)
-
-        def step_gemm1():
-            wave_amd.mxfp4_gemm_grouped(state["q1"], state["s1"], w1, w1s, offs, h1, a_scale_layout=M32, b_scale_layout=M32)
-
-        def step_act():
-            state["q2"], state["s2"] = wave_amd.silu_and_mul_quantize(h1[:, :inter], h1[:, inter:], scale_layout=M32)
-
-        def step_gemm2():
-            wave_amd.mxfp4_gemm_grouped(state["q2"], state["s2"], w2, w2s, offs, out, a_scale_layout=M32, b_scale_layout=M32)
-
-        steps = [("moe_align_block_size", step_align), ("gathered_quantiser", step_gather), ("grouped_gemm_gate_up", step_gemm1),
-                 ("gated_activation_quantiser", step_act), ("grouped_gemm_down", step_gemm2)]
-
-        def layer(count):
-            for _ in range(count):
-                for _, fn in steps:
-                    fn()
-
-        layer(1)
-        torch.cuda.synchronize()
-        _, per_layer, _ = timed(torch, layer, args.steps, args.warmup)
-        each = {}
-        for name, fn in steps:
-            def run(count, fn=fn):
-                for _ in range(count):
-                    fn()
-            each[name] = round(timed(torch, run, args.steps, args.warmup)[1] * 1e6, 2)
-        flops = 2.0 * n_ent * (2 * inter) * hidden + 2.0 * n_ent * hidden * inter
-        tfl = flops / per_layer / 1e12
+        leg = leg_moe_layer(torch, wave_amd, dev, args.steps, args.warmup)
         print(json.dumps(dict(common, **{
             "metric": "MoE expert MLP (align, gather + quantise, grouped GEMM, gated quantiser, grouped GEMM) TFLOPS",
-            "value": round(tfl, 1), "unit": "TFLOP/s", "ms_per_step": round(per_layer * 1e3, 4),
+            "value": leg["tflops"], "unit": "TFLOP/s", "ms_per_step": round(leg["layer_us"] * 1e-3, 4),
             "dtype": "bf16 activations, mxfp4 operands, f32 accumulate, bf16 out", "data": "synthetic (normal activations, uniform weights)",
-            "config": {"workload": f"moe_layer: {tokens} tokens x top-{topk} of {E} experts, hidden {hidden}, intermediate {inter}"},
-            "roofline": {"bound": "mfma", "achieved": round(tfl, 1), "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(tfl / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "persist_gemm_kernel (grouped)",
-                         "launch_us": round(per_layer * 1e6, 2)},
-            "steps_us": each, "sum_of_steps_us": round(sum(each.values()), 2)})))
+            "config": {"workload": leg["workload"]},
+            "roofline": {"bound": "mfma", "achieved": leg["tflops"], "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
+                         "frac": leg["frac_of_mxfp4_peak"], "traffic": None, "kernel": "persist_gemm_kernel (grouped)",
+                         "launch_us": leg["layer_us"]},
+            "steps_us": leg["steps_us"], "sum_of_steps_us": leg["sum_of_steps_us"]})))
         return
 
     if args.workload == "cfg4":
@@ -932,6 +939,8 @@ def main():
         leg = leg_mxfp8(torch, wave_amd, dev, args.steps, args.warmup)
         leg.pop("wall_s_per_step")
         result["mxfp8"] = leg
+        torch.cuda.empty_cache()
+        result["moe_layer"] = leg_moe_layer(torch, wave_amd, dev, min(args.steps, 50), min(args.warmup, 20))
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, m, n, k, seed, srange, args.cpu_rows)

@@ -36,12 +36,13 @@ namespace wave_mxfp4 {
 // only known on the device, where the GEMM and the summing kernel both evaluate this.
 __host__ __device__ inline int tail_parts_rule(int rest, int grid, int k_tiles) {
   if (rest <= 0 || rest * 2 > grid) return 1;
-  const float tile_us = 1.85f * (float)k_tiles;
-  int parts = 1;
-  float best = tile_us;
+  // (whole nanoseconds: the GEMM and the summing kernel must come to the same answer, which floating point
+  // contracted differently in two places would not promise)
+  const int tile_ns = 1850 * k_tiles;
+  int parts = 1, best = tile_ns;
   for (int c = 2; c <= 8 && c * rest <= grid && k_tiles / c >= 4; ++c) {
-    const float us = tile_us / (float)c + 2.0f * (float)rest * (float)c * (256.0f * 256.0f * 4.0f) / 4.0e6f + 6.0f;
-    if (us < best * 0.9f) best = us, parts = c;
+    const int ns = tile_ns / c + 2 * rest * c * (256 * 256 * 4 / 4000) + 6000;
+    if (ns * 10 < best * 9) best = ns, parts = c;
   }
   return parts;
 }

@@ -36,13 +36,16 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
   // wave w owns the contiguous segment [seg0, seg1) of the flat table
   const int per_wave = ((n + kAlignWaves - 1) / kAlignWaves + 63) & ~63;
   const int seg0 = min(n, wave * per_wave), seg1 = min(n, seg0 + per_wave);
-  // (8 steps of 64 ids are fetched together: a step at a time would pay a memory round trip each)
+  // (8 steps of 64 ids are fetched together: a step at a time would pay a memory round trip each; the first
+  // eight steps stay in registers for the placement below: up to 8192 entries are read once)
+  int64_t e_first[8];
   for (int base = seg0; base < seg1; base += 8 * 64) {
     int64_t e[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int i = base + s * 64 + lane;
       e[s] = i < seg1 ? (int64_t)topk_ids[i] : -1;
+      if (base == seg0) e_first[s] = e[s];
     }
 #pragma unroll
     for (int s = 0; s < 8; ++s)
@@ -82,16 +85,10 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
     const int from = starts[e] + counts[e], to = min(starts[e + 1], sorted_len);
     for (int i = from + lane; i < to; i += 64) sorted_ids[i] = n;
   }
-  // the expert of every block, all threads together: the last expert whose run starts at or before the block
-  for (int b = t; b < min(total / block_size, expert_ids_len); b += kAlignThreads) {
-    const int pos = b * block_size;
-    int lo = 0, hi = E - 1;
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) >> 1;
-      if (starts[mid] <= pos) lo = mid; else hi = mid - 1;
-    }
-    // (an empty expert shares its start with the next one; "the last" steps past it)
-    expert_ids[b] = lo;
+  // the expert of every block: a wave per expert fills the blocks of its run (an empty expert has none)
+  for (int e = wave; e < E; e += kAlignWaves) {
+    const int from = starts[e] / block_size, to = min(starts[e + 1] / block_size, expert_ids_len);
+    for (int b = from + lane; b < to; b += 64) expert_ids[b] = e;
   }
 
   // place: a wave walks its segment in order; the lanes of one expert take consecutive positions
@@ -105,7 +102,7 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int i = base8 + s * 64 + lane;
-      e8[s] = i < seg1 ? (int64_t)topk_ids[i] : -1;
+      e8[s] = base8 == seg0 ? e_first[s] : i < seg1 ? (int64_t)topk_ids[i] : -1;
     }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {

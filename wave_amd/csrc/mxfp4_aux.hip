@@ -105,16 +105,20 @@ __global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_la
 }
 
 // Row-major -> MFMA32 for ks % 4 == 0, the conversion in front of every tile
-// GEMM with row-major scales.  A workgroup takes 32 rows x 32 K tiles: 8-byte
-// reads that walk each row contiguously, the even and odd groups of a K tile
-// split with v_perm into the two dwords of its block (lanes r%32 and 32 + r%32),
-// a pass through LDS (block stride 65 dwords: conflict-free both ways), and
-// dword writes that walk the destination contiguously.
+// GEMM with row-major scales.  A workgroup takes 32 blocks of (32 rows x one K
+// tile): 32 rows x 32 K tiles, or for short rows 64 x 16 or 128 x 8, so that all
+// of its threads have a piece whatever K is (with 16 K tiles a row, K = 4096, half
+// of them had none).  8-byte reads that walk each row contiguously, the even and
+// odd groups of a K tile split with v_perm into the two dwords of its block (lanes
+// r%32 and 32 + r%32), a pass through LDS (block stride 65 dwords), and dword
+// writes that walk the destination contiguously.
 // blockIdx.z picks one of two tensors with the same ks (the A and B scales of a
 // GEMM go through one launch; rows of one of them 0 for a single tensor).
 // With gt.table the launch's first workgroup builds the M tile table of a grouped
 // GEMM before its share of the scales (mxfp4_group_table.h): the table only needs
 // the offsets, so it costs the call no launch of its own.
+// K tiles of a row that one workgroup walks, as a power of two: 5, 4 or 3.
+__host__ __device__ inline int scale_wg_kt_log(int k_tiles) { return k_tiles > 16 ? 5 : k_tiles > 8 ? 4 : 3; }
 __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__restrict__ src0,
                                                               uint8_t *__restrict__ dst0, int rows0,
                                                               const uint8_t *__restrict__ src1,
@@ -130,13 +134,14 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
   uint8_t *dst = blockIdx.z ? dst1 : dst0;
   const int rows = blockIdx.z ? rows1 : rows0;
   const int k_tiles = (ks + 7) >> 3;  // ks % 4 == 0: the last K tile may hold 4 groups only (the rest is written as 0)
-  const int rt = blockIdx.x, kt0 = blockIdx.y * 32;  // row tiles along x: up to 2^31 - 1 of them
-  const int row_base = rt * 32;
-  if (rt * 32 >= rows) return;  // the grid is sized for the taller tensor
+  const int kt_log = scale_wg_kt_log(k_tiles), kt_mask = (1 << kt_log) - 1;
+  const int rt0 = blockIdx.x << (5 - kt_log), kt0 = blockIdx.y << kt_log;  // row tiles along x: up to 2^31 - 1 workgroups
+  const int row_base = rt0 * 32;
+  if (row_base >= rows) return;  // the grid is sized for the taller tensor
   const int t = threadIdx.x;
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
-    const int unit = t + 256 * u, r = unit >> 5, ktl = unit & 31;
+    const int unit = t + 256 * u, r = unit >> kt_log, ktl = unit & kt_mask;
     const int row = row_base + r, kt = kt0 + ktl;
     uint2 v = make_uint2(0u, 0u);
     if (row < rows && kt < k_tiles) {
@@ -144,15 +149,17 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
       v.x = *(const uint32_t *)at;
       if (kt * 8 + 4 < ks) v.y = *(const uint32_t *)(at + 4);
     }
-    stage[ktl * 65 + r] = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u);       // groups 0, 2, 4, 6
-    stage[ktl * 65 + 32 + r] = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);  // groups 1, 3, 5, 7
+    const int blk = ((r >> 5) << kt_log) + ktl;
+    stage[blk * 65 + (r & 31)] = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u);       // groups 0, 2, 4, 6
+    stage[blk * 65 + 32 + (r & 31)] = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);  // groups 1, 3, 5, 7
   }
   __syncthreads();
-  uint32_t *out = (uint32_t *)dst + ((int64_t)rt * k_tiles + kt0) * 64;
+  uint32_t *out = (uint32_t *)dst;
 #pragma unroll
   for (int u = 0; u < 8; ++u) {
     const int d = t + 256 * u, blk = d >> 6, lane = d & 63;
-    if (kt0 + blk < k_tiles) out[d] = stage[blk * 65 + lane];
+    const int rt = rt0 + (blk >> kt_log), kt = kt0 + (blk & kt_mask);
+    if (kt < k_tiles && rt * 32 < rows) out[((int64_t)rt * k_tiles + kt) * 64 + lane] = stage[blk * 65 + lane];
   }
 }
 
@@ -324,7 +331,9 @@ hipError_t launch_scale_convert(const uint8_t *src, int src_layout, uint8_t *dst
   if (n == 0) return hipSuccess;
   if (src_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && dst_layout == WAVE_MXFP4_SCALE_MFMA32 && (ks & 3) == 0 &&
       ((uintptr_t)src & 3) == 0 && rows < ((int64_t)1 << 31) && (ksp / 8 + 31) / 32 <= 65535) {
-    dim3 grid((unsigned)(rows_p / 32), (unsigned)((ksp / 8 + 31) / 32), 1);
+    const int kt_log = scale_wg_kt_log((int)(ksp / 8));
+    const int64_t rows_wg = 1024 >> kt_log, per_wg = (int64_t)1 << kt_log;  // rows and K tiles a workgroup takes
+    dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), (unsigned)((ksp / 8 + per_wg - 1) / per_wg), 1);
     scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(src, dst, (int)rows, nullptr, nullptr, 0, (int)ks, GroupTableArgs{});
     return hipGetLastError();
   }
@@ -361,11 +370,13 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
     b_rows = 0;
   }
   const int64_t rows_max = a_rows > b_rows ? a_rows : b_rows;
-  const int64_t rt = (rows_max + 31) / 32;
   if ((ks & 3) != 0 || ks == 0 || ((uintptr_t)a_src & 3) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 3) != 0) ||
       rows_max >= ((int64_t)1 << 31) || ((ks + 7) / 8 + 31) / 32 > 65535 || a_rows <= 0 || b_rows < 0)
     return hipErrorInvalidValue;
-  dim3 grid((unsigned)rt, (unsigned)(((ks + 7) / 8 + 31) / 32), b_rows > 0 ? 2 : 1);
+  const int kt_log = scale_wg_kt_log((int)((ks + 7) / 8));
+  const int64_t rows_wg = 1024 >> kt_log;  // rows a workgroup takes
+  const int64_t k_tiles = (ks + 7) / 8, per_wg = (int64_t)1 << kt_log;
+  dim3 grid((unsigned)((rows_max + rows_wg - 1) / rows_wg), (unsigned)((k_tiles + per_wg - 1) / per_wg), b_rows > 0 ? 2 : 1);
   scale_to_mfma32_kernel<<<grid, 256, 0, stream>>>(a_src, a_dst, (int)a_rows, b_src, b_dst, (int)b_rows, (int)ks,
                                                    table ? *table : GroupTableArgs{});
   return hipGetLastError();

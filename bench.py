@@ -434,6 +434,8 @@ def mfma_ceiling(torch, dev, steps, warmup):
     vp, i32 = ctypes.c_void_p, ctypes.c_int
     probe.wave_probe_mfma_fp4.argtypes = [vp, vp, vp, i32, i32, i32, i32, vp]
     probe.wave_probe_mfma_fp4.restype = i32
+    probe.wave_probe_mfma_fp4_duty.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp]
+    probe.wave_probe_mfma_fp4_duty.restype = i32
     probe.wave_probe_operand_bytes.argtypes = [i32, i32]
     probe.wave_probe_operand_bytes.restype = ctypes.c_size_t
     cus = torch.cuda.get_device_properties(0).multi_processor_count
@@ -447,15 +449,17 @@ def mfma_ceiling(torch, dev, steps, warmup):
                     "zeros": torch.zeros(nbytes, dtype=torch.uint8, device=dev)}
         out = torch.empty(cus * waves * 64, dtype=torch.float32, device=dev)
         ticks = torch.empty(cus, dtype=torch.int64, device=dev)
-        for data in ("random", "zeros"):
+        # idle: s_sleep 1 instructions after every 32 MFMAs (4 waves per CU only): the pipes' duty cycle as a knob
+        for data, idle in [("random", 0), ("zeros", 0)] + ([("random", s) for s in (4, 8, 16)] +
+                                                           [("zeros", s) for s in (4, 8, 16)] if waves == 4 else []):
             src = operands[data]
 
             def run(count):
                 for _ in range(count):
-                    rc = probe.wave_probe_mfma_fp4(src.data_ptr(), out.data_ptr(), ticks.data_ptr(), iters, 110, cus,
-                                                   waves, stream)
+                    rc = probe.wave_probe_mfma_fp4_duty(src.data_ptr(), out.data_ptr(), ticks.data_ptr(), iters, 110,
+                                                        cus, waves, idle, stream)
                     if rc != 0:
-                        raise RuntimeError(f"wave_probe_mfma_fp4: {rc}")
+                        raise RuntimeError(f"wave_probe_mfma_fp4_duty: {rc}")
 
             _, per, settle_ms = timed(torch, run, max(steps // 10, 10), max(warmup // 10, 2))
             mfmas_per_wave = iters * 32
@@ -463,11 +467,11 @@ def mfma_ceiling(torch, dev, steps, warmup):
             # MFMA cycles each SIMD has to issue (32 per instruction, waves / 4 waves per SIMD): the clock if the pipe
             # never idles, a lower bound of it otherwise
             clock_ghz = mfmas_per_wave * 32 * (waves / 4) / per / 1e9
-            rows.append({"operands": data, "waves_per_cu": waves, "launch_ms": round(per * 1e3, 3),
+            rows.append({"operands": data, "waves_per_cu": waves, "idle_sleeps_per_32_mfma": idle, "launch_ms": round(per * 1e3, 3),
                          "tflops": round(flops / per / 1e12, 1),
                          "frac_of_mxfp4_peak": round(flops / per / 1e12 / PEAK_MXFP4_TFLOPS, 4),
                          "mfma_clock_ghz": round(clock_ghz, 3), "settle_ms": round(settle_ms, 1)})
-    best_random = max(r["tflops"] for r in rows if r["operands"] == "random")
+    best_random = max(r["tflops"] for r in rows if r["operands"] == "random" and r["idle_sleeps_per_32_mfma"] == 0)
     return rows, best_random
 
 

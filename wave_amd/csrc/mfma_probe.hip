@@ -23,7 +23,11 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // NT = 256: 4 waves per workgroup, each a 128 x 128 wave tile (4 x 4 MFMA tiles, 16 accumulators).
 // NT = 512: 8 waves, each 64 x 128 (2 x 4 MFMA tiles), the shape of the 8-wave GEMM kernels: two waves per SIMD
 // have 256 registers each.
-template <int NT>
+// GAP: s_sleep 1 instructions (64 cycles each) after the 32 MFMAs of an iteration: with GAP = 8 a wave's matrix
+// pipe idles a third of the time, about the duty cycle of the GEMM kernels (their rate on all-zero operands is
+// 72-74 % of this loop's).  What that loop sustains on random operands is what the GEMM's stalls alone would
+// leave of the MFMA-alone rate; what the GEMM loses beyond that is the energy of its data movement.
+template <int NT, int GAP>
 __global__ void __launch_bounds__(NT) mfma_probe_kernel(const v4i *__restrict__ src, float *__restrict__ out,
                                                         unsigned long long *__restrict__ ticks, int iters, int scale) {
   constexpr int MI = NT == 256 ? 4 : 2, MJ = 4, KT = NT == 256 ? 2 : 4;  // 32 MFMAs per wave and iteration
@@ -52,6 +56,8 @@ __global__ void __launch_bounds__(NT) mfma_probe_kernel(const v4i *__restrict__ 
           const v8i b = {fb[t][j].x, fb[t][j].y, fb[t][j].z, fb[t][j].w, 0, 0, 0, 0};
           acc[i * MJ + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i * MJ + j], 4, 4, 0, scale, 0, scale);
         }
+#pragma unroll
+    for (int g = 0; g < GAP; ++g) __builtin_amdgcn_s_sleep(1);
   }
   const unsigned long long t1 = __builtin_amdgcn_s_memtime();
   float s = 0.f;
@@ -77,18 +83,41 @@ size_t wave_probe_operand_bytes(int workgroups, int waves_per_workgroup) {
 // The sums are never rescaled (that would move all accumulators through the vector registers): pick scale_byte
 // so that iters * 32 products of at most 36 * 2^(2 * (scale_byte - 127)) stay finite, e.g. 110.
 // Returns 0, or -1 for a bad argument, or the hipError_t of the launch.
-int wave_probe_mfma_fp4(const void *operands, float *out, unsigned long long *ticks, int iters, int scale_byte,
-                        int workgroups, int waves_per_workgroup, void *hip_stream) {
+// idle_sleeps: 0, 4, 8 or 16 s_sleep 1 instructions (64 cycles each) after every 32 MFMAs (1024 busy cycles of a
+// wave that has its SIMD to itself): the duty cycle of the matrix pipes as a knob.
+int wave_probe_mfma_fp4_duty(const void *operands, float *out, unsigned long long *ticks, int iters, int scale_byte,
+                             int workgroups, int waves_per_workgroup, int idle_sleeps, void *hip_stream) {
   if (!operands || !out || !ticks || iters < 1 || workgroups < 1 || scale_byte < 0 || scale_byte > 254) return -1;
   hipStream_t stream = (hipStream_t)hip_stream;
   const int s = scale_byte | (scale_byte << 8) | (scale_byte << 16) | (scale_byte << 24);
-  if (waves_per_workgroup == 4)
-    mfma_probe_kernel<256><<<workgroups, 256, 0, stream>>>((const v4i *)operands, out, ticks, iters, s);
-  else if (waves_per_workgroup == 8)
-    mfma_probe_kernel<512><<<workgroups, 512, 0, stream>>>((const v4i *)operands, out, ticks, iters, s);
-  else
+#define WAVE_PROBE_LAUNCH(NT, GAP) \
+  mfma_probe_kernel<NT, GAP><<<workgroups, NT, 0, stream>>>((const v4i *)operands, out, ticks, iters, s)
+  if (waves_per_workgroup == 4) {
+    switch (idle_sleeps) {
+      case 0: WAVE_PROBE_LAUNCH(256, 0); break;
+      case 4: WAVE_PROBE_LAUNCH(256, 4); break;
+      case 8: WAVE_PROBE_LAUNCH(256, 8); break;
+      case 16: WAVE_PROBE_LAUNCH(256, 16); break;
+      default: return -1;
+    }
+  } else if (waves_per_workgroup == 8) {
+    switch (idle_sleeps) {
+      case 0: WAVE_PROBE_LAUNCH(512, 0); break;
+      case 4: WAVE_PROBE_LAUNCH(512, 4); break;
+      case 8: WAVE_PROBE_LAUNCH(512, 8); break;
+      case 16: WAVE_PROBE_LAUNCH(512, 16); break;
+      default: return -1;
+    }
+  } else {
     return -1;
+  }
+#undef WAVE_PROBE_LAUNCH
   return (int)hipGetLastError();
+}
+
+int wave_probe_mfma_fp4(const void *operands, float *out, unsigned long long *ticks, int iters, int scale_byte,
+                        int workgroups, int waves_per_workgroup, void *hip_stream) {
+  return wave_probe_mfma_fp4_duty(operands, out, ticks, iters, scale_byte, workgroups, waves_per_workgroup, 0, hip_stream);
 }
 
 }  // extern "C"

@@ -40,6 +40,7 @@ WORKLOADS = {
     "cfg3_m32": (32, 28672, 8192, "bf16", 2, (120, 134)),
     "cfg3_m64": (64, 28672, 8192, "bf16", 2, (120, 134)),
     "cfg3_m128": (128, 28672, 8192, "bf16", 2, (120, 134)),
+    "cfg3_m256": (256, 28672, 8192, "bf16", 2, (120, 134)),
     "cfg5": (4093, 6144, 7168, "f32", 4, (100, 154)),
 }
 
@@ -895,7 +896,7 @@ def main():
 
     if not args.no_legs and args.workload == "cfg2":
         # the decode shapes of the metric's second half: M = 16 (its target), and M = 1, 32, 64 and 128 beside it
-        for name in ("cfg3_m16", "cfg3_m1", "cfg3_m32", "cfg3_m64", "cfg3_m128"):
+        for name in ("cfg3_m16", "cfg3_m1", "cfg3_m32", "cfg3_m64", "cfg3_m128", "cfg3_m256"):
             dm, dn, dk, _, dseed, drange = WORKLOADS[name]
             dsets = make_gpu_inputs(torch, dm, dn, dk, dseed, drange, dev, copies=4)
             dout = torch.empty(dm, dn, dtype=torch.bfloat16, device=dev)
@@ -922,6 +923,20 @@ def main():
                     "workload": "the same call with B's scales already in MFMA operand order",
                     "launch_us": round(rper * 1e6, 2), "gbps": round(dbytes / rper / 1e9, 1),
                     "frac_of_hbm_peak": round(dbytes / rper / 1e9 / PEAK_HBM_GBPS, 4)}
+                if dm > 128:
+                    # ... and B in b_preshuffle order on top (static weights, preshuffled once, as the reference's
+                    # asymmetric kernels assume), A's scales in MFMA order as the quantiser writes them: A through
+                    # LDS, B straight from global memory into registers
+                    psets = [(x, wave_amd.scale_convert(xs, dm, dk // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32),
+                              wave_amd.b_preshuffle(w), ws32) for (x, xs, w, ws32) in rsets]
+                    _, pper, _ = time_gemm(torch, wave_amd, psets, dout, dsteps, args.warmup, a_scale_layout=L.SCALE_MFMA32,
+                                           b_scale_layout=L.SCALE_MFMA32, b_layout=L.B_PRESHUFFLE)
+                    result["decode_m%d" % dm]["preshuffled_b"] = {
+                        "workload": "the same operands, B in b_preshuffle order and both scale tensors in MFMA operand order",
+                        "kernel": "midb_gemm_kernel", "launch_us": round(pper * 1e6, 2),
+                        "gbps": round(dbytes / pper / 1e9, 1),
+                        "frac_of_hbm_peak": round(dbytes / pper / 1e9 / PEAK_HBM_GBPS, 4)}
+                    del psets
                 del rsets
             del dsets, dout
 

@@ -110,6 +110,13 @@ typedef enum {
    * AUTO takes it when its rounds cost less.  The reference fixes one block shape per compiled kernel
    * (wave_lang/kernel/wave/templates/tagged_mxfp4_gemm.py:38-145); picking it per problem is the library's. */
   WAVE_MXFP4_VARIANT_T256x192_W4x2 = 9,
+  /* M <= 256 against a wide preshuffled B from HBM: one workgroup per strip of 128 columns, 4 waves side by
+   * side along N; A through an LDS ring that takes the whole LDS, B straight from global memory into registers
+   * four K tiles ahead (the reference's asymmetric data flow, tagged_mxfp4_gemm.py:950-991, at a decode-sized M).
+   * Needs b_layout PRESHUFFLE, M <= 256, N % 32 == 0, K % 2048 == 0 (K % 1024 == 0 from M = 129 on), no split,
+   * and MFMA32 scales or the workspace; WAVE_MXFP4_ERR_UNSUPPORTED otherwise.  AUTO takes it for 128 < M <= 256
+   * where it applies and N >= 12288 (below that M variant 8 is as fast on the same operands). */
+  WAVE_MXFP4_VARIANT_MID_M_BDIRECT = 10,
   WAVE_MXFP4_VARIANT_COUNT_
 } wave_mxfp4_variant;
 

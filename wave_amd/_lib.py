@@ -40,6 +40,7 @@ VARIANT_T128x256_W2x2 = 6
 VARIANT_T256x256_W1x4_BDIRECT = 7
 VARIANT_MID_M = 8
 VARIANT_T256x192_W4x2 = 9
+VARIANT_MID_M_BDIRECT = 10
 
 # every symbol include/wave_mxfp4.h declares
 EXPORTS = (

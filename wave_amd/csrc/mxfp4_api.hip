@@ -140,7 +140,15 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
 // Kernels that read both scale tensors in MFMA32 order (the library re-lays them out first when it has scratch).
 // The mid-M kernel also reads row-major scales and scales in e8m0_shuffle order (the reference's format for
 // preshuffled scales) as they are: no pass per call for them.
-bool wants_mfma32_scales(int v) { return is_tile_variant(v) || v == WAVE_MXFP4_VARIANT_MID_M; }
+bool wants_mfma32_scales(int v) {
+  return is_tile_variant(v) || v == WAVE_MXFP4_VARIANT_MID_M || v == WAVE_MXFP4_VARIANT_MID_M_BDIRECT;
+}
+// What the B-direct mid-M kernel takes (the part of it that shape and layout alone decide): K in whole turns of
+// its ring of A, 8 K tiles up to 128 rows and 4 beyond.
+bool midb_shape_ok(int64_t m, int64_t n, int64_t k, int b_layout) {
+  return b_layout == WAVE_MXFP4_B_PRESHUFFLE && m >= 1 && m <= 256 && n % 32 == 0 && k > 0 &&
+         k % (m <= 128 ? 2048 : 1024) == 0;
+}
 bool mid_reads(int layout) {
   return layout == WAVE_MXFP4_SCALE_ROW_MAJOR || layout == WAVE_MXFP4_SCALE_MFMA32 || layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
 }
@@ -298,6 +306,16 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (variant == WAVE_MXFP4_VARIANT_AUTO && v == WAVE_MXFP4_VARIANT_MID_M && split_k > 1)  // (it takes whole K ranges)
     v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
   if (v == WAVE_MXFP4_VARIANT_SKINNY && m > skinny_max_m()) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  // the fallback of the library's own choice of the B-direct mid-M kernel, should the scales not reach MFMA32 order
+  const int v_plain = v;
+  // (measured at N = 28672, K = 8192 against the strip kernel on the same preshuffled B: M = 256 45.8 -> 43.1 us;
+  // at M = 128 the two tie, 28.6 / 28.8 us, and the strip kernel needs neither K in whole turns nor MFMA32 scales)
+  if (variant == WAVE_MXFP4_VARIANT_AUTO && m > 128 && n >= 12288 && split_k <= 1 && midb_shape_ok(m, n, k, b_layout))
+    v = WAVE_MXFP4_VARIANT_MID_M_BDIRECT;
+  if (variant == WAVE_MXFP4_VARIANT_MID_M_BDIRECT) {
+    const bool native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+    if (!midb_shape_ok(m, n, k, b_layout) || split_k > 1 || (!native && !workspace)) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  }
   if (variant == WAVE_MXFP4_VARIANT_MID_M) {
     const bool native = (mid_reads(a_scale_layout) || a_scale_layout == WAVE_MXFP4_SCALE_PER_ROW) && mid_reads(b_scale_layout);
     if (!mid_shape_ok(m, n, k) || split_k > 1 || (!native && !workspace)) return WAVE_MXFP4_ERR_UNSUPPORTED;
@@ -416,8 +434,16 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     if (variant == WAVE_MXFP4_VARIANT_MID_M) return WAVE_MXFP4_ERR_UNSUPPORTED;
     v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
   }
+  if (v == WAVE_MXFP4_VARIANT_MID_M_BDIRECT && !midb_gemm_applies(p)) {
+    if (variant == WAVE_MXFP4_VARIANT_MID_M_BDIRECT) return WAVE_MXFP4_ERR_UNSUPPORTED;
+    v = v_plain == WAVE_MXFP4_VARIANT_MID_M && !mid_gemm_applies(p)
+            ? (m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n))
+            : v_plain;
+  }
   const int vv = v;
-  if (vv == WAVE_MXFP4_VARIANT_MID_M) {
+  if (vv == WAVE_MXFP4_VARIANT_MID_M_BDIRECT) {
+    e = launch_midb_gemm(p, stream);
+  } else if (vv == WAVE_MXFP4_VARIANT_MID_M) {
     e = launch_mid_gemm(p, device_cus(), stream);
   } else if (v == WAVE_MXFP4_VARIANT_NAIVE) {
     e = launch_naive_gemm(p, stream);

@@ -136,6 +136,8 @@ hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2,
 bool persist_prefers_192(const GemmParams &p, int num_cus, int parts256);
 bool asym_gemm_applies(const GemmParams &p, int num_cus, bool forced);
 hipError_t launch_asym_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
+bool midb_gemm_applies(const GemmParams &p);
+hipError_t launch_midb_gemm(const GemmParams &p, hipStream_t stream);
 bool mid_gemm_applies(const GemmParams &p);
 hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream, int bm = 0);
 bool mid_grouped_applies(const GemmParams &p);

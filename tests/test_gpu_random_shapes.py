@@ -2,6 +2,8 @@
 against the exact oracle: the dispatch rules (tile shape by tile count, automatic and explicit splits with uneven
 parts, scale staging, streaming kernel) are exercised at shapes nobody picked by hand."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -76,4 +78,23 @@ def _wide_cases(count, seed):
 
 @pytest.mark.parametrize("case", _wide_cases(18, seed=21), ids=lambda c: f"w{c[0]}-{c[1]}x{c[2]}x{c[3]}")
 def test_random_wide_shape_against_oracle(case):
+    test_random_shape_against_oracle(case)
+
+
+def _midb_cases(count, seed):
+    """Shapes the library's own choice gives to the B-direct mid-M kernel when B is preshuffled (128 < M <= 256,
+    N >= 12288 in whole 32-column tiles, K in whole turns of its ring), with every scale layout and with and
+    without scratch (without it, and with scales that are not in MFMA32 order, the strip kernel takes them)."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        m, n, k = int(rng.integers(129, 257)), 32 * int(rng.integers(384, 1000)), 1024 * int(rng.integers(1, 9))
+        out.append((i, m, n, k, int(rng.integers(0, 3)), int(rng.integers(0, 3)), True, bool(rng.integers(0, 2)),
+                    bool(rng.integers(0, 4) > 0)))
+    return out
+
+
+@pytest.mark.parametrize("case", _midb_cases(int(os.environ.get("WAVE_MIDB_FUZZ", "10")), seed=22),
+                         ids=lambda c: f"b{c[0]}-{c[1]}x{c[2]}x{c[3]}")
+def test_random_preshuffled_mid_shape_against_oracle(case):
     test_random_shape_against_oracle(case)

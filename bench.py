@@ -476,6 +476,33 @@ def mfma_ceiling(torch, dev, steps, warmup):
     return rows, best_random
 
 
+def l2_dma_probe(torch, dev, steps, warmup):
+    """What L2 and Infinity Cache deliver to the CUs' LDS through the GEMM kernels' operand DMA alone
+    (wave_amd/csrc/mfma_probe.hip, dma_probe_kernel): 12 panels of 1 MB (3 per XCD, L2 resident) and 96 (12 MB per
+    XCD: from the Infinity Cache)."""
+    import ctypes
+
+    probe = ctypes.CDLL(os.path.join(ROOT, "wave_amd", "csrc", "libwave_probe.so"))
+    vp, i32 = ctypes.c_void_p, ctypes.c_int
+    probe.wave_probe_l2_dma.argtypes = [vp, i32, i32, i32, vp]
+    probe.wave_probe_l2_dma.restype = i32
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.randint(0, 256, (96 << 20,), dtype=torch.uint8, device=dev)
+    iters, rows = 64, []
+    for panels in (12, 96):
+        def run(count):
+            for _ in range(count):
+                rc = probe.wave_probe_l2_dma(src.data_ptr(), panels, iters, cus, stream)
+                if rc != 0:
+                    raise RuntimeError(f"wave_probe_l2_dma: {rc}")
+
+        _, per, _ = timed(torch, run, max(steps // 30, 5), max(warmup // 30, 2))
+        rows.append({"panels_of_1mb": panels, "footprint_per_xcd_mb": panels * 8 // 32 if panels < 32 else panels // 8,
+                     "launch_ms": round(per * 1e3, 3), "tb_per_s": round(cus * iters * (1 << 20) / per / 1e12, 2)})
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -572,7 +599,8 @@ def main():
             "config": {"workload": "mfma_ceiling: one workgroup per CU, 4 or 8 waves, 8000 x 32 MFMAs per wave and launch"},
             "roofline": {"bound": "mfma", "achieved": best, "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(best / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "mfma_probe_kernel"},
-            "runs": rows, "gemm_8192": gemm_rows})))
+            "runs": rows, "gemm_8192": gemm_rows,
+            "operand_dma_alone": l2_dma_probe(torch, dev, args.steps, args.warmup)})))
         return
 
     if args.workload == "quant_bf16":

@@ -69,9 +69,45 @@ __global__ void __launch_bounds__(NT) mfma_probe_kernel(const v4i *__restrict__ 
   if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
 }
 
+// Second probe: what the L2 (and, with a footprint beyond it, the Infinity Cache) delivers to a CU's LDS through the
+// GEMM kernels' operand DMA, with nothing else going on.  A region is a panel of 256 rows x 4096 bytes (1 MB, the
+// A or B panel of a 256-row tile at K = 8192); a workgroup of 8 waves walks its panel's 32 K tiles of 128 bytes
+// per row `iters` times, one wave instruction = 8 rows x 128 bytes (buffer_load_dwordx4 ... lds), counted waits.
+// Workgroup w reads panel w % panels: with 12 panels an XCD's workgroups share 3 (L2 resident), with 96 they walk
+// 12 MB per XCD, three times its L2.
+#define WAVE_PROBE_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+__global__ void __launch_bounds__(512) dma_probe_kernel(const uint8_t *__restrict__ src, int panels, int iters) {
+  __shared__ __attribute__((aligned(1024))) uint8_t ring[2 * 32 * 1024];
+  constexpr int NW = 8, PITCH = 4096, ND = 256 / 8 / NW;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint8_t *base = src + (size_t)(blockIdx.x % panels) * (256 * PITCH);
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, 256 * PITCH, 0x00020000);
+  const int voff = (lane >> 3) * PITCH + (lane & 7) * 16;
+  for (int it = 0; it < iters; ++it) {
+    for (int kt = 0; kt < 32; ++kt) {
+#pragma unroll
+      for (int d = 0; d < ND; ++d)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, WAVE_PROBE_LDS_PTR(ring + ((kt & 1) * 32 + d * NW + wave) * 1024), 16, voff,
+                                                 ((d * NW + wave) * 8) * PITCH + kt * 128, 0, 0);
+      __builtin_amdgcn_s_waitcnt((12 & 15) | (7 << 4) | (15 << 8));  // vmcnt(12): three K tiles in flight per wave
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+}
+
 }  // namespace
 
 extern "C" {
+
+// One launch of the DMA probe: `workgroups` workgroups of 8 waves, each `iters` x 1 MB from panel (id % panels) of
+// `src` (panels x 1 MB) into its LDS.  Returns 0, -1 for a bad argument, or the hipError_t of the launch.
+int wave_probe_l2_dma(const void *src, int panels, int iters, int workgroups, void *hip_stream) {
+  if (!src || panels < 1 || iters < 1 || workgroups < 1) return -1;
+  dma_probe_kernel<<<workgroups, 512, 0, (hipStream_t)hip_stream>>>((const uint8_t *)src, panels, iters);
+  return (int)hipGetLastError();
+}
+
 
 // Bytes of `operands` one launch reads: 32 fragments of 16 bytes per thread.
 size_t wave_probe_operand_bytes(int workgroups, int waves_per_workgroup) {

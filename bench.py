@@ -476,6 +476,38 @@ def mfma_ceiling(torch, dev, steps, warmup):
     return rows, best_random
 
 
+def read_once_probe(torch, dev, steps, warmup):
+    """A read-once stream of 117 MB (the decode shapes' B: 224 strips of 128 rows x 4 KB) with nothing else going
+    on (wave_amd/csrc/mfma_probe.hip, stream_probe_kernel): from HBM (three sets rotated) and from the Infinity
+    Cache (one set)."""
+    import ctypes
+
+    probe = ctypes.CDLL(os.path.join(ROOT, "wave_amd", "csrc", "libwave_probe.so"))
+    vp, i32 = ctypes.c_void_p, ctypes.c_int
+    probe.wave_probe_read_once.argtypes = [vp, i32, vp, vp]
+    probe.wave_probe_read_once.restype = i32
+    stream = torch.cuda.current_stream().cuda_stream
+    strips, set_bytes = 224, 224 * 128 * 4096
+    src = torch.randint(0, 256, (3 * set_bytes,), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(16, dtype=torch.int32, device=dev)
+    rows = []
+    for name, nsets in (("hbm (3 sets rotated)", 3), ("infinity cache (1 set)", 1)):
+        state = {"i": 0}
+
+        def run(count):
+            for _ in range(count):
+                rc = probe.wave_probe_read_once(src.data_ptr() + (state["i"] % nsets) * set_bytes, strips,
+                                                sink.data_ptr(), stream)
+                state["i"] += 1
+                if rc != 0:
+                    raise RuntimeError(f"wave_probe_read_once: {rc}")
+
+        _, per, _ = timed(torch, run, max(steps, 100), max(warmup, 30))
+        rows.append({"source": name, "bytes": set_bytes, "launch_us": round(per * 1e6, 2),
+                     "tb_per_s": round(set_bytes / per / 1e12, 2)})
+    return rows
+
+
 def l2_dma_probe(torch, dev, steps, warmup):
     """What L2 and Infinity Cache deliver to the CUs' LDS through the GEMM kernels' operand DMA alone
     (wave_amd/csrc/mfma_probe.hip, dma_probe_kernel): 12 panels of 1 MB (3 per XCD, L2 resident) and 96 (12 MB per
@@ -600,7 +632,8 @@ def main():
             "roofline": {"bound": "mfma", "achieved": best, "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(best / PEAK_MXFP4_TFLOPS, 4), "traffic": None, "kernel": "mfma_probe_kernel"},
             "runs": rows, "gemm_8192": gemm_rows,
-            "operand_dma_alone": l2_dma_probe(torch, dev, args.steps, args.warmup)})))
+            "operand_dma_alone": l2_dma_probe(torch, dev, args.steps, args.warmup),
+            "read_once_stream": read_once_probe(torch, dev, args.steps, args.warmup)})))
         return
 
     if args.workload == "quant_bf16":

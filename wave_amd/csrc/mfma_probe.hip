@@ -96,9 +96,56 @@ __global__ void __launch_bounds__(512) dma_probe_kernel(const uint8_t *__restric
   __builtin_amdgcn_s_waitcnt(0);
 }
 
+// Third probe: a read-once stream with nothing else going on, in the access pattern of the decode kernels' B
+// operand: strips of 128 rows x 4096 bytes in 16-row blocks of contiguous rows (b_preshuffle order), one workgroup of
+// four waves per strip, a wave instruction = two 512-byte pieces of one K step into registers (non-temporal), four K
+// tiles in flight per wave, every workgroup starting at a K tile of its own.  Launched over operand sets that
+// together exceed the Infinity Cache it streams from HBM; over one set of 117 MB, from the Infinity Cache.
+__global__ void __launch_bounds__(256) stream_probe_kernel(const uint8_t *__restrict__ b, int nkt, int *sink) {
+  constexpr int KP = 4096, SETS = 4;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint8_t *base = b + (size_t)blockIdx.x * 128 * KP;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, 128 * KP, 0x00020000);
+  const int fr = lane & 31, fg = lane >> 5;
+  const int goff = wave * 32 * KP + (fr >> 4) * 16 * KP + fg * 256 + (fr & 15) * 16;
+  int kt = (int)(blockIdx.x / 8) % nkt;
+  v4i r[SETS][4];
+  v4i acc = {0, 0, 0, 0};
+#pragma unroll
+  for (int s = 0; s < SETS; ++s) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) r[s][t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, goff, (kt * 4 + t) * 512, 2);
+    kt = kt + 1 == nkt ? 0 : kt + 1;
+  }
+  for (int j = SETS; j < nkt; j += SETS) {
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        acc += r[s][t];
+        r[s][t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, goff, (kt * 4 + t) * 512, 2);
+      }
+      kt = kt + 1 == nkt ? 0 : kt + 1;
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < SETS; ++s)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc += r[s][t];
+  if (acc.x == 0x12345678) sink[0] = acc.y + acc.z + acc.w;  // (keeps the loads)
+}
+
 }  // namespace
 
 extern "C" {
+
+// One launch of the stream probe over `strips` strips of 128 x 4096 bytes at `b` (K = 8192: 32 K tiles).
+int wave_probe_read_once(const void *b, int strips, int *sink, void *hip_stream) {
+  if (!b || !sink || strips < 1) return -1;
+  stream_probe_kernel<<<strips, 256, 0, (hipStream_t)hip_stream>>>((const uint8_t *)b, 32, sink);
+  return (int)hipGetLastError();
+}
+
 
 // One launch of the DMA probe: `workgroups` workgroups of 8 waves, each `iters` x 1 MB from panel (id % panels) of
 // `src` (panels x 1 MB) into its LDS.  Returns 0, -1 for a bad argument, or the hipError_t of the launch.

@@ -423,9 +423,10 @@ def leg_dense(torch, wave_amd, dev, name, steps, warmup, variant=0):
             "settle_ms": round(settle_ms, 1)}
 
 
-def mfma_ceiling(torch, dev, steps, warmup):
+def mfma_ceiling(torch, dev, steps, warmup, compact=False):
     """What the matrix pipes sustain on the scaled FP4 MFMA alone (wave_amd/csrc/mfma_probe.hip): random operand
-    bytes against zeros, 4 and 8 waves per CU, one workgroup per CU."""
+    bytes against zeros, 4 and 8 waves per CU, one workgroup per CU.  compact: the 8-wave shape of the GEMM kernels
+    only, random and zeros, no duty-cycle rows (the leg of the default line)."""
     import ctypes
 
     path = os.path.join(ROOT, "wave_amd", "csrc", "libwave_probe.so")
@@ -443,7 +444,7 @@ def mfma_ceiling(torch, dev, steps, warmup):
     stream = torch.cuda.current_stream().cuda_stream
     iters = 8000   # x 32 MFMAs x 32 cycles per wave: about 4 ms per launch at one wave per SIMD
     rows = []
-    for waves in (4, 8):
+    for waves in ((8,) if compact else (4, 8)):
         nbytes = probe.wave_probe_operand_bytes(cus, waves)
         g = torch.Generator(device=dev).manual_seed(11)
         operands = {"random": torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=dev, generator=g),
@@ -462,7 +463,7 @@ def mfma_ceiling(torch, dev, steps, warmup):
                     if rc != 0:
                         raise RuntimeError(f"wave_probe_mfma_fp4_duty: {rc}")
 
-            _, per, settle_ms = timed(torch, run, max(steps // 10, 10), max(warmup // 10, 2))
+            _, per, settle_ms = timed(torch, run, 5 if compact else max(steps // 10, 10), 2 if compact else max(warmup // 10, 2))
             mfmas_per_wave = iters * 32
             flops = cus * waves * mfmas_per_wave * 2.0 * 32 * 32 * 64
             # MFMA cycles each SIMD has to issue (32 per instruction, waves / 4 waves per SIMD): the clock if the pipe
@@ -952,6 +953,28 @@ def main():
                 "frac_of_mxfp4_peak": round(flops / bper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
             }
             del wp
+        if args.workload == "cfg2" and not args.no_legs:
+            # What this chip, in this run, lets the matrix pipes do: the scaled FP4 MFMA alone (no memory traffic,
+            # wave_amd/csrc/mfma_probe.hip) on random and on all-zero operand bytes, and the headline kernel on
+            # all-zero operands (same instruction stream and traffic as on the seeded data, less power per
+            # instruction).  On random bytes the chip is power-limited well below its 2.4 GHz peak clock, so
+            # `frac_of_mfma_alone` is the headline kernel against the ceiling measured beside it, `frac` against
+            # the published peak.
+            rows, _ = mfma_ceiling(torch, dev, args.steps, args.warmup, compact=True)
+            by = {r["operands"]: r for r in rows}
+            zx, zw = torch.zeros_like(x), torch.zeros_like(w)
+            _, zper, _ = time_gemm(torch, wave_amd, [(zx, xs32, zw, ws32)], out, args.steps, args.warmup,
+                                   a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32)
+            del zx, zw
+            result["power_ceiling"] = {
+                "workload": "v_mfma_scale_f32_32x32x64_f8f6f4 alone, 8 waves per CU, 8000 x 32 per wave and launch, on "
+                            "uniformly random bytes and on zeros; the headline kernel on all-zero A and B",
+                "mfma_random_tflops": by["random"]["tflops"], "mfma_random_clock_ghz": by["random"]["mfma_clock_ghz"],
+                "mfma_zero_tflops": by["zeros"]["tflops"], "mfma_zero_clock_ghz": by["zeros"]["mfma_clock_ghz"],
+                "gemm_zero_us": round(zper * 1e6, 2), "gemm_zero_tflops": round(flops / zper / 1e12, 1),
+                "gemm_zero_frac_of_mfma_zero": round(flops / zper / 1e12 / by["zeros"]["tflops"], 4),
+            }
+            roofline["frac_of_mfma_alone"] = round(roofline["achieved"] / by["random"]["tflops"], 4)
         del xs32, ws32
     del sets, out
 

@@ -15,6 +15,7 @@ from oracle import c_oracle
 from oracle import mxfp4_oracle as orc
 from wave_amd import _lib
 
+from gpu_util import F32_TIGHT as F32_TIGHT_
 from gpu_util import (BF16_ABS, BF16_REL, DEV, TILE_VARIANTS, assert_bf16_close, assert_close,
                       assert_f32_close, run_gemm, to_gpu)
 
@@ -341,3 +342,30 @@ def test_configs_with_torch_seeded_inputs(name, m, n, k, dt, seed, lo, hi):
     else:
         rows = sample_rows(m, 8, seed=seed)
         assert_close(c[rows], c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows), dt, name)
+
+
+def test_grouped_persistent_path_survives_malformed_offsets():
+    """Offsets that are not non-decreasing ([0, T, 0, T, ...]: every other group is the whole tensor, 40 tiles of
+    256 rows against a table capacity of 18) are clamped, not validated: the table's last band is cut to the tiles
+    that were written, so the walk reads no unwritten entry (wave_amd/csrc/mxfp4_group_table.h, checked on the CPU
+    by tests/test_group_table_host.py).  The call must return, and every 256-column block of every row of C holds
+    either nothing (a dropped tile) or that row's product with one of the experts that own it."""
+    e, n, k, T = 8, 4096, 1024, 2560
+    x, xs, w, ws, _ = grouped_inputs(e, n, k, T, seed=91)
+    off = np.array([0, T] * 4 + [0], dtype=np.int32)
+    gx, gxs, gw, gws, goff = to_gpu(x, xs, w, ws, off)
+    out = torch.full((T, n), float("nan"), dtype=torch.float32, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, goff, out, variant=_lib.VARIANT_T256x256_W4x2)
+    torch.cuda.synchronize()
+    c = out.cpu().numpy()
+    pick = np.unique(np.concatenate([np.arange(0, T, 61), np.arange(255, T, 256)]))
+    refs = [c_oracle.scaled_gemm_exact(x, w[g], xs, ws[g], rows=pick) for g in (0, 2, 4, 6)]
+    written = 0
+    for i, r in enumerate(pick):
+        for b in range(n // 256):
+            blk = c[r, b * 256:(b + 1) * 256]
+            if np.isnan(blk).all():
+                continue
+            written += 1
+            assert any(np.abs(blk - ref[i, b * 256:(b + 1) * 256]).max() <= F32_TIGHT_ * np.abs(ref[i]).max() for ref in refs), (r, b)
+    assert written > 0

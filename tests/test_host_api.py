@@ -136,10 +136,16 @@ def test_superseded_scratch_buffers_stay_alive():
         assert host._grow_scratch(key, 50, alloc) is small          # large enough: reused
         ptr = small.data_ptr()
         big = host._grow_scratch(key, 1000, alloc)
-        assert big is not small and big.numel() == 1000
+        assert big is not small and big.numel() == 1024  # grown geometrically: the next power of two
         del small
         assert made[0]() is not None and made[0]().data_ptr() == ptr  # still referenced by the module
         assert host._grow_scratch(key, 1000, alloc) is big
+        # a run of slowly growing requests retires less than the live buffer holds
+        before = len(host._retired)
+        for n in range(1025, 9000, 7):
+            last = host._grow_scratch(key, n, alloc)
+        retired = sum(t.numel() for t in host._retired[before:])
+        assert retired < last.numel() and last.numel() == 16384
     finally:
         host._scratch.pop(key, None)
 

@@ -25,6 +25,7 @@
 // contract is the same.
 #include <type_traits>
 
+#include "mxfp4_group_table.h"
 #include "mxfp4_tile_common.h"
 
 namespace wave_mxfp4 {
@@ -54,10 +55,7 @@ __device__ __forceinline__ bool map_grouped_tile(const int32_t *table, int total
   const int seq = (id % kNumXcd) * per_xcd + id / kNumXcd;
   if (seq >= total) return false;
   const int band = __builtin_amdgcn_readfirstlane(table[4 * (1 + seq / tiles_n) + 3]);
-  const int start = band >> 4, height = band & 15;
-  const int in_band = seq - start * tiles_n;
-  tn = in_band / height;
-  tm = start + in_band - tn * height;
+  grouped_tile_of_seq(band, seq, tiles_n, tm, tn);
   return true;
 }
 

@@ -86,7 +86,9 @@ def workspace_bytes(m: int, n: int, k: int, split_k: int = 0, variant: int = _li
 # ordered, so they can share it; different streams get different buffers.
 # A buffer that was handed out is never freed: a HIP graph captured while it was
 # current keeps its address, so a buffer that a larger call supersedes moves to
-# `_retired` and stays allocated until the process ends.
+# `_retired` and stays allocated until the process ends.  Buffers grow geometrically
+# (the request rounded up to a power of two), so what a run of slowly growing problems
+# leaves in `_retired` stays below the size of the live buffer.
 _scratch: dict = {}
 _retired: list = []
 # signatures of mxfp4_gemm calls that passed every check: -> (m, n, k, out dtype code, a scale layout, scratch bytes)
@@ -100,7 +102,7 @@ def _grow_scratch(key, nbytes: int, alloc):
     if buf is None or buf.numel() < nbytes:
         if buf is not None:
             _retired.append(buf)
-        buf = alloc(nbytes)
+        buf = alloc(1 << max(int(nbytes) - 1, 0).bit_length())
         _scratch[key] = buf
     return buf
 

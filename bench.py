@@ -418,9 +418,20 @@ def leg_dense(torch, wave_amd, dev, name, steps, warmup, variant=0):
     out = torch.empty(m, n, dtype=torch.bfloat16 if od == "bf16" else torch.float32, device=dev)
     _, per, settle_ms = time_gemm(torch, wave_amd, sets, out, steps, warmup, variant=variant)
     flops = gemm_flops(m, n, k)
-    return {"workload": f"{name}: M={m} N={n} K={k} {od} out seed {seed}", "launch_us": round(per * 1e6, 2),
-            "tflops": round(flops / per / 1e12, 1), "frac_of_mxfp4_peak": round(flops / per / 1e12 / PEAK_MXFP4_TFLOPS, 4),
-            "settle_ms": round(settle_ms, 1)}
+    leg = {"workload": f"{name}: M={m} N={n} K={k} {od} out seed {seed}", "launch_us": round(per * 1e6, 2),
+           "tflops": round(flops / per / 1e12, 1), "frac_of_mxfp4_peak": round(flops / per / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+           "settle_ms": round(settle_ms, 1)}
+    if variant == 0 and k % 256 == 0:
+        # the same call with both scale tensors in the reference's e8m0_shuffle order (read in place)
+        from wave_amd import _lib as L
+        x, xs, w, ws = sets[0]
+        xsh = wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_E8M0_SHUFFLE)
+        wsh = wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_E8M0_SHUFFLE)
+        _, sper, _ = time_gemm(torch, wave_amd, [(x, xsh, w, wsh)], out, steps, warmup,
+                               a_scale_layout=L.SCALE_E8M0_SHUFFLE, b_scale_layout=L.SCALE_E8M0_SHUFFLE)
+        leg["e8m0_shuffled_scales"] = {"launch_us": round(sper * 1e6, 2), "tflops": round(flops / sper / 1e12, 1),
+                                       "frac_of_mxfp4_peak": round(flops / sper / 1e12 / PEAK_MXFP4_TFLOPS, 4)}
+    return leg
 
 
 def mfma_ceiling(torch, dev, steps, warmup, compact=False):
@@ -934,6 +945,18 @@ def main():
             "launch_us": round(pper * 1e6, 2), "tflops": round(flops / pper / 1e12, 1),
             "frac_of_mxfp4_peak": round(flops / pper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
         }
+        # ... and in e8m0_shuffle order, the format the reference's preshuffled-scale kernels take
+        # (wave_lang/kernel/wave/utils/mxfp_utils.py:113-128): read in place by the persistent kernels
+        xsh = wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_E8M0_SHUFFLE)
+        wsh = wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_E8M0_SHUFFLE)
+        _, sper, _ = time_gemm(torch, wave_amd, [(x, xsh, w, wsh)], out, args.steps, args.warmup,
+                               a_scale_layout=L.SCALE_E8M0_SHUFFLE, b_scale_layout=L.SCALE_E8M0_SHUFFLE)
+        result["e8m0_shuffled_scales"] = {
+            "workload": "the same operands, scales in the reference's e8m0_shuffle order, read in place (no re-layout launch)",
+            "launch_us": round(sper * 1e6, 2), "tflops": round(flops / sper / 1e12, 1),
+            "frac_of_mxfp4_peak": round(flops / sper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+        }
+        del xsh, wsh
         # roofline: the dominant kernel by itself, i.e. this leg's launches (a call with row-major scales is that
         # kernel + the scale re-layout launch in front of it: `call_us`, the figure `value` is computed from)
         roofline["call_us"] = roofline["launch_us"]

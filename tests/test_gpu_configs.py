@@ -360,12 +360,12 @@ def test_grouped_persistent_path_survives_malformed_offsets():
     c = out.cpu().numpy()
     pick = np.unique(np.concatenate([np.arange(0, T, 61), np.arange(255, T, 256)]))
     refs = [c_oracle.scaled_gemm_exact(x, w[g], xs, ws[g], rows=pick) for g in (0, 2, 4, 6)]
-    written = 0
-    for i, r in enumerate(pick):
-        for b in range(n // 256):
-            blk = c[r, b * 256:(b + 1) * 256]
-            if np.isnan(blk).all():
-                continue
-            written += 1
-            assert any(np.abs(blk - ref[i, b * 256:(b + 1) * 256]).max() <= F32_TIGHT_ * np.abs(ref[i]).max() for ref in refs), (r, b)
-    assert written > 0
+    # (tiles of different experts that cover the same rows are written concurrently: an element is one expert's or
+    # another's, and which may differ from element to element)
+    got = c[pick]
+    dropped = np.isnan(got)
+    err = np.min([np.abs(np.where(dropped, ref, got) - ref) for ref in refs], axis=0)
+    assert err.max() <= F32_TIGHT_ * max(np.abs(ref).max() for ref in refs)
+    blocks = dropped.reshape(len(pick), n // 256, 256)
+    assert (blocks.all(axis=2) | ~blocks.any(axis=2)).all(), "a dropped tile is dropped whole"
+    assert not dropped.all()

@@ -29,7 +29,7 @@ CSRC = os.path.join(ROOT, "wave_amd", "csrc")
 #    around the accumulator read-out between two K loops (5 stores + 5 loads per 4096 MFMAs of a wave), none
 #    inside a K loop.
 KNOWN_SCRATCH = {
-    "asym_gemm_kernel<true>": 32,
+    "asym_gemm_kernel<true, false>": 32,
     "tile_gemm_kernel<TileCfg<256, 256, 2, 2>": 160,
     "stream_gemm_kernel<4, true, 1>": 32,
     "stream_gemm_kernel<4, true, 2>": 32,

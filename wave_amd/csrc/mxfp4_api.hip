@@ -323,7 +323,8 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT) {
     // what the B-direct kernel takes, checked before anything is launched: preshuffled B, whole 256-column tiles,
     // an even number (at least 6) of K tiles, no split, scales in MFMA32 order or scratch to bring them there
-    const bool native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+    const bool native = (a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32) ||
+                        (a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE);
     if (b_layout != WAVE_MXFP4_B_PRESHUFFLE || n % 256 != 0 || k % 512 != 0 || k < 1536 || split_k > 1 ||
         (!native && !workspace))
       return WAVE_MXFP4_ERR_UNSUPPORTED;
@@ -331,7 +332,9 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
 
   if (v == WAVE_MXFP4_VARIANT_T256x192_W4x2) {
     // the 256x192 tiles exist in the persistent kernel only: whole tiles along N, more tiles than CUs, no split
-    const bool native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+    const bool native = (a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32) ||
+                        (a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE &&
+                         k % kTileK == 0);
     const int grid = device_cus() / 8 * 8;
     if (n % 192 != 0 || k < 768 || split_k > 1 || (!native && !workspace) || ((m + 255) / 256) * (n / 192) <= grid)
       return WAVE_MXFP4_ERR_UNSUPPORTED;
@@ -387,7 +390,26 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   const bool small_short = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 && p.tiles_per_split <= (splits > 1 ? 12 : 16) &&
                            k % kTileK == 0 &&
                            p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
-  if (wants_mfma32_scales(v) && workspace && !small_short) {
+  // Both tensors in e8m0_shuffle order, the reference's preshuffled format (tagged_mxfp4_gemm.py:334-403,485-536):
+  // the 8-wave persistent kernels read it in place (two dwords and a byte permute per lane instead of one dword),
+  // so a caller that holds its operands the reference's way pays no re-layout launch.
+  bool shuffled_in_place = false;
+  if (p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && splits == 1 &&
+      (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 || v == WAVE_MXFP4_VARIANT_T256x192_W4x2 ||
+       v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT)) {
+    GemmParams q = p;
+    int bm, bn;
+    tile_variant_shape(v, &bm, &bn);
+    q.tiles_m = (int)((m + bm - 1) / bm);
+    q.tiles_n = (int)((n + bn - 1) / bn);
+    if (v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT)
+      shuffled_in_place = asym_gemm_applies(q, device_cus(), true);
+    else
+      shuffled_in_place = (variant == WAVE_MXFP4_VARIANT_AUTO && v == WAVE_MXFP4_VARIANT_T256x256_W4x2 &&
+                           asym_gemm_applies(q, device_cus(), false)) ||
+                          persist_gemm_applies(q, v, device_cus());
+  }
+  if (wants_mfma32_scales(v) && workspace && !small_short && !shuffled_in_place) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
     const bool mid = v == WAVE_MXFP4_VARIANT_MID_M;
     const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads(p.a_scale_layout)) ? a_bytes : 0;

@@ -26,7 +26,9 @@
 // K tile in a fixed order.
 //
 // Taken for preshuffled B, N % 256 == 0, K % 512 == 0 (the B registers alternate between even and
-// odd K tiles), K >= 1536, both scale tensors in MFMA32 order, dense, no split.  Any M.
+// odd K tiles), K >= 1536, both scale tensors in MFMA32 order or both in e8m0_shuffle order (SHUF: the
+// same 256-byte blocks, a lane's four bytes in two dwords 128 bytes apart, put together by a v_perm),
+// dense, no split.  Any M.
 #include <type_traits>
 
 #include "mxfp4_tile_common.h"
@@ -42,16 +44,16 @@ constexpr int kSSlot = kAsymWaves * 1024;       // A scales of one K tile: 2 KB 
 constexpr int kStage = 4096;                    // C staging per wave
 constexpr int kAsymLds = kARing * kASlot + kARing * kSSlot + kAsymWaves * kStage;  // 160 KB
 constexpr int kALd = kAsymBM / 8 / kAsymWaves;  // A DMA instructions per wave and K tile (8)
-// Vector memory operations per wave and K tile: A 8, A scales 1, B 8, B scales 2.
-constexpr int kOpsPerKTile = kALd + 1 + 8 + 2;
+// Vector memory operations per wave and K tile: A 8, A scales 1, B 8, B scales 2 (4 in e8m0_shuffle order).
+constexpr int ops_per_k_tile(bool shuf) { return kALd + 1 + 8 + (shuf ? 4 : 2); }
 // At the wait of K tile g (before its fourth K step) A and its scales of K tile g + 1 must have landed.  They
 // were requested in K tile g - 2 (at the latest as the last operations of its fourth K step: the compiler may
 // order the requests of one K step among themselves), followed by the 19 of K tile g - 1 and the 14 of the first
-// three K steps of K tile g.
-constexpr int kWaitSteady = kOpsPerKTile + 14;
+// three K steps of K tile g (16 with four B scale requests, which go out in the second K step).
+constexpr int wait_steady(bool shuf) { return ops_per_k_tile(shuf) + (shuf ? 16 : 14); }
 static_assert(kAsymLds <= 160 * 1024, "LDS");
 
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool SHUF>
 __device__ __forceinline__ void asym_body(const GemmParams &p) {
   constexpr int BM = kAsymBM, BN = kAsymBN, NW = kAsymWaves;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -107,7 +109,10 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
   // B fragment of the 32x32x64 MFMA straight from b_preshuffle order: lane = (row r = lane % 32, K half = lane / 32)
   const int fr = lane & 31, fg = lane >> 5;
   const int b_goff = wave * 64 * kp + (fr >> 4) * 16 * kp + fg * 256 + (fr & 15) * 16;
-  const int bs_goff = (2 * wave) * k_tiles_blocks + lane * 4;
+  // the lane's dword of a 256-byte scale block (SHUF: the first of its two, the other 128 bytes on)
+  const int s_lane = SHUF ? ((lane >> 5) * 16 + (lane & 15)) * 4 : lane * 4;
+  const uint32_t s_sel = (lane & 16) ? 0x07030501u : 0x06020400u;  // SHUF: the lane's bytes of the two dwords
+  const int bs_goff = (2 * wave) * k_tiles_blocks + s_lane;
   // A fragment reads: row fr of a 32-row block, chunk 2t + fg at its swizzled position
   uint32_t foff[4];
 #pragma unroll
@@ -133,17 +138,21 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
     for (int jn = 0; jn < 2; ++jn)
       dst[jn] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_goff, (kt * 4 + t) * 512 + jn * 32 * kp, 0);
   };
-  auto load_bs = [&](int which, int kt, uint32_t (&dst)[2]) {
+  auto load_bs = [&](int which, int kt, uint32_t (&dst)[2], uint32_t (&dst2)[2]) {
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc_n(bs_base[which], bs_lim[which]);
 #pragma unroll
-    for (int jn = 0; jn < 2; ++jn)
+    for (int jn = 0; jn < 2; ++jn) {
       dst[jn] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, bs_goff, jn * k_tiles_blocks + kt * 256, 0);
+      if constexpr (SHUF)
+        dst2[jn] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, bs_goff, jn * k_tiles_blocks + kt * 256 + 128, 0);
+    }
   };
 
   // ---------------- registers ----------------
   v16f acc[8][2];
   v4i bq[2][4][2];          // [parity of the K tile][K step][jn]
   uint32_t sb_cur[2][2], sb_in[2][2];  // B scales in use / arriving, per parity
+  uint32_t sb_in2[2][2];               // SHUF: the second dword of the arriving ones
   uint32_t sa[2][8];        // A scales per parity
   v4i afr[2][8];            // A fragments, double buffered by K step
 
@@ -154,9 +163,15 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
   };
   auto read_sa = [&](int slot, uint32_t (&dst)[8]) {
     // block i of the tile's eight was fetched by wave i / 2 into the lower half of its kilobyte
-    const uint8_t *base = s_ring + slot * kSSlot + lane * 4;
+    const uint8_t *base = s_ring + slot * kSSlot + s_lane;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dst[i] = *(const uint32_t *)(base + (i >> 1) * 1024 + (i & 1) * 256);
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t d0 = *(const uint32_t *)(base + (i >> 1) * 1024 + (i & 1) * 256);
+      if constexpr (SHUF)
+        dst[i] = __builtin_amdgcn_perm(*(const uint32_t *)(base + (i >> 1) * 1024 + (i & 1) * 256 + 128), d0, s_sel);
+      else
+        dst[i] = d0;
+    }
   };
   auto mfma_step = [&](const v4i (&fa)[8], const v4i (&fb)[2], const uint32_t (&sca)[8], const uint32_t (&scb)[2], auto t_tag,
                        auto zero_tag) {
@@ -217,7 +232,12 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
     // this K tile's B scales were requested two K tiles ago into sb_in: real moves, pinned here (a compiler copy
     // would be folded into a phi of the loop and wait wherever that lands)
 #pragma unroll
-    for (int jn = 0; jn < 2; ++jn) asm volatile("v_mov_b32 %0, %1" : "=v"(sb_cur[PAR][jn]) : "v"(sb_in[PAR][jn]));
+    for (int jn = 0; jn < 2; ++jn) {
+      if constexpr (SHUF)
+        asm volatile("v_perm_b32 %0, %1, %2, %3" : "=v"(sb_cur[PAR][jn]) : "v"(sb_in2[PAR][jn]), "v"(sb_in[PAR][jn]), "v"(s_sel));
+      else
+        asm volatile("v_mov_b32 %0, %1" : "=v"(sb_cur[PAR][jn]) : "v"(sb_in[PAR][jn]));
+    }
     read_a(sl, 1, afr[1]);
     mfma_step(afr[0], bq[PAR][0], sa[PAR], sb_cur[PAR], T0{}, zero_tag);
     issue_a(wa, kta, sl_a, 0, 2);
@@ -229,7 +249,7 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
     mfma_step(afr[1], bq[PAR][1], sa[PAR], sb_cur[PAR], T1{}, Keep{});
     issue_a(wa, kta, sl_a, 2, 4);
     load_b(wb2, ktb2, 0, bq[PAR][0]);
-    load_bs(wb2, ktb2, sb_in[PAR]);
+    load_bs(wb2, ktb2, sb_in[PAR], sb_in2[PAR]);
     order_step();
     __builtin_amdgcn_sched_barrier(0);
 
@@ -332,19 +352,19 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
   issue_as(0, 1, 1);
 #pragma unroll
   for (int t = 0; t < 3; ++t) load_b(0, 0, t, bq[0][t]);
-  load_bs(0, 0, sb_in[0]);
+  load_bs(0, 0, sb_in[0], sb_in2[0]);
   issue_a(0, 2, 2, 0, 2);
   load_b(0, 0, 3, bq[0][3]);
   issue_a(0, 2, 2, 2, 4);
   load_b(0, 1, 0, bq[1][0]);
-  load_bs(0, 1, sb_in[1]);
+  load_bs(0, 1, sb_in[1], sb_in2[1]);
   issue_a(0, 2, 2, 4, 6);
   load_b(0, 1, 1, bq[1][1]);
   issue_a(0, 2, 2, 6, 8);
   issue_as(0, 2, 2);
   load_b(0, 1, 2, bq[1][2]);
   // everything but the last K tile's worth has landed (the one-time cost of filling the pipeline)
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kOpsPerKTile));
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(ops_per_k_tile(SHUF)));
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
@@ -355,6 +375,7 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
   // ---------------- the tiles ----------------
   typedef std::integral_constant<int, 0> Even;
   typedef std::integral_constant<int, 1> Odd;
+  constexpr int kWaitSteady = wait_steady(SHUF);
   typedef std::integral_constant<int, kWaitSteady> WaitSteady;
   typedef std::integral_constant<int, (kWaitSteady + NS > 63 ? 63 : kWaitSteady + NS)> WaitAfterStore;
   int sl = 0;
@@ -399,17 +420,17 @@ __device__ __forceinline__ void asym_body(const GemmParams &p) {
   __builtin_amdgcn_s_waitcnt(0);  // the trailing requests must not outlive the workgroup's LDS and registers
 }
 
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool SHUF = false>
 __global__ void __launch_bounds__(kAsymNT, 1) asym_gemm_kernel(const GemmParams p) {
-  asym_body<OUT_BF16>(p);
+  asym_body<OUT_BF16, SHUF>(p);
 }
 
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool SHUF>
 hipError_t launch_asym_out(const GemmParams &p, int grid_x, hipStream_t stream) {
   static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)asym_gemm_kernel<OUT_BF16>, kAsymLds);
+  hipError_t e = allow_dynamic_lds(once, (const void *)asym_gemm_kernel<OUT_BF16, SHUF>, kAsymLds);
   if (e != hipSuccess) return e;
-  asym_gemm_kernel<OUT_BF16><<<dim3(grid_x, 1, 1), dim3(kAsymNT), kAsymLds, stream>>>(p);
+  asym_gemm_kernel<OUT_BF16, SHUF><<<dim3(grid_x, 1, 1), dim3(kAsymNT), kAsymLds, stream>>>(p);
   return hipGetLastError();
 }
 
@@ -419,7 +440,8 @@ hipError_t launch_asym_out(const GemmParams &p, int grid_x, hipStream_t stream) 
 // fewer tiles than CUs is taken too).
 bool asym_gemm_applies(const GemmParams &p, int num_cus, bool forced) {
   if (!p.b_preshuffled || p.num_groups != 0 || p.tile_table != nullptr || p.splits != 1 || p.partial != nullptr) return false;
-  if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  const bool shuffled = p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
+  if (!shuffled && (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32)) return false;
   if ((p.n & 255) != 0 || (p.k & 511) != 0 || p.k_tiles < 6 || p.m < 1) return false;
   // 32-bit offsets inside one operand tile and one C tile
   if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31)) return false;
@@ -432,7 +454,9 @@ bool asym_gemm_applies(const GemmParams &p, int num_cus, bool forced) {
 
 hipError_t launch_asym_gemm(const GemmParams &p, int num_cus, hipStream_t stream) {
   const int grid = num_cus / kNumXcd * kNumXcd;
-  return p.out_bf16 ? launch_asym_out<true>(p, grid, stream) : launch_asym_out<false>(p, grid, stream);
+  if (p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
+    return p.out_bf16 ? launch_asym_out<true, true>(p, grid, stream) : launch_asym_out<false, true>(p, grid, stream);
+  return p.out_bf16 ? launch_asym_out<true, false>(p, grid, stream) : launch_asym_out<false, false>(p, grid, stream);
 }
 
 }  // namespace wave_mxfp4

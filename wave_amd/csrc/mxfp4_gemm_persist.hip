@@ -91,9 +91,15 @@ enum KtKind {
 // FMT_A / FMT_B: element format codes of the scaled MFMA, 4 = e2m1 (MXFP4); 0 = e4m3, 1 = e5m2 (MXFP8, both
 // operands 8-bit: a 128-byte K tile is then 128 elements = two 64-deep K steps of 32 bytes per lane, the MFMA
 // takes 64 cycles instead of 32, and one MFMA32 scale block serves two K tiles; dense, whole K tiles, no cut).
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, int FMT_A = 4, int FMT_B = 4>
+// SHUF: both scale tensors in e8m0_shuffle order (the reference's preshuffled format,
+// wave_lang/kernel/wave/utils/mxfp_utils.py:113-128), read in place.  It keeps the same 256-byte blocks per 32 rows
+// and K tile in the same order as MFMA32; inside a block the four bytes of a lane (row r, K half h: groups 2t + h of
+// the K steps t = 0..3) sit in two dwords, (16h + r % 16) for t = 0, 2 and 32 further on for t = 1, 3, at bytes
+// (r % 32) / 16 and 2 + (r % 32) / 16: two loads and one v_perm where MFMA32 takes one load and a move.
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, int FMT_A = 4, int FMT_B = 4, bool SHUF = false>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
   constexpr bool FP8 = FMT_A != 4;
+  static_assert(!SHUF || (!FP8 && !GROUPED && !TAIL), "scales in e8m0_shuffle order: dense MXFP4 problems with whole K tiles");
   constexpr bool B4 = FP8 && FMT_B == 4;  // 8-bit A against 4-bit B [N, K/2]: the lower half of B's LDS rows
   static_assert(FMT_A != 4 || FMT_B == 4, "an MXFP4 A against an MXFP8 B is not built");
   static_assert(!FP8 || (!GROUPED && !TAIL && !SPLIT), "MXFP8: dense problems with whole K tiles");
@@ -273,8 +279,10 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
 
   // ---------------- scales (MFMA-native order: one dword per lane, 32 rows and K tile) ----------------
   const int a_srow = ((wave_m * Cfg::WM) >> 5) * k_tiles_blocks, b_srow = ((wave_n * Cfg::WN) >> 5) * k_tiles_blocks;
-  const int s_lane = lane * 4;
+  const int s_lane = SHUF ? ((lane >> 5) * 16 + (lane & 15)) * 4 : lane * 4;
+  const uint32_t s_sel = (lane & 16) ? 0x07030501u : 0x06020400u;  // SHUF: the lane's bytes of its two dwords
   uint32_t raw_a[MT_M], raw_b[MT_N], sc_a[MT_M], sc_b[MT_N];
+  uint32_t raw_a2[SHUF ? MT_M : 1], raw_b2[SHUF ? MT_N : 1];  // SHUF: the dwords of the odd K steps
   auto sblk = [](int kt) { return FP8 ? kt >> 1 : kt; };  // MXFP8: one MFMA32 block serves two K tiles
   auto load_scales = [&](int which, int kt) {
     const __amdgpu_buffer_rsrc_t ra = make_rsrc_n(as_base[which], as_lim[which]), rb = make_rsrc_n(bs_base[which], bs_lim[which]);
@@ -284,11 +292,17 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       a_lane = ((t & 31) + (lane & 32)) * 4 + (t >> 5) * k_tiles_blocks;
     }
 #pragma unroll
-    for (int i = 0; i < MT_M; ++i)
+    for (int i = 0; i < MT_M; ++i) {
       raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256, 0);
+      if constexpr (SHUF)
+        raw_a2[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256 + 128, 0);
+    }
 #pragma unroll
-    for (int j = 0; j < MT_N; ++j)
+    for (int j = 0; j < MT_N; ++j) {
       raw_b[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + sblk(kt) * 256, 0);
+      if constexpr (SHUF)
+        raw_b2[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + sblk(kt) * 256 + 128, 0);
+    }
   };
   // Real register moves, pinned here (a compiler copy would be folded into the
   // loop's phi and wait for the next scale load at the top of every iteration).
@@ -301,6 +315,13 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       for (int i = 0; i < MT_M; ++i) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(sc_a[i]) : "s"(shift), "v"(raw_a[i]));
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) asm volatile("v_lshrrev_b32 %0, %1, %2" : "=v"(sc_b[j]) : "s"(shift), "v"(raw_b[j]));
+    } else if constexpr (SHUF) {
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i)
+        asm volatile("v_perm_b32 %0, %1, %2, %3" : "=v"(sc_a[i]) : "v"(raw_a2[i]), "v"(raw_a[i]), "v"(s_sel));
+#pragma unroll
+      for (int j = 0; j < MT_N; ++j)
+        asm volatile("v_perm_b32 %0, %1, %2, %3" : "=v"(sc_b[j]) : "v"(raw_b2[j]), "v"(raw_b[j]), "v"(s_sel));
     } else {
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(sc_a[i]) : "v"(raw_a[i]));
@@ -651,9 +672,9 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   __builtin_amdgcn_s_waitcnt(0);  // the trailing DMA must not outlive the workgroup's LDS
 }
 
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, bool SHUF = false>
 __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_kernel(const GemmParams p) {
-  persist_body<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>(p);
+  persist_body<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT, 4, 4, SHUF>(p);
 }
 
 template <class Cfg, bool OUT_BF16, int FMT_A, int FMT_B>
@@ -700,13 +721,13 @@ __global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams 
   }
 }
 
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT>
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, bool SHUF = false>
 static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_t stream) {
   static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>,
+  hipError_t e = allow_dynamic_lds(once, (const void *)persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT, SHUF>,
                                    Cfg::LDS_BYTES);
   if (e != hipSuccess) return e;
-  persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT>
+  persist_gemm_kernel<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT, SHUF>
       <<<dim3(grid_x, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
   e = hipGetLastError();
   if (SPLIT && e == hipSuccess) {
@@ -722,6 +743,14 @@ static hipError_t launch_persist_out(const GemmParams &p, int grid_x, hipStream_
 template <class Cfg, bool OUT_BF16>
 static hipError_t launch_persist_dense(const GemmParams &p, int grid_x, hipStream_t stream) {
   const bool tail = (p.k & (kTileK - 1)) != 0;
+  if constexpr (Cfg::NWAVES == 8) {
+    if (p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {  // (both tensors, whole K tiles: persist_gemm_applies)
+      if constexpr (Cfg::BN == 256) {
+        if (p.tail_parts > 1) return launch_persist_out<Cfg, OUT_BF16, false, false, true, true>(p, grid_x, stream);
+      }
+      return launch_persist_out<Cfg, OUT_BF16, false, false, false, true>(p, grid_x, stream);
+    }
+  }
   if constexpr (Cfg::NWAVES == 8 && Cfg::BN == 256) {  // (the 4-wave kernel has no registers to spare for the split bookkeeping)
     if (p.tail_parts > 1)
       return tail ? launch_persist_out<Cfg, OUT_BF16, false, true, true>(p, grid_x, stream)
@@ -791,7 +820,11 @@ bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
   const int bn = variant == WAVE_MXFP4_VARIANT_T256x192_W4x2 ? 192 : 256;
   // (a grouped problem comes with its M tile table, or not at all)
   if ((p.num_groups != 0) != (p.tile_table != nullptr) || p.splits != 1 || p.partial != nullptr) return false;
-  if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  // both scale tensors in MFMA32 order; or, 8-wave kernels on dense problems with whole K tiles, both in
+  // e8m0_shuffle order
+  const bool shuffled = p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE &&
+                        variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 && p.num_groups == 0 && (p.k & (kTileK - 1)) == 0;
+  if (!shuffled && (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32)) return false;
   if (p.n % bn != 0 || p.tiles_n != p.n / bn || p.k_tiles < 3) return false;  // any M
   // a partial last K tile: dense problems with at least four K tiles
   if ((p.k & (kTileK - 1)) != 0 && (p.num_groups != 0 || p.k_tiles < 4)) return false;

@@ -1,7 +1,8 @@
 """The grouped GEMM's M tile table on the CPU: the builder's and the tile walk's own arithmetic
 (wave_amd/csrc/mxfp4_group_table.h, compiled for the host by tests/host_group_table.cpp) over well-formed and
-malformed offsets arrays.  Every tile the walk reaches must be an entry the builder wrote, with its rows inside
-the tensors, its group below the group count, and every (M tile, N tile) visited exactly once.
+malformed offsets arrays, with and without short tiles.  Every tile the walk reaches must be an entry the builder
+wrote, with its rows inside the tensors, its group below the group count, every (M tile, N tile) visited exactly
+once, and every short tile (a group's last tile of few rows) behind all full ones.
 
 The reference's MoE tests build their groups from torch.unique counts and never hand over a malformed array
 (tests/kernel/moe_test.py:175-246); a C ABI that takes a device pointer has to survive one.
@@ -25,7 +26,7 @@ def harness(tmp_path_factory):
 
 
 def run(harness, cases):
-    text = "".join(f"{t} {bm} {tn} {len(off) - 1} {' '.join(str(int(o)) for o in off)}\n" for t, bm, tn, off in cases)
+    text = "".join(f"{t} {bm} {tn} {sr} {len(off) - 1} {' '.join(str(int(o)) for o in off)}\n" for t, bm, tn, sr, off in cases)
     out = subprocess.run([harness], input=text, capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-2000:]
     lines = out.stdout.split("\n")[:-1]
@@ -43,15 +44,18 @@ def test_well_formed_offsets_make_every_tile(harness):
         if rng.random() < 0.3:
             counts[rng.integers(0, groups)] = 0
         off = np.concatenate([[0], np.cumsum(counts)])
-        cases.append((int(off[-1]) + int(rng.integers(0, 300)), bm, int(rng.integers(1, 60)), off))
-    for (t, bm, tn, off), line in zip(cases, run(harness, cases)):
-        assert line == f"ok {sum(-(-int(c) // bm) for c in np.diff(off))}", (t, bm, tn, off.tolist(), line)
+        cases.append((int(off[-1]) + int(rng.integers(0, 300)), bm, int(rng.integers(1, 60)), int(rng.choice([0, 64, 128])), off))
+    for (t, bm, tn, sr, off), line in zip(cases, run(harness, cases)):
+        counts = [int(c) for c in np.diff(off)]
+        shorts = sum(1 for c in counts if c > 0 and c - (-(-c // bm) - 1) * bm <= sr)
+        assert line == f"ok {sum(-(-c // bm) for c in counts)} {shorts}", (t, bm, tn, sr, off.tolist(), line)
 
 
 def test_the_capacity_cut_keeps_the_walk_inside_the_table(harness):
     # the advisor's example: [0, T, 0, T, ...] with T = 2560 and 8 groups is 40 tiles against a capacity of 18
     T = 2560
-    cases = [(T, 256, 7, [0, T] * 4 + [0]), (T, 256, 56, [0, T, 0, T, 0, T, 0, T, T])]
+    cases = [(T, 256, 7, 0, [0, T] * 4 + [0]), (T, 256, 56, 64, [0, T, 0, T, 0, T, 0, T, T]),
+             (T + 40, 256, 5, 64, [0, T + 40] * 4 + [0])]
     rng = np.random.default_rng(1)
     for _ in range(2000):
         groups = int(rng.integers(1, 24))
@@ -67,6 +71,6 @@ def test_the_capacity_cut_keeps_the_walk_inside_the_table(harness):
             off = np.sort(rng.integers(0, total + 1, groups + 1))
             i, j = rng.integers(0, groups + 1, 2)
             off[i], off[j] = off[j], off[i]
-        cases.append((total, int(rng.choice([64, 128, 256])), int(rng.integers(1, 20)), off))
-    bad = [(c[0], c[1], c[2], list(map(int, c[3])), line) for c, line in zip(cases, run(harness, cases)) if not line.startswith("ok")]
+        cases.append((total, int(rng.choice([64, 128, 256])), int(rng.integers(1, 20)), int(rng.choice([0, 16, 64])), off))
+    bad = [(c[0], c[1], c[2], c[3], list(map(int, c[4])), line) for c, line in zip(cases, run(harness, cases)) if not line.startswith("ok")]
     assert not bad, bad[:3]

@@ -98,6 +98,9 @@ bool is_tile_variant(int v) {
 }
 
 // Grouped problems of at most this many rows per expert on average go to the mid-M kernel.
+// Grouped persistent kernel: a group's last M tile of at most this many rows runs as a short tile (all eight waves
+// side by side on 64 rows: an eighth of a full tile's MFMAs), after the full ones.
+constexpr int kGroupedShortRows = 64;
 constexpr int64_t kGroupedMidMaxAvgRows = 152;  // (rows per block up to 192: the 256-row block loses to the tile kernels)
 
 // What the mid-M kernel takes (the part of it that the shape alone decides).
@@ -708,9 +711,12 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
     const auto rm_or_native = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
     if (rm_or_native(p.a_scale_layout) && rm_or_native(p.b_scale_layout) && persist_gemm_applies(q, v, device_cus())) {
       const bool a_native = p.a_scale_layout == WAVE_MXFP4_SCALE_MFMA32, b_native = p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
-      const GroupTableArgs gt{offsets, num_groups, 256, (int)total_rows, table};
+      // (a problem of few rounds cuts a sparse last round along K instead: no short tiles then)
+      const bool cut_tail = v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && grouped_tail_bytes(total_rows, n, k, num_groups) != 0;
+      const int short_rows = v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && !cut_tail ? kGroupedShortRows : 0;
+      const GroupTableArgs gt{offsets, num_groups, 256, short_rows, (int)total_rows, table};
       if (a_native && b_native)
-        e = launch_grouped_tile_table(offsets, num_groups, 256, total_rows, table, stream);
+        e = launch_grouped_tile_table(offsets, num_groups, 256, short_rows, total_rows, table, stream);
       else
         e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, a_native ? 0 : total_rows, p.b_scale, ws_b,
                                         b_native ? 0 : (int64_t)num_groups * n, p.ks, stream, &gt);
@@ -718,7 +724,7 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
         if (!a_native) q.a_scale = ws_a;
         if (!b_native) q.b_scale = ws_b;
         q.b_scale_group_stride = n * (int64_t)p.ksp;
-        if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && grouped_tail_bytes(total_rows, n, k, num_groups) != 0)
+        if (cut_tail)
           q.tail_partial = (float *)(ws_b + round_up_256((size_t)num_groups * scale_buffer_bytes(n, k)));
         return record_hip(launch_persist_gemm(q, v, device_cus(), stream));
       }

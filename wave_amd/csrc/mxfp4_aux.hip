@@ -127,8 +127,8 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
   __shared__ uint32_t stage[32 * 65];
   if (gt.table != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
     __shared__ int wave_sums[4];
-    __shared__ int carry;
-    build_group_tile_table<256>(gt, wave_sums, &carry);
+    __shared__ int carry[2];
+    build_group_tile_table<256>(gt, wave_sums, carry);
   }
   const uint8_t *src = blockIdx.z ? src1 : src0;
   uint8_t *dst = blockIdx.z ? dst1 : dst0;

@@ -35,7 +35,7 @@ struct GemmParams {
   float *partial;          // split-K slices [splits, M, N] f32, or null
   const int32_t *offsets;  // grouped: device [E+1]; else null
   const int32_t *tile_table;  // grouped, persistent kernel: device table of M tiles (int32 x 4 each: entry 0 =
-                              // {count}, entry 1 + t = {first row, rows, expert}); A's scales are laid out per tile
+                              // {tiles, full tiles}, entry 1 + t = {first row, rows, expert, band}: mxfp4_group_table.h)
   int m, n, k;
   int kp;              // K / 2
   int ks;              // K / 32
@@ -173,7 +173,9 @@ hipError_t launch_e8m0_shuffle(const uint8_t *scale, uint8_t *out, int64_t rows,
 // What the builder of a grouped GEMM's M tile table takes (mxfp4_group_table.h); table == nullptr: none to build.
 struct GroupTableArgs {
   const int32_t *offsets;
-  int num_groups, bm, total_rows;
+  int num_groups, bm;
+  int short_rows;  // a group's last tile of at most this many rows goes to the table's short tiles (0: none do)
+  int total_rows;
   int32_t *table;
 };
 // (with `table`, the launch's first workgroup also builds the M tile table of a grouped GEMM; a_rows == 0: B alone)
@@ -182,8 +184,8 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
                                        const GroupTableArgs *table = nullptr);
 hipError_t launch_scale_pair_shuffle_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int64_t a_rows, const uint8_t *b_src,
                                                uint8_t *b_dst, int64_t b_rows, int64_t ks, hipStream_t stream);
-hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int64_t total_rows, int32_t *table,
-                                     hipStream_t stream);
+hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int short_rows, int64_t total_rows,
+                                     int32_t *table, hipStream_t stream);
 hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t kp,
                                hipStream_t stream);
 

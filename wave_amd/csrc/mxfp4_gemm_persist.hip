@@ -50,13 +50,10 @@ __host__ __device__ inline int tail_parts_rule(int rest, int grid, int k_tiles) 
 
 // Tile id -> (M tile, N tile) of a grouped problem: the same XCD regrouping as map_tile, but the bands the sequence
 // walks column by column are the table's (at most 8 tiles of one expert), not fixed runs of 8 tile rows.
-__device__ __forceinline__ bool map_grouped_tile(const int32_t *table, int total, int tiles_n, int id, int &tm, int &tn) {
-  const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
-  const int seq = (id % kNumXcd) * per_xcd + id / kNumXcd;
-  if (seq >= total) return false;
-  const int band = __builtin_amdgcn_readfirstlane(table[4 * (1 + seq / tiles_n) + 3]);
-  grouped_tile_of_seq(band, seq, tiles_n, tm, tn);
-  return true;
+// (the full tiles first, then the table's short tiles: grouped_tile_of_id)
+__device__ __forceinline__ bool map_grouped_tile(const int32_t *table, int tiles, int full, int tiles_n, int id, int &tm, int &tn) {
+  return grouped_tile_of_id(tiles, full, tiles_n, id,
+                            [table](int t) { return __builtin_amdgcn_readfirstlane(table[4 * (1 + t) + 3]); }, tm, tn);
 }
 
 enum KtKind {
@@ -112,9 +109,16 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
   const int kp = p.kp, nkt = p.k_tiles;
-  const int tiles_m = GROUPED ? p.tile_table[0] : p.tiles_m;
+  // SHORTS: a grouped problem's short tiles (a group's last M tile of at most 64 rows, listed behind the full ones
+  // in the table) run after all full tiles, with the eight waves side by side on the tile's 64 rows (each 64 x 32:
+  // two MFMAs per K step instead of eight).  The operand streams, their waits and the barrier are the full
+  // tile's, request for request, so full and short tiles follow each other in any order.
+  constexpr bool SHORTS = GROUPED && !SPLIT && !FP8 && Cfg::NWAVES == 8 && Cfg::BN == 256 && Cfg::WAVES_M == 4;
+  const int tiles_m = GROUPED ? __builtin_amdgcn_readfirstlane(p.tile_table[0]) : p.tiles_m;
+  const int tiles_full = GROUPED ? __builtin_amdgcn_readfirstlane(p.tile_table[1]) : tiles_m;
   const int total = tiles_m * p.tiles_n;
-  const int padded = (total + kNumXcd - 1) / kNumXcd * kNumXcd;
+  // ids of the tile walk (the padding ids of the XCD regrouping included)
+  const int padded = GROUPED ? grouped_walk_ids(tiles_m, tiles_full, p.tiles_n) : (total + kNumXcd - 1) / kNumXcd * kNumXcd;
   const int k_tiles_blocks = (p.ksp >> 3) * 256;  // bytes of one 32-row scale tile row
 
   // ---------------- the tile sequence of this workgroup ----------------
@@ -129,10 +133,11 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   int m0[2], n0[2], a_lim[2], as_lim[2], b_lim[2], bs_lim[2], c_rows[2], nkt_of[2], part_of[2];
   int a_row32[2] = {0, 0};  // grouped: the tile's first row inside its 32-row scale block
   bool tail_on[2];
+  bool is_short[2] = {false, false};
   const int m_blocks = (p.m + 31) >> 5;
   const int b_kt_stride = p.b_preshuffled ? 2048 : B4 ? kTileKBytes / 2 : kTileKBytes;
   auto map_grouped = [&](int id, int &tm, int &tn) -> bool {
-    return map_grouped_tile(p.tile_table, total, p.tiles_n, id, tm, tn);
+    return map_grouped_tile(p.tile_table, tiles_m, tiles_full, p.tiles_n, id, tm, tn);
   };
   // (grouped: the tile count, and with it whether the last round is cut, is only known here)
   const int tail_parts = !SPLIT ? 1
@@ -168,6 +173,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       b_base[which] = p.b + (int64_t)expert * p.b_group_stride + (int64_t)n0[which] * kp;
       bs_base[which] = p.b_scale + (int64_t)expert * p.b_scale_group_stride + (int64_t)(n0[which] >> 5) * k_tiles_blocks;
       a_row32[which] = first & 31;
+      is_short[which] = SHORTS && tm >= tiles_full;
       as_base[which] = p.a_scale + (int64_t)(first >> 5) * k_tiles_blocks;
       as_lim[which] = (int)min((int64_t)(m_blocks - (first >> 5)) * k_tiles_blocks, (int64_t)0x7FFFFFFF);
     } else {
@@ -198,8 +204,22 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     }
     return true;
   };
-  int pid = blockIdx.x;
-  if (!set_tile(0, pid)) return;
+  // Item `step` of this workgroup's walk is tile id blockIdx.x + step * gridDim.x: all its full tiles, then its short
+  // ones.  (Measured at 8 experts x 14336 x 4096, 8192 rows in multinomial groups, 1792 full and 224 short tiles:
+  // short tiles placed between the full ones instead - at a position that differs from workgroup to workgroup, or
+  // from XCD to XCD - so that their requests for B meet less competition, took 11-12 us longer: the workgroups of
+  // an XCD then no longer run the tiles of a band together, and what they share of A and B is fetched again.)
+  const int grid = (int)gridDim.x;
+  const int walk_items = (int)blockIdx.x < padded ? (padded - (int)blockIdx.x + grid - 1) / grid : 0;
+  auto id_of = [&](int step) -> int { return (int)blockIdx.x + step * grid; };
+  // (padding ids of the XCD regrouping map to no tile: the walk steps over them)
+  int step = 0;
+  if constexpr (SHORTS) {
+    while (step < walk_items && !set_tile(0, id_of(step))) ++step;
+    if (step >= walk_items) return;
+  } else {
+    if (!set_tile(0, id_of(0))) return;
+  }
 
   // ---------------- global -> LDS addressing (see the one-tile kernel) ----------------
   const int ld_row0 = wave * 8 + (lane >> 3);
@@ -277,6 +297,34 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     }
   };
 
+  // short tile: the wave's operands are rows 0..63 of A (two fragments) and its own 32 rows of B (one)
+  auto read_frags_short = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], FragB(&fb)[MT_N]) {
+    if constexpr (SHORTS) {
+      const uint8_t *ba = smem + slot_a * SLOT + foff[t];
+      const uint8_t *bb = smem + slot_b * SLOT + wave * 32 * kTileKBytes + foff[t];
+      fa[0] = *(const v4i *)ba;
+      fa[1] = *(const v4i *)(ba + 32 * kTileKBytes);
+      fb[0] = *(const v4i *)bb;
+    }
+  };
+
+  // The first fragments of the NEXT output tile, full or short (one sequence of six reads with that tile's bases,
+  // not a branch between two sequences: the fragment registers of two paths would have to meet in one place, and
+  // the register allocation of the whole loop fell apart over that.  A short tile has one fragment of B: its
+  // three surplus reads repeat it.)
+  auto read_frags_next_tile = [&](int slot_a, int slot_b, Frag(&fa)[MT_M], FragB(&fb)[MT_N]) {
+    if constexpr (SHORTS) {
+      const bool ns = is_short[1];
+      const uint8_t *ba = smem + slot_a * SLOT + (ns ? 0u : a_fbase) + foff[0];
+      const uint8_t *bb = smem + slot_b * SLOT + (ns ? (uint32_t)(wave * 32 * kTileKBytes) : b_fbase) + foff[0];
+      const int b_step = ns ? 0 : 32 * kTileKBytes;
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) fa[i] = *(const v4i *)(ba + i * 32 * kTileKBytes);
+#pragma unroll
+      for (int jj = 0; jj < MT_N; ++jj) fb[jj] = *(const v4i *)(bb + jj * b_step);
+    }
+  };
+
   // ---------------- scales (MFMA-native order: one dword per lane, 32 rows and K tile) ----------------
   const int a_srow = ((wave_m * Cfg::WM) >> 5) * k_tiles_blocks, b_srow = ((wave_n * Cfg::WN) >> 5) * k_tiles_blocks;
   const int s_lane = SHUF ? ((lane >> 5) * 16 + (lane & 15)) * 4 : lane * 4;
@@ -291,17 +339,21 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       const int t = a_row32[which] + (lane & 31);
       a_lane = ((t & 31) + (lane & 32)) * 4 + (t >> 5) * k_tiles_blocks;
     }
+    // (a short tile: the blocks of rows 0..63 and of the wave's 32 columns; the three further B requests stay, for
+    // the count of requests in flight, and read blocks that are not used)
+    const int a_sr = SHORTS && is_short[which] ? 0 : a_srow;
+    const int b_sr = SHORTS && is_short[which] ? wave * k_tiles_blocks : b_srow;
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
-      raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256, 0);
+      raw_a[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, a_sr + i * k_tiles_blocks + sblk(kt) * 256, 0);
       if constexpr (SHUF)
-        raw_a2[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, a_srow + i * k_tiles_blocks + sblk(kt) * 256 + 128, 0);
+        raw_a2[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, a_sr + i * k_tiles_blocks + sblk(kt) * 256 + 128, 0);
     }
 #pragma unroll
     for (int j = 0; j < MT_N; ++j) {
-      raw_b[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + sblk(kt) * 256, 0);
+      raw_b[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_sr + j * k_tiles_blocks + sblk(kt) * 256, 0);
       if constexpr (SHUF)
-        raw_b2[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_srow + j * k_tiles_blocks + sblk(kt) * 256 + 128, 0);
+        raw_b2[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rb, s_lane, b_sr + j * k_tiles_blocks + sblk(kt) * 256 + 128, 0);
     }
   };
   // Real register moves, pinned here (a compiler copy would be folded into the
@@ -356,6 +408,24 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       }
     }
   };
+  // short tile: 64 rows x the wave's 32 columns, accumulated in acc[0][0] and acc[1][0]
+  auto mfma_short = [&](const Frag(&fa)[MT_M], const FragB(&fb)[MT_N], auto t_tag, auto zero_tag) {
+    if constexpr (SHORTS) {
+      constexpr int T = decltype(t_tag)::value;
+      constexpr bool ZERO = decltype(zero_tag)::value;
+      const v8i vb = v8i{fb[0].x, fb[0].y, fb[0].z, fb[0].w, 0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const v8i va = v8i{fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
+        v16f c = acc[i][0];
+        if (ZERO) {
+#pragma unroll
+          for (int g = 0; g < 16; ++g) c[g] = 0.f;
+        }
+        acc[i][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, c, 4, 4, T, (int)sc_b[0], T, (int)sc_a[i]);
+      }
+    }
+  };
   typedef std::integral_constant<int, 0> T0;
   typedef std::integral_constant<int, 1> T1;
   typedef std::integral_constant<int, 2> T2;
@@ -396,9 +466,30 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     }
   };
   // PENDING: the C stores of the previous output tile are in the queue (every tile but the first).
-  auto k_tile = [&](int j, int sa, int sb, auto kind_tag, auto pending_tag) {
+  // SHORT: the current output tile is a short tile (its MFMAs and fragment reads; everything else is the same)
+  auto order_phase_short = [&]() {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  };
+  auto k_tile = [&](int j, int sa, int sb, auto kind_tag, auto pending_tag, auto short_tag) {
     constexpr int KIND = decltype(kind_tag)::value;
     constexpr bool PENDING = decltype(pending_tag)::value;
+    constexpr bool SHORT = decltype(short_tag)::value;
+    static_assert(!SHORT || SHORTS, "short tiles: the grouped 8-wave kernel");
+    auto rd = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], FragB(&fb)[MT_N]) {
+      if constexpr (SHORT) read_frags_short(slot_a, slot_b, t, fa, fb);
+      else read_frags(slot_a, slot_b, t, fa, fb);
+    };
+    auto mm = [&](const Frag(&fa)[MT_M], const FragB(&fb)[MT_N], auto t_tag, auto zero_tag) {
+      if constexpr (SHORT) mfma_short(fa, fb, t_tag, zero_tag);
+      else mfma_block(fa, fb, t_tag, zero_tag);
+    };
+    auto order = [&]() {
+      if constexpr (SHORT) order_phase_short();
+      else order_phase();
+    };
     static_assert(TAIL || KIND != kSteadyTail, "kSteadyTail belongs to the TAIL kernels");
     constexpr int W1 = KIND == kBound2 ? 1 : 0;                      // output tile of K tile j+1
     constexpr int W2 = (KIND == kBound1 || KIND == kBound2) ? 1 : 0;  // ... of K tile j+2
@@ -438,23 +529,23 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       __builtin_amdgcn_sched_barrier(0);
       return;
     }
-    read_frags(sa, sb, 1, fa1, fb1);
-    mfma_block(fa0, fb0, T0{}, Zero{});
+    rd(sa, sb, 1, fa1, fb1);
+    mm(fa0, fb0, T0{}, Zero{});
     if (KIND != kFirst) issue_g2l(W1, 1, kt1, sb1, B_LD / 2, B_LD);
     if (TAIL && KIND == kBound1) flip_tail(b_goff);  // the second half of B of the partial K tile is out: back
     if (TAIL && KIND == kSteadyTail) flip_tail(a_goff);
-    order_phase();
+    order();
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(sa, sb, 2, fa0, fb0);
-    mfma_block(fa1, fb1, T1{}, Keep{});
+    rd(sa, sb, 2, fa0, fb0);
+    mm(fa1, fb1, T1{}, Keep{});
     issue_g2l(W2, 0, kt2, sa2, 0, A_LD / 2);
-    order_phase();
+    order();
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(sa, sb, 3, fa1, fb1);
-    mfma_block(fa0, fb0, T2{}, Keep{});
+    rd(sa, sb, 3, fa1, fb1);
+    mm(fa0, fb0, T2{}, Keep{});
     issue_g2l(W2, 0, kt2, sa2, A_LD / 2, A_LD);
     if (TAIL && KIND == kSteadyTail) flip_tail(a_goff), flip_tail(b_goff);  // A back; B until kBound1's first phase
-    order_phase();
+    order();
     __builtin_amdgcn_sched_barrier(0);
     // Everything this wave issued up to B(j+1) has landed.  Younger than that:
     // the A_LD instructions of A(j+2) and, in the first K tile after a
@@ -468,10 +559,15 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(sa1, sb1, 0, fa0, fb0);
-    mfma_block(fa1, fb1, T3{}, Keep{});
+    // the first fragments of the next K tile; at the end of an output tile they are the next tile's, in ITS shape
+    if constexpr (SHORTS && KIND == kBound2) {
+      read_frags_next_tile(sa1, sb1, fa0, fb0);
+    } else {
+      rd(sa1, sb1, 0, fa0, fb0);
+    }
+    mm(fa1, fb1, T3{}, Keep{});
     issue_g2l(W2, 1, kt2, sa, 0, B_LD / 2);
-    order_phase();
+    order();
     __builtin_amdgcn_sched_barrier(0);
     canon_scales(kt1);
     load_scales(W2, kt2);
@@ -590,6 +686,42 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     }
   };
 
+  // A short tile's C: acc[i][0][4q + e] is row 32 i + lane % 32, column 32 wave + 8q + 4 (lane / 32) + e of the tile;
+  // eight stores of 8 or 16 bytes per lane, then as many more beyond the descriptor (dropped, but counted) as
+  // bring the number of store instructions to a full tile's, which the first wait of the next tile counts on.
+  auto store_short = [&](uint8_t *cbase, int ldc, int tn0, int rows) {
+    if constexpr (SHORTS) {
+      constexpr int ELT = OUT_BF16 ? 2 : 4;
+      const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc_n(cbase, (int)min((int64_t)rows * ldc * ELT, (int64_t)0x7FFFFFFF));
+      int lane_v = lane;
+      asm volatile("" : "+v"(lane_v));
+      const int fr = lane_v & 31, fg = lane_v >> 5;
+      const int col0 = tn0 + wave * 32 + fg * 4;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v16f &a = acc[i][0];
+          const int off = ((i * 32 + fr) * ldc + col0 + q * 8) * ELT;
+          if constexpr (OUT_BF16) {
+            typedef __bf16 bf4 __attribute__((ext_vector_type(4)));
+            const bf4 h = {(__bf16)a[4 * q], (__bf16)a[4 * q + 1], (__bf16)a[4 * q + 2], (__bf16)a[4 * q + 3]};
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2i, h), c_rsrc, off, 0, 2);
+          } else {
+            const v4f v = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), c_rsrc, off, 0, 2);
+          }
+        }
+      }
+      // (each to an address of its own, far beyond the descriptor and not next to another: the compiler deletes a
+      // store that a later one overwrites, and joins neighbours into one instruction)
+#pragma unroll
+      for (int d = 8; d < (OUT_BF16 ? NS_BF16 : NS_F32); ++d)
+        __builtin_amdgcn_raw_buffer_store_b32(0, c_rsrc, 0x40000000 + 64 * d, 0, 0);
+      asm volatile("" ::: "memory");
+    }
+  };
+
   // ---------------- prologue of the first tile ----------------
   issue_g2l(0, 0, 0, 0, 0, A_LD);
   issue_g2l(0, 1, 0, 1, 0, B_LD);
@@ -602,7 +734,10 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   asm volatile("" ::: "memory");
   canon_scales(0);
   load_scales(0, 1);
-  read_frags(0, 1, 0, fa0, fb0);
+  bool short_first = false;
+  if constexpr (SHORTS) short_first = is_short[0];
+  if (short_first) read_frags_short(0, 1, 0, fa0, fb0);
+  else read_frags(0, 1, 0, fa0, fb0);
   __builtin_amdgcn_sched_barrier(0);
 
   // ---------------- the tiles ----------------
@@ -614,30 +749,36 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   int sa = 0, part_stage = -1;
   auto next_slot = [&](int s) { return s + 2 >= RING ? s + 2 - RING : s + 2; };
   auto b_slot = [&](int s) { return s + 1 >= RING ? 0 : s + 1; };
-  auto run_tile = [&](auto pending_tag) -> bool {
-    const int npid = pid + (int)gridDim.x;
-    const bool has_next = set_tile(1, npid);
+  // Returns 0: that was the workgroup's last tile; 1: a full tile follows; 2: a short tile follows.
+  auto run_tile = [&](auto pending_tag, auto short_tag) -> int {
+    constexpr bool SHORT = decltype(short_tag)::value;
+    int nstep = step + 1;
+    bool has_next = set_tile(1, id_of(nstep));
+    if constexpr (SHORTS) {
+      while (!has_next && nstep + 1 < walk_items) has_next = set_tile(1, id_of(++nstep));
+    }
     if (!has_next) {
       m0[1] = m0[0], n0[1] = n0[0], a_lim[1] = a_lim[0], as_lim[1] = as_lim[0], c_rows[1] = c_rows[0];
       b_lim[1] = b_lim[0], bs_lim[1] = bs_lim[0];
       nkt_of[1] = nkt_of[0], part_of[1] = part_of[0], tail_on[1] = tail_on[0], a_row32[1] = a_row32[0];
       a_base[1] = a_base[0], b_base[1] = b_base[0], as_base[1] = as_base[0], bs_base[1] = bs_base[0];
+      is_short[1] = is_short[0];
     }
     const int nk = SPLIT ? nkt_of[0] : nkt;  // K tiles of this item
-    k_tile(0, sa, b_slot(sa), std::integral_constant<int, kFirst>{}, pending_tag);
+    k_tile(0, sa, b_slot(sa), std::integral_constant<int, kFirst>{}, pending_tag, short_tag);
     sa = next_slot(sa);
     for (int j = 1; j < nk - (TAIL ? 3 : 2); ++j) {
-      k_tile(j, sa, b_slot(sa), std::integral_constant<int, kSteady>{}, pending_tag);
+      k_tile(j, sa, b_slot(sa), std::integral_constant<int, kSteady>{}, pending_tag, short_tag);
       sa = next_slot(sa);
     }
     if constexpr (TAIL) {  // nk >= 4
-      k_tile(nk - 3, sa, b_slot(sa), std::integral_constant<int, kSteadyTail>{}, pending_tag);
+      k_tile(nk - 3, sa, b_slot(sa), std::integral_constant<int, kSteadyTail>{}, pending_tag, short_tag);
       sa = next_slot(sa);
     }
-    k_tile(nk - 2, sa, b_slot(sa), std::integral_constant<int, kBound1>{}, pending_tag);
+    k_tile(nk - 2, sa, b_slot(sa), std::integral_constant<int, kBound1>{}, pending_tag, short_tag);
     sa = next_slot(sa);
     const int stage_slot = b_slot(sa);
-    k_tile(nk - 1, sa, stage_slot, std::integral_constant<int, kBound2>{}, pending_tag);
+    k_tile(nk - 1, sa, stage_slot, std::integral_constant<int, kBound2>{}, pending_tag, short_tag);
     // second half of B(1) of the next tile, ahead of the C stores (its first
     // half went into slot `sa` in the last phase above)
     if constexpr (!FP8) issue_g2l(1, 1, 1, sa, B_LD / 2, B_LD);
@@ -645,27 +786,42 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     __builtin_amdgcn_sched_barrier(0);
     if (SPLIT && part_of[0] >= 0) {  // a part of a tile of the last round: always the workgroup's last item,
       part_stage = stage_slot;       // stored after the loop (a second store path in here costs the loop registers)
-      return false;
+      return 0;
     }
-    store_tile(stage_slot, (uint8_t *)p.c + (int64_t)m0[0] * p.n * (OUT_BF16 ? 2 : 4), p.n, n0[0], c_rows[0],
-               std::false_type{});
-    if (!has_next) return false;
+    if constexpr (SHORT)
+      store_short((uint8_t *)p.c + (int64_t)m0[0] * p.n * (OUT_BF16 ? 2 : 4), p.n, n0[0], c_rows[0]);
+    else
+      store_tile(stage_slot, (uint8_t *)p.c + (int64_t)m0[0] * p.n * (OUT_BF16 ? 2 : 4), p.n, n0[0], c_rows[0],
+                 std::false_type{});
+    if (!has_next) return 0;
     // the staging slot is the next target of the A stream: all waves must be done reading it
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    pid = npid;
+    step = nstep;
     m0[0] = m0[1], n0[0] = n0[1], a_lim[0] = a_lim[1], as_lim[0] = as_lim[1], c_rows[0] = c_rows[1];
     b_lim[0] = b_lim[1], bs_lim[0] = bs_lim[1];
     nkt_of[0] = nkt_of[1], part_of[0] = part_of[1], tail_on[0] = tail_on[1], a_row32[0] = a_row32[1];
     a_base[0] = a_base[1], b_base[0] = b_base[1], as_base[0] = as_base[1], bs_base[0] = bs_base[1];
-    return true;
+    is_short[0] = is_short[1];
+    return SHORTS && is_short[0] ? 2 : 1;
   };
-  if (run_tile(std::false_type{})) {
-    while (run_tile(std::true_type{})) {
+  int more = 2;
+  if (!short_first) more = run_tile(std::false_type{}, std::false_type{});
+  if constexpr (SHORTS) {
+    if (short_first) {
+      // no tile before this one: as many dropped stores as a tile's, so that the first wait of the first short
+      // tile finds the queue it counts on (one instantiation then serves every short tile)
+      const __amdgpu_buffer_rsrc_t none = make_rsrc_n(p.c, 0);
+#pragma unroll
+      for (int d = 0; d < (OUT_BF16 ? NS_BF16 : NS_F32); ++d) __builtin_amdgcn_raw_buffer_store_b32(0, none, 64 * d, 0, 0);
+      asm volatile("" ::: "memory");
     }
+    while (more != 0) more = more == 2 ? run_tile(std::true_type{}, std::true_type{}) : run_tile(std::true_type{}, std::false_type{});
+  } else {
+    while (more == 1) more = run_tile(std::true_type{}, std::false_type{});
   }
   if (SPLIT && part_stage >= 0)
     store_tile(part_stage, (uint8_t *)(p.tail_partial + (int64_t)part_of[0] * BM * BN), BN, 0, BM, std::true_type{});
@@ -697,7 +853,7 @@ __global__ void __launch_bounds__(256) persist_tail_sum_kernel(const GemmParams 
   const int r = blockIdx.x / (BM / kSumRows), band = blockIdx.x % (BM / kSumRows);
   if (GROUPED && (parts <= 1 || whole + r >= padded)) return;
   int tm, tn;
-  if (!(GROUPED ? map_grouped_tile(p.tile_table, total, p.tiles_n, whole + r, tm, tn)
+  if (!(GROUPED ? map_grouped_tile(p.tile_table, tiles_m, p.tile_table[1], p.tiles_n, whole + r, tm, tn)
                 : map_tile(whole + r, p.tiles_m, p.tiles_n, tm, tn)))
     return;  // a padding id
   int m_first = tm * BM, m_end = p.m;

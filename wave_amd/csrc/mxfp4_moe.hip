@@ -149,15 +149,16 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
 // The M tile table of a grouped GEMM (mxfp4_group_table.h) by a launch of its own.
 __global__ void __launch_bounds__(kAlignThreads) grouped_tile_table_kernel(const GroupTableArgs g) {
   __shared__ int wave_sums[kAlignWaves];
-  __shared__ int carry;
-  build_group_tile_table<kAlignThreads>(g, wave_sums, &carry);
+  __shared__ int carry[2];
+  build_group_tile_table<kAlignThreads>(g, wave_sums, carry);
 }
 
 }  // namespace
 
-hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int64_t total_rows, int32_t *table,
-                                     hipStream_t stream) {
-  grouped_tile_table_kernel<<<1, kAlignThreads, 0, stream>>>(GroupTableArgs{offsets, num_groups, bm, (int)total_rows, table});
+hipError_t launch_grouped_tile_table(const int32_t *offsets, int num_groups, int bm, int short_rows, int64_t total_rows,
+                                     int32_t *table, hipStream_t stream) {
+  grouped_tile_table_kernel<<<1, kAlignThreads, 0, stream>>>(
+      GroupTableArgs{offsets, num_groups, bm, short_rows, (int)total_rows, table});
   return hipGetLastError();
 }
 

@@ -315,6 +315,36 @@ int wave_mxfp4_silu_and_mul_quantize(const void *gate, const void *up, int64_t l
                                      void *q, void *scale, int64_t rows, int64_t n, int scale_layout,
                                      void *hip_stream);
 
+/* The first GEMM of a gated expert MLP with the activation and the quantiser of
+ * the second GEMM's operand fused into its C write: the reference's chain
+ * "gate/up GEMM -> silu_and_mul -> (quantise) -> down GEMM"
+ * (tests/kernel/moe_test.py:113-129; templates/test_kernels.py:74 notes the fused
+ * dynamic quantisation as not done there).  b [num_groups, 2 I, K/2] and its
+ * scales hold each expert's gate projection [I, K] and up projection [I, K]
+ * INTERLEAVED in blocks of 32 rows (wave_mxfp4_interleave_gate_up, once per
+ * weight); n = 2 I.  Instead of C [total_rows, n] the call writes
+ * q [total_rows, I / 2] packed e2m1 and scale (e8m0 per row and 32 columns,
+ * act_scale_layout = WAVE_MXFP4_SCALE_MFMA32, the order the second GEMM reads) of
+ * silu(gate) * up, bit-identical to wave_mxfp4_gemm_grouped (bf16 out) followed
+ * by wave_mxfp4_silu_and_mul_quantize on its two halves.  num_groups = 0 with
+ * offsets = NULL is the dense problem.  Served by the persistent 256x256 kernel
+ * only: I % 128 == 0, K % 256 == 0, K >= 768, more 256x256 tiles than CUs, a
+ * workspace of wave_mxfp4_grouped_workspace_bytes(total_rows, n, k, max(num_groups, 1))
+ * bytes, scales row-major or MFMA32, B row-major; WAVE_MXFP4_ERR_UNSUPPORTED
+ * otherwise (the caller then runs the two calls).  Rows past the last offset
+ * are left untouched, as are the padding rows of an MFMA32 scale tensor. */
+int wave_mxfp4_gemm_gated_quantize(const void *a, const void *a_scale, const void *b, const void *b_scale, void *q,
+                                   void *scale, const int32_t *offsets, int num_groups, int64_t total_rows, int64_t n,
+                                   int64_t k, int a_scale_layout, int b_scale_layout, int act_scale_layout,
+                                   void *workspace, size_t workspace_bytes, void *hip_stream);
+
+/* Row interleave for wave_mxfp4_gemm_gated_quantize: src is [2 * half_rows,
+ * row_bytes] bytes, gate rows first, up rows behind them (packed weights
+ * [2 I, K/2] or their row-major scales [2 I, K/32]); dst receives blocks of 32
+ * rows alternating gate, up, gate, ...  half_rows % 32 == 0.  (No counterpart
+ * in the reference, which keeps the two projections apart.) */
+int wave_mxfp4_interleave_gate_up(const void *src, void *dst, int64_t half_rows, int64_t row_bytes, void *hip_stream);
+
 /* Text for a status code; never NULL (the reference reports errors as
  * exceptions carrying hipGetErrorName/String, runtime.cpp:96-109). */
 const char *wave_mxfp4_status_string(int status);

@@ -8,7 +8,9 @@ from .mxfp4 import (
     dequant,
     e8m0_shuffle,
     e8m0_to_f32,
+    interleave_gate_up,
     mxfp4_gemm,
+    mxfp4_gemm_gated_quantize,
     mxfp4_gemm_grouped,
     moe_align_block_size,
     mxfp4_to_f32,
@@ -26,7 +28,9 @@ __all__ = [
     "dequant",
     "e8m0_shuffle",
     "e8m0_to_f32",
+    "interleave_gate_up",
     "mxfp4_gemm",
+    "mxfp4_gemm_gated_quantize",
     "mxfp4_gemm_grouped",
     "moe_align_block_size",
     "mxfp4_to_f32",

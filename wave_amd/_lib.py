@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # WAVE_MXFP4_LIB points at another build of the same ABI (e.g. an experiment)
 LIB_PATH = os.environ.get("WAVE_MXFP4_LIB") or os.path.join(_HERE, "csrc", "libwave_mxfp4.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 # status codes of include/wave_mxfp4.h
 OK = 0
@@ -64,6 +64,8 @@ EXPORTS = (
     "wave_mxfp4_moe_align_block_size",
     "wave_mxfp4_silu_and_mul",
     "wave_mxfp4_silu_and_mul_quantize",
+    "wave_mxfp4_gemm_gated_quantize",
+    "wave_mxfp4_interleave_gate_up",
     "wave_mxfp4_status_string",
     "wave_mxfp4_last_hip_error",
     "wave_mxfp4_abi_version",
@@ -123,6 +125,10 @@ def load():
     lib.wave_mxfp4_silu_and_mul.restype = i32
     lib.wave_mxfp4_silu_and_mul_quantize.argtypes = [p, p, i64, i64, i32, p, p, i64, i64, i32, p]
     lib.wave_mxfp4_silu_and_mul_quantize.restype = i32
+    lib.wave_mxfp4_gemm_gated_quantize.argtypes = [p, p, p, p, p, p, p, i32, i64, i64, i64, i32, i32, i32, p, sz, p]
+    lib.wave_mxfp4_gemm_gated_quantize.restype = i32
+    lib.wave_mxfp4_interleave_gate_up.argtypes = [p, p, i64, i64, p]
+    lib.wave_mxfp4_interleave_gate_up.restype = i32
     lib.wave_mxfp4_status_string.argtypes = [i32]
     lib.wave_mxfp4_status_string.restype = ctypes.c_char_p
     lib.wave_mxfp4_last_hip_error.argtypes = []

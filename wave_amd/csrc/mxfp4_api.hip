@@ -21,7 +21,7 @@ int record_hip(hipError_t e) {
 inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 inline bool bad_enum(int v, int count) { return v < 0 || v >= count; }
 
-constexpr int kAbiVersion = 9;
+constexpr int kAbiVersion = 10;
 constexpr int64_t kMaxDim = (int64_t)1 << 30;
 
 // Shape checks shared by the dense and grouped entry points.
@@ -757,6 +757,71 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
   const int tv = needs_generic_k(p) ? WAVE_MXFP4_VARIANT_T128x128_W2x2 : v;
   size_grid(tv);
   return record_hip(launch_tile_gemm(p, tv, stream));
+}
+
+int wave_mxfp4_interleave_gate_up(const void *src, void *dst, int64_t half_rows, int64_t row_bytes, void *hip_stream) {
+  if (half_rows < 0 || row_bytes < 0 || half_rows % 32 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (half_rows == 0 || row_bytes == 0) return WAVE_MXFP4_OK;
+  if (!src || !dst) return WAVE_MXFP4_ERR_NULL_POINTER;
+  return record_hip(launch_interleave_rows((const uint8_t *)src, (uint8_t *)dst, half_rows, row_bytes, 32, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp4_gemm_gated_quantize(const void *a, const void *a_scale, const void *b, const void *b_scale, void *q,
+                                   void *scale, const int32_t *offsets, int num_groups, int64_t total_rows, int64_t n,
+                                   int64_t k, int a_scale_layout, int b_scale_layout, int act_scale_layout,
+                                   void *workspace, size_t workspace_bytes, void *hip_stream) {
+  if (num_groups < 0 || num_groups > 65536) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  int rc = check_common(a, a_scale, b, b_scale, q, total_rows, n, k, WAVE_MXFP4_OUT_BF16, a_scale_layout, b_scale_layout,
+                        WAVE_MXFP4_B_ROW_MAJOR, WAVE_MXFP4_VARIANT_AUTO);
+  if (rc <= 0) return rc;
+  if (!scale) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (bad_enum(act_scale_layout, 3)) return WAVE_MXFP4_ERR_BAD_ENUM;
+  if (act_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return WAVE_MXFP4_ERR_UNSUPPORTED;  // (what the next GEMM reads)
+  if (num_groups > 0 && !offsets) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (num_groups > 0 && !aligned(offsets, 4)) return WAVE_MXFP4_ERR_MISALIGNED;
+  const auto rm_or_native = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
+  if (n % 256 != 0 || k % kTileK != 0 || k < 3 * kTileK || !rm_or_native(a_scale_layout) || !rm_or_native(b_scale_layout))
+    return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (!workspace || !aligned(workspace, 256)) return workspace ? WAVE_MXFP4_ERR_MISALIGNED : WAVE_MXFP4_ERR_UNSUPPORTED;
+  hipStream_t stream = (hipStream_t)hip_stream;
+  const int groups = num_groups > 0 ? num_groups : 1;
+  if (workspace_bytes < wave_mxfp4_grouped_workspace_bytes(total_rows, n, k, groups) || (int64_t)groups * n > 0x7FFFFFFF)
+    return WAVE_MXFP4_ERR_UNSUPPORTED;
+
+  GemmParams p;
+  fill_params(p, a, a_scale, b, b_scale, q, total_rows, n, k, WAVE_MXFP4_OUT_BF16, a_scale_layout, b_scale_layout,
+              WAVE_MXFP4_B_ROW_MAJOR);
+  p.epi_scale = (uint8_t *)scale;
+  p.epi_scale_layout = act_scale_layout;
+  p.tiles_m = (int)(num_groups > 0 ? total_rows / 256 + num_groups : (total_rows + 255) / 256);
+  p.tiles_n = (int)(n / 256);
+  int32_t *table = (int32_t *)workspace;
+  uint8_t *ws_a = (uint8_t *)workspace + grouped_table_bytes(total_rows, groups);
+  uint8_t *ws_b = ws_a + grouped_a_scale_bytes(total_rows, k);
+  const bool a_native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32, b_native = b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+  if (num_groups > 0) {
+    p.offsets = offsets;
+    p.num_groups = num_groups;
+    p.b_group_stride = n * (k / 2);
+    p.b_scale_group_stride = b_native ? ((n + 31) / 32 * 32) * (int64_t)p.ksp : n * (int64_t)p.ks;
+    p.tile_table = table;
+  }
+  GemmParams q32 = p;
+  q32.a_scale_layout = q32.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+  if (!persist_gated_applies(q32, device_cus())) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  hipError_t e = hipSuccess;
+  const GroupTableArgs gt{offsets, num_groups, 256, 0, (int)total_rows, table};
+  if (a_native && b_native) {
+    if (num_groups > 0) e = launch_grouped_tile_table(offsets, num_groups, 256, 0, total_rows, table, stream);
+  } else {
+    e = launch_scale_pair_to_mfma32(p.a_scale, ws_a, a_native ? 0 : total_rows, p.b_scale, ws_b,
+                                    b_native ? 0 : (int64_t)groups * n, p.ks, stream, num_groups > 0 ? &gt : nullptr);
+  }
+  if (e != hipSuccess) return e == hipErrorInvalidValue ? WAVE_MXFP4_ERR_UNSUPPORTED : record_hip(e);
+  if (!a_native) q32.a_scale = ws_a;
+  if (!b_native) q32.b_scale = ws_b;
+  q32.b_scale_group_stride = n * (int64_t)p.ksp;
+  return record_hip(launch_persist_gated(q32, device_cus(), stream));
 }
 
 int wave_mxfp4_to_f32(const void *q, float *out, int64_t rows, int64_t kp, void *hip_stream) {

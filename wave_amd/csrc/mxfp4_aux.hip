@@ -203,6 +203,21 @@ __global__ void b_preshuffle_kernel(const uint8_t *__restrict__ b, uint8_t *__re
   }
 }
 
+// Rows of a [2 * half_rows, row_bytes] matrix whose first half is a gate projection and whose second half the
+// matching up projection, interleaved in blocks of `block` rows: out block 2 b = gate rows block b, out block
+// 2 b + 1 = up rows block b.  One thread per 4 bytes (row_bytes % 4 == 0) or per byte.
+template <typename T>
+__global__ void interleave_rows_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t half_rows, int64_t row_units,
+                                       int block) {
+  const int64_t total = 2 * half_rows * row_units;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / row_units, c = i - r * row_units;
+    const int64_t blk = r / block, in = r - blk * block;
+    const int64_t from = (blk & 1 ? half_rows : 0) + (blk >> 1) * block + in;
+    dst[i] = src[from * row_units + c];
+  }
+}
+
 // C = sum over splits of partial[s], converted to the output type.  Fixed
 // summation order, so the result does not depend on scheduling.
 __global__ void splitk_reduce_kernel(const float *__restrict__ partial, void *__restrict__ c, int64_t mn,
@@ -392,6 +407,18 @@ hipError_t launch_b_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int
   const int64_t n = rows * (kp / 16);
   if (n == 0) return hipSuccess;
   b_preshuffle_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(b, out, rows, kp);
+  return hipGetLastError();
+}
+
+hipError_t launch_interleave_rows(const uint8_t *src, uint8_t *dst, int64_t half_rows, int64_t row_bytes, int block,
+                                  hipStream_t stream) {
+  const int64_t n = 2 * half_rows * row_bytes;
+  if (n == 0) return hipSuccess;
+  if (row_bytes % 4 == 0 && ((uintptr_t)src & 3) == 0 && ((uintptr_t)dst & 3) == 0)
+    interleave_rows_kernel<uint32_t><<<blocks_for(n / 4, kThreads), kThreads, 0, stream>>>(
+        (const uint32_t *)src, (uint32_t *)dst, half_rows, row_bytes / 4, block);
+  else
+    interleave_rows_kernel<uint8_t><<<blocks_for(n, kThreads), kThreads, 0, stream>>>(src, dst, half_rows, row_bytes, block);
   return hipGetLastError();
 }
 

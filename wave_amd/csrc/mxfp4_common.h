@@ -53,6 +53,8 @@ struct GemmParams {
   int tiles_m, tiles_n;
   int64_t b_group_stride;        // bytes between experts in b
   int64_t b_scale_group_stride;  // bytes between experts in b_scale
+  uint8_t *epi_scale;            // gated epilogue: the activation's e8m0 scales (c then holds its packed codes)
+  int epi_scale_layout;          // ... their layout (MFMA32)
 };
 
 // e2m1 code -> f32.  Bit 3 is the sign; codes 0..7 are 0, .5, 1, 1.5, 2, 3, 4, 6.
@@ -134,6 +136,10 @@ hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hi
 bool persist_gemm_fp8_applies(const GemmParams &p, int num_cus);
 hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2, int b_fmt, hipStream_t stream);
 bool persist_prefers_192(const GemmParams &p, int num_cus, int parts256);
+bool persist_gated_applies(const GemmParams &p, int num_cus);
+hipError_t launch_persist_gated(const GemmParams &p, int num_cus, hipStream_t stream);
+hipError_t launch_interleave_rows(const uint8_t *src, uint8_t *dst, int64_t half_rows, int64_t row_bytes, int block,
+                                  hipStream_t stream);
 bool asym_gemm_applies(const GemmParams &p, int num_cus, bool forced);
 hipError_t launch_asym_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
 bool midb_gemm_applies(const GemmParams &p);

@@ -93,9 +93,22 @@ enum KtKind {
 // and K tile in the same order as MFMA32; inside a block the four bytes of a lane (row r, K half h: groups 2t + h of
 // the K steps t = 0..3) sit in two dwords, (16h + r % 16) for t = 0, 2 and 32 further on for t = 1, 3, at bytes
 // (r % 32) / 16 and 2 + (r % 32) / 16: two loads and one v_perm where MFMA32 takes one load and a move.
-template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, int FMT_A = 4, int FMT_B = 4, bool SHUF = false>
+// GATED: the step behind the first GEMM of a gated MLP, fused into the C write.  B holds the gate and up projections
+// interleaved in blocks of 32 rows (rows 64 b .. 64 b + 31: gate rows 32 b .., rows 64 b + 32 .. 64 b + 63: up rows
+// 32 b ..), so that a wave's accumulator tiles (i, 2 jp) and (i, 2 jp + 1) hold gate and up of the same 32 rows x 32
+// columns of the activation, element for element in the same lane.  The kernel writes, instead of C [M, N], the
+// MXFP4 quantisation of silu(gate) * up [M, N / 2]: packed e2m1 to p.c ([M, N / 4] bytes) and one e8m0 scale per
+// row and 32 columns to p.epi_scale (MFMA32 order, what the next GEMM reads).  Arithmetic as in the unfused pair of kernels, bit for
+// bit: gate and up rounded to bf16 (the GEMM's output there), silu(g) * u in f32 with the hardware exp2 and
+// reciprocal, rounded to bf16, then the quantiser's scale rule and conversion (mxfp4_quant.hip).  A row's 32
+// columns sit in two lanes (l and l + 32), which exchange their maxima and halves of their codes with
+// v_permlane32_swap.
+template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, int FMT_A = 4, int FMT_B = 4, bool SHUF = false,
+          bool GATED = false>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
   constexpr bool FP8 = FMT_A != 4;
+  static_assert(!GATED || (!FP8 && !TAIL && !SPLIT && OUT_BF16 && Cfg::NWAVES == 8 && Cfg::BN == 256),
+                "gated epilogue: whole K tiles, no cut, the 8-wave 256x256 tiles");
   static_assert(!SHUF || (!FP8 && !GROUPED && !TAIL), "scales in e8m0_shuffle order: dense MXFP4 problems with whole K tiles");
   constexpr bool B4 = FP8 && FMT_B == 4;  // 8-bit A against 4-bit B [N, K/2]: the lower half of B's LDS rows
   static_assert(FMT_A != 4 || FMT_B == 4, "an MXFP4 A against an MXFP8 B is not built");
@@ -113,7 +126,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // in the table) run after all full tiles, with the eight waves side by side on the tile's 64 rows (each 64 x 32:
   // two MFMAs per K step instead of eight).  The operand streams, their waits and the barrier are the full
   // tile's, request for request, so full and short tiles follow each other in any order.
-  constexpr bool SHORTS = GROUPED && !SPLIT && !FP8 && Cfg::NWAVES == 8 && Cfg::BN == 256 && Cfg::WAVES_M == 4;
+  constexpr bool SHORTS = GROUPED && !SPLIT && !FP8 && !GATED && Cfg::NWAVES == 8 && Cfg::BN == 256 && Cfg::WAVES_M == 4;
   const int tiles_m = GROUPED ? __builtin_amdgcn_readfirstlane(p.tile_table[0]) : p.tiles_m;
   const int tiles_full = GROUPED ? __builtin_amdgcn_readfirstlane(p.tile_table[1]) : tiles_m;
   const int total = tiles_m * p.tiles_n;
@@ -448,7 +461,8 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
 
   // C store instructions per wave and tile (1 KB each)
   constexpr int NS_BF16 = Cfg::WM * Cfg::WN * 2 / 1024, NS_F32 = Cfg::WM * Cfg::WN * 4 / 1024;
-  constexpr int kWaitFirstBf16 = NS_BF16 + A_LD > 63 ? 63 : NS_BF16 + A_LD;
+  constexpr int NS_GATED = MT_M * (MT_N / 2) * 2;  // per accumulator pair: one store of codes, one of scale bytes
+  constexpr int kWaitFirstBf16 = GATED ? NS_GATED + A_LD : NS_BF16 + A_LD > 63 ? 63 : NS_BF16 + A_LD;
   constexpr int kWaitFirstF32 = NS_F32 + A_LD > 63 ? 63 : NS_F32 + A_LD;
 
   // ---------------- one K tile (phases as in the one-tile kernel) ----------------
@@ -686,6 +700,83 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     }
   };
 
+  // The gated, quantised C (GATED): see the head of this function.
+  auto store_gated = [&](int tile_m0, int tn0, int rows) {
+    if constexpr (GATED) {
+      typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+      int lane_v = lane;
+      asm volatile("" : "+v"(lane_v));
+      const int fr = lane_v & 31, fg = lane_v >> 5;
+      const int qrow = p.n >> 2;                       // bytes of a row of codes
+      const int act_ks = p.n >> 6;                     // scale groups of a row
+      const __amdgpu_buffer_rsrc_t q_rsrc =
+          make_rsrc_n((uint8_t *)p.c + (int64_t)tile_m0 * qrow, (int)min((int64_t)rows * qrow, (int64_t)0x7FFFFFFF));
+      const int s_kt = (act_ks + 7) >> 3;               // K tiles of the activation (MFMA32 blocks per 32 rows)
+      const __amdgpu_buffer_rsrc_t s_rsrc = make_rsrc_n(p.epi_scale, rsrc_bytes((int64_t)((p.m + 31) >> 5) * s_kt * 256));
+      // (the accumulators are complete here: without this the last K tile's MFMAs are moved down between the
+      // conversions below, with their operand fragments parked in scratch memory)
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i)
+#pragma unroll
+        for (int j = 0; j < MT_N; ++j) asm volatile("" : "+v"(acc[i][j]));
+#pragma unroll
+      for (int i = 0; i < MT_M; ++i) {
+        const int r_tile = wave_m * Cfg::WM + i * 32 + fr;   // row inside the tile
+#pragma unroll
+        for (int jp = 0; jp < MT_N / 2; ++jp) {
+          const v16f &ga = acc[i][2 * jp], &ua = acc[i][2 * jp + 1];
+          uint32_t h[8];
+          uint32_t lo = 0, hi = 0;
+#pragma unroll
+          for (int w = 0; w < 8; ++w) {
+            // the GEMM's bf16 output of the unfused pipeline, then its activation kernel's arithmetic
+            const bf16x2 g2 = {(__bf16)ga[2 * w], (__bf16)ga[2 * w + 1]}, u2 = {(__bf16)ua[2 * w], (__bf16)ua[2 * w + 1]};
+            const uint32_t gb = __builtin_bit_cast(uint32_t, g2), ub = __builtin_bit_cast(uint32_t, u2);
+            const float g0 = __builtin_bit_cast(float, gb << 16), g1 = __builtin_bit_cast(float, gb & 0xFFFF0000u);
+            const float u0 = __builtin_bit_cast(float, ub << 16), u1 = __builtin_bit_cast(float, ub & 0xFFFF0000u);
+            const float r0 = g0 * u0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g0 * -1.44269504088896340736f));
+            const float r1 = g1 * u1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g1 * -1.44269504088896340736f));
+            const bf16x2 o = {(__bf16)r0, (__bf16)r1};
+            h[w] = __builtin_bit_cast(uint32_t, o);
+            lo = max(lo, h[w] & 0x7FFFu);
+            hi = max(hi, (h[w] >> 16) & 0x7FFFu);
+          }
+          // the group's largest magnitude: this lane's 16 columns and the other lane's
+          const uint32_t mine = max(lo, hi);
+          const auto both = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
+          const uint32_t amax = max(both[0], both[1]) << 16;
+          const uint32_t e = (amax + 0x200000u) >> 23;
+          const uint32_t sb = e >= 255u ? 254u : (e > 2u ? e - 2u : 0u);
+          const float sf = __builtin_bit_cast(float, sb ? sb << 23 : 0x00400000u);
+          // codes: dword 0 = columns 8q + 4 fg + 0..3 of q = 0, 1, dword 1 = of q = 2, 3 (two bytes each)
+          uint32_t c0 = 0, c1 = 0;
+          c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[0]), sf, 0);
+          c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[1]), sf, 1);
+          c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[2]), sf, 2);
+          c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[3]), sf, 3);
+          c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[4]), sf, 0);
+          c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[5]), sf, 1);
+          c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[6]), sf, 2);
+          c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[7]), sf, 3);
+          // lanes 0..31 get the upper lanes' dword 0, lanes 32..63 the lower lanes' dword 1: each lane then holds
+          // 8 consecutive bytes of its row's 16 (the lower lanes bytes 0..7, the upper lanes bytes 8..15)
+          const auto sw = __builtin_amdgcn_permlane32_swap(c0, c1, false, false);
+          v2i out;
+          out.x = (int)__builtin_amdgcn_perm(sw[1], sw[0], 0x05040100u);
+          out.y = (int)__builtin_amdgcn_perm(sw[1], sw[0], 0x07060302u);
+          const int g = (tn0 >> 6) + wave_n * (MT_N / 2) + jp;  // the activation's scale group
+          __builtin_amdgcn_raw_buffer_store_b64(out, q_rsrc, r_tile * qrow + g * 16 + fg * 8, 0, 0);
+          // one scale byte per row, from the lower lanes; rows past the tile's own are some other tile's
+          const int r_abs = tile_m0 + r_tile;
+          const int s_off = ((r_abs >> 5) * s_kt + (g >> 3)) * 256 + (((g & 1) << 5) | (r_abs & 31)) * 4 + ((g & 7) >> 1);
+          __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sb, s_rsrc, fg == 0 && r_tile < rows ? s_off : (int)0x80000000, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);  // one pair of accumulator tiles at a time through the vector registers
+        }
+      }
+      asm volatile("" ::: "memory");
+    }
+  };
+
   // A short tile's C: acc[i][0][4q + e] is row 32 i + lane % 32, column 32 wave + 8q + 4 (lane / 32) + e of the tile;
   // eight stores of 8 or 16 bytes per lane, then as many more beyond the descriptor (dropped, but counted) as
   // bring the number of store instructions to a full tile's, which the first wait of the next tile counts on.
@@ -788,7 +879,9 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       part_stage = stage_slot;       // stored after the loop (a second store path in here costs the loop registers)
       return 0;
     }
-    if constexpr (SHORT)
+    if constexpr (GATED)
+      store_gated(m0[0], n0[0], c_rows[0]);
+    else if constexpr (SHORT)
       store_short((uint8_t *)p.c + (int64_t)m0[0] * p.n * (OUT_BF16 ? 2 : 4), p.n, n0[0], c_rows[0]);
     else
       store_tile(stage_slot, (uint8_t *)p.c + (int64_t)m0[0] * p.n * (OUT_BF16 ? 2 : 4), p.n, n0[0], c_rows[0],
@@ -831,6 +924,11 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
 template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, bool SHUF = false>
 __global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_kernel(const GemmParams p) {
   persist_body<Cfg, OUT_BF16, GROUPED, TAIL, SPLIT, 4, 4, SHUF>(p);
+}
+
+template <class Cfg, bool GROUPED>
+__global__ void __launch_bounds__(Cfg::NT, 1) persist_gemm_gated_kernel(const GemmParams p) {
+  persist_body<Cfg, true, GROUPED, false, false, 4, 4, false, true>(p);
 }
 
 template <class Cfg, bool OUT_BF16, int FMT_A, int FMT_B>
@@ -1025,6 +1123,33 @@ hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2,
   if (b_fmt == 2) return a_e5m2 ? launch_persist_fp8_fmt<1, 4>(p, grid, stream) : launch_persist_fp8_fmt<0, 4>(p, grid, stream);
   if (a_e5m2) return b_fmt ? launch_persist_fp8_fmt<1, 1>(p, grid, stream) : launch_persist_fp8_fmt<1, 0>(p, grid, stream);
   return b_fmt ? launch_persist_fp8_fmt<0, 1>(p, grid, stream) : launch_persist_fp8_fmt<0, 0>(p, grid, stream);
+}
+
+// The gated, quantising kernel: the 8-wave 256x256 tiles, dense or grouped by table, whole K tiles, N = twice the
+// activation's width in whole 256-column tiles, MFMA32 scales, more tiles than workgroups.
+bool persist_gated_applies(const GemmParams &p, int num_cus) {
+  if (!p.out_bf16 || p.epi_scale == nullptr || (p.k & (kTileK - 1)) != 0 || p.tail_partial != nullptr || p.tail_parts > 1)
+    return false;
+  if (p.epi_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
+  if ((int64_t)p.m * (p.n >> 6) >= ((int64_t)1 << 31) || (int64_t)((p.m + 31) >> 5) * (((p.n >> 6) + 7) >> 3) * 256 >= ((int64_t)1 << 31))
+    return false;
+  return persist_gemm_applies(p, WAVE_MXFP4_VARIANT_T256x256_W4x2, num_cus);
+}
+
+hipError_t launch_persist_gated(const GemmParams &p, int num_cus, hipStream_t stream) {
+  typedef TileCfg<256, 256, 4, 2> Cfg;
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  static LdsAttrOnce once[2];
+  const bool grouped = p.tile_table != nullptr;
+  const void *fn = grouped ? (const void *)persist_gemm_gated_kernel<Cfg, true> : (const void *)persist_gemm_gated_kernel<Cfg, false>;
+  const hipError_t e = allow_dynamic_lds(once[grouped ? 1 : 0], fn, Cfg::LDS_BYTES);
+  if (e != hipSuccess) return e;
+  if (grouped)
+    persist_gemm_gated_kernel<Cfg, true><<<dim3(grid, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  else
+    persist_gemm_gated_kernel<Cfg, false><<<dim3(grid, 1, 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream>>>(p);
+  return hipGetLastError();
 }
 
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream) {

@@ -496,6 +496,62 @@ def silu_and_mul_quantize(gate: torch.Tensor, up: torch.Tensor, *, scale_layout:
     return q, scales
 
 
+def interleave_gate_up(t: torch.Tensor) -> torch.Tensor:
+    """``[..., 2I, C]`` uint8 (gate rows, then up rows: packed weights or their row-major scales) -> the same shape
+    with blocks of 32 rows alternating gate, up, ...: the weight order :func:`mxfp4_gemm_gated_quantize` takes."""
+    lib = _lib.load()
+    t = _as_u8(t, "t")
+    if t.dim() < 2 or t.shape[-2] % 64 != 0:
+        raise ValueError("expected [..., 2I, C] with I a multiple of 32")
+    out = torch.empty_like(t)
+    flat_in, flat_out = t.reshape(-1, t.shape[-2], t.shape[-1]), out.view(-1, t.shape[-2], t.shape[-1])
+    with _on_device(t.device):
+        for e in range(flat_in.shape[0]):
+            st = lib.wave_mxfp4_interleave_gate_up(flat_in[e].data_ptr(), flat_out[e].data_ptr(), t.shape[-2] // 2,
+                                                   t.shape[-1], _stream_ptr(t.device))
+            _lib.check(st, "wave_mxfp4_interleave_gate_up")
+    return out
+
+
+def mxfp4_gemm_gated_quantize(x, x_scales, w_il, w_scales_il, offsets=None, *, a_scale_layout=_lib.SCALE_ROW_MAJOR,
+                              b_scale_layout=_lib.SCALE_ROW_MAJOR, act_scale_layout=_lib.SCALE_MFMA32, workspace=None):
+    """The first GEMM of a gated expert MLP with :func:`silu_and_mul_quantize` fused into its output: ``w_il``
+    ``[E, 2I, K/2]`` (or ``[2I, K/2]`` with ``offsets=None``: dense) holds gate and up projections interleaved by
+    :func:`interleave_gate_up`, as do its scales.  Returns ``(q [rows, I/2], scales)`` of ``silu(gate) * up``, the
+    same bits as ``mxfp4_gemm_grouped`` (bf16 out) followed by ``silu_and_mul_quantize``.  Raises ``ValueError``
+    (status "unsupported") where the fused kernel does not apply; the caller then runs the two calls."""
+    lib = _lib.load()
+    x, w_il = _as_u8(x, "x"), _as_u8(w_il, "w_il")
+    x_scales, w_scales_il = _as_u8(x_scales, "x_scales"), _as_u8(w_scales_il, "w_scales_il")
+    grouped = offsets is not None
+    if x.dim() != 2 or w_il.dim() != (3 if grouped else 2):
+        raise ValueError("x must be [rows, K/2] and w_il [E, 2I, K/2] (grouped) or [2I, K/2] (dense)")
+    rows, kp = x.shape
+    e = w_il.shape[0] if grouped else 0
+    n = w_il.shape[-2]
+    if w_il.shape[-1] != kp:
+        raise ValueError(f"x and w_il disagree on K/2: {kp} vs {w_il.shape[-1]}")
+    if n % 64 != 0:
+        raise ValueError("w_il: 2I must be a multiple of 64")
+    k, inter = kp * 2, n // 2
+    if grouped and (offsets.dtype != torch.int32 or not offsets.is_cuda or offsets.numel() != e + 1):
+        raise ValueError("offsets: expected a contiguous int32 GPU tensor of E + 1 entries")
+    _scale_rows_ok(x_scales, rows, k // 32, a_scale_layout, "x_scales")
+    q = torch.empty(rows, inter // 2, dtype=torch.uint8, device=x.device)
+    scales = _new_scales(rows, inter // 32, act_scale_layout, x.device)
+    if workspace is None:
+        workspace = _workspace(x.device, int(lib.wave_mxfp4_grouped_workspace_bytes(rows, n, k, max(e, 1))))
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    with _on_device(x.device):
+        st = lib.wave_mxfp4_gemm_gated_quantize(x.data_ptr(), x_scales.data_ptr(), w_il.data_ptr(), w_scales_il.data_ptr(),
+                                                q.data_ptr(), scales.data_ptr(), offsets.data_ptr() if grouped else None,
+                                                e, rows, n, k, a_scale_layout, b_scale_layout, act_scale_layout, ws_ptr,
+                                                ws_bytes, _stream_ptr(x.device))
+    _lib.check(st, "wave_mxfp4_gemm_gated_quantize")
+    return q, scales
+
+
 _FP8_FORMATS = {torch.float8_e4m3fn: _lib.MXFP8_E4M3, torch.float8_e5m2: _lib.MXFP8_E5M2}
 
 

@@ -133,8 +133,11 @@ def test_expert_mlp_chain_with_resident_scale_layouts(size):
     -> gathered quantiser -> grouped GEMM (gate and up) -> gated activation fused into the quantiser -> grouped
     GEMM (down), every scale tensor written or kept in MFMA32 order so that no re-layout launch sits between the
     steps.  Each step against the oracle applied to the device's output of the step before: bytes exact for the
-    quantisers, the GEMMs within the bf16 bound.  "serving": a few rows per expert (mid-M kernel); "prefill": more
-    256x256 tiles than CUs (table-driven persistent kernel, groups starting at rows that are no multiples of 32)."""
+    quantisers, the GEMMs within the bf16 bound.  "serving": a few rows per expert (with activation scales in
+    MFMA32 order that is the one-tile-per-workgroup kernel; the mid-M kernel, which takes row-major activation
+    scales, has the same shapes in test_gpu_grouped_mid.py); "prefill": more 256x256 tiles than CUs (table-driven
+    persistent kernel, groups starting at rows that are no multiples of 32), where the first GEMM with the
+    activation and the quantiser fused into its C write must give the chain's q2 / s2 bit for bit."""
     tokens, topk, experts, hidden, inter = (40, 2, 8, 1024, 2048) if size == "serving" else (2600, 2, 4, 1024, 2048)
     m32 = _lib.SCALE_MFMA32
     rng = np.random.default_rng(31)
@@ -181,6 +184,14 @@ def test_expert_mlp_chain_with_resident_scale_layouts(size):
     want_q2, want_s2 = qo.quantize_mxfp4(stored.float().cpu().numpy())
     assert np.array_equal(q2.cpu().numpy(), want_q2)
     assert np.array_equal(wave_amd.scale_convert(s2, rows, inter // 32, m32, _lib.SCALE_ROW_MAJOR).cpu().numpy(), want_s2)
+    if size == "prefill":
+        # the same three steps as one call: interleaved gate / up weights, activation + quantiser in the C write
+        w1_il = wave_amd.interleave_gate_up(gw1)
+        w1s_il = torch.stack([wave_amd.scale_convert(wave_amd.interleave_gate_up(torch.from_numpy(w1s[e]).to(DEV)), 2 * inter,
+                                                     hidden // 32, _lib.SCALE_ROW_MAJOR, m32) for e in range(experts)])
+        fq2, fs2 = wave_amd.mxfp4_gemm_gated_quantize(q1, s1, w1_il, w1s_il, g_off, a_scale_layout=m32, b_scale_layout=m32)
+        assert np.array_equal(fq2.cpu().numpy(), want_q2)
+        assert np.array_equal(wave_amd.scale_convert(fs2, rows, inter // 32, m32, _lib.SCALE_ROW_MAJOR).cpu().numpy(), want_s2)
     ref_act = mo.silu_and_mul(h1_host[:, :inter], h1_host[:, inter:])
     got_act = stored.float().cpu().numpy().astype(np.float64)
     assert np.abs(got_act - ref_act).max() <= 2.0 ** -7 * max(1.0, np.abs(ref_act).max())

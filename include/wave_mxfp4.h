@@ -155,8 +155,13 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
  * split-K partial sums, the parts of a sparsely filled last round of tiles) is
  * a fixed array of wave_mxfp4_static_scratch_bytes() = 16 MiB inside the
  * library's device image, one per GPU, held until the process ends.  The call
- * allocates and frees nothing.  A problem whose
- * wave_mxfp4_workspace_bytes(m, n, k, split_k, variant) exceeds that size is
+ * allocates and frees nothing, provided wave_mxfp4_static_scratch_bytes() was
+ * called once on that device beforehand (set-up: it looks the array's address
+ * up, which may load the library's code object; without it the first
+ * wave_mxfp4_gemm_static of a device does the lookup itself).  A problem whose
+ * scratch (wave_mxfp4_workspace_bytes(m, n, k, split_k, variant), less the parts
+ * this call's layouts do not use: scale tensors already in MFMA32 order are read
+ * in place) exceeds that size is
  * rejected with WAVE_MXFP4_ERR_WORKSPACE (wave_mxfp4_last_hip_error() then
  * holds the two sizes); 8192^3 needs 6.3 MB.  All calls on one GPU share the
  * array: calls that overlap in time on one GPU (different streams, or threads

@@ -64,3 +64,70 @@ def test_static_scratch_rejects_what_does_not_fit():
     # argument errors come before the size test
     assert lib.wave_mxfp4_gemm_static(None, p, p, p, p, 64, 64, 256, 0, 0, 0, 0, 1, 0, None) == _lib.ERR_NULL_POINTER
     assert lib.wave_mxfp4_gemm_static(p, p, p, p, p, 64, 64, 48, 0, 0, 0, 0, 1, 0, None) == _lib.ERR_BAD_SHAPE
+
+
+def test_static_entry_allocates_nothing_and_replays_from_a_captured_graph():
+    """After the set-up call (wave_mxfp4_static_scratch_bytes, which looks the array's address up) and one call per
+    kernel (which loads it), calls leave the device's free memory where it was; a call captured into a HIP graph
+    replays with the eager bits, with eager calls on the same array between the replays; and a problem of 16384^3
+    whose scales are already in MFMA32 order is not refused for the scratch other layouts of that shape would need."""
+    lib = _lib.load()
+    assert lib.wave_mxfp4_static_scratch_bytes() == 16 << 20
+    m, n, k = 2304, 2048, 1024   # re-laid scales in the scratch, the persistent kernel
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=91, scale_lo=120, scale_hi=134)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    small = torch.empty(64, 256, dtype=torch.float32, device=DEV)
+
+    def call(stream, dst=out):
+        st = lib.wave_mxfp4_gemm_static(gx.data_ptr(), gxs.data_ptr(), gw.data_ptr(), gws.data_ptr(), dst.data_ptr(),
+                                        dst.shape[0], dst.shape[1], k, _lib.OUT_BF16 if dst.dtype == torch.bfloat16 else _lib.OUT_F32,
+                                        0, 0, 0, 0, 0, stream)
+        assert st == _lib.OK, (st, lib.wave_mxfp4_last_hip_error())
+
+    cur = torch.cuda.current_stream().cuda_stream
+    call(cur)
+    call(cur, small)
+    torch.cuda.synchronize()
+    eager = out.clone()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        call(cur)
+        call(cur, small)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the calls changed the device's free memory"
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        call(stream.cuda_stream)
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(stream)
+    for replay in range(3):
+        out.fill_(float("nan"))
+        call(cur, small)   # an eager call on the same array between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {replay}"
+
+    # the size gate counts what the call's own layouts need: at 32768 x 16384 x 16384 row-major scales would be re-laid
+    # into 25 MB of scratch (refused), scales already in MFMA32 order are read in place (served)
+    bm, big = 32768, 16384
+    g = torch.Generator(device=DEV).manual_seed(5)
+    bx = torch.randint(0, 256, (bm, big // 2), dtype=torch.uint8, device=DEV, generator=g)
+    bw = torch.randint(0, 256, (big, big // 2), dtype=torch.uint8, device=DEV, generator=g)
+    bxs = torch.randint(122, 131, (bm, big // 32), dtype=torch.uint8, device=DEV, generator=g)   # any bytes, any order
+    bws = torch.randint(122, 131, (big, big // 32), dtype=torch.uint8, device=DEV, generator=g)
+    got = torch.empty(bm, big, dtype=torch.bfloat16, device=DEV)
+    want = torch.empty(bm, big, dtype=torch.bfloat16, device=DEV)
+    args = (bx.data_ptr(), bxs.data_ptr(), bw.data_ptr(), bws.data_ptr())
+    assert lib.wave_mxfp4_gemm_static(*args, got.data_ptr(), bm, big, big, _lib.OUT_BF16, 0, 0, 0, 1, 0, cur) == _lib.ERR_WORKSPACE
+    m32 = _lib.SCALE_MFMA32
+    assert lib.wave_mxfp4_gemm_static(*args, got.data_ptr(), bm, big, big, _lib.OUT_BF16, m32, m32, 0, 1, 0, cur) == _lib.OK
+    assert lib.wave_mxfp4_gemm(*args, want.data_ptr(), bm, big, big, _lib.OUT_BF16, m32, m32, 0, 1, None, 0, 0, cur) == _lib.OK
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)

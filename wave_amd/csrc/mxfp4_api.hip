@@ -519,7 +519,26 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   return record_hip(e);
 }
 
-size_t wave_mxfp4_static_scratch_bytes(void) { return kStaticScratchBytes; }
+// Also the set-up call: it looks the array's address up for the current device, which may load the library's code
+// object and allocate inside the runtime, so that wave_mxfp4_gemm_static itself never does.
+size_t wave_mxfp4_static_scratch_bytes(void) {
+  void *ignored = nullptr;
+  (void)static_scratch_for_current_device(&ignored);
+  return kStaticScratchBytes;
+}
+
+// Scratch one call needs: wave_mxfp4_workspace_bytes is the most any layout of the same shape can take; scale
+// tensors that come in MFMA32 order are read where they are, and only a_scale_layout PER_ROW spreads rows out.
+static size_t call_scratch_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant, int asl, int bsl) {
+  size_t need = wave_mxfp4_workspace_bytes(m, n, k, split_k, variant);
+  const auto take = [&need](size_t bytes) { need = need > bytes ? need - bytes : 0; };
+  if (asl != WAVE_MXFP4_SCALE_PER_ROW) take(round_up_256((size_t)m * (size_t)(k / 32)));
+  if (wants_mfma32_scales(pick_variant(m, n, k, variant))) {
+    if (asl == WAVE_MXFP4_SCALE_MFMA32) take(round_up_256(scale_buffer_bytes(m, k)));
+    if (bsl == WAVE_MXFP4_SCALE_MFMA32) take(round_up_256(scale_buffer_bytes(n, k)));
+  }
+  return need;
+}
 
 int wave_mxfp4_gemm_static(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c, int64_t m,
                            int64_t n, int64_t k, int out_dtype, int a_scale_layout, int b_scale_layout, int b_layout,
@@ -529,11 +548,11 @@ int wave_mxfp4_gemm_static(const void *a, const void *a_scale, const void *b, co
                               variant);
   if (rc <= 0) return rc;
   if (split_k < 0) return WAVE_MXFP4_ERR_BAD_SPLIT;
-  if (wave_mxfp4_workspace_bytes(m, n, k, split_k, variant) > kStaticScratchBytes) {
+  const size_t need = call_scratch_bytes(m, n, k, split_k, variant, a_scale_layout, b_scale_layout);
+  if (need > kStaticScratchBytes) {
     snprintf(g_hip_error, sizeof(g_hip_error),
              "wave_mxfp4_gemm_static: %lld x %lld x %lld with split_k %d needs %zu bytes of scratch, the static "
-             "buffer holds %zu", (long long)m, (long long)n, (long long)k, split_k,
-             wave_mxfp4_workspace_bytes(m, n, k, split_k, variant), kStaticScratchBytes);
+             "buffer holds %zu", (long long)m, (long long)n, (long long)k, split_k, need, kStaticScratchBytes);
     return WAVE_MXFP4_ERR_WORKSPACE;
   }
   void *scratch = nullptr;

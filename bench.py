@@ -977,10 +977,14 @@ def main():
         wsh = wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_E8M0_SHUFFLE)
         _, sper, _ = time_gemm(torch, wave_amd, [(x, xsh, w, wsh)], out, args.steps, args.warmup,
                                a_scale_layout=L.SCALE_E8M0_SHUFFLE, b_scale_layout=L.SCALE_E8M0_SHUFFLE)
+        _, iper, _ = time_gemm(torch, wave_amd, [(x, xsh, w, wsh)], out, args.steps, args.warmup, workspace=False,
+                               a_scale_layout=L.SCALE_E8M0_SHUFFLE, b_scale_layout=L.SCALE_E8M0_SHUFFLE)
         result["e8m0_shuffled_scales"] = {
-            "workload": "the same operands, scales in the reference's e8m0_shuffle order, read in place (no re-layout launch)",
+            "workload": "the same operands, scales in the reference's e8m0_shuffle order: with scratch (re-laid by one "
+                        "launch, the library's choice), and without (read in place by the persistent kernel)",
             "launch_us": round(sper * 1e6, 2), "tflops": round(flops / sper / 1e12, 1),
             "frac_of_mxfp4_peak": round(flops / sper / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+            "in_place_no_scratch_us": round(iper * 1e6, 2),
         }
         del xsh, wsh
         # roofline: the dominant kernel by itself, i.e. this leg's launches (a call with row-major scales is that

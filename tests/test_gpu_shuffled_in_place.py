@@ -2,8 +2,8 @@
 place (wave_lang/kernel/wave/utils/mxfp_utils.py:113-128; the reference's preshuffled-scale kernel families read
 that format straight from global memory, wave_lang/kernel/wave/templates/tagged_mxfp4_gemm.py:334-403,485-536).
 
-Each case runs without any workspace, so that no re-layout pass can stand in for the in-place read, and is held to
-two bars: rows of every M tile against the exact oracle, and every element bit-equal to the same kernel fed the
+The cases run without any workspace (with one the library re-lays the scales first, which is faster), so that no
+re-layout pass can stand in for the in-place read, and are held to two bars: rows of every M tile against the exact oracle, and every element bit-equal to the same kernel fed the
 same scales in MFMA32 order (the two differ only in how a lane finds its four scale bytes)."""
 
 import numpy as np
@@ -66,13 +66,18 @@ def test_bdirect_kernel_reads_shuffled_scales_in_place(dt):
         check(x, xs, w, ws, dt, shuf, m32, f"B-direct, variant {variant}")
 
 
-def test_sparse_last_round_cut_along_k_with_shuffled_scales():
-    """288 tiles on 256 CUs: with scratch for the parts the last round's 32 tiles are cut along K; the scales are
-    still read in place."""
+def test_with_scratch_the_library_re_lays_shuffled_scales_and_gives_the_same_bits():
+    """With a workspace the call converts the shuffled scales to MFMA32 order first (one 5 us launch costs less than
+    the kernel's doubled scale requests) and may cut a sparse last round along K (288 tiles on 256 CUs); without
+    one it reads them in place.  Same bits either way where the summation order is the same (no cut: K = 1024)."""
     m, n, k = 4608, 4096, 8192
     x, xs, w, ws = orc.make_inputs(m, n, k, seed=12, scale_lo=120, scale_hi=134)
     shuf, m32 = both_layouts(x, xs, w, ws, torch.bfloat16, _lib.VARIANT_T256x256_W4x2, workspace=None)
-    check(x, xs, w, ws, torch.bfloat16, shuf, m32, "cut last round")
+    check(x, xs, w, ws, torch.bfloat16, shuf, m32, "scratch: re-laid, last round cut")
+    x, xs, w, ws = orc.make_inputs(4100, 4096, 1024, seed=13, scale_lo=120, scale_hi=134)
+    with_ws, _ = both_layouts(x, xs, w, ws, torch.float32, _lib.VARIANT_T256x256_W4x2, workspace=None)
+    without, _ = both_layouts(x, xs, w, ws, torch.float32, _lib.VARIANT_T256x256_W4x2, workspace=False)
+    assert np.array_equal(with_ws, without)
 
 
 def test_nan_and_extreme_scales_stay_in_their_rows_and_columns():

@@ -394,10 +394,14 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
                            k % kTileK == 0 &&
                            p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
   // Both tensors in e8m0_shuffle order, the reference's preshuffled format (tagged_mxfp4_gemm.py:334-403,485-536):
-  // the 8-wave persistent kernels read it in place (two dwords and a byte permute per lane instead of one dword),
-  // so a caller that holds its operands the reference's way pays no re-layout launch.
+  // the 8-wave persistent kernels can read it in place (two dwords and a byte permute per lane instead of one
+  // dword), which a caller without scratch gets.  With scratch the re-layout launch stays: the kernel's scale
+  // requests are not free (twelve per wave and K tile instead of six: 8192^3 251.9 against 243.9 us), and at
+  // 5.2 us the launch costs less than they do.
+  const size_t relayout_bytes = round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
   bool shuffled_in_place = false;
   if (p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && p.b_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE && splits == 1 &&
+      !(workspace && ws_used + relayout_bytes <= workspace_bytes) &&
       (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 || v == WAVE_MXFP4_VARIANT_T256x192_W4x2 ||
        v == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT)) {
     GemmParams q = p;

@@ -998,12 +998,9 @@ template <class Cfg, bool OUT_BF16>
 static hipError_t launch_persist_dense(const GemmParams &p, int grid_x, hipStream_t stream) {
   const bool tail = (p.k & (kTileK - 1)) != 0;
   if constexpr (Cfg::NWAVES == 8) {
-    if (p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE) {  // (both tensors, whole K tiles: persist_gemm_applies)
-      if constexpr (Cfg::BN == 256) {
-        if (p.tail_parts > 1) return launch_persist_out<Cfg, OUT_BF16, false, false, true, true>(p, grid_x, stream);
-      }
+    // (both tensors, whole K tiles: persist_gemm_applies; a call without scratch, so no cut of the last round)
+    if (p.a_scale_layout == WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
       return launch_persist_out<Cfg, OUT_BF16, false, false, false, true>(p, grid_x, stream);
-    }
   }
   if constexpr (Cfg::NWAVES == 8 && Cfg::BN == 256) {  // (the 4-wave kernel has no registers to spare for the split bookkeeping)
     if (p.tail_parts > 1)

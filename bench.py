@@ -592,6 +592,9 @@ def main():
                          "expert, the mid-M kernel beside the tile kernels; moe_layer: one mixture-of-experts MLP end to end "
                          "(alignment, gathered quantiser, grouped GEMM, gated quantiser, grouped GEMM), step by step and whole")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
+    ap.add_argument("--resident-scales", action="store_true",
+                    help="decode_sweep: both scale tensors handed over in MFMA32 order (no re-layout launch for any kernel)")
+    ap.add_argument("--preshuffled-b", action="store_true", help="decode_sweep: B in b_preshuffle order")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-legs", "--no-decode", dest="no_legs", action="store_true",
                     help="cfg2 only: skip the legs beside the headline (decode shapes, quantiser, cfg4, cfg5, mxfp8)")
@@ -695,24 +698,42 @@ def main():
 
         SETTLE["ms"] = 20.0
         rows = []
+        # --resident-scales: both scale tensors handed over in MFMA32 order (static weights, activations from the
+        # quantiser), where no kernel needs a re-layout launch and the library's choice follows other borders;
+        # --preshuffled-b on top: B in b_preshuffle order, the B-direct mid-M kernel among the candidates
+        resident, pre = args.resident_scales, args.preshuffled_b
+        grid_n = (12288, 14336, 20480, 28672, 40960, 57344) if resident else (8192, 14336, 28672, 57344)
+        grid_m = (16, 32, 48, 64, 96, 128, 192, 256) if resident else (1, 16, 32, 64, 128, 256)
+        kw = {}
+        if resident:
+            kw.update(a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32)
+        if pre:
+            kw.update(b_layout=L.B_PRESHUFFLE)
         for k in (8192, 4096):
-            for n in (8192, 14336, 28672, 57344):
-                for m in (1, 16, 32, 64, 128, 256):
+            for n in grid_n:
+                for m in grid_m:
                     copies = max(2, min(6, int(600e6 / (n * k / 2))))
                     sets = make_gpu_inputs(torch, m, n, k, 2, (120, 134), dev, copies=copies)
+                    if resident or pre:
+                        sets = [(x, wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32) if resident else xs,
+                                 wave_amd.b_preshuffle(w) if pre else w,
+                                 wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32) if resident else ws)
+                                for x, xs, w, ws in sets]
                     out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
                     us = {}
                     names = [("mid", L.VARIANT_MID_M, 1)]
                     if m <= 64:
                         names.append(("stream", L.VARIANT_SKINNY, 1))
-                    else:
+                    if m > 64 or (resident and m >= 32):
                         names += [("t128x128", L.VARIANT_T128x128_W2x2, 0), ("t128x256", L.VARIANT_T128x256_W2x2, 0),
                                   ("t256x256", L.VARIANT_T256x256_W4x2, 0)]
+                    if pre and k % (2048 if m <= 128 else 1024) == 0:
+                        names.append(("midb", L.VARIANT_MID_M_BDIRECT, 1))
                     # (the library's choice is timed first and last and the shorter time kept: right behind the
                     # power-hungry tile kernels the same launch reads up to 5 % long)
                     names = [("auto", L.VARIANT_AUTO, 0)] + names + [("auto", L.VARIANT_AUTO, 0)]
                     for name, v, split in names:
-                        _, per, _ = time_gemm(torch, wave_amd, sets, out, min(args.steps, 100), 20, variant=v, split_k=split)
+                        _, per, _ = time_gemm(torch, wave_amd, sets, out, min(args.steps, 100), 20, variant=v, split_k=split, **kw)
                         us[name] = min(us.get(name, 1e9), round(per * 1e6, 2))
                     nbytes = gemm_bytes(m, n, k, 2)
                     rows.append({"m": m, "n": n, "k": k, "us": us, "bytes": nbytes,
@@ -725,7 +746,9 @@ def main():
             "ms_per_step": round(sum(r["us"]["auto"] for r in rows) * 1e-3, 3),
             "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out",
             "data": "synthetic (seeded uniform nibbles and scales), weights from HBM",
-            "config": {"workload": f"decode_sweep: {len(rows)} shapes M x N x K, bf16 out, seed 2"}, "shapes": rows})))
+            "config": {"workload": f"decode_sweep: {len(rows)} shapes M x N x K, bf16 out, seed 2" +
+                       (", both scale tensors in MFMA32 order" if resident else ", row-major scales") +
+                       (", B in b_preshuffle order" if pre else "")}, "shapes": rows})))
         return
 
     if args.workload == "moe_serving":

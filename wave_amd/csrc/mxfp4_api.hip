@@ -66,7 +66,11 @@ void fill_params(GemmParams &p, const void *a, const void *as, const void *b, co
   p.b_preshuffled = bl == WAVE_MXFP4_B_PRESHUFFLE;
 }
 
-int pick_tile_variant(int64_t m, int64_t n) {
+int pick_tile_variant(int64_t m, int64_t n, bool native_scales) {
+  // One tile row of at most 128 rows, both scale tensors already in MFMA32 order: 256-row tiles would be half
+  // empty, and up to two 128x128 workgroups per CU run side by side (weights from HBM: 128 x 57344 x 8192 68.1 us
+  // on 256x256 tiles, 59.9 on 128x128; 64 x 57344 x 4096: 34.5 against 28.1 us).  Measured up to N = 65536.
+  if (native_scales && m <= 128 && n <= 65536) return WAVE_MXFP4_VARIANT_T128x128_W2x2;
   const int64_t t256 = ((m + 255) / 256) * ((n + 255) / 256);
   // 8 waves: measured 4-5 % ahead of 4 at 8192^3.  Up to 128 tiles of 256x256 leave half the CUs idle; the same
   // problem as up to 512 tiles of 128x128 fills them with two workgroups each (1024 x 8192 x 16384: 87 -> 82 us).
@@ -108,7 +112,7 @@ bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
   return m >= 1 && m <= mid_max_m() && k % kTileK == 0 && k >= 4 * kTileK && n % 4 == 0;
 }
 
-int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
+int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scales, bool b_preshuffled) {
   int v = variant;
   if (v == WAVE_MXFP4_VARIANT_AUTO) {
     // Reading B once from HBM bounds these problems, and the mid-M kernel gives B and A rings of their own.
@@ -132,10 +136,36 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant) {
                        : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096)
                        : m > 16 ? n >= 12288 && n <= 320 * cus
                                 : n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus);
+      // Both scale tensors already in MFMA32 order (static weights, activations from the quantiser): no kernel
+      // needs a re-layout launch in front, and the mid-M kernel cannot narrow its strips (a wave's strip is a
+      // 32-row scale block), which moves some borders.  Measured with the weights from HBM on a grid of M = 16 ..
+      // 256, N = 12288 .. 57344, K = 4096 / 8192 (us, mid-M -> the kernel taken instead):
+      //   16 < M <= 48 at K >= 8192 up to N = 16384: the streaming kernel (32 x 12288: 17.4 -> 14.6, 48 x 12288:
+      //     19.3 -> 17.8, 32 x 14336: 17.7 -> 16.5; at N = 20480 the mid-M kernel leads, 18.9 against 20.2)
+      //   M <= 64 at K >= 8192 with a second round of strips that is at most a quarter full: the streaming kernel
+      //     (32 x 40960: 35.6 -> 33.4, 48 x 40960: 40.6 -> 37.1; preshuffled B: 40.5 -> 34.7, 45.1 -> 38.0;
+      //     at N = 57344, three quarters full, the mid-M kernel leads again, 40.4 against 45.8)
+      //   48 <= M <= 128 at K <= 4096 between one and two rounds of strips, B row-major: the 128x128 tiles
+      //     (48 x 40960 x 4096: 25.0 -> 23.1, 128 x 40960: 29.2 -> 27.9, 96 x 57344: 31.0 -> 29.3)
+      //   128 < M <= 192 at K <= 4096 up to N = 16384: the tiles (192 x 12288 x 4096: 16.5 -> 13.9)
+      // (With one operand set that stays in the 256 MB memory-side cache the tile kernels look 10-30 % better than
+      // this on most of the grid; the borders above are for weights that come from HBM.)
+      if (mid && native_scales) {
+        const int64_t strips = (n + 127) / 128;
+        const bool second_round = strips > cus && strips <= 2 * cus;
+        // (K = 8192: the streaming kernel's longest K range without a split; up to 16 rows it also leads at
+        // K = 4096 on that quarter-full second round, 16 x 40960 x 4096: 19.2 -> 17.4, preshuffled B 21.4 -> 17.6)
+        const bool k_whole = k >= 8192 && k <= (int64_t)kTileK * stream_max_k_tiles();
+        if ((k_whole && m > 16 && m <= 48 && strips <= 128) ||
+            ((k_whole || m <= 16) && m <= 64 && second_round && 4 * strips <= 5 * cus))
+          return WAVE_MXFP4_VARIANT_SKINNY;
+        if (k <= 4096 && ((m >= 48 && m <= 128 && second_round && !b_preshuffled) || (m > 128 && m <= 192 && strips <= 128)))
+          return pick_tile_variant(m, n, true);
+      }
       if (mid) return WAVE_MXFP4_VARIANT_MID_M;
     }
     if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;
-    v = pick_tile_variant(m, n);
+    v = pick_tile_variant(m, n, native_scales);
   }
   return v;
 }
@@ -270,9 +300,7 @@ static size_t scale_buffer_bytes(int64_t rows, int64_t k) {
 }
 static size_t round_up_256(size_t v) { return (v + 255) / 256 * 256; }
 
-size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant) {
-  if (m <= 0 || n <= 0 || k <= 0 || split_k < 0 || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_)) return 0;
-  const int v = pick_variant(m, n, k, variant);
+static size_t workspace_bytes_of(int64_t m, int64_t n, int64_t k, int split_k, int v) {
   size_t bytes = round_up_256((size_t)m * (size_t)(k / 32));  // per-row A scales spread out to [M, K/32]
   if (v == WAVE_MXFP4_VARIANT_NAIVE) return bytes;
   int splits = split_k;
@@ -293,6 +321,14 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
   return bytes;
 }
 
+size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant) {
+  if (m <= 0 || n <= 0 || k <= 0 || split_k < 0 || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_)) return 0;
+  // the library's own choice of kernel depends on the scale layouts of the call: the larger of the two
+  const size_t plain = workspace_bytes_of(m, n, k, split_k, pick_variant(m, n, k, variant, false, false));
+  const size_t native = workspace_bytes_of(m, n, k, split_k, pick_variant(m, n, k, variant, true, false));
+  return plain > native ? plain : native;
+}
+
 int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
                     int64_t m, int64_t n, int64_t k, int out_dtype, int a_scale_layout,
                     int b_scale_layout, int b_layout, int split_k, void *workspace,
@@ -305,15 +341,23 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
 
   GemmParams p;
   fill_params(p, a, a_scale, b, b_scale, c, m, n, k, out_dtype, a_scale_layout, b_scale_layout, b_layout);
-  int v = pick_variant(m, n, k, variant);
+  const bool native_scales = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+  int v = pick_variant(m, n, k, variant, native_scales, b_layout == WAVE_MXFP4_B_PRESHUFFLE);
   if (variant == WAVE_MXFP4_VARIANT_AUTO && v == WAVE_MXFP4_VARIANT_MID_M && split_k > 1)  // (it takes whole K ranges)
-    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
+    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n, native_scales);
   if (v == WAVE_MXFP4_VARIANT_SKINNY && m > skinny_max_m()) return WAVE_MXFP4_ERR_UNSUPPORTED;
   // the fallback of the library's own choice of the B-direct mid-M kernel, should the scales not reach MFMA32 order
   const int v_plain = v;
   // (measured at N = 28672, K = 8192 against the strip kernel on the same preshuffled B: M = 256 45.8 -> 43.1 us;
-  // at M = 128 the two tie, 28.6 / 28.8 us, and the strip kernel needs neither K in whole turns nor MFMA32 scales)
-  if (variant == WAVE_MXFP4_VARIANT_AUTO && m > 128 && n >= 12288 && split_k <= 1 && midb_shape_ok(m, n, k, b_layout))
+  // past one round of strips the 256x256 tiles lead, 256 x 40960 x 8192: 74.0 against 65.6.
+  // Up to 128 rows the strip kernel needs neither K in whole turns nor MFMA32 scales; with both scale tensors
+  // already in MFMA32 order the B-direct kernel leads there too, weights from HBM: 128 x 28672 x 8192 32.7 -> 28.1,
+  // 128 x 20480 29.5 -> 24.4, 96 x 20480 x 4096 15.4 -> 13.5, 48 x 20480 x 8192 23.6 -> 20.7, 128 x 57344 x 8192
+  // 63.4 -> 54.9; at N <= 16384, K = 8192 the streaming kernel keeps M < 64: 32 x 12288 14.9 against 18.4.)
+  const int64_t cus_n = 128 * (int64_t)device_cus();  // columns of one round of strips
+  if (variant == WAVE_MXFP4_VARIANT_AUTO && n >= 12288 && split_k <= 1 && midb_shape_ok(m, n, k, b_layout) &&
+      (m > 128 ? n <= cus_n
+               : native_scales && n <= 2 * cus_n && (m >= 64 || (m >= 32 && n <= cus_n && (n >= 20480 || k <= 4096)))))
     v = WAVE_MXFP4_VARIANT_MID_M_BDIRECT;
   if (variant == WAVE_MXFP4_VARIANT_MID_M_BDIRECT) {
     const bool native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
@@ -461,12 +505,12 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     // (the library's own choice without scratch for the scales, or offsets beyond 32 bits: the kernels that
     // served these shapes before)
     if (variant == WAVE_MXFP4_VARIANT_MID_M) return WAVE_MXFP4_ERR_UNSUPPORTED;
-    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n);
+    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n, native_scales);
   }
   if (v == WAVE_MXFP4_VARIANT_MID_M_BDIRECT && !midb_gemm_applies(p)) {
     if (variant == WAVE_MXFP4_VARIANT_MID_M_BDIRECT) return WAVE_MXFP4_ERR_UNSUPPORTED;
     v = v_plain == WAVE_MXFP4_VARIANT_MID_M && !mid_gemm_applies(p)
-            ? (m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n))
+            ? (m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n, native_scales))
             : v_plain;
   }
   const int vv = v;
@@ -537,7 +581,8 @@ static size_t call_scratch_bytes(int64_t m, int64_t n, int64_t k, int split_k, i
   size_t need = wave_mxfp4_workspace_bytes(m, n, k, split_k, variant);
   const auto take = [&need](size_t bytes) { need = need > bytes ? need - bytes : 0; };
   if (asl != WAVE_MXFP4_SCALE_PER_ROW) take(round_up_256((size_t)m * (size_t)(k / 32)));
-  if (wants_mfma32_scales(pick_variant(m, n, k, variant))) {
+  const bool native_scales = asl == WAVE_MXFP4_SCALE_MFMA32 && bsl == WAVE_MXFP4_SCALE_MFMA32;
+  if (wants_mfma32_scales(pick_variant(m, n, k, variant, native_scales, false))) {
     if (asl == WAVE_MXFP4_SCALE_MFMA32) take(round_up_256(scale_buffer_bytes(m, k)));
     if (bsl == WAVE_MXFP4_SCALE_MFMA32) take(round_up_256(scale_buffer_bytes(n, k)));
   }
@@ -705,8 +750,8 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
       return record_hip(launch_mid_gemm(p, device_cus(), stream, (int)bm));
     }
   }
-  const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_tile_variant(total_rows > 64 ? total_rows : 65, n)
-                                                   : pick_variant(total_rows, n, k, variant);
+  const int v = variant == WAVE_MXFP4_VARIANT_AUTO ? pick_tile_variant(total_rows > 64 ? total_rows : 65, n, false)
+                                                   : pick_variant(total_rows, n, k, variant, false, false);
   if (v == WAVE_MXFP4_VARIANT_NAIVE) return record_hip(launch_naive_gemm(p, stream));
   int bm, bn;
   auto size_grid = [&](int tile_variant) {

@@ -211,15 +211,16 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
 size_t wave_mxfp4_grouped_workspace_bytes(int64_t total_rows, int64_t n, int64_t k, int num_groups);
 
 /* Element format of the MXFP8 operands (OCP MX: e4m3 is the "fn" variant without
- * infinities, e5m2 is IEEE-like).  WAVE_MXFP8_B_E2M1 is for b_format only: 8-bit
- * activations against MXFP4 weights, B [N, K/2] packed as in wave_mxfp4_gemm. */
-typedef enum { WAVE_MXFP8_E4M3 = 0, WAVE_MXFP8_E5M2 = 1, WAVE_MXFP8_B_E2M1 = 2 } wave_mxfp8_format;
+ * infinities, e5m2 is IEEE-like).  WAVE_MXFP8_E2M1 (= WAVE_MXFP8_B_E2M1, its older name) marks one operand, A or
+ * B but not both, as MXFP4: [rows, K/2] packed as in wave_mxfp4_gemm, against an 8-bit other operand. */
+typedef enum { WAVE_MXFP8_E4M3 = 0, WAVE_MXFP8_E5M2 = 1, WAVE_MXFP8_B_E2M1 = 2, WAVE_MXFP8_E2M1 = 2 } wave_mxfp8_format;
 
 /* The same block-scaled GEMM on MXFP8 operands: A [M, K] of a_format and
  * B [N, K] of b_format, one byte per element (the formats may differ: cbsz /
- * blgp 0 / 1 of the instruction; b_format WAVE_MXFP8_B_E2M1: B [N, K/2], two e2m1
- * per byte, blgp 4 - the mixed operand types the reference's scaled MMA admits,
- * wave_lang/kernel/wave/constraints.py:425-431), scales [R, K/32] e8m0 row-major,
+ * blgp 0 / 1 of the instruction; WAVE_MXFP8_E2M1 for one of them: that operand [rows, K/2], two e2m1
+ * per byte, cbsz / blgp 4 - the mixed operand types the reference's scaled MMA admits in either order,
+ * wave_lang/kernel/wave/constraints.py:425-431; both e2m1 is wave_mxfp4_gemm's and WAVE_MXFP4_ERR_UNSUPPORTED here),
+ * scales [R, K/32] e8m0 row-major,
  * C f32 or bf16.  Replaces the kernel of tests/kernel/wave_gemm_mxfp_test.py:416-501
  * (tkl.f8e5m2 operands through the same scaled MFMA).  K % 128 == 0; variant
  * AUTO, T256x256_W2x2, T256x256_W4x2 or T128x128_W2x2.  `workspace` is optional scratch of

@@ -20,7 +20,7 @@ import numpy as np
 from .mxfp4_oracle import SCALE_GROUP_SIZE, e8m0_to_f32, mxfp4_to_f32
 
 E4M3, E5M2 = 0, 1
-E2M1 = 2   # second operand only: packed MXFP4 weights [N, K/2] against 8-bit activations (the mixed operand
+E2M1 = 2   # one operand of the two: packed MXFP4 [rows, K/2] against an 8-bit other (the mixed operand
            # types of the scaled MMA, wave_lang/kernel/wave/constraints.py:425-431; the reference holds no test of
            # it, the restatement is the composition of the two pinned decodes and the same f64 product)
 
@@ -55,13 +55,15 @@ def fp8_to_f64(x: np.ndarray, fmt: int) -> np.ndarray:
 def scaled_gemm_mxfp8(x, w_t, x_scales, w_scales, fmt) -> np.ndarray:
     """x [M, K], w_t [N, K] uint8 codes, scales [R, K/32] e8m0 -> C [M, N] float64
     (tests/kernel/wave_gemm_mxfp_test.py:80-91 with w_t = w.T).  ``fmt`` is one
-    format for both operands or a pair (x format, w_t format)."""
+    format for both operands or a pair (x format, w_t format); an E2M1 operand is
+    [rows, K/2] packed, decoded by the MXFP4 oracle's table."""
     fmt_x, fmt_w = fmt if isinstance(fmt, (tuple, list)) else (fmt, fmt)
     xs = e8m0_to_f32(np.asarray(x_scales, dtype=np.uint8)).astype(np.float64).repeat(SCALE_GROUP_SIZE, axis=1)
     ws = e8m0_to_f32(np.asarray(w_scales, dtype=np.uint8)).astype(np.float64).repeat(SCALE_GROUP_SIZE, axis=1)
-    a = fp8_to_f64(x, fmt_x) * xs
-    b = (mxfp4_to_f32(np.asarray(w_t, dtype=np.uint8)).astype(np.float64) if fmt_w == E2M1 else fp8_to_f64(w_t, fmt_w)) * ws
-    return a @ b.T
+    def decode(codes, f):
+        return mxfp4_to_f32(np.asarray(codes, dtype=np.uint8)).astype(np.float64) if f == E2M1 else fp8_to_f64(codes, f)
+
+    return (decode(x, fmt_x) * xs) @ (decode(w_t, fmt_w) * ws).T
 
 
 def make_inputs_mxfp8(m, n, k, seed, fmt, scale_lo=124, scale_hi=127):
@@ -82,7 +84,10 @@ def make_inputs_mxfp8(m, n, k, seed, fmt, scale_lo=124, scale_hi=127):
         lower = (v - vals[idx - 1]) <= (vals[idx] - v)
         return codes[np.where(lower, idx - 1, idx)]
 
-    x = quantise(rng.standard_normal((m, k)), fmt_x)
+    if fmt_x == E2M1:
+        x = rng.integers(0, 256, size=(m, k // 2), dtype=np.uint8)
+    else:
+        x = quantise(rng.standard_normal((m, k)), fmt_x)
     if fmt_w == E2M1:   # uniform nibbles, as the MXFP4 generator draws them
         w_t = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
     else:

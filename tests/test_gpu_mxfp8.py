@@ -99,6 +99,50 @@ def test_mxfp8_activations_against_mxfp4_weights(m, n, k, vname, fmt_x):
     assert_f32_close(run(x, xs, w_t, ws, fmt, variant=VARIANTS[vname]), ref, f"{vname} {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("fmt_w", [o8.E5M2, o8.E4M3], ids=["e5m2", "e4m3"])
+@pytest.mark.parametrize("vname", sorted(VARIANTS))
+@pytest.mark.parametrize("m,n,k", [(128, 128, 128), (256, 256, 512), (300, 200, 384), (1, 40, 256), (257, 33, 1152),
+                                   (1024, 1024, 1024)])
+def test_mxfp4_activations_against_mxfp8_weights(m, n, k, vname, fmt_w):
+    """Packed e2m1 A [M, K/2] against 8-bit B: the other order of the mixed operand types
+    (wave_lang/kernel/wave/constraints.py:425-431; the reference holds no test of either)."""
+    fmt = (o8.E2M1, fmt_w)
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=m + n + k + 5, fmt=fmt, scale_lo=120, scale_hi=134)
+    assert x.shape == (m, k // 2) and w_t.shape == (n, k)
+    ref = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, fmt)
+    assert_f32_close(run(x, xs, w_t, ws, fmt, variant=VARIANTS[vname]), ref, f"{vname} {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_mxfp4_against_mxfp8_one_hot_and_more_tiles_than_cus(out_dtype):
+    """One-hot rows of B (1.0 at one position, scale 1) read back columns of dequantised A exactly (every e2m1
+    value times a power of two is a bf16 number), on 272 tiles: the persistent kernel with the scratch buffer."""
+    m, n, k = 4352, 4096, 512
+    fmt = (o8.E2M1, o8.E5M2)
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=4, fmt=fmt, scale_lo=118, scale_hi=136)
+    w_t[:] = 0
+    ws[:] = 127
+    one = int(np.nonzero(o8.E5M2_TABLE == 1.0)[0][0])
+    pos = (np.arange(n) * 37) % k
+    w_t[np.arange(n), pos] = one
+    c = run(x, xs, w_t, ws, fmt, out_dtype=out_dtype)
+    from oracle import mxfp4_oracle as o4
+    a = o4.mxfp4_to_f32(x).astype(np.float64) * o4.e8m0_to_f32(xs).astype(np.float64).repeat(32, axis=1)
+    assert np.array_equal(c, a[:, pos].astype(np.float32))
+
+
+def test_both_operands_e2m1_is_refused():
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(64, 64, 256, seed=1, fmt=(o8.E2M1, o8.E2M1))
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    out = torch.empty(64, 64, dtype=torch.float32, device=DEV)
+    with pytest.raises(ValueError):
+        wave_amd.mxfp8_gemm(gx, gxs, gw, gws, out, elem_format=(o8.E2M1, o8.E2M1))
+    lib = _lib.load()
+    st = lib.wave_mxfp8_gemm(gx.data_ptr(), gxs.data_ptr(), gw.data_ptr(), gws.data_ptr(), out.data_ptr(), 64, 64, 256,
+                             _lib.MXFP8_E2M1, _lib.MXFP8_E2M1, 0, None, 0, 0, None)
+    assert st == _lib.ERR_UNSUPPORTED
+
+
 def test_mxfp8_against_mxfp4_one_hot_and_more_tiles_than_cus():
     """One-hot rows of A (1.0 at one position, scale 1) read back columns of dequantised B exactly, on 272 tiles
     (the persistent kernel with the scratch buffer, one tile per workgroup without: the same bits)."""
@@ -191,7 +235,8 @@ def test_mxfp8_argument_errors():
         ("ws", None), ("wsb", 0), ("variant", 0), ("stream", None))])
     assert g(k=192) == _lib.ERR_BAD_SHAPE
     assert g(m=-1) == _lib.ERR_BAD_SHAPE
-    assert g(fmt=2) == _lib.ERR_BAD_ENUM
+    assert g(fmt=3) == _lib.ERR_BAD_ENUM
+    assert g(fmt=2, fmt_b=2) == _lib.ERR_UNSUPPORTED   # (both e2m1: the MXFP4 entry point's)
     assert g(fmt_b=-1) == _lib.ERR_BAD_ENUM
     assert g(od=3) == _lib.ERR_BAD_ENUM
     assert g(variant=_lib.VARIANT_SKINNY) == _lib.ERR_UNSUPPORTED

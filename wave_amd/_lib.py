@@ -29,6 +29,7 @@ SCALE_ROW_MAJOR, SCALE_E8M0_SHUFFLE, SCALE_MFMA32, SCALE_PER_ROW = 0, 1, 2, 3
 B_ROW_MAJOR, B_PRESHUFFLE = 0, 1
 IN_F32, IN_BF16, IN_F16 = 0, 1, 2
 MXFP8_E4M3, MXFP8_E5M2, MXFP8_B_E2M1 = 0, 1, 2
+MXFP8_E2M1 = MXFP8_B_E2M1  # one operand (x or w_t, not both) packed MXFP4 against an 8-bit other
 
 VARIANT_AUTO = 0
 VARIANT_T256x256_W2x2 = 1

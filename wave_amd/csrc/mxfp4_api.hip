@@ -623,12 +623,14 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
                     size_t workspace_bytes, int variant, void *hip_stream) {
   if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim || k % 128 != 0)
     return WAVE_MXFP4_ERR_BAD_SHAPE;
-  if (bad_enum(a_format, 2) || bad_enum(b_format, 3) || bad_enum(out_dtype, 2) ||
+  if (bad_enum(a_format, 3) || bad_enum(b_format, 3) || bad_enum(out_dtype, 2) ||
       bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_))
     return WAVE_MXFP4_ERR_BAD_ENUM;
   if (variant != WAVE_MXFP4_VARIANT_AUTO && variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 &&
       variant != WAVE_MXFP4_VARIANT_T256x256_W4x2 && variant != WAVE_MXFP4_VARIANT_T128x128_W2x2)
     return WAVE_MXFP4_ERR_UNSUPPORTED;
+  // (one 4-bit operand at most: two are wave_mxfp4_gemm's)
+  if (a_format == WAVE_MXFP8_B_E2M1 && b_format == WAVE_MXFP8_B_E2M1) return WAVE_MXFP4_ERR_UNSUPPORTED;
   if (m == 0 || n == 0) return WAVE_MXFP4_OK;
   if (!c) return WAVE_MXFP4_ERR_NULL_POINTER;
   if (k > 0 && (!a || !a_scale || !b || !b_scale)) return WAVE_MXFP4_ERR_NULL_POINTER;
@@ -673,8 +675,8 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   }
   // large dense problems on the 8-wave tiles with re-laid scales: the persistent kernel
   if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && persist_gemm_fp8_applies(p, device_cus()))
-    return record_hip(launch_persist_gemm_fp8(p, device_cus(), a_format == WAVE_MXFP8_E5M2, b_format, stream));
-  return record_hip(launch_tile_gemm_fp8(p, v, a_format == WAVE_MXFP8_E5M2, b_format, stream));
+    return record_hip(launch_persist_gemm_fp8(p, device_cus(), a_format, b_format, stream));
+  return record_hip(launch_tile_gemm_fp8(p, v, a_format, b_format, stream));
 }
 
 // Scratch of a grouped call: [M tile table | A scales | B scales].

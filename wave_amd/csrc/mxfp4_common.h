@@ -130,11 +130,11 @@ inline hipError_t allow_dynamic_lds(LdsAttrOnce &once, const void *kernel, int b
   return e;
 }
 
-hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_fmt, hipStream_t stream);
+hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_fmt, int b_fmt, hipStream_t stream);
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus);
 hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hipStream_t stream);
 bool persist_gemm_fp8_applies(const GemmParams &p, int num_cus);
-hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2, int b_fmt, hipStream_t stream);
+hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_fmt, int b_fmt, hipStream_t stream);
 bool persist_prefers_192(const GemmParams &p, int num_cus, int parts256);
 bool persist_gated_applies(const GemmParams &p, int num_cus);
 hipError_t launch_persist_gated(const GemmParams &p, int num_cus, hipStream_t stream);

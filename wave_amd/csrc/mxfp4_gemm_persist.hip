@@ -106,12 +106,12 @@ enum KtKind {
 template <class Cfg, bool OUT_BF16, bool GROUPED, bool TAIL, bool SPLIT, int FMT_A = 4, int FMT_B = 4, bool SHUF = false,
           bool GATED = false>
 __device__ __forceinline__ void persist_body(const GemmParams &p) {
-  constexpr bool FP8 = FMT_A != 4;
+  constexpr bool FP8 = FMT_A != 4 || FMT_B != 4;
   static_assert(!GATED || (!FP8 && !TAIL && !SPLIT && OUT_BF16 && Cfg::NWAVES == 8 && Cfg::BN == 256),
                 "gated epilogue: whole K tiles, no cut, the 8-wave 256x256 tiles");
   static_assert(!SHUF || (!FP8 && !GROUPED && !TAIL), "scales in e8m0_shuffle order: dense MXFP4 problems with whole K tiles");
   constexpr bool B4 = FP8 && FMT_B == 4;  // 8-bit A against 4-bit B [N, K/2]: the lower half of B's LDS rows
-  static_assert(FMT_A != 4 || FMT_B == 4, "an MXFP4 A against an MXFP8 B is not built");
+  constexpr bool A4 = FP8 && FMT_A == 4;  // 4-bit A [M, K/2] against 8-bit B, the same way round
   static_assert(!FP8 || (!GROUPED && !TAIL && !SPLIT), "MXFP8: dense problems with whole K tiles");
   constexpr int BM = Cfg::BM, BN = Cfg::BN, MT_M = Cfg::MT_M, MT_N = Cfg::MT_N;
   constexpr int NWAVES = Cfg::NWAVES, A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
@@ -200,11 +200,11 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     // B and its scales end with the tensor (grouped: with the expert's)
     b_lim[which] = rsrc_bytes(((int64_t)p.n - n0[which]) * (B4 ? kp >> 1 : kp));
     bs_lim[which] = rsrc_bytes((int64_t)(((p.n + 31) >> 5) - (n0[which] >> 5)) * k_tiles_blocks);
-    a_base[which] = p.a + (int64_t)m0[which] * kp;
+    a_base[which] = p.a + (int64_t)m0[which] * (A4 ? kp >> 1 : kp);
     // (grouped: A ends with the tile's own rows.  The rows of the next group would do as padding, their results
     // are dropped, but zeros cost the matrix pipes far less power than data does, and power is what bounds the
     // kernel.)
-    a_lim[which] = (int)min((int64_t)max(GROUPED ? c_rows[which] : p.m - m0[which], 0) * kp, (int64_t)0x7FFFFFFF);
+    a_lim[which] = (int)min((int64_t)max(GROUPED ? c_rows[which] : p.m - m0[which], 0) * (A4 ? kp >> 1 : kp), (int64_t)0x7FFFFFFF);
     if (SPLIT) {  // the item's K range starts at K tile kt_lo: move the bases there
       a_base[which] += kt_lo * kTileKBytes;
       a_lim[which] = max(a_lim[which] - kt_lo * kTileKBytes, 0);
@@ -240,12 +240,14 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   // DMA instruction d of a wave fills rows 8*NWAVES*d further down: one per-lane
   // offset per operand, the rest is scalar (registers are what this kernel is short of).
   const int kpb = B4 ? kp >> 1 : kp;  // bytes of a row of B
-  int a_goff = ld_row0 * kp + ld_chunk * 16;
+  const int kpa = A4 ? kp >> 1 : kp;  // bytes of a row of A
+  int a_goff = ld_row0 * kpa + ld_chunk * 16;
+  if (A4 && ld_chunk >= 4) a_goff = (int)0x80000000;  // the upper half of the LDS row: no request, zeros
   int b_goff = p.b_preshuffled ? (ld_row0 >> 4) * 16 * kp + (ld_row0 & 15) * 16 + (ld_chunk >> 1) * 512 +
                                            (ld_chunk & 1) * 256
                                      : ld_row0 * kpb + ld_chunk * 16;
   if (B4 && ld_chunk >= 4) b_goff = (int)0x80000000;  // the upper half of the LDS row: no request, zeros
-  const int ld_step = NWAVES * 8 * kp;  // bytes between consecutive d, either layout (8*NWAVES is a multiple of 16)
+  const int ld_step = NWAVES * 8 * kpa;  // bytes between consecutive d, either layout (8*NWAVES is a multiple of 16)
   const int ld_step_b = NWAVES * 8 * kpb;
   const bool tail_lane = TAIL && ld_chunk >= ((p.k & (kTileK - 1)) >> 5);
   auto flip_tail = [&](int &goff) { goff ^= tail_lane && (!SPLIT || tail_on[0]) ? (int)0x80000000 : 0; };
@@ -256,7 +258,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
     uint8_t *dst_tile = smem + slot * SLOT;
     const __amdgpu_buffer_rsrc_t rsrc =
         op == 0 ? make_rsrc_n(a_base[which], a_lim[which]) : make_rsrc_n(b_base[which], b_lim[which]);
-    const int soff = op == 0 ? kt * kTileKBytes : kt * b_kt_stride;
+    const int soff = op == 0 ? kt * (A4 ? kTileKBytes / 2 : kTileKBytes) : kt * b_kt_stride;
 #pragma unroll
     for (int d = d0; d < d1; ++d) {
       uint8_t *dst = dst_tile + (d * NWAVES + wave) * 1024;
@@ -276,9 +278,9 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
   }
   const uint32_t a_fbase = (uint32_t)(wave_m * Cfg::WM * kTileKBytes);
   const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
-  typedef typename std::conditional<FP8, v8i, v4i>::type Frag;
+  typedef typename std::conditional<FP8 && !A4, v8i, v4i>::type Frag;
   typedef typename std::conditional<FP8 && !B4, v8i, v4i>::type FragB;
-  uint32_t foff_b4[2];  // 8-bit A against 4-bit B: K step s of B is the chunk 2s + fg of the row's lower half
+  uint32_t foff_b4[2];  // a 4-bit operand against an 8-bit one: its K step s is the chunk 2s + fg of the row's lower half
 #pragma unroll
   for (int t = 0; t < 2; ++t) foff_b4[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
   auto read_frags = [&](int slot_a, int slot_b, int t, Frag(&fa)[MT_M], FragB(&fb)[MT_N]) {
@@ -286,9 +288,13 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
       const uint8_t *ta = smem + slot_a * SLOT + a_fbase, *tb = smem + slot_b * SLOT + b_fbase;
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) {
-        const v4i lo = *(const v4i *)(ta + foff[2 * t] + i * 32 * kTileKBytes);
-        const v4i hi = *(const v4i *)(ta + foff[2 * t + 1] + i * 32 * kTileKBytes);
-        fa[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        if constexpr (A4) {
+          fa[i] = *(const v4i *)(ta + foff_b4[t] + i * 32 * kTileKBytes);
+        } else {
+          const v4i lo = *(const v4i *)(ta + foff[2 * t] + i * 32 * kTileKBytes);
+          const v4i hi = *(const v4i *)(ta + foff[2 * t + 1] + i * 32 * kTileKBytes);
+          fa[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
       }
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
@@ -405,7 +411,7 @@ __device__ __forceinline__ void persist_body(const GemmParams &p) {
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
       v8i va;
-      if constexpr (FP8) va = fa[i];
+      if constexpr (FP8 && !A4) va = fa[i];
       else va = v8i{fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
@@ -1114,9 +1120,12 @@ static hipError_t launch_persist_fp8_fmt(const GemmParams &p, int grid_x, hipStr
                     : launch_persist_fp8_out<Cfg, false, FMT_A, FMT_B>(p, grid_x, stream);
 }
 
-// b_fmt: 0 = e4m3, 1 = e5m2, 2 = e2m1 (packed, two per byte)
-hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_e5m2, int b_fmt, hipStream_t stream) {
+// a_fmt, b_fmt: 0 = e4m3, 1 = e5m2, 2 = e2m1 (packed, two per byte; one operand at most)
+hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_fmt, int b_fmt, hipStream_t stream) {
   const int grid = num_cus / kNumXcd * kNumXcd;
+  if (a_fmt == 2 && b_fmt == 2) return hipErrorInvalidValue;  // (both 4-bit: the MXFP4 entry point)
+  if (a_fmt == 2) return b_fmt ? launch_persist_fp8_fmt<4, 1>(p, grid, stream) : launch_persist_fp8_fmt<4, 0>(p, grid, stream);
+  const int a_e5m2 = a_fmt;
   if (b_fmt == 2) return a_e5m2 ? launch_persist_fp8_fmt<1, 4>(p, grid, stream) : launch_persist_fp8_fmt<0, 4>(p, grid, stream);
   if (a_e5m2) return b_fmt ? launch_persist_fp8_fmt<1, 1>(p, grid, stream) : launch_persist_fp8_fmt<1, 0>(p, grid, stream);
   return b_fmt ? launch_persist_fp8_fmt<0, 1>(p, grid, stream) : launch_persist_fp8_fmt<0, 0>(p, grid, stream);

@@ -127,12 +127,12 @@ constexpr int kSlabMaxPitch = (kSlabMaxKTiles + 2) * 8;  // bytes per row: the K
 // K step takes one 16-byte chunk of B per lane, as in MXFP4.
 template <class Cfg, int MODE, int FMT = 4, int FMT_B = FMT>
 __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
-  static_assert(FMT != 4 || FMT_B == 4, "an MXFP4 A against an MXFP8 B is not built");
   constexpr bool GENERIC_K = MODE == kGenericK;
   constexpr bool NATIVE = MODE == kNative;
   constexpr bool SC_LDS = MODE == kDirectLds;
-  constexpr bool FP8 = FMT != 4;
+  constexpr bool FP8 = FMT != 4 || FMT_B != 4;
   constexpr bool B4 = FP8 && FMT_B == 4;  // 8-bit A against 4-bit B
+  constexpr bool A4 = FP8 && FMT == 4;    // 4-bit A against 8-bit B
   static_assert(!SC_LDS || (!FP8 && Cfg::LDS_BYTES + (Cfg::BM + Cfg::BN) * kSlabMaxPitch <= 160 * 1024),
                 "scale rows in LDS: MXFP4 on a tile whose ring leaves room");
   static_assert(!FP8 || MODE != kGenericK, "MXFP8 needs whole K tiles");
@@ -191,9 +191,10 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   // are 8*NWAVES rows apart (a multiple of 16), so the chunk does not depend on d.
   const int kp = p.kp;
   const int kpb = B4 ? kp >> 1 : kp;  // bytes of a row of B
+  const int kpa = A4 ? kp >> 1 : kp;  // ... of A
   // (every descriptor ends with its tensor, or its expert's part of it: an access past it reads zeros instead of
   // a neighbour's memory)
-  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(p.a + (int64_t)m0 * kp, rsrc_bytes(((int64_t)p.m - m0) * kp));
+  const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(p.a + (int64_t)m0 * kpa, rsrc_bytes(((int64_t)p.m - m0) * kpa));
   // preshuffle keeps 16-row blocks contiguous
   const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc_n(b_ptr + (int64_t)n0 * kpb, rsrc_bytes(((int64_t)p.n - n0) * kpb));
   const int ld_row0 = wave * 8 + (lane >> 3);
@@ -205,7 +206,10 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   //   preshuffle : (r/16)*16*kp + (c/2)*512 + (c%2)*256 + (r%16)*16
   int a_goff[A_LD], b_goff[B_LD];
 #pragma unroll
-  for (int d = 0; d < A_LD; ++d) a_goff[d] = min(ld_row0 + d * NWAVES * 8, a_row_lim) * kp + ld_chunk * 16;
+  for (int d = 0; d < A_LD; ++d) {
+    a_goff[d] = min(ld_row0 + d * NWAVES * 8, a_row_lim) * kpa + ld_chunk * 16;
+    if (A4 && ld_chunk >= 4) a_goff[d] = (int)0x80000000;  // the upper half of the LDS row: no request, zeros
+  }
 #pragma unroll
   for (int d = 0; d < B_LD; ++d) {
     const int r = min(ld_row0 + d * NWAVES * 8, b_row_lim);
@@ -244,7 +248,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
     // (fp4 +0.0), so they add nothing whatever their scale.
     const bool tail = GENERIC_K && tail_chunks != 0 && kt == p.k_tiles - 1;
     const v4i zero = {0, 0, 0, 0};
-    const int soff = op == 0 ? kt * kTileKBytes : kt * b_kt_stride;
+    const int soff = op == 0 ? kt * (A4 ? kTileKBytes / 2 : kTileKBytes) : kt * b_kt_stride;
 #pragma unroll
     for (int d = d0; d < d1; ++d) {
       uint8_t *dst = dst_tile + (d * NWAVES + wave) * 1024;
@@ -277,9 +281,9 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
   const uint32_t a_fbase = (uint32_t)(wave_m * Cfg::WM * kTileKBytes);
   const uint32_t b_fbase = (uint32_t)(wave_n * Cfg::WN * kTileKBytes);
 
-  typedef typename std::conditional<FP8, v8i, v4i>::type Frag;
+  typedef typename std::conditional<FP8 && !A4, v8i, v4i>::type Frag;
   typedef typename std::conditional<FP8 && !B4, v8i, v4i>::type FragB;
-  // (8-bit A against 4-bit B: K step s of B is the chunk 2s + fg of the row's lower half)
+  // (a 4-bit operand against an 8-bit one: its K step s is the chunk 2s + fg of the row's lower half)
   uint32_t foff_b4[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) foff_b4[t] = (uint32_t)(fr * kTileKBytes + (((t * 2 + fg) ^ ((fr >> 1) & 7)) << 4));
@@ -288,9 +292,13 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
       const uint8_t *ta = smem + slot_a * SLOT + a_fbase, *tb = smem + slot_b * SLOT + b_fbase;
 #pragma unroll
       for (int i = 0; i < MT_M; ++i) {
-        const v4i lo = *(const v4i *)(ta + foff[2 * t] + i * 32 * kTileKBytes);
-        const v4i hi = *(const v4i *)(ta + foff[2 * t + 1] + i * 32 * kTileKBytes);
-        fa[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        if constexpr (A4) {
+          fa[i] = *(const v4i *)(ta + foff_b4[t] + i * 32 * kTileKBytes);
+        } else {
+          const v4i lo = *(const v4i *)(ta + foff[2 * t] + i * 32 * kTileKBytes);
+          const v4i hi = *(const v4i *)(ta + foff[2 * t + 1] + i * 32 * kTileKBytes);
+          fa[i] = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
       }
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
@@ -481,7 +489,7 @@ __device__ __forceinline__ void tile_gemm_body(const GemmParams &p) {
 #pragma unroll
     for (int i = 0; i < MT_M; ++i) {
       v8i va;
-      if constexpr (FP8) va = fa[i];
+      if constexpr (FP8 && !A4) va = fa[i];
       else va = v8i{fa[i].x, fa[i].y, fa[i].z, fa[i].w, 0, 0, 0, 0};
 #pragma unroll
       for (int j = 0; j < MT_N; ++j) {
@@ -836,19 +844,22 @@ static hipError_t launch_fp8_by_scales(const GemmParams &p, hipStream_t stream) 
   return native ? launch_cfg<Cfg, kNative, FMT_A, FMT_B>(p, stream) : launch_cfg<Cfg, kDirect, FMT_A, FMT_B>(p, stream);
 }
 
-// b_fmt: 0 = e4m3, 1 = e5m2, 2 = e2m1 (packed, two per byte)
+// a_fmt, b_fmt: 0 = e4m3, 1 = e5m2, 2 = e2m1 (packed, two per byte; one operand at most)
 template <class Cfg>
-static hipError_t launch_fp8_formats(const GemmParams &p, int a_e5m2, int b_fmt, hipStream_t stream) {
+static hipError_t launch_fp8_formats(const GemmParams &p, int a_fmt, int b_fmt, hipStream_t stream) {
+  if (a_fmt == 2 && b_fmt == 2) return hipErrorInvalidValue;  // (both 4-bit: the MXFP4 entry point)
+  if (a_fmt == 2) return b_fmt ? launch_fp8_by_scales<Cfg, 4, 1>(p, stream) : launch_fp8_by_scales<Cfg, 4, 0>(p, stream);
+  const int a_e5m2 = a_fmt;
   if (b_fmt == 2) return a_e5m2 ? launch_fp8_by_scales<Cfg, 1, 4>(p, stream) : launch_fp8_by_scales<Cfg, 0, 4>(p, stream);
   if (a_e5m2) return b_fmt ? launch_fp8_by_scales<Cfg, 1, 1>(p, stream) : launch_fp8_by_scales<Cfg, 1, 0>(p, stream);
   return b_fmt ? launch_fp8_by_scales<Cfg, 0, 1>(p, stream) : launch_fp8_by_scales<Cfg, 0, 0>(p, stream);
 }
 
 // MXFP8: `p` describes the byte geometry (kp = K bytes per row, ks = K/32, k_tiles = K/128).
-hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_e5m2, int b_fmt, hipStream_t stream) {
-  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_fp8_formats<Cfg256x256w4>(p, a_e5m2, b_fmt, stream);
-  if (variant == WAVE_MXFP4_VARIANT_T256x256_W4x2) return launch_fp8_formats<Cfg256x256w8>(p, a_e5m2, b_fmt, stream);
-  if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2) return launch_fp8_formats<Cfg128x128w4>(p, a_e5m2, b_fmt, stream);
+hipError_t launch_tile_gemm_fp8(const GemmParams &p, int variant, int a_fmt, int b_fmt, hipStream_t stream) {
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W2x2) return launch_fp8_formats<Cfg256x256w4>(p, a_fmt, b_fmt, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T256x256_W4x2) return launch_fp8_formats<Cfg256x256w8>(p, a_fmt, b_fmt, stream);
+  if (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2) return launch_fp8_formats<Cfg128x128w4>(p, a_fmt, b_fmt, stream);
   return hipErrorInvalidValue;
 }
 

@@ -563,9 +563,10 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
     ``x.view(torch.int8)`` of ``float8_e5m2`` tensors).  float8 tensors carry
     their format; for uint8 / int8 views pass ``elem_format``, one value for both
     operands or a pair ``(x format, w_t format)`` (default e5m2, the
-    reference's ``tkl.f8e5m2``).  With ``MXFP8_B_E2M1`` as the second format
-    ``w_t`` is ``[N, K/2]`` packed MXFP4 (8-bit activations against 4-bit weights,
-    the mixed operands of wave_lang/kernel/wave/constraints.py:425-431).
+    reference's ``tkl.f8e5m2``).  With ``MXFP8_E2M1`` as one of the two formats that
+    operand is ``[rows, K/2]`` packed MXFP4 against the 8-bit other (8-bit activations
+    against 4-bit weights or the other way round, the mixed operands of
+    wave_lang/kernel/wave/constraints.py:425-431; both 4-bit is :func:`mxfp4_gemm`).
     ``workspace`` as in :func:`mxfp4_gemm`."""
     lib = _lib.load()
     given = tuple(elem_format) if isinstance(elem_format, (tuple, list)) else (elem_format, elem_format)
@@ -583,12 +584,15 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
     x, w_t = ops
     x_scales = _as_u8(x_scales, "x_scales")
     w_scales = _as_u8(w_scales, "w_scales")
-    if fmts[0] == _lib.MXFP8_B_E2M1:
-        raise ValueError("x must be an 8-bit format (MXFP8_B_E2M1 is for w_t only)")
-    w_cols = x.shape[1] // 2 if fmts[1] == _lib.MXFP8_B_E2M1 and x.dim() == 2 else (x.shape[1] if x.dim() == 2 else -1)
-    if x.dim() != 2 or w_t.dim() != 2 or w_t.shape[1] != w_cols:
-        raise ValueError("x must be [M, K] and w_t [N, K] ([N, K/2] for packed e2m1)")
-    m, k = x.shape
+    x4, w4 = fmts[0] == _lib.MXFP8_E2M1, fmts[1] == _lib.MXFP8_E2M1
+    if x4 and w4:
+        raise ValueError("both operands e2m1: that is mxfp4_gemm")
+    if x.dim() != 2 or w_t.dim() != 2:
+        raise ValueError("x must be [M, K] and w_t [N, K] ([rows, K/2] for a packed e2m1 operand)")
+    k = x.shape[1] * 2 if x4 else x.shape[1]
+    if w_t.shape[1] != (k // 2 if w4 else k):
+        raise ValueError("x must be [M, K] and w_t [N, K] ([rows, K/2] for a packed e2m1 operand)")
+    m = x.shape[0]
     n = w_t.shape[0]
     if k % 128:
         raise ValueError(f"K = {k} must be a multiple of 128")

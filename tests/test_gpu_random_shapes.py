@@ -98,3 +98,22 @@ def _midb_cases(count, seed):
                          ids=lambda c: f"b{c[0]}-{c[1]}x{c[2]}x{c[3]}")
 def test_random_preshuffled_mid_shape_against_oracle(case):
     test_random_shape_against_oracle(case)
+
+
+def _resident_cases(count, seed):
+    """Shapes on either side of the borders the library's own choice follows when both scale tensors come in MFMA32
+    order (streaming kernel, mid-M kernel, 128x128 tiles, B-direct mid-M kernel from 32 rows on with a preshuffled
+    B): up to 256 rows, N from 12288 to past one round of 128-column strips, K = 2048 / 4096 / 8192."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        m = int(rng.choice([rng.integers(1, 17), rng.integers(17, 65), rng.integers(65, 129), rng.integers(129, 257)]))
+        n = 32 * int(rng.choice([rng.integers(384, 513), rng.integers(513, 1025), rng.integers(1025, 1400)]))
+        k = int(rng.choice([2048, 4096, 8192]))
+        out.append((i, m, n, k, 2, 2, bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 4) > 0)))
+    return out
+
+
+@pytest.mark.parametrize("case", _resident_cases(12, seed=23), ids=lambda c: f"r{c[0]}-{c[1]}x{c[2]}x{c[3]}")
+def test_random_resident_scale_shape_against_oracle(case):
+    test_random_shape_against_oracle(case)

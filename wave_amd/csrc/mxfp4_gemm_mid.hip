@@ -65,8 +65,12 @@ struct MidCfg {
   // from L2 at the same moment as all the others, needs the deeper ring.  With no B traffic at all the kernel
   // took 17 / 22 us at two K tiles of A ahead: its latency, not B's, set the pace.
   //   (DA, DB) = (3, 7) / (3, 5) / (2, 5): 29.9 / 33.1 / 43.5     (6, 5) / (5, 3) / (3, 3): 27.9 / 31.4 / 39.0
-  static constexpr int DA = TWO_PER_CU ? 3 : BM <= 64 ? 6 : BM <= 128 ? 5 : BM <= 192 ? 3 : 2;  // K tiles of A in LDS
-  static constexpr int DB = TWO_PER_CU ? 3 : BM <= 32 ? 7 : BM <= 64 ? 5 : BM <= 192 ? 3 : 4;   // K tiles of B in the ring
+  // The 256-row block, whose K tile of A is 32 KB, takes (3, 2): a third K tile of A is worth more than B's third
+  // and fourth (M = 256 / 224 / 200 at N = 28672, K = 8192 with (2, 4): 45.0 / 43.2 / 42.7 us, with (3, 2): 43.6 /
+  // 41.1 / 39.9); at 192 rows (4, 2) against (3, 3) is a draw (36.4 / 35.6 against 37.7 / 35.0 us with row-major /
+  // MFMA32 scales) and (3, 3) stays.
+  static constexpr int DA = TWO_PER_CU ? 3 : BM <= 64 ? 6 : BM <= 128 ? 5 : 3;  // K tiles of A in LDS
+  static constexpr int DB = TWO_PER_CU ? 3 : BM <= 32 ? 7 : BM <= 64 ? 5 : BM <= 192 ? 3 : 2;   // K tiles of B in the ring
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
   static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
   // Scale groups of A in LDS: the one being read, (j / 4), up to the one requested with A(j + DA - 1); a group's

@@ -65,12 +65,16 @@ struct MidCfg {
   // from L2 at the same moment as all the others, needs the deeper ring.  With no B traffic at all the kernel
   // took 17 / 22 us at two K tiles of A ahead: its latency, not B's, set the pace.
   //   (DA, DB) = (3, 7) / (3, 5) / (2, 5): 29.9 / 33.1 / 43.5     (6, 5) / (5, 3) / (3, 3): 27.9 / 31.4 / 39.0
+  // Deeper still for A at the small blocks, re-measured later on the same shape: 32 rows (6, 7) -> (10, 6) 22.9 ->
+  // 22.7 us, 64 rows (6, 5) -> (8, 4) 24.4 -> 24.3 (23.75 -> 23.4 with MFMA32 scales); at 128 rows (6, 2) lost
+  // against (5, 3), 33.0 against 28.9 us.  A producer with more than 63 requests in flight is held at the counter's
+  // limit by the hardware, and its wait is clamped there (it then waits for a few requests more than it must).
   // The 256-row block, whose K tile of A is 32 KB, takes (3, 2): a third K tile of A is worth more than B's third
   // and fourth (M = 256 / 224 / 200 at N = 28672, K = 8192 with (2, 4): 45.0 / 43.2 / 42.7 us, with (3, 2): 43.6 /
   // 41.1 / 39.9); at 192 rows (4, 2) against (3, 3) is a draw (36.4 / 35.6 against 37.7 / 35.0 us with row-major /
   // MFMA32 scales) and (3, 3) stays.
-  static constexpr int DA = TWO_PER_CU ? 3 : BM <= 64 ? 6 : BM <= 128 ? 5 : 3;  // K tiles of A in LDS
-  static constexpr int DB = TWO_PER_CU ? 3 : BM <= 32 ? 7 : BM <= 64 ? 5 : BM <= 192 ? 3 : 2;   // K tiles of B in the ring
+  static constexpr int DA = TWO_PER_CU ? 3 : BM <= 32 ? 10 : BM <= 64 ? 8 : BM <= 128 ? 5 : 3;  // K tiles of A in LDS
+  static constexpr int DB = TWO_PER_CU ? 3 : BM <= 32 ? 6 : BM <= 64 ? 4 : BM <= 192 ? 3 : 2;   // K tiles of B in the ring
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
   static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
   // Scale groups of A in LDS: the one being read, (j / 4), up to the one requested with A(j + DA - 1); a group's
@@ -84,7 +88,7 @@ struct MidCfg {
   static constexpr int A_LD = BM / 8;                                    // A DMA instructions per K tile (producer)
   static_assert(LDS <= (TWO_PER_CU ? 80 : 160) * 1024, "LDS");
   static_assert(MT_M % WM == 0 && B_RING >= kMidCW * 32 * 32 * 4, "whole row blocks per wave; the waves' C staging fits the ring");
-  static_assert((DA - 2) * A_LD + 8 <= 63 && 4 * (LB - 1) + 2 <= 63, "vmcnt range");
+  static_assert(4 * (LB - 1) + 2 <= 63, "vmcnt range");
 };
 
 // A_RM / B_RM: the operand's scales are row-major (else MFMA32 order, or with A_SH / B_SH e8m0_shuffle order: the
@@ -162,7 +166,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     int slot_next = DA - 1;  // slot of the K tile requested next
     for (int j = v0; j < vend; ++j) {
       // A(j) has landed: younger than it are A(j + 1 .. j + DA - 2) and at most one scale group
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((DA - 2) * Cfg::A_LD));
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((DA - 2) * Cfg::A_LD < 63 ? (DA - 2) * Cfg::A_LD : 63));
       asm volatile("" ::: "memory");
       __builtin_amdgcn_s_barrier();  // A(j) visible to the compute waves; they are done with A(j - 1)
       asm volatile("" ::: "memory");

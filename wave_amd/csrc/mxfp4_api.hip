@@ -119,9 +119,11 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     // Measured at K = 2048 .. 8192 (us, other kernel -> mid-M):
     //   64 < M <= 192 against the tile kernels: from N = 12288 on (128 x 12288 x 8192: 29.7 -> 23.3,
     //     128 x 24576: 43.4 -> 27.6; 128 x 8192 loses, 19.3 -> 22.8) and, for 96 < M at K <= 4096, from N = 8192 on
-    //     (128 x 8192 x 4096: 18.0 -> 13.6); 192 < M <= 256 on one round of strips from N = 24576 on (256 x 24576:
-    //     51.5 -> 43.9, 256 x 32768: 59.0 -> 50.5; 256 x 16384 loses, 38.3 -> 39.9, and so does 256 x 40960,
-    //     71.5 -> 88.0: two rounds of 256-row blocks against 160 tiles of 256 x 256)
+    //     (128 x 8192 x 4096: 18.0 -> 13.6); 192 < M <= 256 on one round of strips from N = 20480 on (256 x 24576:
+    //     51.5 -> 43.9, 256 x 32768: 59.0 -> 50.5, 256 x 20480: 43.6 -> 37.7 and 24.1 -> 21.4 at K = 4096 since the
+    //     256-row block holds three K tiles of A; 256 x 16384 lost before that, 38.3 -> 39.9, 256 x 14336 x 4096
+    //     still does, 15.0 -> 20.7, and so does 256 x 40960, 71.5 -> 88.0: two rounds of 256-row blocks against 160
+    //     tiles of 256 x 256)
     //   32 < M <= 64 against the streaming kernel: from N = 12288 on (48 x 28672 x 8192: 28.0 -> 22.5), and from
     //     N = 4096 on at K <= 4096 (64 x 8192 x 4096: 14.5 -> 10.7; 48 x 8192 x 8192 loses, 14.4 -> 17.3)
     //   16 < M <= 32: N from 12288 up to 320 columns per CU (32 x 28672 x 8192: 24.8 -> 22.2; past one round of
@@ -131,7 +133,7 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     //     a tie or 2 % lost at K = 8192: 16 x 40960 29.8 -> 30.3), beyond at any K (16 x 57344 x 8192: 41.4 -> 38.3)
     if (mid_shape_ok(m, n, k)) {
       const int64_t cus = device_cus();
-      const bool mid = m > 192  ? n >= 24576 && n <= 128 * cus
+      const bool mid = m > 192  ? n >= 20480 && n <= 128 * cus
                        : m > 64 ? n >= 12288 || (k <= 4096 && n >= 8192 && m > 96)
                        : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096)
                        : m > 16 ? n >= 12288 && n <= 320 * cus

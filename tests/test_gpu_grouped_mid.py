@@ -1,7 +1,8 @@
 """GPU: the grouped GEMM at a small batch (a few rows per expert: the decode step of a mixture of experts, the
 per-expert loop of tests/kernel/moe_test.py:175-246 at serving sizes) through the mid-M kernel, one workgroup per
 (expert, strip of columns), against the exact oracle applied per group: ragged and empty groups, groups of more rows
-than one block, N that ends inside a strip, row-major and MFMA32 expert scales, preshuffled expert weights, both
+than one block, N that ends inside a strip, row-major and MFMA32 expert scales, activation scales row-major or in
+MFMA32 order, preshuffled expert weights, both
 output types, rows past the last offset left alone, and the library's own choice of it."""
 
 import numpy as np
@@ -38,9 +39,12 @@ def reference(x, xs, w, ws, off):
     return out
 
 
-def run(x, xs, w, ws, off, dt, lb=RM, pre=False, **kw):
+def run(x, xs, w, ws, off, dt, lb=RM, pre=False, la=RM, **kw):
     e, n, k = w.shape[0], w.shape[1], x.shape[1] * 2
     gx, gxs, gw, gws, goff = to_gpu(x, xs, w, ws, off)
+    if la != RM:   # one tensor over all rows: its 32-row blocks straddle the groups
+        gxs = wave_amd.scale_convert(gxs, x.shape[0], k // 32, RM, la)
+        kw["a_scale_layout"] = la
     if pre:
         gw = torch.stack([wave_amd.b_preshuffle(gw[g]) for g in range(e)])
     if lb != RM:
@@ -69,6 +73,36 @@ def test_grouped_mid_ragged_groups(e, n, k, rows, lb, pre, dt):
     x, xs, w, ws, off = inputs(e, n, k, rows, seed=e + rows)
     c = run(x, xs, w, ws, off, dt, lb=lb, pre=pre, variant=V)
     check(c, reference(x, xs, w, ws, off), dt, f"E={e} {rows}x{n}x{k}")
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("lb,pre", [(RM, False), (M32, False), (M32, True), (SH, False)])
+@pytest.mark.parametrize("e,n,k,rows", [(8, 160, 1024, 40), (5, 1008, 1280, 333), (16, 96, 2048, 16), (3, 4096, 1024, 700),
+                                        (40, 1024, 2048, 300), (8, 512, 1024, 8 * 200)])
+def test_grouped_mid_activation_scales_in_mfma32_order(e, n, k, rows, lb, pre, dt):
+    """The activations' scales as the gathered quantiser writes them for the tile kernels: one [rows, K/32] tensor in
+    MFMA32 order whose 32-row blocks ignore the group borders, so a group's block of rows starts at any row of a
+    scale block and reads one block more than its rows span.  Same groups as above (one-row groups, groups of more
+    rows than the block, more strips than CUs) and 200 rows per expert on average (the 192-row block: the
+    256-row block has no room for the extra scale block); every block height is reached through the average."""
+    x, xs, w, ws, off = inputs(e, n, k, rows, seed=e + rows + 1)
+    c = run(x, xs, w, ws, off, dt, lb=lb, pre=pre, la=M32, variant=V)
+    check(c, reference(x, xs, w, ws, off), dt, f"E={e} {rows}x{n}x{k} A scales MFMA32")
+
+
+def test_grouped_mid_mfma32_activation_scales_nan_stays_in_its_row():
+    """A NaN scale (byte 255) in the last row of one group and the first row of the next: exactly those two rows of C
+    are NaN, although both groups' blocks read the scale block the rows share."""
+    e, n, k, rows = 4, 256, 1024, 100
+    x, xs, w, ws, off = inputs(e, n, k, rows, seed=9, lo=124, hi=130)
+    r = int(off[2])
+    assert 0 < r < rows and off[1] < off[2] < off[3]
+    xs[r - 1, 5] = 255
+    xs[r, 17] = 255
+    c = run(x, xs, w, ws, off, torch.float32, la=M32, variant=V)
+    nan_rows = np.isnan(c).all(axis=1)
+    assert np.array_equal(np.nonzero(nan_rows)[0], [r - 1, r])
+    assert not np.isnan(np.delete(c, [r - 1, r], axis=0)).any()
 
 
 @pytest.mark.parametrize("force_empty", [(0,), (3, 4), (7,), (0, 1, 2, 3, 4, 5, 6)])

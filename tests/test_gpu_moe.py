@@ -133,9 +133,9 @@ def test_expert_mlp_chain_with_resident_scale_layouts(size):
     -> gathered quantiser -> grouped GEMM (gate and up) -> gated activation fused into the quantiser -> grouped
     GEMM (down), every scale tensor written or kept in MFMA32 order so that no re-layout launch sits between the
     steps.  Each step against the oracle applied to the device's output of the step before: bytes exact for the
-    quantisers, the GEMMs within the bf16 bound.  "serving": a few rows per expert (with activation scales in
-    MFMA32 order that is the one-tile-per-workgroup kernel; the mid-M kernel, which takes row-major activation
-    scales, has the same shapes in test_gpu_grouped_mid.py); "prefill": more 256x256 tiles than CUs (table-driven
+    quantisers, the GEMMs within the bf16 bound.  "serving": a few rows per expert (the mid-M kernel, one workgroup
+    per expert and strip, whose blocks of rows start inside the 32-row blocks of the activations' MFMA32 scales:
+    80 routed rows over 8 experts, 8 x 16 and 8 x 8 strips); "prefill": more 256x256 tiles than CUs (table-driven
     persistent kernel, groups starting at rows that are no multiples of 32), where the first GEMM with the
     activation and the quantiser fused into its C write must give the chain's q2 / s2 bit for bit."""
     tokens, topk, experts, hidden, inter = (40, 2, 8, 1024, 2048) if size == "serving" else (2600, 2, 4, 1024, 2048)

@@ -52,10 +52,12 @@ constexpr int kMidOnce = 2;  // the "nt" bit: B is read exactly once
 // one's prologue and C write run under the other's stream.  For problems of more workgroups than CUs (measured, 8
 // experts x 14336 x 4096 at one row per expert: 47.0 -> 40.2 us, 6.2 TB/s; 64 experts x 2048 x 7168: 80.8 -> 74.1 us,
 // 6.75 TB/s); with one workgroup per CU or fewer the deep rings are the better use of the LDS.
-template <int BM_, bool B_RM_, bool TWO_PER_CU_ = false>
+// A_OFF: A's scales are in MFMA32 order and the block of rows may start inside one of their 32-row blocks (a group
+// of a grouped problem starts at any row): the images hold one block more.
+template <int BM_, bool B_RM_, bool TWO_PER_CU_ = false, bool A_OFF_ = false>
 struct MidCfg {
   static constexpr int BM = BM_, MT_M = BM / 32;
-  static constexpr bool B_RM = B_RM_, TWO_PER_CU = TWO_PER_CU_;
+  static constexpr bool B_RM = B_RM_, TWO_PER_CU = TWO_PER_CU_, A_OFF = A_OFF_;
   static_assert(!TWO_PER_CU || BM == 32, "only the 32-row block leaves room for two workgroups");
   // The four compute waves sit WM x (4 / WM) on the strip: two row halves times two pairs of column groups from
   // BM = 64 on (one A fragment per two MFMAs), side by side on one row block at BM = 32.
@@ -76,7 +78,7 @@ struct MidCfg {
   static constexpr int DA = TWO_PER_CU ? 3 : BM <= 32 ? 10 : BM <= 64 ? 8 : BM <= 128 ? 5 : 3;  // K tiles of A in LDS
   static constexpr int DB = TWO_PER_CU ? 3 : BM <= 32 ? 6 : BM <= 64 ? 4 : BM <= 192 ? 3 : 2;   // K tiles of B in the ring
   static constexpr int LB = DB - 1;                                      // B is requested LB K tiles ahead
-  static constexpr int AS_SLOT = MT_M * 1024;                            // A scales of 4 K tiles (1 KB per 32 rows)
+  static constexpr int AS_SLOT = (MT_M + (A_OFF ? 1 : 0)) * 1024;        // A scales of 4 K tiles (1 KB per 32 rows)
   // Scale groups of A in LDS: the one being read, (j / 4), up to the one requested with A(j + DA - 1); a group's
   // slot may be overwritten only when the group before it in that slot is no longer read: more than
   // ceil((DA - 1) / 4) slots (a power of two, for the slot index).
@@ -99,7 +101,8 @@ struct MidCfg {
 // at `b_base` (one expert's, for a grouped problem) with its scales at `bs_base`, C rows at `c_base`.
 template <class Cfg, bool A_RM, bool B_SH, bool A_SH>
 __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, const uint8_t *a_base, const uint8_t *as_base,
-                                         const uint8_t *b_base, const uint8_t *bs_base, uint8_t *c_base, const int m_rows) {
+                                         const uint8_t *b_base, const uint8_t *bs_base, uint8_t *c_base, const int m_rows,
+                                         const int a_row32 = 0) {
   constexpr bool B_RM = Cfg::B_RM;
   constexpr int MT_M = Cfg::MT_M, DA = Cfg::DA, DB = Cfg::DB, LB = Cfg::LB;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -130,7 +133,8 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
   if (wave == kMidCW) {
     // ================= the producer wave: A and its scales =================
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc_n(a_base, (int)min((int64_t)m_rows * kp, (int64_t)0x7FFFFFFF));
-    const int64_t as_bytes = a_rowmajor ? (int64_t)m_rows * p.ks : (int64_t)((m_rows + 31) >> 5) * k_tiles_blocks;
+    // (blocked: `as_base` is the 32-row block that holds the first row, row a_row32 of it)
+    const int64_t as_bytes = a_rowmajor ? (int64_t)m_rows * p.ks : (int64_t)((a_row32 + m_rows + 31) >> 5) * k_tiles_blocks;
     const __amdgpu_buffer_rsrc_t as_rsrc = make_rsrc_n(as_base, (int)min(as_bytes, (int64_t)0x7FFFFFFF));
     const int row0 = lane >> 3;  // instruction d fills rows 8d .. 8d + 7
     // chunk position lane % 8 of row r holds chunk (lane % 8) ^ ((r / 2) % 8); 8d is a multiple of 8, so the
@@ -153,7 +157,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     auto issue_as = [&](int g) {
       const int soff = g < g_end ? group4_of(g) * as_gstep : (int)0x80000000;
 #pragma unroll
-      for (int i = 0; i < MT_M; ++i)
+      for (int i = 0; i < MT_M + (Cfg::A_OFF ? 1 : 0); ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(as_rsrc, WAVE_LDS_PTR(as_ring + (g & (Cfg::AS_SLOTS - 1)) * Cfg::AS_SLOT + i * 1024), 16,
                                                  as_goff, soff + i * as_istep, 0, 0);
     };
@@ -266,13 +270,16 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     const uint32_t d1 = *(const uint32_t *)(blk + 128 + fg * 64 + (fr & 15) * 4);
     return __builtin_amdgcn_perm(d1, d0, 0x06020400u + (uint32_t)(fr >> 4) * 0x01010101u);
   };
+  // MFMA32 order, a block of rows that starts at row a_row32 of a 32-row scale block: the lane's row fr of row block
+  // i is row (a_row32 + fr) % 32 of image i + (a_row32 + fr) / 32
+  const int a_lane_off = Cfg::A_OFF ? ((a_row32 + fr) >> 5) * 1024 + ((fg << 5) | ((a_row32 + fr) & 31)) * 4 : lane * 4;
   auto lane_scales = [&](const uint8_t *img, auto rm_tag, int j) -> uint32_t {
     if constexpr (decltype(rm_tag)::value) {
       return pick_scales(*(const v4i *)(img + ((j & 2) << 8) + fr * 16), j);
     } else if constexpr (A_SH) {
       return shuffled_scales(img + (j & 3) * 256);
     } else {
-      return *(const uint32_t *)(img + (j & 3) * 256 + lane * 4);
+      return *(const uint32_t *)(img + (j & 3) * 256 + a_lane_off);
     }
   };
   // B, row-major: the piece (j / 2) % 4 of row fr in the swizzled 32 x 64-byte image of the K tile's group of 8
@@ -465,15 +472,16 @@ __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p,
   if constexpr (!GROUPED) {
     mid_body<Cfg, A_RM, B_SH, A_SH>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
   } else {
-    static_assert(A_RM, "a group may start at any row: A's scales row-major");
+    static_assert(A_RM || (Cfg::A_OFF && !A_SH), "a group may start at any row: A's scales row-major, or MFMA32 with room for the block it starts in");
     const int e = blockIdx.y;
     const int lo = __builtin_amdgcn_readfirstlane(min(max(p.offsets[e], 0), p.m));
     const int hi = __builtin_amdgcn_readfirstlane(min(max(p.offsets[e + 1], lo), p.m));
     const uint8_t *b = p.b + (int64_t)e * p.b_group_stride, *bs = p.b_scale + (int64_t)e * p.b_scale_group_stride;
     const int elt = p.out_bf16 ? 2 : 4;
     for (int m0 = lo; m0 < hi; m0 += Cfg::BM) {
-      mid_body<Cfg, A_RM, B_SH, A_SH>(p, wv, p.a + (int64_t)m0 * p.kp, p.a_scale + (int64_t)m0 * p.ks, b, bs,
-                          (uint8_t *)p.c + (int64_t)m0 * p.n * elt, min(Cfg::BM, hi - m0));
+      const uint8_t *as = A_RM ? p.a_scale + (int64_t)m0 * p.ks : p.a_scale + (int64_t)(m0 >> 5) * p.k_tiles * 256;
+      mid_body<Cfg, A_RM, B_SH, A_SH>(p, wv, p.a + (int64_t)m0 * p.kp, as, b, bs,
+                          (uint8_t *)p.c + (int64_t)m0 * p.n * elt, min(Cfg::BM, hi - m0), A_RM ? 0 : m0 & 31);
       // every wave is done with the rings (the C staging's reads included) before the next block's requests
       __builtin_amdgcn_s_waitcnt(0);
       asm volatile("" ::: "memory");
@@ -514,9 +522,15 @@ hipError_t launch_mid_layouts(const GemmParams &p, int wv, hipStream_t stream) {
 template <int BM, bool TWO = false>
 hipError_t launch_mid_cfg(const GemmParams &p, int wv, hipStream_t stream) {
   const bool a_rm = p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR, b_rm = p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
-  if (p.num_groups != 0)  // (row-major A scales: checked by mid_grouped_applies)
+  if (p.num_groups != 0) {  // (A's scales row-major or MFMA32: checked by mid_grouped_applies)
+    if constexpr (BM <= 192) {
+      if (!a_rm)
+        return b_rm ? launch_mid_layouts<MidCfg<BM, true, TWO, true>, false, true>(p, wv, stream)
+                    : launch_mid_layouts<MidCfg<BM, false, TWO, true>, false, true>(p, wv, stream);
+    }
     return b_rm ? launch_mid_layouts<MidCfg<BM, true, TWO>, true, true>(p, wv, stream)
                 : launch_mid_layouts<MidCfg<BM, false, TWO>, true, true>(p, wv, stream);
+  }
   if (a_rm)
     return b_rm ? launch_mid_layouts<MidCfg<BM, true, TWO>, true, false>(p, wv, stream)
                 : launch_mid_layouts<MidCfg<BM, false, TWO>, true, false>(p, wv, stream);
@@ -566,7 +580,7 @@ bool mid_gemm_applies(const GemmParams &p) {
 // per expert.
 bool mid_grouped_applies(const GemmParams &p) {
   if (p.num_groups <= 0 || p.num_groups > 65535 || p.offsets == nullptr || p.splits != 1 || p.partial != nullptr) return false;
-  if (p.a_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR) return false;
+  if (p.a_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
   if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 &&
       p.b_scale_layout != WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
     return false;
@@ -581,6 +595,8 @@ bool mid_grouped_applies(const GemmParams &p) {
 // rows takes several blocks).
 hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream, int bm) {
   if (bm <= 0) bm = p.m;
+  // (a group's block with A scales in MFMA32 order holds one scale block more: no room for it beside 256 rows)
+  if (p.num_groups != 0 && p.a_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && bm > 192) bm = 192;
   // more strips than CUs at the 32-row block: two workgroups per CU
   const int64_t strips = (int64_t)((p.n + kMidBN - 1) / kMidBN) * (p.num_groups != 0 ? p.num_groups : 1);
   const bool two = bm <= 32 && strips > num_cus;

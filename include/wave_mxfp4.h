@@ -333,10 +333,15 @@ int wave_mxfp4_silu_and_mul_quantize(const void *gate, const void *up, int64_t l
  * act_scale_layout = WAVE_MXFP4_SCALE_MFMA32, the order the second GEMM reads) of
  * silu(gate) * up, bit-identical to wave_mxfp4_gemm_grouped (bf16 out) followed
  * by wave_mxfp4_silu_and_mul_quantize on its two halves.  num_groups = 0 with
- * offsets = NULL is the dense problem.  Served by the persistent 256x256 kernel
- * only: I % 128 == 0, K % 256 == 0, K >= 768, more 256x256 tiles than CUs, a
- * workspace of wave_mxfp4_grouped_workspace_bytes(total_rows, n, k, max(num_groups, 1))
- * bytes, scales row-major or MFMA32, B row-major; WAVE_MXFP4_ERR_UNSUPPORTED
+ * offsets = NULL is the dense problem.  Served by two kernels: the persistent
+ * 256x256 kernel (more 256x256 tiles than CUs), and, for a small batch routed
+ * over the experts (grouped, at most 152 rows per expert on average, the
+ * experts' B scales resident in MFMA32 order, at least half as many
+ * 128-column strips over all experts as CUs), the mid-M kernel that
+ * wave_mxfp4_gemm_grouped gives such a batch to.  Either way I % 128 == 0,
+ * K % 256 == 0, K >= 1024 (768 on the persistent kernel), a workspace of
+ * wave_mxfp4_grouped_workspace_bytes(total_rows, n, k, max(num_groups, 1)) bytes,
+ * scales row-major or MFMA32, B row-major; WAVE_MXFP4_ERR_UNSUPPORTED
  * otherwise (the caller then runs the two calls).  Rows past the last offset
  * are left untouched, as are the padding rows of an MFMA32 scale tensor. */
 int wave_mxfp4_gemm_gated_quantize(const void *a, const void *a_scale, const void *b, const void *b_scale, void *q,

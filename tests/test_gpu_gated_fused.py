@@ -124,3 +124,56 @@ def test_rows_past_the_last_offset_are_left_alone_and_small_problems_are_refused
     assert lib.wave_mxfp4_gemm_gated_quantize(gx.data_ptr(), gxs.data_ptr(), w_il.data_ptr(), ws_il.data_ptr(), q.data_ptr(),
                                               s.data_ptr(), off.data_ptr(), 3, rows, 2 * inter, k, RM, RM, RM,
                                               scratch.data_ptr(), ws_bytes, stream) == _lib.ERR_UNSUPPORTED
+
+
+# ---- a small batch routed over the experts: the same epilogue in the grouped mid-M kernel ----
+
+def run_small_batch(counts, inter, k, seed, a_native, slack_rows=0):
+    """Resident weight scales (MFMA32) and a batch the grouped call gives to the mid-M kernel: far too few 256x256
+    tiles for the persistent kernel, so a fused call that succeeds ran the mid-M kernel.  Against the chain through
+    the same kernel (grouped GEMM, variant MID_M, bf16 out, then silu_and_mul_quantize), bit for bit."""
+    e, n = len(counts), 2 * inter
+    valid = int(sum(counts))
+    rows = valid + slack_rows
+    x, xs, _, _ = orc.make_inputs(rows, 1, k, seed, scale_lo=122, scale_hi=128)
+    rng = np.random.default_rng(seed + 1)
+    w = rng.integers(0, 256, size=(e, n, k // 2), dtype=np.uint8)
+    ws = rng.integers(120, 127, size=(e, n, k // 32), dtype=np.uint8)
+    gx, gxs, gw, gws = to_gpu(x, xs, w, ws)
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)).to(DEV)
+    c = torch.full((rows, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    wave_amd.mxfp4_gemm_grouped(gx, gxs, gw, gws, off, c, variant=_lib.VARIANT_MID_M)
+    q_ref, s_ref = wave_amd.silu_and_mul_quantize(c[:valid, :inter], c[:valid, inter:], scale_layout=RM)
+    w_il, ws_il = wave_amd.interleave_gate_up(gw), wave_amd.interleave_gate_up(gws)
+    ws_il = torch.stack([wave_amd.scale_convert(ws_il[g], n, k // 32, RM, M32) for g in range(e)])
+    a_s, la = gxs, RM
+    if a_native:
+        a_s, la = wave_amd.scale_convert(gxs, rows, k // 32, RM, M32), M32
+    lib = _lib.load()
+    q = torch.full((rows, inter // 2), 0xAB, dtype=torch.uint8, device=DEV)
+    s = torch.full(((rows + 31) // 32 * 32, (inter // 32 + 7) // 8 * 8), 0xCD, dtype=torch.uint8, device=DEV)
+    ws_bytes = int(lib.wave_mxfp4_grouped_workspace_bytes(rows, n, k, e))
+    scratch = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=DEV)
+    st = lib.wave_mxfp4_gemm_gated_quantize(gx.data_ptr(), a_s.data_ptr(), w_il.data_ptr(), ws_il.data_ptr(), q.data_ptr(),
+                                            s.data_ptr(), off.data_ptr(), e, rows, n, k, la, M32, M32,
+                                            scratch.data_ptr(), scratch.numel(), torch.cuda.current_stream().cuda_stream)
+    assert st == _lib.OK, st
+    torch.cuda.synchronize()
+    assert torch.equal(q[:valid], q_ref), "packed codes differ from the unfused chain"
+    assert bool((q[valid:] == 0xAB).all()), "rows past the last offset were written"
+    s_rm = wave_amd.scale_convert(s, rows, inter // 32, M32, RM)
+    assert torch.equal(s_rm[:valid], s_ref), "scales differ from the unfused chain"
+    assert bool((s_rm[valid:] == 0xCD).all()), "scales of rows past the last offset were written"
+    codes = torch.bincount((q[:valid].flatten() & 15).to(torch.int64), minlength=16)
+    assert int((codes > 0).sum()) >= 12 and len(torch.unique(s_rm[:valid])) >= 3
+
+
+@pytest.mark.parametrize("a_native", [False, True], ids=["a_scales_row_major", "a_scales_mfma32"])
+@pytest.mark.parametrize("counts,inter,k", [
+    ([16, 9, 0, 31, 22, 1, 40, 13], 1024, 1024),              # blocks of 64 rows, one live row block in most
+    ([70, 20, 64, 65, 3, 0, 50, 47], 1792, 2048),             # blocks of 64 rows, two groups of a second pass
+    ([100, 0, 260, 33, 1, 150, 97, 128], 1024, 1024),         # blocks of 128 rows, a group of three passes
+    ([150, 160, 140, 155, 149, 132, 141, 143], 1024, 1536),   # blocks of 192 rows
+], ids=["bm64_sparse", "bm64", "bm128", "bm192"])
+def test_small_batch_fused_in_the_mid_kernel_matches_the_chain(counts, inter, k, a_native):
+    run_small_batch(counts, inter, k, seed=sum(counts) + k, a_native=a_native, slack_rows=37)

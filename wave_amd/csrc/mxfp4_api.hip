@@ -878,6 +878,17 @@ int wave_mxfp4_gemm_gated_quantize(const void *a, const void *a_scale, const voi
     p.b_scale_group_stride = b_native ? ((n + 31) / 32 * 32) * (int64_t)p.ksp : n * (int64_t)p.ks;
     p.tile_table = table;
   }
+  // A small batch routed over the experts (the range the grouped call gives to the mid-M kernel): the same
+  // epilogue in that kernel, one launch, no table, the scales read as they are.
+  if (num_groups > 0 && b_native && mid_gated_applies(p)) {
+    const int64_t avg = (total_rows + num_groups - 1) / num_groups;
+    if (avg <= kGroupedMidMaxAvgRows && (int64_t)num_groups * (n / 128) >= device_cus() / 2) {
+      int64_t bm = (5 * avg + 3) / 4 < total_rows ? (5 * avg + 3) / 4 : total_rows;
+      bm = bm > 192 ? 192 : (bm + 63) / 64 * 64;
+      p.tile_table = nullptr;
+      return record_hip(launch_mid_gated(p, stream, (int)bm));
+    }
+  }
   GemmParams q32 = p;
   q32.a_scale_layout = q32.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
   if (!persist_gated_applies(q32, device_cus())) return WAVE_MXFP4_ERR_UNSUPPORTED;

@@ -99,10 +99,16 @@ struct MidCfg {
 // a branch on the layout inside the K loop makes the compiler wait for every outstanding request at the join.
 // One strip of one block of `m_rows` <= BM rows: A [m_rows, kp] at `a_base` with its scales at `as_base`, B [N, kp]
 // at `b_base` (one expert's, for a grouped problem) with its scales at `bs_base`, C rows at `c_base`.
-template <class Cfg, bool A_RM, bool B_SH, bool A_SH>
+// GATED: the first GEMM of a gated MLP with the step behind it in its C write, as in the persistent kernel
+// (mxfp4_gemm_persist.hip): B holds gate and up rows interleaved in blocks of 32, so the two column groups of a wave
+// are gate and up of the same 32 activation columns, element for element in the same lane; written are the MXFP4
+// codes of silu(gate) * up ([rows, N / 4] bytes at `c_base`) and one e8m0 scale per row and 32 columns in MFMA32
+// order at p.epi_scale (row `m_abs0` + the block's row).  The arithmetic of the unfused pair of kernels, bit for bit.
+template <class Cfg, bool A_RM, bool B_SH, bool A_SH, bool GATED = false>
 __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, const uint8_t *a_base, const uint8_t *as_base,
                                          const uint8_t *b_base, const uint8_t *bs_base, uint8_t *c_base, const int m_rows,
-                                         const int a_row32 = 0) {
+                                         const int a_row32 = 0, const int m_abs0 = 0) {
+  static_assert(!GATED || (Cfg::WM == 2 && !Cfg::B_RM && !B_SH), "gated epilogue: a wave holds a gate and an up group; B scales MFMA32");
   constexpr bool B_RM = Cfg::B_RM;
   constexpr int MT_M = Cfg::MT_M, DA = Cfg::DA, DB = Cfg::DB, LB = Cfg::LB;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -402,6 +408,65 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 
+  if constexpr (GATED) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const int qrow = p.n >> 2;    // bytes of a row of codes
+    const int act_ks = p.n >> 6;  // scale groups of a row of the activation
+    const int s_kt = (act_ks + 7) >> 3;
+    const __amdgpu_buffer_rsrc_t q_rsrc = make_rsrc_n(c_base, (int)min((int64_t)m_rows * qrow, (int64_t)0x7FFFFFFF));
+    const __amdgpu_buffer_rsrc_t s_rsrc = make_rsrc_n(p.epi_scale, rsrc_bytes((int64_t)((p.m + 31) >> 5) * s_kt * 256));
+    const int g = (n0 >> 6) + wn;  // the activation's scale group: the strip's pair of column groups of this wave
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      if (i >= live) break;
+      const int r_tile = (WM * i + wm) * 32 + fr;
+      const v16f &ga = acc[i][0], &ua = acc[i][1];
+      uint32_t h[8];
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        // the GEMM's bf16 output of the unfused pipeline, then its activation kernel's arithmetic
+        const bf16x2 g2 = {(__bf16)ga[2 * w], (__bf16)ga[2 * w + 1]}, u2 = {(__bf16)ua[2 * w], (__bf16)ua[2 * w + 1]};
+        const uint32_t gb = __builtin_bit_cast(uint32_t, g2), ub = __builtin_bit_cast(uint32_t, u2);
+        const float g0 = __builtin_bit_cast(float, gb << 16), g1 = __builtin_bit_cast(float, gb & 0xFFFF0000u);
+        const float u0 = __builtin_bit_cast(float, ub << 16), u1 = __builtin_bit_cast(float, ub & 0xFFFF0000u);
+        const float r0 = g0 * u0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g0 * -1.44269504088896340736f));
+        const float r1 = g1 * u1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g1 * -1.44269504088896340736f));
+        const bf16x2 o = {(__bf16)r0, (__bf16)r1};
+        h[w] = __builtin_bit_cast(uint32_t, o);
+        lo = max(lo, h[w] & 0x7FFFu);
+        hi = max(hi, (h[w] >> 16) & 0x7FFFu);
+      }
+      // the group's largest magnitude: this lane's 16 columns and the other lane's
+      const uint32_t mine = max(lo, hi);
+      const auto both = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
+      const uint32_t amax = max(both[0], both[1]) << 16;
+      const uint32_t e = (amax + 0x200000u) >> 23;
+      const uint32_t sb = e >= 255u ? 254u : (e > 2u ? e - 2u : 0u);
+      const float sf = __builtin_bit_cast(float, sb ? sb << 23 : 0x00400000u);
+      uint32_t c0 = 0, c1 = 0;
+      c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[0]), sf, 0);
+      c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[1]), sf, 1);
+      c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[2]), sf, 2);
+      c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c0, __builtin_bit_cast(bf16x2, h[3]), sf, 3);
+      c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[4]), sf, 0);
+      c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[5]), sf, 1);
+      c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[6]), sf, 2);
+      c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(c1, __builtin_bit_cast(bf16x2, h[7]), sf, 3);
+      // lanes 0..31 get the upper lanes' dword 0, lanes 32..63 the lower lanes' dword 1: each lane then holds
+      // 8 consecutive bytes of its row's 16 (the lower lanes bytes 0..7, the upper lanes bytes 8..15)
+      const auto sw = __builtin_amdgcn_permlane32_swap(c0, c1, false, false);
+      v2i out;
+      out.x = (int)__builtin_amdgcn_perm(sw[1], sw[0], 0x05040100u);
+      out.y = (int)__builtin_amdgcn_perm(sw[1], sw[0], 0x07060302u);
+      // (rows past the block's own lie past the end of the descriptor: dropped)
+      __builtin_amdgcn_raw_buffer_store_b64(out, q_rsrc, r_tile * qrow + g * 16 + fg * 8, 0, 0);
+      const int r_abs = m_abs0 + r_tile;
+      const int s_off = ((r_abs >> 5) * s_kt + (g >> 3)) * 256 + (((g & 1) << 5) | (r_abs & 31)) * 4 + ((g & 7) >> 1);
+      __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sb, s_rsrc, fg == 0 && r_tile < m_rows ? s_off : (int)0x80000000, 0, 0);
+    }
+    return;
+  }
   // ---------------- C: accumulators -> the wave's ring -> global ----------------
   // acc[i][jn][4q + e] is row lane % 32, column 8q + 4 * (lane / 32) + e of the 32 x 32 tile (row block
   // WM i + wm, group NJ wn + jn).  A tile is staged as 32 rows of eight 4-column pieces and stored 8 rows per
@@ -466,22 +531,22 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
 // GROUPED: blockIdx.y is the expert; its rows offsets[e] .. offsets[e + 1] (clamped to [0, M], not validated) are
 // taken BM at a time - a group of more rows than BM streams its expert's B once per block of rows, which is what
 // the table-driven persistent kernel is for; this one is for the few rows per expert of a small batch.
-template <class Cfg, bool A_RM, bool GROUPED, bool B_SH, bool A_SH>
+template <class Cfg, bool A_RM, bool GROUPED, bool B_SH, bool A_SH, bool GATED = false>
 __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p, const int wv) {
   static_assert(!(A_RM && A_SH), "one layout");
   if constexpr (!GROUPED) {
-    mid_body<Cfg, A_RM, B_SH, A_SH>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
+    mid_body<Cfg, A_RM, B_SH, A_SH, GATED>(p, wv, p.a, p.a_scale, p.b, p.b_scale, (uint8_t *)p.c, p.m);
   } else {
     static_assert(A_RM || (Cfg::A_OFF && !A_SH), "a group may start at any row: A's scales row-major, or MFMA32 with room for the block it starts in");
     const int e = blockIdx.y;
     const int lo = __builtin_amdgcn_readfirstlane(min(max(p.offsets[e], 0), p.m));
     const int hi = __builtin_amdgcn_readfirstlane(min(max(p.offsets[e + 1], lo), p.m));
     const uint8_t *b = p.b + (int64_t)e * p.b_group_stride, *bs = p.b_scale + (int64_t)e * p.b_scale_group_stride;
-    const int elt = p.out_bf16 ? 2 : 4;
+    const int64_t c_row = GATED ? p.n >> 2 : (int64_t)p.n * (p.out_bf16 ? 2 : 4);  // bytes of a row of what is written
     for (int m0 = lo; m0 < hi; m0 += Cfg::BM) {
       const uint8_t *as = A_RM ? p.a_scale + (int64_t)m0 * p.ks : p.a_scale + (int64_t)(m0 >> 5) * p.k_tiles * 256;
-      mid_body<Cfg, A_RM, B_SH, A_SH>(p, wv, p.a + (int64_t)m0 * p.kp, as, b, bs,
-                          (uint8_t *)p.c + (int64_t)m0 * p.n * elt, min(Cfg::BM, hi - m0), A_RM ? 0 : m0 & 31);
+      mid_body<Cfg, A_RM, B_SH, A_SH, GATED>(p, wv, p.a + (int64_t)m0 * p.kp, as, b, bs,
+                          (uint8_t *)p.c + (int64_t)m0 * c_row, min(Cfg::BM, hi - m0), A_RM ? 0 : m0 & 31, m0);
       // every wave is done with the rings (the C staging's reads included) before the next block's requests
       __builtin_amdgcn_s_waitcnt(0);
       asm volatile("" ::: "memory");
@@ -491,14 +556,14 @@ __global__ void __launch_bounds__(kMidNT, 1) mid_gemm_kernel(const GemmParams p,
   }
 }
 
-template <class Cfg, bool A_RM, bool GROUPED, bool B_SH, bool A_SH = false>
+template <class Cfg, bool A_RM, bool GROUPED, bool B_SH, bool A_SH = false, bool GATED = false>
 hipError_t launch_mid_kernel(const GemmParams &p, int wv, hipStream_t stream) {
   static LdsAttrOnce once;
-  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH, A_SH>, Cfg::LDS);
+  hipError_t e = allow_dynamic_lds(once, (const void *)mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH, A_SH, GATED>, Cfg::LDS);
   if (e != hipSuccess) return e;
   const int bn = kMidCW * wv;
   const dim3 grid((p.n + bn - 1) / bn, GROUPED ? p.num_groups : 1, 1);
-  mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH, A_SH><<<grid, dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
+  mid_gemm_kernel<Cfg, A_RM, GROUPED, B_SH, A_SH, GATED><<<grid, dim3(kMidNT), Cfg::LDS, stream>>>(p, wv);
   return hipGetLastError();
 }
 
@@ -607,6 +672,28 @@ hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream,
   if (bm <= 128) return launch_mid_cfg<128>(p, wv, stream);
   if (bm <= 192) return launch_mid_cfg<192>(p, wv, stream);
   return launch_mid_cfg<256>(p, wv, stream);
+}
+
+// The gated, quantising form (grouped): blocks of 64, 128 or 192 rows (a wave needs both column groups of a pair: the
+// 32-row block's four waves side by side do not have them), both B scale tensors in MFMA32 order, whole 128-column
+// strips of gate / up pairs.
+bool mid_gated_applies(const GemmParams &p) {
+  return mid_grouped_applies(p) && p.epi_scale != nullptr && p.epi_scale_layout == WAVE_MXFP4_SCALE_MFMA32 &&
+         p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && !p.b_preshuffled && p.out_bf16 && (p.n & 127) == 0 &&
+         (int64_t)p.m * (p.n >> 2) < ((int64_t)1 << 31);
+}
+
+template <int BM>
+static hipError_t launch_mid_gated_bm(const GemmParams &p, hipStream_t stream) {
+  if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR)
+    return launch_mid_kernel<MidCfg<BM, false, false, false>, true, true, false, false, true>(p, 32, stream);
+  return launch_mid_kernel<MidCfg<BM, false, false, true>, false, true, false, false, true>(p, 32, stream);
+}
+
+hipError_t launch_mid_gated(const GemmParams &p, hipStream_t stream, int bm) {
+  if (bm <= 64) return launch_mid_gated_bm<64>(p, stream);
+  if (bm <= 128) return launch_mid_gated_bm<128>(p, stream);
+  return launch_mid_gated_bm<192>(p, stream);
 }
 
 }  // namespace wave_mxfp4

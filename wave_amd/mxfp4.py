@@ -518,8 +518,10 @@ def mxfp4_gemm_gated_quantize(x, x_scales, w_il, w_scales_il, offsets=None, *, a
     """The first GEMM of a gated expert MLP with :func:`silu_and_mul_quantize` fused into its output: ``w_il``
     ``[E, 2I, K/2]`` (or ``[2I, K/2]`` with ``offsets=None``: dense) holds gate and up projections interleaved by
     :func:`interleave_gate_up`, as do its scales.  Returns ``(q [rows, I/2], scales)`` of ``silu(gate) * up``, the
-    same bits as ``mxfp4_gemm_grouped`` (bf16 out) followed by ``silu_and_mul_quantize``.  Raises ``ValueError``
-    (status "unsupported") where the fused kernel does not apply; the caller then runs the two calls."""
+    same bits as ``mxfp4_gemm_grouped`` (bf16 out) followed by ``silu_and_mul_quantize``.  Large batches run the
+    persistent kernel, small grouped ones (up to 152 rows per expert on average) with ``b_scale_layout`` MFMA32 the
+    mid-M kernel.  Raises ``ValueError`` (status "unsupported") where neither applies; the caller then runs the
+    two calls."""
     lib = _lib.load()
     x, w_il = _as_u8(x, "x"), _as_u8(w_il, "w_il")
     x_scales, w_scales_il = _as_u8(x_scales, "x_scales"), _as_u8(w_scales_il, "w_scales_il")

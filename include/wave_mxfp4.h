@@ -231,6 +231,32 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
                     size_t workspace_bytes, int variant, void *hip_stream);
 size_t wave_mxfp8_workspace_bytes(int64_t m, int64_t n, int64_t k);
 
+/* An 8-bit B [rows, K] (one byte per element) into the order a B-direct kernel
+ * reads with one coalesced 16-byte load per lane and half MFMA operand: the
+ * 8-bit counterpart of b_preshuffle (mxfp_utils.py:98-110, which the
+ * reference defines for packed MXFP4 rows only; this layout is this
+ * library's).  Blocks of 32 rows x 128 bytes (one K tile), 4096 bytes each,
+ * block (r / 32, kt) at ((r / 32) * (K / 128) + kt) * 4096; inside a block
+ * the 16-byte pieces follow each other as [K step s = 0..1][half h = 0..1]
+ * [lane l = 0..63], and lane l = 32 * g + r' holds row r' of the block, bytes
+ * 64 * s + 32 * h + 16 * g .. + 15 of the K tile (the scaled MFMA takes a
+ * lane's 32 bytes of an 8-bit operand as two halves 32 bytes apart in K).
+ * rows % 32 == 0, K % 128 == 0; not in place. */
+int wave_mxfp8_b_preshuffle(const void *b, void *out, int64_t rows, int64_t k, void *hip_stream);
+
+/* wave_mxfp8_gemm with B in wave_mxfp8_b_preshuffle order: A through LDS, B
+ * straight from global memory into registers (the schedule of
+ * wave_lang/kernel/wave/schedules/gemm_mxfp4_double_buffer.py:1781-2222 on the
+ * operands of tests/kernel/wave_gemm_mxfp_test.py:416-501).  Both operands
+ * 8-bit (e4m3 / e5m2 in any pairing), N % 256 == 0, K % 256 == 0, K >= 768, any
+ * M; each scale tensor row-major or WAVE_MXFP4_SCALE_MFMA32 (with a row-major
+ * one the workspace of wave_mxfp8_workspace_bytes(m, n, k) bytes is required:
+ * it is re-laid out there first).  WAVE_MXFP4_ERR_UNSUPPORTED otherwise. */
+int wave_mxfp8_gemm_b_preshuffled(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
+                                  int64_t m, int64_t n, int64_t k, int a_format, int b_format, int out_dtype,
+                                  int a_scale_layout, int b_scale_layout, void *workspace, size_t workspace_bytes,
+                                  void *hip_stream);
+
 /* Packed e2m1 [rows, kp] -> f32 [rows, 2*kp] through the 16-entry table, code 8
  * gives -0.0 (mxfp_utils.py:60-83).  Bit-exact. */
 int wave_mxfp4_to_f32(const void *q, float *out, int64_t rows, int64_t kp, void *hip_stream);

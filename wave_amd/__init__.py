@@ -14,6 +14,7 @@ from .mxfp4 import (
     mxfp4_gemm_grouped,
     moe_align_block_size,
     mxfp4_to_f32,
+    mxfp8_b_preshuffle,
     mxfp8_gemm,
     quantize_mxfp4,
     quantize_mxfp4_rows,
@@ -34,6 +35,7 @@ __all__ = [
     "mxfp4_gemm_grouped",
     "moe_align_block_size",
     "mxfp4_to_f32",
+    "mxfp8_b_preshuffle",
     "mxfp8_gemm",
     "quantize_mxfp4",
     "quantize_mxfp4_rows",

@@ -53,6 +53,8 @@ EXPORTS = (
     "wave_mxfp4_grouped_workspace_bytes",
     "wave_mxfp8_gemm",
     "wave_mxfp8_workspace_bytes",
+    "wave_mxfp8_b_preshuffle",
+    "wave_mxfp8_gemm_b_preshuffled",
     "wave_mxfp4_to_f32",
     "wave_mxfp4_e8m0_to_f32",
     "wave_mxfp4_dequant",
@@ -102,6 +104,10 @@ def load():
     lib.wave_mxfp8_workspace_bytes.argtypes = [i64, i64, i64]
     lib.wave_mxfp8_workspace_bytes.restype = sz
     lib.wave_mxfp8_gemm.restype = i32
+    lib.wave_mxfp8_b_preshuffle.argtypes = [p, p, i64, i64, p]
+    lib.wave_mxfp8_b_preshuffle.restype = i32
+    lib.wave_mxfp8_gemm_b_preshuffled.argtypes = [p, p, p, p, p, i64, i64, i64, i32, i32, i32, i32, i32, p, sz, p]
+    lib.wave_mxfp8_gemm_b_preshuffled.restype = i32
     lib.wave_mxfp4_to_f32.argtypes = [p, p, i64, i64, p]
     lib.wave_mxfp4_to_f32.restype = i32
     lib.wave_mxfp4_e8m0_to_f32.argtypes = [p, p, i64, p]

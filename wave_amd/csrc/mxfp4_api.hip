@@ -681,6 +681,68 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   return record_hip(launch_tile_gemm_fp8(p, v, a_format, b_format, stream));
 }
 
+int wave_mxfp8_b_preshuffle(const void *b, void *out, int64_t rows, int64_t k, void *hip_stream) {
+  if (rows < 0 || k < 0 || rows % 32 != 0 || k % 128 != 0) return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (rows == 0 || k == 0) return WAVE_MXFP4_OK;
+  if (!b || !out) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (b == out) return WAVE_MXFP4_ERR_UNSUPPORTED;  // not in place
+  if (!aligned(b, 16) || !aligned(out, 16)) return WAVE_MXFP4_ERR_MISALIGNED;
+  return record_hip(launch_b8_preshuffle((const uint8_t *)b, (uint8_t *)out, rows, k, (hipStream_t)hip_stream));
+}
+
+int wave_mxfp8_gemm_b_preshuffled(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
+                                  int64_t m, int64_t n, int64_t k, int a_format, int b_format, int out_dtype,
+                                  int a_scale_layout, int b_scale_layout, void *workspace, size_t workspace_bytes,
+                                  void *hip_stream) {
+  if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim || k % 128 != 0 || n % 32 != 0)
+    return WAVE_MXFP4_ERR_BAD_SHAPE;
+  if (bad_enum(a_format, 3) || bad_enum(b_format, 3) || bad_enum(out_dtype, 2) || bad_enum(a_scale_layout, 4) ||
+      bad_enum(b_scale_layout, 4))
+    return WAVE_MXFP4_ERR_BAD_ENUM;
+  const auto rm_or_native = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
+  // (the preshuffled order is defined for 8-bit rows; the kernel that reads it takes whole 256-column tiles and
+  // pairs of K tiles)
+  if (a_format == WAVE_MXFP8_E2M1 || b_format == WAVE_MXFP8_E2M1 || !rm_or_native(a_scale_layout) ||
+      !rm_or_native(b_scale_layout) || n % 256 != 0 || k % 256 != 0 || k < 768)
+    return WAVE_MXFP4_ERR_UNSUPPORTED;
+  if (m == 0 || n == 0) return WAVE_MXFP4_OK;
+  if (!c || !a || !a_scale || !b || !b_scale) return WAVE_MXFP4_ERR_NULL_POINTER;
+  if (!aligned(a, 16) || !aligned(b, 16) || !aligned(a_scale, 4) || !aligned(b_scale, 4) || !aligned(c, 16))
+    return WAVE_MXFP4_ERR_MISALIGNED;
+  if (k * 256 >= ((int64_t)1 << 31)) return WAVE_MXFP4_ERR_UNSUPPORTED;  // 32-bit offsets inside a tile
+  if (workspace && !aligned(workspace, 256)) return WAVE_MXFP4_ERR_MISALIGNED;
+  hipStream_t stream = (hipStream_t)hip_stream;
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.a = (const uint8_t *)a, p.a_scale = (const uint8_t *)a_scale;
+  p.b = (const uint8_t *)b, p.b_scale = (const uint8_t *)b_scale;
+  p.c = c;
+  p.m = (int)m, p.n = (int)n, p.k = (int)k;
+  p.kp = (int)k;  // bytes per operand row
+  p.ks = (int)(k / 32);
+  p.ksp = p.ks;  // (K % 256 == 0)
+  p.k_tiles = (int)(k / 128);
+  p.tiles_per_split = p.k_tiles;
+  p.splits = 1;
+  p.out_bf16 = out_dtype == WAVE_MXFP4_OUT_BF16;
+  p.tiles_m = (int)((m + 255) / 256);
+  p.tiles_n = (int)(n / 256);
+  const bool a_native = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32, b_native = b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
+  if (!a_native || !b_native) {
+    // the row-major ones into MFMA32 order first (one launch)
+    const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k));
+    if (!workspace || workspace_bytes < wave_mxfp8_workspace_bytes(m, n, k)) return WAVE_MXFP4_ERR_UNSUPPORTED;
+    const hipError_t e = launch_scale_pair_to_mfma32(p.a_scale, (uint8_t *)workspace, a_native ? 0 : m, p.b_scale,
+                                                     (uint8_t *)workspace + a_bytes, b_native ? 0 : n, p.ks, stream);
+    if (e != hipSuccess) return e == hipErrorInvalidValue ? WAVE_MXFP4_ERR_UNSUPPORTED : record_hip(e);
+    if (!a_native) p.a_scale = (const uint8_t *)workspace;
+    if (!b_native) p.b_scale = (const uint8_t *)workspace + a_bytes;
+  }
+  p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+  if (!asym8_gemm_applies(p, device_cus())) return WAVE_MXFP4_ERR_UNSUPPORTED;
+  return record_hip(launch_asym8_gemm(p, device_cus(), a_format, b_format, stream));
+}
+
 // Scratch of a grouped call: [M tile table | A scales | B scales].
 static size_t grouped_table_bytes(int64_t total_rows, int num_groups) {
   return round_up_256((size_t)(1 + total_rows / 256 + num_groups) * 16);

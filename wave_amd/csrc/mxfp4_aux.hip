@@ -203,6 +203,20 @@ __global__ void b_preshuffle_kernel(const uint8_t *__restrict__ b, uint8_t *__re
   }
 }
 
+// 8-bit B [rows, k] -> the order the B-direct MXFP8 kernel reads (mxfp8_gemm_asym.hip): blocks of 32 rows x 128
+// bytes, block (n / 32, kt) at ((n / 32) * (k / 128) + kt) * 4096, its 16-byte pieces as [K step][half][lane],
+// lane = 32 * g + r holding row r's bytes 64 * step + 32 * half + 16 * g .. + 15.  One thread per piece of the result.
+__global__ void b8_preshuffle_kernel(const uint8_t *__restrict__ b, uint8_t *__restrict__ out, int64_t rows, int64_t k) {
+  const int64_t total = rows * (k >> 4), k_tiles = k >> 7;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t blk = i >> 8, nb = blk / k_tiles, kt = blk - nb * k_tiles;
+    const int piece = (int)(i & 255), q = piece >> 6, lane = piece & 63;
+    const int64_t row = nb * 32 + (lane & 31);
+    const int64_t col = kt * 128 + (q >> 1) * 64 + (q & 1) * 32 + (lane >> 5) * 16;
+    *(v4i *)(out + i * 16) = *(const v4i *)(b + row * k + col);
+  }
+}
+
 // Rows of a [2 * half_rows, row_bytes] matrix whose first half is a gate projection and whose second half the
 // matching up projection, interleaved in blocks of `block` rows: out block 2 b = gate rows block b, out block
 // 2 b + 1 = up rows block b.  One thread per 4 bytes (row_bytes % 4 == 0) or per byte.
@@ -399,6 +413,13 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
 
 hipError_t launch_scale_spread_rows(const uint8_t *src, uint8_t *dst, int64_t rows, int64_t ks, hipStream_t stream) {
   scale_spread_rows_kernel<<<blocks_for(rows * ks, 256), 256, 0, stream>>>(src, dst, rows, ks);
+  return hipGetLastError();
+}
+
+hipError_t launch_b8_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t k, hipStream_t stream) {
+  const int64_t n = rows * (k / 16);
+  if (n == 0) return hipSuccess;
+  b8_preshuffle_kernel<<<blocks_for(n, kThreads), kThreads, 0, stream>>>(b, out, rows, k);
   return hipGetLastError();
 }
 

@@ -140,6 +140,9 @@ bool persist_gated_applies(const GemmParams &p, int num_cus);
 hipError_t launch_persist_gated(const GemmParams &p, int num_cus, hipStream_t stream);
 hipError_t launch_interleave_rows(const uint8_t *src, uint8_t *dst, int64_t half_rows, int64_t row_bytes, int block,
                                   hipStream_t stream);
+bool asym8_gemm_applies(const GemmParams &p, int num_cus);
+hipError_t launch_asym8_gemm(const GemmParams &p, int num_cus, int a_fmt, int b_fmt, hipStream_t stream);
+hipError_t launch_b8_preshuffle(const uint8_t *b, uint8_t *out, int64_t rows, int64_t k, hipStream_t stream);
 bool asym_gemm_applies(const GemmParams &p, int num_cus, bool forced);
 hipError_t launch_asym_gemm(const GemmParams &p, int num_cus, hipStream_t stream);
 bool midb_gemm_applies(const GemmParams &p);

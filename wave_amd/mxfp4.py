@@ -557,8 +557,29 @@ def mxfp4_gemm_gated_quantize(x, x_scales, w_il, w_scales_il, offsets=None, *, a
 _FP8_FORMATS = {torch.float8_e4m3fn: _lib.MXFP8_E4M3, torch.float8_e5m2: _lib.MXFP8_E5M2}
 
 
+def mxfp8_b_preshuffle(b: torch.Tensor) -> torch.Tensor:
+    """``[N, K]`` 8-bit weights (uint8 / int8 / float8) -> the same bytes in the order the B-direct MXFP8 kernel
+    reads with one coalesced 16-byte load per lane (blocks of 32 rows x 128 bytes; the layout is this library's:
+    the reference's ``b_preshuffle``, wave_lang/kernel/wave/utils/mxfp_utils.py:98-110, covers packed MXFP4 rows
+    only).  N % 32 == 0, K % 128 == 0.  For :func:`mxfp8_gemm` with ``b_preshuffled=True``."""
+    lib = _lib.load()
+    dt = b.dtype
+    if dt in _FP8_FORMATS or dt == torch.int8:
+        b = b.view(torch.uint8)
+    b = _as_u8(b, "b")
+    if b.dim() != 2:
+        raise ValueError("b must be [N, K]")
+    rows, k = b.shape
+    out = torch.empty_like(b)
+    with _on_device(b.device):
+        st = lib.wave_mxfp8_b_preshuffle(b.data_ptr(), out.data_ptr(), rows, k, _stream_ptr(b.device))
+    _lib.check(st, "wave_mxfp8_b_preshuffle")
+    return out.view(dt)
+
+
 def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
-               variant=_lib.VARIANT_AUTO, workspace=None) -> None:
+               variant=_lib.VARIANT_AUTO, workspace=None, b_preshuffled=False,
+               a_scale_layout=_lib.SCALE_ROW_MAJOR, b_scale_layout=_lib.SCALE_ROW_MAJOR) -> None:
     """``out[M, N] = (x * scales) @ (w_t * scales).T`` for MXFP8 operands:
     ``x [M, K]``, ``w_t [N, K]`` one byte per element, scales ``[R, K/32]`` e8m0
     (tests/kernel/wave_gemm_mxfp_test.py:416-501, which passes
@@ -569,7 +590,10 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
     operand is ``[rows, K/2]`` packed MXFP4 against the 8-bit other (8-bit activations
     against 4-bit weights or the other way round, the mixed operands of
     wave_lang/kernel/wave/constraints.py:425-431; both 4-bit is :func:`mxfp4_gemm`).
-    ``workspace`` as in :func:`mxfp4_gemm`."""
+    ``workspace`` as in :func:`mxfp4_gemm`.  ``b_preshuffled=True``: ``w_t`` comes from
+    :func:`mxfp8_b_preshuffle` and the B-direct kernel runs (both operands 8-bit, N % 256 == 0,
+    K % 256 == 0, K >= 768; ``ValueError`` "unsupported" otherwise); only that call takes scale
+    tensors in MFMA32 order (``a_scale_layout`` / ``b_scale_layout``)."""
     lib = _lib.load()
     given = tuple(elem_format) if isinstance(elem_format, (tuple, list)) else (elem_format, elem_format)
     if len(given) != 2:
@@ -598,8 +622,10 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
     n = w_t.shape[0]
     if k % 128:
         raise ValueError(f"K = {k} must be a multiple of 128")
-    _scale_rows_ok(x_scales, m, k // 32, _lib.SCALE_ROW_MAJOR, "x_scales")
-    _scale_rows_ok(w_scales, n, k // 32, _lib.SCALE_ROW_MAJOR, "w_scales")
+    if not b_preshuffled and (a_scale_layout != _lib.SCALE_ROW_MAJOR or b_scale_layout != _lib.SCALE_ROW_MAJOR):
+        raise ValueError("scales in another order than row-major: only with b_preshuffled=True")
+    _scale_rows_ok(x_scales, m, k // 32, a_scale_layout, "x_scales")
+    _scale_rows_ok(w_scales, n, k // 32, b_scale_layout, "w_scales")
     od = _check_out(out, (m, n))
     ws_ptr, ws_bytes = None, 0
     if workspace is None:
@@ -608,6 +634,13 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
         workspace = None
     if workspace is not None:
         ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    if b_preshuffled:
+        with _on_device(x.device):
+            st = lib.wave_mxfp8_gemm_b_preshuffled(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
+                                                   out.data_ptr(), m, n, k, fmts[0], fmts[1], od, a_scale_layout,
+                                                   b_scale_layout, ws_ptr, ws_bytes, _stream_ptr(x.device))
+        _lib.check(st, "wave_mxfp8_gemm_b_preshuffled")
+        return
     with _on_device(x.device):
         st = lib.wave_mxfp8_gemm(x.data_ptr(), x_scales.data_ptr(), w_t.data_ptr(), w_scales.data_ptr(),
                                  out.data_ptr(), m, n, k, fmts[0], fmts[1], od, ws_ptr, ws_bytes, variant,

@@ -25,11 +25,12 @@ CSRC = os.path.join(ROOT, "wave_amd", "csrc")
 # library picks by itself for the shapes the throughput figures are quoted on:
 #  * the 4-wave one-tile-per-workgroup 256x256 kernel (variant T256x256_W2x2; AUTO takes the 8-wave one),
 #  * the streaming kernel's 49..64-row instantiation with one or two waves along K (all 512 registers hold A).
-#  * the B-direct kernel with bf16 output: a handful of registers are spilled and reloaded once per OUTPUT TILE,
+#  * the B-direct kernels with bf16 output: a handful of registers are spilled and reloaded once per OUTPUT TILE,
 #    around the accumulator read-out between two K loops (5 stores + 5 loads per 4096 MFMAs of a wave), none
 #    inside a K loop.
 KNOWN_SCRATCH = {
     "asym_gemm_kernel<true, false>": 32,
+    "asym8_gemm_kernel<true,": 32,
     "tile_gemm_kernel<TileCfg<256, 256, 2, 2>": 160,
     "stream_gemm_kernel<4, true, 1>": 32,
     "stream_gemm_kernel<4, true, 2>": 32,

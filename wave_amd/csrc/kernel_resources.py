@@ -33,7 +33,7 @@ FIELDS = {
 }
 
 # kernels whose main loops the throughput figures depend on
-HOT = ("persist_gemm_kernel", "persist_gemm_gated_kernel", "persist_gemm_fp8_kernel", "asym_gemm_kernel", "tile_gemm_kernel", "stream_gemm_kernel", "mid_gemm_kernel", "midb_gemm_kernel",
+HOT = ("persist_gemm_kernel", "persist_gemm_gated_kernel", "persist_gemm_fp8_kernel", "asym_gemm_kernel", "asym8_gemm_kernel", "tile_gemm_kernel", "stream_gemm_kernel", "mid_gemm_kernel", "midb_gemm_kernel",
        "quantize_kernel")
 
 

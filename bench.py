@@ -440,7 +440,15 @@ def leg_mxfp8(torch, wave_amd, dev, steps, warmup, variant=0):
             wave_amd.mxfp8_gemm(x, xs, w4, ws, out, elem_format=(L.MXFP8_E5M2, L.MXFP8_B_E2M1), variant=variant)
 
     _, mper, _ = timed(torch, run_mixed, steps, warmup)
+    w4p = wave_amd.b_preshuffle(w4)
     del w4
+
+    def run_mixed_pre(count):
+        for _ in range(count):
+            wave_amd.mxfp8_gemm(x, xs, w4p, ws, out, elem_format=(L.MXFP8_E5M2, L.MXFP8_B_E2M1), b_preshuffled=True)
+
+    _, mpper, _ = timed(torch, run_mixed_pre, steps, warmup)
+    del w4p
     # the same problem with B in the library's preshuffled 8-bit order (B straight into registers), scales as the
     # call above hands them over (row-major, re-laid out by a launch of the call) and resident in MFMA32 order;
     # and both kernels on zero operands (no switching power: what the schedules reach at the full clock)
@@ -481,6 +489,7 @@ def leg_mxfp8(torch, wave_amd, dev, steps, warmup, variant=0):
     pre = dict(rate(pper), workload="the same problem, B in wave_mxfp8_b_preshuffle order (B-direct kernel), per call "
                                     "with the launch that re-lays the row-major scales out",
                kernel="asym8_gemm_kernel", resident_scales=rate(pper32),
+               e5m2_x_e2m1=dict(rate(mpper), workload="8-bit activations against MXFP4 weights in b_preshuffle order"),
                zero_operands={"symmetric_us": round(zper * 1e6, 2), "b_direct_us": round(zpper * 1e6, 2)})
     return {"workload": f"mxfp8: M={m} N={n} K={k} e5m2 x e5m2, f32 out, seed 5", "kernel": "persist_gemm_fp8_kernel",
             "b_preshuffled": pre,

@@ -247,11 +247,14 @@ int wave_mxfp8_b_preshuffle(const void *b, void *out, int64_t rows, int64_t k, v
 /* wave_mxfp8_gemm with B in wave_mxfp8_b_preshuffle order: A through LDS, B
  * straight from global memory into registers (the schedule of
  * wave_lang/kernel/wave/schedules/gemm_mxfp4_double_buffer.py:1781-2222 on the
- * operands of tests/kernel/wave_gemm_mxfp_test.py:416-501).  Both operands
- * 8-bit (e4m3 / e5m2 in any pairing), N % 256 == 0, K % 256 == 0, K >= 768, any
- * M; each scale tensor row-major or WAVE_MXFP4_SCALE_MFMA32 (with a row-major
- * one the workspace of wave_mxfp8_workspace_bytes(m, n, k) bytes is required:
- * it is re-laid out there first).  WAVE_MXFP4_ERR_UNSUPPORTED otherwise. */
+ * operands of tests/kernel/wave_gemm_mxfp_test.py:416-501).  A 8-bit (e4m3 /
+ * e5m2), B 8-bit in any pairing with it, or b_format = WAVE_MXFP8_E2M1: then b
+ * is packed MXFP4 [N, K/2] in wave_mxfp4_b_preshuffle order (the weights of
+ * the MXFP4 B-direct kernels, here against 8-bit activations).  N % 256 == 0,
+ * K % 256 == 0, K >= 768, any M; each scale tensor row-major or
+ * WAVE_MXFP4_SCALE_MFMA32 (with a row-major one the workspace of
+ * wave_mxfp8_workspace_bytes(m, n, k) bytes is required: it is re-laid out
+ * there first).  WAVE_MXFP4_ERR_UNSUPPORTED otherwise. */
 int wave_mxfp8_gemm_b_preshuffled(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
                                   int64_t m, int64_t n, int64_t k, int a_format, int b_format, int out_dtype,
                                   int a_scale_layout, int b_scale_layout, void *workspace, size_t workspace_bytes,

@@ -43,7 +43,8 @@ def test_preshuffle_matches_its_definition():
 def run(x, xs, w_t, ws, fmt, out_dtype=torch.float32, resident=False):
     gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
     m, n, k = x.shape[0], w_t.shape[0], x.shape[1]
-    wp = wave_amd.mxfp8_b_preshuffle(gw)
+    b4 = isinstance(fmt, tuple) and fmt[1] == o8.E2M1
+    wp = wave_amd.b_preshuffle(gw) if b4 else wave_amd.mxfp8_b_preshuffle(gw)
     out = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
     kw = {}
     if resident:
@@ -55,7 +56,8 @@ def run(x, xs, w_t, ws, fmt, out_dtype=torch.float32, resident=False):
     return out
 
 
-FMTS = {"e5m2": o8.E5M2, "e4m3": o8.E4M3, "e4m3_x_e5m2": (o8.E4M3, o8.E5M2), "e5m2_x_e4m3": (o8.E5M2, o8.E4M3)}
+FMTS = {"e5m2": o8.E5M2, "e4m3": o8.E4M3, "e4m3_x_e5m2": (o8.E4M3, o8.E5M2), "e5m2_x_e4m3": (o8.E5M2, o8.E4M3),
+        "e5m2_x_e2m1": (o8.E5M2, o8.E2M1), "e4m3_x_e2m1": (o8.E4M3, o8.E2M1)}
 
 
 @pytest.mark.parametrize("fname", sorted(FMTS))
@@ -71,7 +73,7 @@ def test_against_oracle(m, n, k, fname):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("fname", ["e5m2", "e4m3_x_e5m2"])
+@pytest.mark.parametrize("fname", ["e5m2", "e4m3_x_e5m2", "e5m2_x_e2m1"])
 @pytest.mark.parametrize("m,n,k", [(4352, 4096, 768), (4100, 4352, 1024), (2050, 8448, 1536)])
 def test_more_tiles_than_cus_same_bits_as_the_row_major_call(m, n, k, fname, out_dtype):
     """272 / 289 / 297 tiles on 256 workgroups: every workgroup walks two output tiles, its request streams run
@@ -110,6 +112,22 @@ def test_one_hot_rows_read_back_every_position_of_b():
     assert np.array_equal(c.astype(np.float64), deq[:, pos].T)
 
 
+def test_one_hot_rows_read_back_every_position_of_a_4_bit_b():
+    """The same through packed e2m1 weights in b_preshuffle order: every e2m1 value times a power of two is exact."""
+    m, n, k = 4352, 4096, 768
+    fmt = (o8.E4M3, o8.E2M1)
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=10, fmt=fmt, scale_lo=118, scale_hi=136)
+    x[:] = 0
+    xs[:] = 127
+    one = int(np.nonzero(o8.E4M3_TABLE == 1.0)[0][0])
+    pos = (np.arange(m) * 37) % k
+    x[np.arange(m), pos] = one
+    c = run(x, xs, w_t, ws, fmt).cpu().numpy()
+    from oracle import mxfp4_oracle as o4
+    b = o4.mxfp4_to_f32(w_t).astype(np.float64) * o4.e8m0_to_f32(ws).astype(np.float64).repeat(32, axis=1)
+    assert np.array_equal(c, b[:, pos].T.astype(np.float32))
+
+
 def test_what_the_kernel_does_not_serve_is_refused():
     m, n, k = 64, 256, 768
     x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=1, fmt=o8.E5M2)
@@ -128,7 +146,6 @@ def test_what_the_kernel_does_not_serve_is_refused():
     assert call(n_=128) == _lib.ERR_UNSUPPORTED            # whole 256-column tiles only
     assert call(k_=512) == _lib.ERR_UNSUPPORTED            # K >= 768
     assert call(k_=640) == _lib.ERR_UNSUPPORTED            # pairs of K tiles
-    assert call(fb=_lib.MXFP8_E2M1) == _lib.ERR_UNSUPPORTED
     assert call(fa=_lib.MXFP8_E2M1) == _lib.ERR_UNSUPPORTED
     assert call(la=_lib.SCALE_E8M0_SHUFFLE) == _lib.ERR_UNSUPPORTED
     assert call(ws_ptr=None, ws_bytes=0) == _lib.ERR_UNSUPPORTED   # row-major scales need the scratch

@@ -700,9 +700,9 @@ int wave_mxfp8_gemm_b_preshuffled(const void *a, const void *a_scale, const void
       bad_enum(b_scale_layout, 4))
     return WAVE_MXFP4_ERR_BAD_ENUM;
   const auto rm_or_native = [](int l) { return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32; };
-  // (the preshuffled order is defined for 8-bit rows; the kernel that reads it takes whole 256-column tiles and
-  // pairs of K tiles)
-  if (a_format == WAVE_MXFP8_E2M1 || b_format == WAVE_MXFP8_E2M1 || !rm_or_native(a_scale_layout) ||
+  // (A is 8-bit; a 4-bit B comes in the MXFP4 b_preshuffle order; the kernel takes whole 256-column tiles and pairs of
+  // K tiles)
+  if (a_format == WAVE_MXFP8_E2M1 || !rm_or_native(a_scale_layout) ||
       !rm_or_native(b_scale_layout) || n % 256 != 0 || k % 256 != 0 || k < 768)
     return WAVE_MXFP4_ERR_UNSUPPORTED;
   if (m == 0 || n == 0) return WAVE_MXFP4_OK;

@@ -19,7 +19,10 @@
 //     a lane's 32 bytes of an 8-bit operand as two halves 32 bytes apart in K.)
 //   * Scales: both tensors in MFMA32 order; one 256-byte block serves two K tiles (bytes 0, 1 of a lane's dword
 //     for the even one, 2, 3 for the odd one, picked by the instruction's byte selector, a constant per phase).
-// Taken for N % 256 == 0, K % 256 == 0, K >= 768, both operands 8-bit (e4m3 / e5m2 in any pairing), dense.  Any M.
+//   * FMT_B = 4: 8-bit A against packed MXFP4 B [N, K/2] in the reference's b_preshuffle order
+//     (wave_lang/kernel/wave/utils/mxfp_utils.py:98-110), read as the MXFP4 B-direct kernel reads it: a K step is
+//     one 16-byte load per lane and column half, four B loads per K tile instead of eight.
+// Taken for N % 256 == 0, K % 256 == 0, K >= 768, A 8-bit (e4m3 / e5m2), B 8-bit or e2m1, dense.  Any M.
 #include <type_traits>
 
 #include "mxfp4_tile_common.h"
@@ -36,24 +39,28 @@ constexpr int kStage = 4096;               // C staging per wave
 constexpr int kLds = kARing * kASlot + kARing * kSSlot + kNW * kStage;  // 160 KB
 constexpr int kALd = kBM / 8 / kNW;        // A DMA instructions per wave and K tile (8)
 // Vector memory operations per wave and K tile: A 8, A scales 1, B 8 (two K steps x two column halves x two
-// 16-byte halves), B scales 2.
-constexpr int kOpsPerKTile = kALd + 1 + 8 + 2;
+// 16-byte halves; a 4-bit B: one 16-byte load each, 4), B scales 2.
+constexpr int ops_per_k_tile(bool b4) { return kALd + 1 + (b4 ? 4 : 8) + 2; }
 // At the wait of K tile g (before its fourth phase) A and its scales of K tile g + 1 must have landed.  They were
-// requested in K tile g - 2 (at the latest as the last operations of its fourth phase), followed by the 19 of
-// K tile g - 1 and the 4 + 4 + 6 of the first three phases of K tile g.
-constexpr int kWaitSteady = kOpsPerKTile + 14;
+// requested in K tile g - 2 (at the latest as the last operations of its fourth phase), followed by the 19 (15) of
+// K tile g - 1 and the 4 + 4 + 6 (3 + 3 + 5) of the first three phases of K tile g.
+constexpr int wait_steady(bool b4) { return ops_per_k_tile(b4) + (b4 ? 11 : 14); }
 static_assert(kLds <= 160 * 1024, "LDS");
 
 template <bool OUT_BF16, int FMT_A, int FMT_B>
 __device__ __forceinline__ void asym8_body(const GemmParams &p) {
   constexpr int BM = kBM, BN = kBN, NW = kNW;
+  constexpr bool B4 = FMT_B == 4;
+  static_assert(FMT_A == 0 || FMT_A == 1, "A is 8-bit");
+  typedef typename std::conditional<B4, v4i, v8i>::type FragB;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   uint8_t *const s_ring = smem + kARing * kASlot;
   uint8_t *const c_stage = s_ring + kARing * kSSlot;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kp = p.kp, nkt = p.k_tiles;  // bytes of an operand row, K tiles of 128 bytes
+  const int kp = p.kp, nkt = p.k_tiles;  // bytes of a row of A, K tiles of 128 elements
+  const int kpb = B4 ? kp >> 1 : kp;     // bytes of a row of B
   const int total = p.tiles_m * p.tiles_n;
   const int padded = (total + kNumXcd - 1) / kNumXcd * kNumXcd;
   const int s_stride = (nkt >> 1) * 256;  // bytes of one 32-row block row of scales (MFMA32 order, K % 256 == 0)
@@ -72,8 +79,8 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
     as_base[which] = p.a_scale + (int64_t)(m0[which] >> 5) * s_stride;
     as_lim[which] = (int)min((int64_t)max(m_blocks - (m0[which] >> 5), 0) * s_stride, (int64_t)0x7FFFFFFF);
     // the 32-row blocks of a column tile are contiguous: they start at byte n0 * kp
-    b_base[which] = p.b + (int64_t)n0[which] * kp;
-    b_lim[which] = (int)min((int64_t)(p.n - n0[which]) * kp, (int64_t)0x7FFFFFFF);
+    b_base[which] = p.b + (int64_t)n0[which] * kpb;
+    b_lim[which] = (int)min((int64_t)(p.n - n0[which]) * kpb, (int64_t)0x7FFFFFFF);
     bs_base[which] = p.b_scale + (int64_t)(n0[which] >> 5) * s_stride;
     bs_lim[which] = (int)min((int64_t)((p.n - n0[which]) >> 5) * s_stride, (int64_t)0x7FFFFFFF);
     return true;
@@ -98,7 +105,8 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
   const int as_goff = lane < 32 ? (2 * wave + (lane >> 4)) * s_stride + (lane & 15) * 16 : (int)0x80000000;
   const int fr = lane & 31, fg = lane >> 5;
   // B: the lane's 16 bytes of a kilobyte; the wave's 64 columns are the 32-row blocks 2 * wave and 2 * wave + 1
-  const int b_goff = wave * 64 * kp + lane * 16;
+  // (4-bit B in b_preshuffle order: 16-row blocks, a K step of a block 512 bytes, lane = (row fr, K half fg))
+  const int b_goff = B4 ? wave * 64 * kpb + (fr >> 4) * 16 * kpb + fg * 256 + (fr & 15) * 16 : wave * 64 * kp + lane * 16;
   const int bs_goff = (2 * wave) * s_stride + lane * 4;
   // A fragment reads: row fr of a 32-row block; K step s takes the chunks 4 s + fg and 4 s + 2 + fg
   uint32_t foff[4];
@@ -120,12 +128,16 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
                                              (kt >> 1) * 256, 0, 0);
   };
   // the B fragment of K step s for the 32-column half jn of the wave's 64 columns
-  auto load_b = [&](int which, int kt, int s, int jn, v8i &dst) {
+  auto load_b = [&](int which, int kt, int s, int jn, FragB &dst) {
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc_n(b_base[which], b_lim[which]);
-    const int soff = jn * 32 * kp + kt * 4096 + s * 2048;
-    const v4i lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_goff, soff, 0);
-    const v4i hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_goff, soff + 1024, 0);
-    dst = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    if constexpr (B4) {
+      dst = __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_goff, jn * 32 * kpb + (kt * 2 + s) * 512, 0);
+    } else {
+      const int soff = jn * 32 * kp + kt * 4096 + s * 2048;
+      const v4i lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_goff, soff, 0);
+      const v4i hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, b_goff, soff + 1024, 0);
+      dst = v8i{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
   };
   auto load_bs = [&](int which, int kt, uint32_t (&dst)[2]) {
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc_n(bs_base[which], bs_lim[which]);
@@ -136,7 +148,7 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
 
   // ---------------- registers ----------------
   v16f acc[8][2];
-  v8i bq[2][2][2];                     // [parity of the K tile][K step][jn]
+  FragB bq[2][2][2];                   // [parity of the K tile][K step][jn]
   uint32_t sb_cur[2][2], sb_in[2][2];  // B scales in use / arriving, per parity
   uint32_t sa[2][8];                   // A scales per parity
   v8i afr[2][4];                       // A fragments of four row blocks, double buffered by phase
@@ -159,7 +171,7 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
     for (int i = 0; i < 8; ++i) dst[i] = *(const uint32_t *)(base + (i >> 1) * 1024 + (i & 1) * 256);
   };
   // T: the byte of the scale dwords (2 * parity of the K tile + K step); HH: which four row blocks
-  auto mfma_phase = [&](const v8i (&fa)[4], const v8i (&fb)[2], const uint32_t (&sca)[8], const uint32_t (&scb)[2],
+  auto mfma_phase = [&](const v8i (&fa)[4], const FragB (&fb)[2], const uint32_t (&sca)[8], const uint32_t (&scb)[2],
                         auto t_tag, auto hh_tag, auto zero_tag) {
     constexpr int T = decltype(t_tag)::value;
     constexpr int HH = decltype(hh_tag)::value;
@@ -175,7 +187,10 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
         }
         // operands swapped (B rows as the matrix A of the instruction): a lane's 4 accumulator registers of a
         // group are 4 consecutive N
-        acc[4 * HH + i][jn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[jn], fa[i], c, FMT_B, FMT_A, T, (int)scb[jn], T,
+        v8i vb;
+        if constexpr (B4) vb = v8i{fb[jn].x, fb[jn].y, fb[jn].z, fb[jn].w, 0, 0, 0, 0};
+        else vb = fb[jn];
+        acc[4 * HH + i][jn] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, fa[i], c, FMT_B, FMT_A, T, (int)scb[jn], T,
                                                                               (int)sca[4 * HH + i]);
       }
     }
@@ -344,7 +359,7 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
   issue_as(0, 2, 2);
   load_b(0, 1, 0, 1, bq[1][0][1]);
   // everything but the last K tile's worth has landed (the one-time cost of filling the pipeline)
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kOpsPerKTile));
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(ops_per_k_tile(B4)));
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
@@ -355,6 +370,7 @@ __device__ __forceinline__ void asym8_body(const GemmParams &p) {
   // ---------------- the tiles ----------------
   typedef std::integral_constant<int, 0> Even;
   typedef std::integral_constant<int, 1> Odd;
+  constexpr int kWaitSteady = wait_steady(B4);
   typedef std::integral_constant<int, kWaitSteady> WaitSteady;
   typedef std::integral_constant<int, (kWaitSteady + NS > 63 ? 63 : kWaitSteady + NS)> WaitAfterStore;
   int sl = 0;
@@ -420,8 +436,8 @@ hipError_t launch_fmt(const GemmParams &p, int grid_x, hipStream_t stream) {
 
 }  // namespace
 
-// Whether the kernel serves this problem (`p` in byte geometry: kp = K bytes of a row, k_tiles = K / 128; B in the
-// preshuffled 8-bit order, both scale tensors in MFMA32 order).
+// Whether the kernel serves this problem (`p` in the geometry of an 8-bit A: kp = K bytes of a row, k_tiles = K / 128;
+// B in the preshuffled 8-bit order, or packed MXFP4 in b_preshuffle order; both scale tensors in MFMA32 order).
 bool asym8_gemm_applies(const GemmParams &p, int num_cus) {
   if (p.num_groups != 0 || p.tile_table != nullptr || p.splits != 1 || p.partial != nullptr) return false;
   if (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32) return false;
@@ -432,11 +448,15 @@ bool asym8_gemm_applies(const GemmParams &p, int num_cus) {
   return num_cus / kNumXcd * kNumXcd >= kNumXcd;
 }
 
-// a_fmt, b_fmt: 0 = e4m3, 1 = e5m2
+// a_fmt: 0 = e4m3, 1 = e5m2; b_fmt: the same, or 2 = e2m1
 hipError_t launch_asym8_gemm(const GemmParams &p, int num_cus, int a_fmt, int b_fmt, hipStream_t stream) {
   const int grid = num_cus / kNumXcd * kNumXcd;
-  if (a_fmt == 0) return b_fmt == 0 ? launch_fmt<0, 0>(p, grid, stream) : b_fmt == 1 ? launch_fmt<0, 1>(p, grid, stream) : hipErrorInvalidValue;
-  if (a_fmt == 1) return b_fmt == 0 ? launch_fmt<1, 0>(p, grid, stream) : b_fmt == 1 ? launch_fmt<1, 1>(p, grid, stream) : hipErrorInvalidValue;
+  if (a_fmt == 0)
+    return b_fmt == 0 ? launch_fmt<0, 0>(p, grid, stream) : b_fmt == 1 ? launch_fmt<0, 1>(p, grid, stream)
+           : b_fmt == 2 ? launch_fmt<0, 4>(p, grid, stream) : hipErrorInvalidValue;
+  if (a_fmt == 1)
+    return b_fmt == 0 ? launch_fmt<1, 0>(p, grid, stream) : b_fmt == 1 ? launch_fmt<1, 1>(p, grid, stream)
+           : b_fmt == 2 ? launch_fmt<1, 4>(p, grid, stream) : hipErrorInvalidValue;
   return hipErrorInvalidValue;
 }
 

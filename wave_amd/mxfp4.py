@@ -591,7 +591,8 @@ def mxfp8_gemm(x, x_scales, w_t, w_scales, out, *, elem_format=None,
     against 4-bit weights or the other way round, the mixed operands of
     wave_lang/kernel/wave/constraints.py:425-431; both 4-bit is :func:`mxfp4_gemm`).
     ``workspace`` as in :func:`mxfp4_gemm`.  ``b_preshuffled=True``: ``w_t`` comes from
-    :func:`mxfp8_b_preshuffle` and the B-direct kernel runs (both operands 8-bit, N % 256 == 0,
+    :func:`mxfp8_b_preshuffle` (a packed e2m1 ``w_t`` from :func:`b_preshuffle`) and the B-direct kernel
+    runs (``x`` 8-bit, N % 256 == 0,
     K % 256 == 0, K >= 768; ``ValueError`` "unsupported" otherwise); only that call takes scale
     tensors in MFMA32 order (``a_scale_layout`` / ``b_scale_layout``)."""
     lib = _lib.load()

@@ -177,3 +177,25 @@ def run_small_batch(counts, inter, k, seed, a_native, slack_rows=0):
 ], ids=["bm64_sparse", "bm64", "bm128", "bm192"])
 def test_small_batch_fused_in_the_mid_kernel_matches_the_chain(counts, inter, k, a_native):
     run_small_batch(counts, inter, k, seed=sum(counts) + k, a_native=a_native, slack_rows=37)
+
+
+def _small_batch_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        e = int(rng.integers(4, 17))
+        avg = int(rng.integers(1, 140))
+        counts = rng.multinomial(avg * e, rng.dirichlet(np.full(e, 2.0))).tolist()
+        inter = 128 * int(rng.integers(1, 13))
+        while e * (2 * inter // 128) < 128:   # experts x strips of 128 columns: at least half the CUs
+            inter += 128
+        out.append((i, counts, inter, 256 * int(rng.integers(4, 9)), bool(rng.integers(0, 2)), int(rng.integers(0, 40))))
+    return out
+
+
+@pytest.mark.parametrize("case", _small_batch_cases(10, seed=77), ids=lambda c: f"{c[0]}-E{len(c[1])}-rows{sum(c[1])}-I{c[2]}-K{c[3]}")
+def test_random_small_batches_fused_in_the_mid_kernel(case):
+    """Seeded expert counts dealt unevenly (Dirichlet weights: empty experts, experts of several blocks), 4 .. 16
+    experts, every block height the library picks."""
+    i, counts, inter, k, a_native, slack = case
+    run_small_batch(counts, inter, k, seed=900 + i, a_native=a_native, slack_rows=slack)

@@ -151,3 +151,31 @@ def test_what_the_kernel_does_not_serve_is_refused():
     assert call(ws_ptr=None, ws_bytes=0) == _lib.ERR_UNSUPPORTED   # row-major scales need the scratch
     assert call(fa=3) == _lib.ERR_BAD_ENUM
     assert call(n_=100) == _lib.ERR_BAD_SHAPE
+
+
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    names = sorted(FMTS)
+    return [(i, int(rng.integers(1, 1400)), 256 * int(rng.integers(1, 9)), 256 * int(rng.integers(3, 11)),
+             names[int(rng.integers(0, len(names)))], bool(rng.integers(0, 2)), bool(rng.integers(0, 2)))
+            for i in range(count)]
+
+
+@pytest.mark.parametrize("case", _random_cases(16, seed=31), ids=lambda c: f"{c[0]}-{c[1]}x{c[2]}x{c[3]}-{c[4]}")
+def test_random_shapes_same_bits_as_the_row_major_call_and_close_to_the_oracle(case):
+    """Seeded shapes nobody picked by hand (1 .. 6 x 8 tiles, K = 768 .. 2560): the row-major call runs the tile
+    kernel or the symmetric persistent one, all with the K steps in the same order."""
+    i, m, n, k, fname, bf16, resident = case
+    fmt = FMTS[fname]
+    out_dtype = torch.bfloat16 if bf16 else torch.float32
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=500 + i, fmt=fmt, scale_lo=118, scale_hi=136)
+    c = run(x, xs, w_t, ws, fmt, out_dtype=out_dtype, resident=resident)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    other = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    wave_amd.mxfp8_gemm(gx, gxs, gw, gws, other, elem_format=fmt)
+    torch.cuda.synchronize()
+    assert torch.equal(c, other), case
+    if not bf16:
+        rows = np.unique(np.r_[0:min(m, 3), m // 2, m - 1])
+        ref = o8.scaled_gemm_mxfp8(x[rows], w_t, xs[rows], ws, fmt)
+        assert_f32_close(c.cpu().numpy()[rows], ref, str(case))

@@ -109,6 +109,7 @@ __global__ void __launch_bounds__(kAlignThreads) moe_align_kernel(const IdT *__r
       const int i = base8 + s * 64 + lane;
       const bool valid = e8[s] >= 0 && e8[s] < E;
       const int e = valid ? (int)e8[s] : -1;
+      if (__ballot(valid) == 0) continue;  // (a short table: most of the eight steps hold no entry at all)
       if (E <= kFewExperts) {
         // few experts: one ballot per expert, no search for the experts that occur
         int pos = -1;

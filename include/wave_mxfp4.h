@@ -367,7 +367,7 @@ int wave_mxfp4_silu_and_mul_quantize(const void *gate, const void *up, int64_t l
  * over the experts (grouped, at most 152 rows per expert on average, the
  * experts' B scales resident in MFMA32 order, at least half as many
  * 128-column strips over all experts as CUs), the mid-M kernel that
- * wave_mxfp4_gemm_grouped gives such a batch to.  Either way I % 128 == 0,
+ * wave_mxfp4_gemm_grouped gives such a batch to, on the same block height.  Either way I % 128 == 0,
  * K % 256 == 0, K >= 1024 (768 on the persistent kernel), a workspace of
  * wave_mxfp4_grouped_workspace_bytes(total_rows, n, k, max(num_groups, 1)) bytes,
  * scales row-major or MFMA32, B row-major; WAVE_MXFP4_ERR_UNSUPPORTED

@@ -170,11 +170,12 @@ def run_small_batch(counts, inter, k, seed, a_native, slack_rows=0):
 
 @pytest.mark.parametrize("a_native", [False, True], ids=["a_scales_row_major", "a_scales_mfma32"])
 @pytest.mark.parametrize("counts,inter,k", [
-    ([16, 9, 0, 31, 22, 1, 40, 13], 1024, 1024),              # blocks of 64 rows, one live row block in most
+    ([16, 9, 0, 31, 22, 1, 40, 13], 1024, 1024),              # blocks of 32 rows (gate / up exchanged through LDS)
+    ([10, 20, 5, 0, 33, 12, 7, 25], 2304, 1024),              # the same, more strips than CUs: two workgroups per CU
     ([70, 20, 64, 65, 3, 0, 50, 47], 1792, 2048),             # blocks of 64 rows, two groups of a second pass
     ([100, 0, 260, 33, 1, 150, 97, 128], 1024, 1024),         # blocks of 128 rows, a group of three passes
     ([150, 160, 140, 155, 149, 132, 141, 143], 1024, 1536),   # blocks of 192 rows
-], ids=["bm64_sparse", "bm64", "bm128", "bm192"])
+], ids=["bm32", "bm32_two_per_cu", "bm64", "bm128", "bm192"])
 def test_small_batch_fused_in_the_mid_kernel_matches_the_chain(counts, inter, k, a_native):
     run_small_batch(counts, inter, k, seed=sum(counts) + k, a_native=a_native, slack_rows=37)
 

@@ -946,9 +946,9 @@ int wave_mxfp4_gemm_gated_quantize(const void *a, const void *a_scale, const voi
     const int64_t avg = (total_rows + num_groups - 1) / num_groups;
     if (avg <= kGroupedMidMaxAvgRows && (int64_t)num_groups * (n / 128) >= device_cus() / 2) {
       int64_t bm = (5 * avg + 3) / 4 < total_rows ? (5 * avg + 3) / 4 : total_rows;
-      bm = bm > 192 ? 192 : (bm + 63) / 64 * 64;
+      bm = bm > 192 ? 192 : bm <= 32 ? 32 : (bm + 63) / 64 * 64;
       p.tile_table = nullptr;
-      return record_hip(launch_mid_gated(p, stream, (int)bm));
+      return record_hip(launch_mid_gated(p, device_cus(), stream, (int)bm));
     }
   }
   GemmParams q32 = p;

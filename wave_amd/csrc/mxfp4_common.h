@@ -151,7 +151,7 @@ bool mid_gemm_applies(const GemmParams &p);
 hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream, int bm = 0);
 bool mid_grouped_applies(const GemmParams &p);
 bool mid_gated_applies(const GemmParams &p);
-hipError_t launch_mid_gated(const GemmParams &p, hipStream_t stream, int bm);
+hipError_t launch_mid_gated(const GemmParams &p, int num_cus, hipStream_t stream, int bm);
 int mid_max_m();
 int persist_tail_parts(const GemmParams &p, int variant, int num_cus, size_t *partial_bytes);
 hipError_t launch_skinny_gemm(const GemmParams &p, hipStream_t stream);

@@ -108,7 +108,7 @@ template <class Cfg, bool A_RM, bool B_SH, bool A_SH, bool GATED = false>
 __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, const uint8_t *a_base, const uint8_t *as_base,
                                          const uint8_t *b_base, const uint8_t *bs_base, uint8_t *c_base, const int m_rows,
                                          const int a_row32 = 0, const int m_abs0 = 0) {
-  static_assert(!GATED || (Cfg::WM == 2 && !Cfg::B_RM && !B_SH), "gated epilogue: a wave holds a gate and an up group; B scales MFMA32");
+  static_assert(!GATED || (!Cfg::B_RM && !B_SH), "gated epilogue: B scales in MFMA32 order (column groups of 32)");
   constexpr bool B_RM = Cfg::B_RM;
   constexpr int MT_M = Cfg::MT_M, DA = Cfg::DA, DB = Cfg::DB, LB = Cfg::LB;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -186,6 +186,7 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
       slot_next = slot_next + 1 == DA ? 0 : slot_next + 1;
     }
     __builtin_amdgcn_s_barrier();  // (the compute waves' barrier in front of their C staging)
+    if constexpr (GATED && Cfg::WM == 1) __builtin_amdgcn_s_barrier();  // (... and the one of their gate / up exchange)
     __builtin_amdgcn_s_waitcnt(0);
     return;
   }
@@ -415,21 +416,22 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
     const int s_kt = (act_ks + 7) >> 3;
     const __amdgpu_buffer_rsrc_t q_rsrc = make_rsrc_n(c_base, (int)min((int64_t)m_rows * qrow, (int64_t)0x7FFFFFFF));
     const __amdgpu_buffer_rsrc_t s_rsrc = make_rsrc_n(p.epi_scale, rsrc_bytes((int64_t)((p.m + 31) >> 5) * s_kt * 256));
-    const int g = (n0 >> 6) + wn;  // the activation's scale group: the strip's pair of column groups of this wave
+    // the wave's 16 values of a row as 8 bf16 pairs: what the unfused GEMM would have stored
+    auto pack_bf16 = [](const v16f &a, uint32_t (&out)[8]) {
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
-      if (i >= live) break;
-      const int r_tile = (WM * i + wm) * 32 + fr;
-      const v16f &ga = acc[i][0], &ua = acc[i][1];
+      for (int w = 0; w < 8; ++w) {
+        const bf16x2 h = {(__bf16)a[2 * w], (__bf16)a[2 * w + 1]};
+        out[w] = __builtin_bit_cast(uint32_t, h);
+      }
+    };
+    // silu(gate) * up of one row block and activation scale group `g`, quantised: the activation kernel's arithmetic
+    auto emit = [&](int r_tile, int g, const uint32_t (&gb)[8], const uint32_t (&ub)[8]) {
       uint32_t h[8];
       uint32_t lo = 0, hi = 0;
 #pragma unroll
       for (int w = 0; w < 8; ++w) {
-        // the GEMM's bf16 output of the unfused pipeline, then its activation kernel's arithmetic
-        const bf16x2 g2 = {(__bf16)ga[2 * w], (__bf16)ga[2 * w + 1]}, u2 = {(__bf16)ua[2 * w], (__bf16)ua[2 * w + 1]};
-        const uint32_t gb = __builtin_bit_cast(uint32_t, g2), ub = __builtin_bit_cast(uint32_t, u2);
-        const float g0 = __builtin_bit_cast(float, gb << 16), g1 = __builtin_bit_cast(float, gb & 0xFFFF0000u);
-        const float u0 = __builtin_bit_cast(float, ub << 16), u1 = __builtin_bit_cast(float, ub & 0xFFFF0000u);
+        const float g0 = __builtin_bit_cast(float, gb[w] << 16), g1 = __builtin_bit_cast(float, gb[w] & 0xFFFF0000u);
+        const float u0 = __builtin_bit_cast(float, ub[w] << 16), u1 = __builtin_bit_cast(float, ub[w] & 0xFFFF0000u);
         const float r0 = g0 * u0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g0 * -1.44269504088896340736f));
         const float r1 = g1 * u1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g1 * -1.44269504088896340736f));
         const bf16x2 o = {(__bf16)r0, (__bf16)r1};
@@ -464,6 +466,37 @@ __device__ __forceinline__ void mid_body(const GemmParams &p, const int wv, cons
       const int r_abs = m_abs0 + r_tile;
       const int s_off = ((r_abs >> 5) * s_kt + (g >> 3)) * 256 + (((g & 1) << 5) | (r_abs & 31)) * 4 + ((g & 7) >> 1);
       __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sb, s_rsrc, fg == 0 && r_tile < m_rows ? s_off : (int)0x80000000, 0, 0);
+    };
+    if constexpr (WM == 2) {
+      // the wave's column groups 2 wn and 2 wn + 1 are gate and up of the activation's group (n0 / 64) + wn
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        if (i >= live) break;
+        uint32_t gb[8], ub[8];
+        pack_bf16(acc[i][0], gb);
+        pack_bf16(acc[i][1], ub);
+        emit((WM * i + wm) * 32 + fr, (n0 >> 6) + wn, gb, ub);
+      }
+    } else {
+      // one row block, the waves side by side: wave 2q holds the gate, wave 2q + 1 the up values of the
+      // activation's group (n0 / 64) + q, element for element in the same lane and register.  The up waves hand
+      // theirs over through the ring (free since the barrier above): 8 dwords per lane, lane-contiguous.
+      uint8_t *xch = b_ring + (wave >> 1) * 2048 + lane * 4;
+      uint32_t gb[8], ub[8];
+      pack_bf16(acc[0][0], gb);
+      if (wave & 1) {
+#pragma unroll
+        for (int w = 0; w < 8; ++w) *(uint32_t *)(xch + w * 256) = gb[w];
+      }
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (!(wave & 1)) {
+#pragma unroll
+        for (int w = 0; w < 8; ++w) ub[w] = *(const uint32_t *)(xch + w * 256);
+        emit(fr, (n0 >> 6) + (wave >> 1), gb, ub);
+      }
     }
     return;
   }
@@ -674,23 +707,27 @@ hipError_t launch_mid_gemm(const GemmParams &p, int num_cus, hipStream_t stream,
   return launch_mid_cfg<256>(p, wv, stream);
 }
 
-// The gated, quantising form (grouped): blocks of 64, 128 or 192 rows (a wave needs both column groups of a pair: the
-// 32-row block's four waves side by side do not have them), both B scale tensors in MFMA32 order, whole 128-column
-// strips of gate / up pairs.
+// The gated, quantising form (grouped): blocks of 32 (the up waves hand their values to the gate waves through LDS),
+// 64, 128 or 192 rows (a wave holds both column groups of a pair), the experts' B scales in MFMA32 order, whole
+// 128-column strips of gate / up pairs.
 bool mid_gated_applies(const GemmParams &p) {
   return mid_grouped_applies(p) && p.epi_scale != nullptr && p.epi_scale_layout == WAVE_MXFP4_SCALE_MFMA32 &&
          p.b_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && !p.b_preshuffled && p.out_bf16 && (p.n & 127) == 0 &&
          (int64_t)p.m * (p.n >> 2) < ((int64_t)1 << 31);
 }
 
-template <int BM>
+template <int BM, bool TWO = false>
 static hipError_t launch_mid_gated_bm(const GemmParams &p, hipStream_t stream) {
   if (p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR)
-    return launch_mid_kernel<MidCfg<BM, false, false, false>, true, true, false, false, true>(p, 32, stream);
-  return launch_mid_kernel<MidCfg<BM, false, false, true>, false, true, false, false, true>(p, 32, stream);
+    return launch_mid_kernel<MidCfg<BM, false, TWO, false>, true, true, false, false, true>(p, 32, stream);
+  return launch_mid_kernel<MidCfg<BM, false, TWO, true>, false, true, false, false, true>(p, 32, stream);
 }
 
-hipError_t launch_mid_gated(const GemmParams &p, hipStream_t stream, int bm) {
+hipError_t launch_mid_gated(const GemmParams &p, int num_cus, hipStream_t stream, int bm) {
+  // (the 32-row block: two workgroups per CU when there are more strips than CUs, as in launch_mid_gemm)
+  if (bm <= 32)
+    return (int64_t)(p.n / kMidBN) * p.num_groups > num_cus ? launch_mid_gated_bm<32, true>(p, stream)
+                                                           : launch_mid_gated_bm<32>(p, stream);
   if (bm <= 64) return launch_mid_gated_bm<64>(p, stream);
   if (bm <= 128) return launch_mid_gated_bm<128>(p, stream);
   return launch_mid_gated_bm<192>(p, stream);

@@ -179,3 +179,31 @@ def test_random_shapes_same_bits_as_the_row_major_call_and_close_to_the_oracle(c
         rows = np.unique(np.r_[0:min(m, 3), m // 2, m - 1])
         ref = o8.scaled_gemm_mxfp8(x[rows], w_t, xs[rows], ws, fmt)
         assert_f32_close(c.cpu().numpy()[rows], ref, str(case))
+
+
+def test_a_beyond_2_gib():
+    """A of 2.15 GB (262444 rows of 8192 bytes): the descriptors are based at each tile, so rows on either side of
+    the 2 GiB byte boundary (row 262144), the first and last tiles and rows at random must come out right; the
+    symmetric kernel on the row-major B gives every element a second opinion."""
+    m, n, k = 262144 + 300, 256, 8192
+    fmt = o8.E4M3
+    g = torch.Generator(device=DEV).manual_seed(77)
+    x = torch.randint(0, 256, (m, k), dtype=torch.uint8, device=DEV, generator=g)
+    x = torch.where((x & 0x7F) == 0x7F, x - 1, x)   # (no NaN codes)
+    w = torch.randint(0, 256, (n, k), dtype=torch.uint8, device=DEV, generator=g)
+    w = torch.where((w & 0x7F) == 0x7F, w - 1, w)
+    xs = torch.randint(122, 132, (m, k // 32), dtype=torch.uint8, device=DEV, generator=g)
+    ws = torch.randint(122, 132, (n, k // 32), dtype=torch.uint8, device=DEV, generator=g)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    wave_amd.mxfp8_gemm(x, xs, wave_amd.mxfp8_b_preshuffle(w), ws, out, elem_format=fmt, b_preshuffled=True)
+    other = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    wave_amd.mxfp8_gemm(x, xs, w, ws, other, elem_format=fmt)
+    torch.cuda.synchronize()
+    assert torch.equal(out, other)
+    rng = np.random.default_rng(5)
+    rows = np.unique(np.concatenate([[0, 1, 255, 256, 262143, 262144, 262145, m - 2, m - 1], rng.integers(0, m, 24)]))
+    idx = torch.from_numpy(rows).to(DEV)
+    ref = o8.scaled_gemm_mxfp8(x[idx].cpu().numpy(), w.cpu().numpy(), xs[idx].cpu().numpy(), ws.cpu().numpy(), fmt)
+    got = out[idx].float().cpu().numpy()
+    tol = 2.0 ** -7 * np.abs(ref) + 1e-4 * np.abs(ref).max()
+    assert (np.abs(got - ref) <= tol).all(), "beyond one bf16 ulp + 1e-4 * max"

@@ -331,7 +331,9 @@ def leg_moe_layer(torch, wave_amd, dev, steps_, warmup_, tokens=4096):
                     fn()
             each[name] = round(timed(torch, run, steps_, warmup_)[1] * 1e6, 2)
         return {"layer_us": round(per_layer * 1e6, 2), "tflops": round(flops / per_layer / 1e12, 1),
-                "frac_of_mxfp4_peak": round(flops / per_layer / 1e12 / PEAK_MXFP4_TFLOPS, 4), "steps_us": each,
+                "frac_of_mxfp4_peak": round(flops / per_layer / 1e12 / PEAK_MXFP4_TFLOPS, 4),
+                "gb_per_s": round(layer_bytes / per_layer / 1e9, 1),
+                "frac_of_hbm_peak": round(layer_bytes / per_layer / 1e9 / PEAK_HBM_GBPS, 4), "steps_us": each,
                 "sum_of_steps_us": round(sum(each.values()), 2)}
 
     # the layer as the library runs it best: activation and quantiser in the first GEMM's C write; and the chain of
@@ -1193,6 +1195,10 @@ def main():
         result["mxfp8"] = leg
         torch.cuda.empty_cache()
         result["moe_layer"] = leg_moe_layer(torch, wave_amd, dev, min(args.steps, 50), min(args.warmup, 20))
+        torch.cuda.empty_cache()
+        # the same layer at a serving batch (16 rows per expert): every weight read once for a handful of rows, the
+        # layer priced against HBM (frac_of_hbm_peak)
+        result["moe_layer_serving"] = leg_moe_layer(torch, wave_amd, dev, args.steps, args.warmup, tokens=64)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, m, n, k, seed, srange, args.cpu_rows)

@@ -95,3 +95,17 @@ def make_inputs_mxfp8(m, n, k, seed, fmt, scale_lo=124, scale_hi=127):
     xs = rng.integers(scale_lo, scale_hi + 1, size=(m, k // 32), dtype=np.uint8)
     ws = rng.integers(scale_lo, scale_hi + 1, size=(n, k // 32), dtype=np.uint8)
     return x, xs, w_t, ws
+
+
+def b8_preshuffle(b: np.ndarray) -> np.ndarray:
+    """The library's preshuffled order of an 8-bit B ``[N, K]`` (declared in include/wave_mxfp4.h beside
+    wave_mxfp8_b_preshuffle; the reference defines ``b_preshuffle``, mxfp_utils.py:98-110, for packed MXFP4 rows
+    only, so this layout has no reference counterpart and is pinned against its own byte formula in the test
+    suite): blocks of 32 rows x 128 bytes, block (n // 32, kt) first by row block then by K tile, inside a block
+    the 16-byte pieces as [K step][half][g][row], the piece of (step, half, g, row) holding that row's bytes
+    64 * step + 32 * half + 16 * g .. + 15 of the K tile.  Same shape out, N % 32 == 0, K % 128 == 0."""
+    n, k = b.shape
+    if n % 32 or k % 128:
+        raise ValueError("N must be a multiple of 32 and K of 128")
+    t = b.reshape(n // 32, 32, k // 128, 2, 2, 2, 16)  # row block, row, K tile, step, half, g, byte
+    return np.ascontiguousarray(t.transpose(0, 2, 3, 4, 5, 1, 6)).reshape(n, k)

@@ -1,6 +1,6 @@
 """GPU: the MXFP8 GEMM with B in the library's preshuffled 8-bit order (wave_mxfp8_b_preshuffle,
-wave_mxfp8_gemm_b_preshuffled): A through LDS, B straight into registers.  The layout against a numpy restatement
-of its definition; the GEMM against the oracle (oracle/mxfp8_oracle.py; bound as in test_gpu_mxfp8.py, the
+wave_mxfp8_gemm_b_preshuffled): A through LDS, B straight into registers.  The layout against the numpy statement
+of its definition (oracle/mxfp8_oracle.py, pinned byte by byte in tests/test_oracle_mxfp8.py); the GEMM against the oracle (oracle/mxfp8_oracle.py; bound as in test_gpu_mxfp8.py, the
 reference's own test tests/kernel/wave_gemm_mxfp_test.py:416-501 uses atol 2e-3 / rtol 1e-3), bit for bit against
 wave_mxfp8_gemm on the row-major operand (same products, same order of the K steps), and exactly on one-hot rows,
 which read back single elements of dequantised B and so pin every position of the layout."""
@@ -20,19 +20,12 @@ pytestmark = pytest.mark.gpu
 RM, M32 = _lib.SCALE_ROW_MAJOR, _lib.SCALE_MFMA32
 
 
-def np_preshuffle(b):
-    """[N, K] bytes -> blocks (n / 32, kt) of 4096 bytes, pieces of 16 bytes as [K step][half][g][row]."""
-    n, k = b.shape
-    t = b.reshape(n // 32, 32, k // 128, 2, 2, 2, 16)  # nb, r, kt, s, h, g, byte
-    return t.transpose(0, 2, 3, 4, 5, 1, 6).reshape(n, k)
-
-
 def test_preshuffle_matches_its_definition():
     rng = np.random.default_rng(0)
     for n, k in [(32, 128), (64, 384), (256, 1024), (96, 2176)]:
         b = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
         got = wave_amd.mxfp8_b_preshuffle(torch.from_numpy(b).to(DEV)).cpu().numpy()
-        assert np.array_equal(got, np_preshuffle(b)), (n, k)
+        assert np.array_equal(got, o8.b8_preshuffle(b)), (n, k)
     gb = torch.zeros(48, 128, dtype=torch.uint8, device=DEV)
     with pytest.raises(ValueError):
         wave_amd.mxfp8_b_preshuffle(gb)          # rows % 32

@@ -74,3 +74,29 @@ def test_generator_rounds_to_nearest_code():
     x, xs, w_t, ws = o8.make_inputs_mxfp8(8, 8, 128, seed=0, fmt=o8.E4M3)
     assert x.dtype == np.uint8 and xs.shape == (8, 4) and np.isfinite(o8.fp8_to_f64(x, o8.E4M3)).all()
     assert ((xs >= 124) & (xs <= 127)).all()
+
+
+def test_b8_preshuffle_is_the_stated_byte_formula_and_a_bijection():
+    """Byte (r, c) of B lands at ((r // 32) * (K // 128) + c // 128) * 4096 + (step * 2 + half) * 1024 +
+    (32 * g + r % 32) * 16 + c % 16 with step = c % 128 // 64, half = c % 64 // 32, g = c % 32 // 16: the formula
+    of include/wave_mxfp4.h, byte by byte, against the reshape / transpose statement."""
+    for n, k in [(32, 128), (96, 384), (64, 1024)]:
+        b = np.arange(n * k, dtype=np.int64).reshape(n, k)      # every byte its own label
+        got = o8.b8_preshuffle(b).reshape(-1)
+        assert sorted(got.tolist()) == list(range(n * k))
+        r, c = np.divmod(np.arange(n * k), k)
+        cc = c % 128
+        dst = ((r // 32) * (k // 128) + c // 128) * 4096 + ((cc // 64) * 2 + (cc % 64) // 32) * 1024 \
+            + (32 * ((cc % 32) // 16) + r % 32) * 16 + c % 16
+        want = np.empty(n * k, dtype=np.int64)
+        want[dst] = np.arange(n * k)
+        assert np.array_equal(got, want), (n, k)
+    # a lane's two 16-byte halves of a K step are 32 bytes apart in K, 1024 bytes apart in the block
+    b = np.arange(32 * 128, dtype=np.int64).reshape(32, 128)
+    p = o8.b8_preshuffle(b).reshape(-1)
+    lane, step = 37, 1   # g = 1, row 5
+    lo = p[(step * 2 + 0) * 1024 + lane * 16:][:16]
+    hi = p[(step * 2 + 1) * 1024 + lane * 16:][:16]
+    assert np.array_equal(lo, b[5, 64 + 16:64 + 32]) and np.array_equal(hi, b[5, 64 + 48:64 + 64])
+    with pytest.raises(ValueError):
+        o8.b8_preshuffle(np.zeros((48, 128), dtype=np.uint8))

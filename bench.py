@@ -976,7 +976,7 @@ def main():
                           "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                           "frac": round(leg["algorithmic_bytes"] / leg["layer_us"] / 1e3 / PEAK_HBM_GBPS, 4), "traffic": None,
                           "kernel": "mid_gemm_kernel (grouped), all steps of the layer", "launch_us": leg["layer_us"]}
-                         if leg["rows_per_expert"] <= 152 else
+                         if leg["rows_per_expert"] <= 160 else
                          {"bound": "mfma", "achieved": leg["tflops"], "peak": PEAK_MXFP4_TFLOPS, "unit": "TFLOP/s",
                           "frac": leg["frac_of_mxfp4_peak"], "traffic": None, "kernel": "persist_gemm_kernel (grouped)",
                           "launch_us": leg["layer_us"]}),

@@ -194,8 +194,10 @@ size_t wave_mxfp4_static_scratch_bytes(void);
  * problems of at most four rounds of 256x256 tiles over the CUs the size
  * includes 256 KB per CU for the f32 parts of a sparsely filled last round,
  * whose tiles are then cut along K and summed by a second launch.
- * A small batch (AUTO: at most 152 rows per expert on average, and enough
- * experts x 128-column strips to occupy half the CUs) runs on the mid-M kernel,
+ * A small batch (AUTO: at most 160 rows per expert on average - or more where
+ * the tile kernels would leave CUs idle for whole rounds, e.g. few column tiles
+ * and a long K - and enough experts x 128-column strips to occupy half the CUs)
+ * runs on the mid-M kernel,
  * one workgroup per (expert, strip), with no table and no scale re-layout: the
  * call is then bound by reading every expert's B once.  It needs K % 256 == 0,
  * K >= 1024, N % 4 == 0, A's scales row-major and B's in any of the three orders;
@@ -364,7 +366,8 @@ int wave_mxfp4_silu_and_mul_quantize(const void *gate, const void *up, int64_t l
  * by wave_mxfp4_silu_and_mul_quantize on its two halves.  num_groups = 0 with
  * offsets = NULL is the dense problem.  Served by two kernels: the persistent
  * 256x256 kernel (more 256x256 tiles than CUs), and, for a small batch routed
- * over the experts (grouped, at most 152 rows per expert on average, the
+ * over the experts (grouped, the batches wave_mxfp4_gemm_grouped gives to the
+ * mid-M kernel: at most 160 rows per expert on average and some beyond, the
  * experts' B scales resident in MFMA32 order, at least half as many
  * 128-column strips over all experts as CUs), the mid-M kernel that
  * wave_mxfp4_gemm_grouped gives such a batch to, on the same block height.  Either way I % 128 == 0,

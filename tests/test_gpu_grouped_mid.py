@@ -144,3 +144,29 @@ def test_grouped_mid_unsupported_cases_are_refused():
     x, xs, w, ws, off = inputs(e, n, k, rows, seed=9)
     with pytest.raises((ValueError, RuntimeError)):
         run(x, xs, w, ws, off, torch.float32, variant=V)
+
+
+@pytest.mark.parametrize("la", [RM, M32], ids=["a_scales_row_major", "a_scales_mfma32"])
+@pytest.mark.parametrize("e,n,k,rows", [
+    (8, 4096, 1024, 1280),    # 160 rows per expert: one pass of the 192-row block
+    (8, 4096, 1024, 2048),    # 256: the 128x256 tiles would take two sparsely filled rounds, two passes here
+    (8, 4096, 1024, 3072),    # 384: less than two rounds of 256x256 tiles, three passes here
+    (16, 2048, 1024, 2900),   # 181 per expert
+    (8, 4096, 1024, 4500),    # 563 per expert: back on the tile kernels (two well-filled rounds)
+    (4, 4096, 1024, 1300),    # few experts of many rows: the tile kernels
+])
+def test_library_choice_beyond_160_rows_per_expert(e, n, k, rows, la):
+    """Whichever kernel the library picks for a grouped problem of 160 .. 560 rows per expert (its estimate of the
+    rounds either side would take; the groups of several 192-row passes among them), every group's rows against the
+    exact oracle on the first, the last and 64 random columns, and bit-equal to the mid-M kernel asked for by name
+    where that is what ran (same K order on every kernel: the two agree to the last bit anyway)."""
+    x, xs, w, ws, off = inputs(e, n, k, rows, seed=e + rows, lo=120, hi=132)
+    rng = np.random.default_rng(rows)
+    cols = np.unique(np.concatenate([[0, 1, 127, 128, n - 1], rng.integers(0, n, 64)]))
+    ref = reference(x, xs, w[:, cols], ws[:, cols], off)
+    for dt in (torch.bfloat16, torch.float32):
+        c = run(x, xs, w, ws, off, dt, lb=M32, la=la)
+        assert not np.isnan(c).any(), "unwritten elements"
+        check(c[:, cols], ref, dt, f"E={e} {rows}x{n}x{k} library's choice")
+        by_name = run(x, xs, w, ws, off, dt, lb=M32, la=la, variant=V)
+        assert np.array_equal(c, by_name)

@@ -95,6 +95,44 @@ int device_cus() {
   return cached[dev];
 }
 
+constexpr int64_t kGroupedMidMaxAvgRows = 160;  // (one pass of the 192-row block over every expert, as good as always)
+// Whether the mid-M kernel is the faster home of a grouped problem (one workgroup per expert and 128-column strip,
+// every expert's B streamed once per block of rows).  Up to 160 rows per expert on average it was, on every shape
+// measured (4..32 experts, N = 2048..28672, K = 4096..14336, multinomial groups).  Beyond, a group takes several
+// passes of 192-row blocks, and what decides is how the tile kernels' rounds come out: a problem of less than two
+// rounds of 256x256 tiles, or one that runs on the smaller tiles, leaves CUs idle for whole rounds (8 experts x 4096
+// x 14336, 1280..2560 rows: 140..190 us against 67..125 us here), while one of many well-filled rounds does not
+// (8 x 28672 x 4096, 1536 rows: 147 against 185 us).  Both sides are priced in K tiles per workgroup and round with
+// factors fitted to 49 such measurements (the choice was within 9 % of the better kernel on all of them).
+static bool grouped_mid_pays(int64_t total_rows, int num_groups, int64_t n, int64_t k) {
+  const int64_t cus = device_cus();
+  const int64_t strips = (int64_t)num_groups * ((n + 127) / 128);
+  if (2 * strips < cus) return false;
+  const int64_t avg = (total_rows + num_groups - 1) / num_groups;
+  if (avg <= kGroupedMidMaxAvgRows) return true;
+  (void)k;  // (both estimates are proportional to K)
+  // passes of 192-row blocks, in halves: groups dealt at random spread about a tenth around the average
+  const double passes_raw = (double)avg * 1.1 / 192.0;
+  const double passes = passes_raw < 1.0 ? 1.0 : (double)((int64_t)(passes_raw * 2.0 + 0.999)) / 2.0;
+  const double rounds_mid = strips > cus ? (double)strips / (double)cus : 1.0;
+  const double t_mid = rounds_mid * passes * 0.9;
+  const int v = pick_tile_variant(total_rows, n, false);
+  const double n256 = (double)((n + 255) / 256), n128 = (double)((n + 127) / 128);
+  double t_alt;
+  if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2) {
+    const double rounds = ((double)total_rows / 256.0 + num_groups) * n256 / (double)cus;
+    if (rounds >= 2.0) return false;
+    t_alt = (rounds < 1.0 ? 1.0 : rounds) * 1.9;
+  } else if (v == WAVE_MXFP4_VARIANT_T128x256_W2x2) {
+    const double tiles = ((double)total_rows / 128.0 + num_groups) * n256;
+    t_alt = (double)((int64_t)((tiles + (double)cus - 1.0) / (double)cus)) * 1.1;
+  } else {
+    const double tiles = ((double)total_rows / 128.0 + num_groups) * n128;
+    t_alt = (double)((int64_t)((tiles + 2.0 * (double)cus - 1.0) / (2.0 * (double)cus))) * 1.1;
+  }
+  return t_mid < t_alt;
+}
+
 bool is_tile_variant(int v) {
   int bm, bn;
   tile_variant_shape(v, &bm, &bn);
@@ -105,7 +143,6 @@ bool is_tile_variant(int v) {
 // Grouped persistent kernel: a group's last M tile of at most this many rows runs as a short tile (all eight waves
 // side by side on 64 rows: an eighth of a full tile's MFMAs), after the full ones.
 constexpr int kGroupedShortRows = 64;
-constexpr int64_t kGroupedMidMaxAvgRows = 152;  // (rows per block up to 192: the 256-row block loses to the tile kernels)
 
 // What the mid-M kernel takes (the part of it that the shape alone decides).
 bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
@@ -798,13 +835,13 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
     return WAVE_MXFP4_ERR_UNSUPPORTED;
   // A small batch routed over the experts: every expert's B is read once for a handful of rows, so the call is
   // bound by streaming B, like the dense mid-M problem.  One workgroup per (expert, strip of columns), no table, no
-  // re-layout of the scales.  AUTO takes it up to 152 rows per expert on average (measured at 8 experts, N = 14336,
-  // K = 4096 against the table-driven tile kernels), when there are enough strips to put most CUs to work.
+  // re-layout of the scales.  AUTO takes it where grouped_mid_pays() says so: up to 160 rows per expert on average,
+  // and beyond where the tile kernels' rounds would come out sparsely filled.
   if (variant == WAVE_MXFP4_VARIANT_MID_M || variant == WAVE_MXFP4_VARIANT_AUTO) {
     const bool fits = mid_grouped_applies(p);
     if (variant == WAVE_MXFP4_VARIANT_MID_M && !fits) return WAVE_MXFP4_ERR_UNSUPPORTED;
     const int64_t avg = (total_rows + num_groups - 1) / num_groups;
-    const bool pays = avg <= kGroupedMidMaxAvgRows && (int64_t)num_groups * ((n + 127) / 128) >= device_cus() / 2;
+    const bool pays = grouped_mid_pays(total_rows, num_groups, n, k);
     if (fits && (variant == WAVE_MXFP4_VARIANT_MID_M || pays)) {
       // rows per block: a quarter more than the average group, 32 or in steps of 64, at most the whole batch.  A
       // group of more rows takes a second pass over its expert's B, which costs that expert's share of the call;
@@ -813,6 +850,8 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
       // 65.4 -> 63.3, 84.3 -> 72.5 us), because the rings are sized for the block, not for the rows that arrive.
       int64_t bm = (5 * avg + 3) / 4 < total_rows ? (5 * avg + 3) / 4 : total_rows;
       bm = bm > 256 ? 256 : bm <= 32 ? 32 : (bm + 63) / 64 * 64;
+      // (the library's own choice above 152 rows per expert was measured, and is priced, on 192-row blocks)
+      if (variant == WAVE_MXFP4_VARIANT_AUTO && bm > 192) bm = 192;
       return record_hip(launch_mid_gemm(p, device_cus(), stream, (int)bm));
     }
   }
@@ -944,7 +983,7 @@ int wave_mxfp4_gemm_gated_quantize(const void *a, const void *a_scale, const voi
   // epilogue in that kernel, one launch, no table, the scales read as they are.
   if (num_groups > 0 && b_native && mid_gated_applies(p)) {
     const int64_t avg = (total_rows + num_groups - 1) / num_groups;
-    if (avg <= kGroupedMidMaxAvgRows && (int64_t)num_groups * (n / 128) >= device_cus() / 2) {
+    if (grouped_mid_pays(total_rows, num_groups, n, k)) {
       int64_t bm = (5 * avg + 3) / 4 < total_rows ? (5 * avg + 3) / 4 : total_rows;
       bm = bm > 192 ? 192 : bm <= 32 ? 32 : (bm + 63) / 64 * 64;
       p.tile_table = nullptr;

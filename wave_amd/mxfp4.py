@@ -519,7 +519,8 @@ def mxfp4_gemm_gated_quantize(x, x_scales, w_il, w_scales_il, offsets=None, *, a
     ``[E, 2I, K/2]`` (or ``[2I, K/2]`` with ``offsets=None``: dense) holds gate and up projections interleaved by
     :func:`interleave_gate_up`, as do its scales.  Returns ``(q [rows, I/2], scales)`` of ``silu(gate) * up``, the
     same bits as ``mxfp4_gemm_grouped`` (bf16 out) followed by ``silu_and_mul_quantize``.  Large batches run the
-    persistent kernel, small grouped ones (up to 152 rows per expert on average) with ``b_scale_layout`` MFMA32 the
+    persistent kernel, small grouped ones (the batches :func:`mxfp4_gemm_grouped` gives to the mid-M kernel: up to 160 rows per expert on
+    average and some beyond) with ``b_scale_layout`` MFMA32 the
     mid-M kernel.  Raises ``ValueError`` (status "unsupported") where neither applies; the caller then runs the
     two calls."""
     lib = _lib.load()

@@ -175,7 +175,9 @@ def run_small_batch(counts, inter, k, seed, a_native, slack_rows=0):
     ([70, 20, 64, 65, 3, 0, 50, 47], 1792, 2048),             # blocks of 64 rows, two groups of a second pass
     ([100, 0, 260, 33, 1, 150, 97, 128], 1024, 1024),         # blocks of 128 rows, a group of three passes
     ([150, 160, 140, 155, 149, 132, 141, 143], 1024, 1536),   # blocks of 192 rows
-], ids=["bm32", "bm32_two_per_cu", "bm64", "bm128", "bm192"])
+    ([250, 260, 240, 255, 249, 232, 241, 243], 2048, 1024),   # two passes of 192-row blocks (few column tiles: the
+                                                              # tile kernels would leave CUs idle for whole rounds)
+], ids=["bm32", "bm32_two_per_cu", "bm64", "bm128", "bm192", "bm192_two_passes"])
 def test_small_batch_fused_in_the_mid_kernel_matches_the_chain(counts, inter, k, a_native):
     run_small_batch(counts, inter, k, seed=sum(counts) + k, a_native=a_native, slack_rows=37)
 

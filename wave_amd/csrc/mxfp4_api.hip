@@ -203,6 +203,12 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
       }
       if (mid) return WAVE_MXFP4_VARIANT_MID_M;
     }
+    // 32 < M <= 64 against a narrow B with a long K: few column tiles, and the streaming kernel's workgroups each
+    // walk all of K with four row blocks of accumulators; the 128x128 tiles with the library's split along K put
+    // more CUs to work (us, streaming -> tiles; 64 x 1024 x 8192: 20.8 -> 12.2, 48 x 4096 x 8192: 17.9 -> 13.0,
+    // 40 x 2048 x 14336: 19.7 -> 18.1, 64 x 3072 x 14336: 25.1 -> 19.8; at N = 4096, K = 14336 the streaming kernel
+    // leads again, 16.1 against 19.5, and at K <= 4096 the two are within a microsecond)
+    if (m > 32 && m <= skinny_max_m() && k > 4096 && n <= (k <= 8192 ? 4096 : 3072)) return pick_tile_variant(m, n, native_scales);
     if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;
     v = pick_tile_variant(m, n, native_scales);
   }

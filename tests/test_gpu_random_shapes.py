@@ -117,3 +117,18 @@ def _resident_cases(count, seed):
 @pytest.mark.parametrize("case", _resident_cases(12, seed=23), ids=lambda c: f"r{c[0]}-{c[1]}x{c[2]}x{c[3]}")
 def test_random_resident_scale_shape_against_oracle(case):
     test_random_shape_against_oracle(case)
+
+
+@pytest.mark.parametrize("m,n,k", [(33, 512, 8192), (48, 3000, 8192), (64, 1024, 14336), (64, 4096, 8192), (40, 3072, 16384),
+                                   (64, 4100, 8192), (32, 1024, 8192)])
+def test_narrow_b_long_k_against_oracle(m, n, k):
+    """32 < M <= 64 against a B of at most 4096 rows with K > 4096: the library's own choice is the 128x128 tiles
+    with its split along K (the last two cases lie just outside that range: the streaming kernel).  Every row
+    against the exact oracle, both output types, with and without scratch."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + n, scale_lo=120, scale_hi=134)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    for dt in (torch.float32, torch.bfloat16):
+        for kw in ({}, {"workspace": False}):
+            got = run_gemm(x, xs, w_t, ws, dt, **kw)
+            assert not np.isnan(got).any()
+            assert_close(got, ref, dt, f"{m}x{n}x{k} {dt} {kw}")

@@ -72,13 +72,15 @@ int pick_tile_variant(int64_t m, int64_t n, bool native_scales) {
   // on 256x256 tiles, 59.9 on 128x128; 64 x 57344 x 4096: 34.5 against 28.1 us).  Measured up to N = 65536.
   if (native_scales && m <= 128 && n <= 65536) return WAVE_MXFP4_VARIANT_T128x128_W2x2;
   const int64_t t256 = ((m + 255) / 256) * ((n + 255) / 256);
+  // 129..256 tiles of 128x256: one workgroup per CU on at least half of them, at nearly twice the MFMA duty of
+  // the 128x128 kernel (1024 x 5120 x 16000: 72 -> 60 us; 1024 x 8192: 80 -> 76 us).  Also where a ragged M makes
+  // that up to 170 tiles of 256x256, which would leave a third of the CUs idle (1100 x 7168 x 8192: 252 tiles of
+  // 128x256 against 140 of 256x256, 49.3 -> 41.8 us; x 4096: 31.3 -> 27.0).
+  const int64_t t128x256 = ((m + 127) / 128) * ((n + 255) / 256);
+  if (t128x256 > 128 && t128x256 <= 256 && t256 <= 170) return WAVE_MXFP4_VARIANT_T128x256_W2x2;
   // 8 waves: measured 4-5 % ahead of 4 at 8192^3.  Up to 128 tiles of 256x256 leave half the CUs idle; the same
   // problem as up to 512 tiles of 128x128 fills them with two workgroups each (1024 x 8192 x 16384: 87 -> 82 us).
   if (t256 > 128) return WAVE_MXFP4_VARIANT_T256x256_W4x2;
-  // 129..256 tiles of 128x256: one workgroup per CU on at least half of them, at nearly twice the MFMA duty of
-  // the 128x128 kernel (1024 x 5120 x 16000: 72 -> 60 us; 1024 x 8192: 80 -> 76 us)
-  const int64_t t128x256 = ((m + 127) / 128) * ((n + 255) / 256);
-  if (t128x256 > 128 && t128x256 <= 256) return WAVE_MXFP4_VARIANT_T128x256_W2x2;
   return WAVE_MXFP4_VARIANT_T128x128_W2x2;
 }
 
@@ -702,9 +704,13 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
     return record_hip(launch_naive_gemm(p, stream));
   }
   int v = variant;
-  if (v == WAVE_MXFP4_VARIANT_AUTO)
-    v = ((m + 255) / 256) * ((n + 255) / 256) >= 128 ? WAVE_MXFP4_VARIANT_T256x256_W4x2  // 8 waves: 498 -> 476 us at 8192^3
-                                                     : WAVE_MXFP4_VARIANT_T128x128_W2x2;
+  if (v == WAVE_MXFP4_VARIANT_AUTO) {
+    // (up to 512 tiles of 128x128 are one round of two workgroups per CU, where up to 170 tiles of 256x256 leave
+    // CUs idle: 2048 x 4096 x 4096 57.2 -> 38.6 us, 1100 x 7168 x 4096 57.0 -> 39.7; from 576 on the two are level)
+    const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128);
+    v = t128 > 512 && ((m + 255) / 256) * ((n + 255) / 256) >= 128 ? WAVE_MXFP4_VARIANT_T256x256_W4x2  // 8 waves: 498 -> 476 us at 8192^3
+                                                                   : WAVE_MXFP4_VARIANT_T128x128_W2x2;
+  }
   int bm, bn;
   tile_variant_shape(v, &bm, &bn);
   p.tiles_m = (int)((m + bm - 1) / bm);

@@ -106,7 +106,11 @@ constexpr int64_t kGroupedMidMaxAvgRows = 160;  // (one pass of the 192-row bloc
 // x 14336, 1280..2560 rows: 140..190 us against 67..125 us here), while one of many well-filled rounds does not
 // (8 x 28672 x 4096, 1536 rows: 147 against 185 us).  Both sides are priced in K tiles per workgroup and round with
 // factors fitted to 49 such measurements (the choice was within 9 % of the better kernel on all of them).
-static bool grouped_mid_pays(int64_t total_rows, int num_groups, int64_t n, int64_t k) {
+// `bm_cap`: the tallest block the call may use (256 rows with row-major activation scales, 192 with MFMA32 ones);
+// `*bm_max`: the block height the estimate was made for.
+static bool grouped_mid_pays(int64_t total_rows, int num_groups, int64_t n, int64_t k, int bm_cap = 192,
+                             int *bm_max = nullptr) {
+  if (bm_max) *bm_max = 192;
   const int64_t cus = device_cus();
   const int64_t strips = (int64_t)num_groups * ((n + 127) / 128);
   if (2 * strips < cus) return false;
@@ -115,9 +119,17 @@ static bool grouped_mid_pays(int64_t total_rows, int num_groups, int64_t n, int6
   (void)k;  // (both estimates are proportional to K)
   // passes of 192-row blocks, in halves: groups dealt at random spread about a tenth around the average
   const double passes_raw = (double)avg * 1.1 / 192.0;
-  const double passes = passes_raw < 1.0 ? 1.0 : (double)((int64_t)(passes_raw * 2.0 + 0.999)) / 2.0;
+  double passes = passes_raw < 1.0 ? 1.0 : (double)((int64_t)(passes_raw * 2.0 + 0.999)) / 2.0;
+  double per_pass = 0.9;
+  // Where one 256-row block still holds every group and the 192-row block needs a second pass, the taller block
+  // (a fifth slower per pass) is taken if the call may (8 x 4096 x 14336, 1536 rows, row-major scales: 106 -> 79 us;
+  // 8 x 8192 x 8192: 123 -> 90)
+  if (bm_cap >= 256 && passes > 1.0 && avg <= 208) {
+    passes = 1.0, per_pass = 1.1;
+    if (bm_max) *bm_max = 256;
+  }
   const double rounds_mid = strips > cus ? (double)strips / (double)cus : 1.0;
-  const double t_mid = rounds_mid * passes * 0.9;
+  const double t_mid = rounds_mid * passes * per_pass;
   const int v = pick_tile_variant(total_rows, n, false);
   const double n256 = (double)((n + 255) / 256), n128 = (double)((n + 127) / 128);
   double t_alt;
@@ -853,7 +865,8 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
     const bool fits = mid_grouped_applies(p);
     if (variant == WAVE_MXFP4_VARIANT_MID_M && !fits) return WAVE_MXFP4_ERR_UNSUPPORTED;
     const int64_t avg = (total_rows + num_groups - 1) / num_groups;
-    const bool pays = grouped_mid_pays(total_rows, num_groups, n, k);
+    int bm_max = 192;
+    const bool pays = grouped_mid_pays(total_rows, num_groups, n, k, p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR ? 256 : 192, &bm_max);
     if (fits && (variant == WAVE_MXFP4_VARIANT_MID_M || pays)) {
       // rows per block: a quarter more than the average group, 32 or in steps of 64, at most the whole batch.  A
       // group of more rows takes a second pass over its expert's B, which costs that expert's share of the call;
@@ -862,8 +875,8 @@ int wave_mxfp4_gemm_grouped(const void *a, const void *a_scale, const void *b, c
       // 65.4 -> 63.3, 84.3 -> 72.5 us), because the rings are sized for the block, not for the rows that arrive.
       int64_t bm = (5 * avg + 3) / 4 < total_rows ? (5 * avg + 3) / 4 : total_rows;
       bm = bm > 256 ? 256 : bm <= 32 ? 32 : (bm + 63) / 64 * 64;
-      // (the library's own choice above 152 rows per expert was measured, and is priced, on 192-row blocks)
-      if (variant == WAVE_MXFP4_VARIANT_AUTO && bm > 192) bm = 192;
+      // (the library's own choice beyond one 192-row block per expert is priced on the block height it names)
+      if (variant == WAVE_MXFP4_VARIANT_AUTO && bm > 192) bm = bm_max;
       return record_hip(launch_mid_gemm(p, device_cus(), stream, (int)bm));
     }
   }

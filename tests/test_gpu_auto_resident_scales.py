@@ -41,6 +41,8 @@ def run(gx, gxs, gw, gws, m, n, dt, layout, b_layout):
     (32, 20480, 4096),    # one round of strips, preshuffled B: the B-direct kernel from 32 rows
     (100, 28672, 2048),
     (256, 40960, 1024),   # above 128 rows the B-direct kernel serves one round of strips only
+    (96, 8192, 4096),     # K <= 4096, preshuffled B: the B-direct kernel from N = 8192 and 48 rows on
+    (48, 10240, 2048),
 ])
 def test_library_choice_with_resident_scales(m, n, k, pre):
     x, xs, w, ws = orc.make_inputs(m, n, k, seed=m + n + k, scale_lo=116, scale_hi=138)

@@ -414,7 +414,10 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   // 128 x 20480 29.5 -> 24.4, 96 x 20480 x 4096 15.4 -> 13.5, 48 x 20480 x 8192 23.6 -> 20.7, 128 x 57344 x 8192
   // 63.4 -> 54.9; at N <= 16384, K = 8192 the streaming kernel keeps M < 64: 32 x 12288 14.9 against 18.4.)
   const int64_t cus_n = 128 * (int64_t)device_cus();  // columns of one round of strips
-  if (variant == WAVE_MXFP4_VARIANT_AUTO && n >= 12288 && split_k <= 1 && midb_shape_ok(m, n, k, b_layout) &&
+  // (with resident scales and K <= 4096 it leads from N = 8192 on for 48 rows and more: 128 x 8192 x 4096 15.5 -> 12.5,
+  // 48 rows 12.4 -> 11.2, 256 rows 20.0 -> 18.0; at N = 4096 the 128x128 tiles are level or ahead)
+  const int64_t midb_min_n = native_scales && k <= 4096 && m >= 48 ? 8192 : 12288;
+  if (variant == WAVE_MXFP4_VARIANT_AUTO && n >= midb_min_n && split_k <= 1 && midb_shape_ok(m, n, k, b_layout) &&
       (m > 128 ? n <= cus_n
                : native_scales && n <= 2 * cus_n && (m >= 64 || (m >= 32 && n <= cus_n && (n >= 20480 || k <= 4096)))))
     v = WAVE_MXFP4_VARIANT_MID_M_BDIRECT;

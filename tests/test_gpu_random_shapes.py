@@ -132,3 +132,19 @@ def test_narrow_b_long_k_against_oracle(m, n, k):
             got = run_gemm(x, xs, w_t, ws, dt, **kw)
             assert not np.isnan(got).any()
             assert_close(got, ref, dt, f"{m}x{n}x{k} {dt} {kw}")
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 8192, 9216), (16, 8448, 11008), (16, 4096, 14080), (64, 2048, 12032),
+                                   (8, 12288, 6400), (16, 4096, 6400), (5, 8192, 13824), (33, 8192, 14080)])
+def test_decode_rows_with_uneven_k_tiles_against_oracle(m, n, k):
+    """Up to 64 rows with a count of K tiles that the streaming kernel cannot deal evenly over its waves (25, 36, 43,
+    47, 54 and 55 tiles: the K of Llama-2 down projections among them): the library's own choice is the mid-M
+    kernel against a wide B and the 128x128 tiles with a split along K against a narrow one.  Every row against the
+    exact oracle, both output types, with and without scratch."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + k, scale_lo=120, scale_hi=134)
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+    for dt in (torch.float32, torch.bfloat16):
+        for kw in ({}, {"workspace": False}):
+            got = run_gemm(x, xs, w_t, ws, dt, **kw)
+            assert not np.isnan(got).any()
+            assert_close(got, ref, dt, f"{m}x{n}x{k} {dt} {kw}")

@@ -163,6 +163,25 @@ bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
   return m >= 1 && m <= mid_max_m() && k % kTileK == 0 && k >= 4 * kTileK && n % 4 == 0;
 }
 
+int auto_split(int64_t m, int64_t n, int64_t k, int variant);
+
+// Whether the streaming kernel would run this K in its counted-wait mode: the library's split leaves every
+// workgroup the same number of whole K tiles, and one, two or four waves share them evenly, at most eight each
+// (launch_stream_gemm).  Otherwise it runs its predicated mode with full waits, or a split into many parts:
+// 16 x 28672 x 14080 (55 K tiles: five parts of eleven) 148.7 us against 36.4 on the mid-M kernel, K = 11008 and
+// 13824 (43 and 54 K tiles) alike, where K = 14336 (two parts of 28) takes 27.
+static bool stream_runs_counted(int64_t n, int64_t k) {
+  if (k % kTileK != 0) return false;
+  const int64_t k_tiles = k / kTileK;
+  const int s = auto_split(1, n, k, WAVE_MXFP4_VARIANT_SKINNY);
+  if (s < 1 || k_tiles % s != 0) return false;
+  const int64_t per = k_tiles / s;
+  if (per > stream_max_k_tiles()) return false;
+  for (int c = 1; c <= 4; c *= 2)
+    if (per % c == 0 && per / c <= 8) return true;
+  return false;
+}
+
 int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scales, bool b_preshuffled) {
   int v = variant;
   if (v == WAVE_MXFP4_VARIANT_AUTO) {
@@ -209,8 +228,9 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
         // (K = 8192: the streaming kernel's longest K range without a split; up to 16 rows it also leads at
         // K = 4096 on that quarter-full second round, 16 x 40960 x 4096: 19.2 -> 17.4, preshuffled B 21.4 -> 17.6)
         const bool k_whole = k >= 8192 && k <= (int64_t)kTileK * stream_max_k_tiles();
-        if ((k_whole && m > 16 && m <= 48 && strips <= 128) ||
-            ((k_whole || m <= 16) && m <= 64 && second_round && 4 * strips <= 5 * cus))
+        if (stream_runs_counted(n, k) &&
+            ((k_whole && m > 16 && m <= 48 && strips <= 128) ||
+             ((k_whole || m <= 16) && m <= 64 && second_round && 4 * strips <= 5 * cus)))
           return WAVE_MXFP4_VARIANT_SKINNY;
         if (k <= 4096 && ((m >= 48 && m <= 128 && second_round && !b_preshuffled) || (m > 128 && m <= 192 && strips <= 128)))
           return pick_tile_variant(m, n, true);
@@ -223,6 +243,15 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     // 40 x 2048 x 14336: 19.7 -> 18.1, 64 x 3072 x 14336: 25.1 -> 19.8; at N = 4096, K = 14336 the streaming kernel
     // leads again, 16.1 against 19.5, and at K <= 4096 the two are within a microsecond)
     if (m > 32 && m <= skinny_max_m() && k > 4096 && n <= (k <= 8192 ? 4096 : 3072)) return pick_tile_variant(m, n, native_scales);
+    // A K that the streaming kernel cannot deal evenly over its waves (see stream_runs_counted): the mid-M kernel
+    // against a wide B, the 128x128 tiles with the library's split against a narrow one (us, streaming -> taken:
+    // 16 x 28672 x 12032 69.1 -> 30.9, 1 x 12288 x 9216 22.2 -> 16.7, 16 x 28672 x 6400 35.6 -> 19.2;
+    // 16 x 4096 x 14080 30.0 -> 16.2, 64 x 4096 x 12032 28.3 -> 15.7)
+    if (m <= skinny_max_m() && k % kTileK == 0 && !stream_runs_counted(n, k)) {
+      if (n >= 8192 && mid_shape_ok(m, n, k)) return WAVE_MXFP4_VARIANT_MID_M;
+      // (up to 32 K tiles one workgroup still streams a narrow B faster than the tiles: 16 x 4096 x 6400 9.1 against 11.7)
+      if (k > 8192) return pick_tile_variant(m, n, native_scales);
+    }
     if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;
     v = pick_tile_variant(m, n, native_scales);
   }

@@ -148,3 +148,17 @@ def test_decode_rows_with_uneven_k_tiles_against_oracle(m, n, k):
             got = run_gemm(x, xs, w_t, ws, dt, **kw)
             assert not np.isnan(got).any()
             assert_close(got, ref, dt, f"{m}x{n}x{k} {dt} {kw}")
+
+
+@pytest.mark.parametrize("m,n,k", [(2773, 1408, 1024), (3300, 1152, 2304), (5600, 640, 1280)])
+def test_half_empty_last_column_tile_against_oracle(m, n, k):
+    """An N that leaves the last 256-column tile half empty, with more than 128 tiles of 128x256 but at most 256 of
+    128x128: the library's own choice is the latter.  Sampled rows against the exact oracle, the whole output
+    against the 128x128 tiles by name (the same K order per element: the same bits)."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + n, scale_lo=120, scale_hi=134)
+    rows = np.unique(np.concatenate([np.arange(0, m, 41), np.arange(m - 5, m)]))
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    for dt in (torch.float32, torch.bfloat16):
+        got = run_gemm(x, xs, w_t, ws, dt)
+        assert_close(got[rows], ref, dt, f"{m}x{n}x{k} {dt}")
+        assert np.array_equal(got, run_gemm(x, xs, w_t, ws, dt, variant=_lib.VARIANT_T128x128_W2x2))

@@ -61,3 +61,22 @@ def test_tile192_rejects_what_it_does_not_take():
     x, xs, w, ws = orc.make_inputs(4352, 4096, 1024, seed=1)     # N % 192 != 0
     with pytest.raises((RuntimeError, ValueError)):
         run(x, xs, w, ws, torch.float32, variant=V, split_k=1)
+
+
+def test_tile192_auto_choice_where_n_is_not_in_whole_256_column_tiles():
+    """N = 102 x 192 = 76.5 x 256: the 256x256 tiles would run one per workgroup in two whole rounds over the CUs
+    (4 x 77 = 308 tiles), the library's own choice is the persistent kernel on 4 x 102 tiles of 256x192.  The same
+    bits as that kernel by name, sampled rows against the exact oracle, and a shape of one round (3 x 77 tiles) that
+    stays on the wider tiles."""
+    m, n, k = 896, 19584, 1024
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=9, scale_lo=110, scale_hi=142)
+    for dt in (torch.float32, torch.bfloat16):
+        auto = run(x, xs, w, ws, dt)
+        assert np.array_equal(auto, run(x, xs, w, ws, dt, variant=V, split_k=1))
+        rows = np.unique(np.concatenate([np.arange(0, m, 61), np.arange(m - 8, m), [255, 256]]))
+        assert_close(auto[rows], c_oracle.scaled_gemm_exact(x, w, xs, ws, rows=rows), dt, "rows vs oracle")
+    m = 640
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=10, scale_lo=110, scale_hi=142)
+    auto = run(x, xs, w, ws, torch.float32)
+    rows = np.arange(0, m, 53)
+    assert_close(auto[rows], c_oracle.scaled_gemm_exact(x, w, xs, ws, rows=rows), torch.float32, "one round")

@@ -77,6 +77,10 @@ int pick_tile_variant(int64_t m, int64_t n, bool native_scales) {
   // that up to 170 tiles of 256x256, which would leave a third of the CUs idle (1100 x 7168 x 8192: 252 tiles of
   // 128x256 against 140 of 256x256, 49.3 -> 41.8 us; x 4096: 31.3 -> 27.0).
   const int64_t t128x256 = ((m + 127) / 128) * ((n + 255) / 256);
+  // (an N that leaves the last 256-column tile half empty can make that no more than 256 tiles of 128x128: one round
+  // of one workgroup per CU at 0.53-0.62 us per K tile against 0.67-1.0; 2773 x 1408 x 3584: 21.8 -> 17.3 us, x 16128:
+  // 54.6 -> 47.2)
+  if (t128x256 > 128 && ((m + 127) / 128) * ((n + 127) / 128) <= 256) return WAVE_MXFP4_VARIANT_T128x128_W2x2;
   if (t128x256 > 128 && t128x256 <= 256 && t256 <= 170) return WAVE_MXFP4_VARIANT_T128x256_W2x2;
   // 8 waves: measured 4-5 % ahead of 4 at 8192^3.  Up to 128 tiles of 256x256 leave half the CUs idle; the same
   // problem as up to 512 tiles of 128x128 fills them with two workgroups each (1024 x 8192 x 16384: 87 -> 82 us).
@@ -649,6 +653,12 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
       }
     } else if (tv == WAVE_MXFP4_VARIANT_T256x192_W4x2) {
       return WAVE_MXFP4_ERR_UNSUPPORTED;  // (no one-tile-per-workgroup kernel of that shape)
+    } else if (GemmParams p192 = p; variant == WAVE_MXFP4_VARIANT_AUTO && tv == WAVE_MXFP4_VARIANT_T256x256_W4x2 &&
+                                    persist_192_over_tile_kernel(p, device_cus()) &&
+                                    (p192.tiles_n = (int)(n / 192),
+                                     persist_gemm_applies(p192, WAVE_MXFP4_VARIANT_T256x192_W4x2, device_cus()))) {
+      // N in whole 192-column tiles but not in whole 256-column ones
+      e = launch_persist_gemm(p192, WAVE_MXFP4_VARIANT_T256x192_W4x2, device_cus(), stream);
     } else {
       e = launch_tile_gemm(p, tv, stream);
     }

@@ -136,6 +136,7 @@ hipError_t launch_persist_gemm(const GemmParams &p, int variant, int num_cus, hi
 bool persist_gemm_fp8_applies(const GemmParams &p, int num_cus);
 hipError_t launch_persist_gemm_fp8(const GemmParams &p, int num_cus, int a_fmt, int b_fmt, hipStream_t stream);
 bool persist_prefers_192(const GemmParams &p, int num_cus, int parts256);
+bool persist_192_over_tile_kernel(const GemmParams &p, int num_cus);
 bool persist_gated_applies(const GemmParams &p, int num_cus);
 hipError_t launch_persist_gated(const GemmParams &p, int num_cus, hipStream_t stream);
 hipError_t launch_interleave_rows(const uint8_t *src, uint8_t *dst, int64_t half_rows, int64_t row_bytes, int block,

@@ -1069,6 +1069,22 @@ bool persist_prefers_192(const GemmParams &p, int num_cus, int parts256) {
   return 0.785 * rounds(t192, 1) < 0.95 * rounds(t256, parts256);
 }
 
+// The same question where N is a multiple of 192 but not of 256: the 256x256 tiles then run one per workgroup, in
+// whole rounds over the CUs, and the persistent kernel on 256x192 tiles is the alternative from more tiles than
+// workgroups on, at any number of tile rows (896 x 19584 x 3584: 308 tiles in two rounds 63.3 us, 408 narrower tiles
+// 51.7; 1183 x 19584: 66.8 -> 55.4; 640 x 19584, 231 tiles in one round, stays: 38.1 against 45.4; 1536 x 19584,
+// 462 against 612 tiles, stays: 70.7 against 76.4).
+bool persist_192_over_tile_kernel(const GemmParams &p, int num_cus) {
+  if (p.num_groups != 0 || p.n % 192 != 0 || p.n % 256 == 0 || p.splits != 1) return false;
+  const int grid = num_cus / kNumXcd * kNumXcd;
+  if (grid < kNumXcd) return false;
+  const int64_t tm = (p.m + 255) / 256, t256 = tm * ((p.n + 255) / 256), t192 = tm * (p.n / 192);
+  if (t192 <= grid) return false;
+  const double f = (double)(t192 % grid) / grid;
+  const double r192 = (double)(t192 / grid) + (f == 0.0 ? 0.0 : 0.4 + 0.6 * f);
+  return 0.785 * r192 < (double)((t256 + num_cus - 1) / num_cus);
+}
+
 // Whether the persistent kernel serves this problem with `num_cus` CUs.
 bool persist_gemm_applies(const GemmParams &p, int variant, int num_cus) {
   if (variant != WAVE_MXFP4_VARIANT_T256x256_W2x2 && variant != WAVE_MXFP4_VARIANT_T256x256_W4x2 &&

@@ -144,7 +144,8 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
 
 /* Scratch bytes wave_mxfp4_gemm can use for (m, n, k, split_k, variant): the
  * split-K partials (for split_k == 0, of the split the library would pick by
- * itself) plus the re-laid-out scales of both operands. */
+ * itself; given less, it takes fewer parts) plus the re-laid-out scales of both
+ * operands. */
 size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant);
 
 /*
@@ -163,7 +164,10 @@ size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, 
  * this call's layouts do not use: scale tensors already in MFMA32 order are read
  * in place) exceeds that size is
  * rejected with WAVE_MXFP4_ERR_WORKSPACE (wave_mxfp4_last_hip_error() then
- * holds the two sizes); 8192^3 needs 6.3 MB.  All calls on one GPU share the
+ * holds the two sizes); 8192^3 needs 6.3 MB.  With split_k == 0 what has to fit
+ * is the call without a split: the library's own split takes as many parts as
+ * the array holds beside the scales, as wave_mxfp4_gemm does with a workspace
+ * of that size.  All calls on one GPU share the
  * array: calls that overlap in time on one GPU (different streams, or threads
  * without ordering) race on it; calls on one stream are ordered and safe.
  */

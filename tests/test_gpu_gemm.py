@@ -103,6 +103,21 @@ def test_split_k_equals_unsplit(vname, splits, out_dtype):
     assert np.array_equal(got, again)
 
 
+@pytest.mark.parametrize("splits", [3, 5, 6, 7, 8])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_split_k_part_counts(splits, out_dtype):
+    """Every part count the library's own split can take (the sum over the parts has an unrolled form per count),
+    on the 128x128 and 128x256 tiles, with an M x N that is and is not a multiple of four."""
+    for m, n in ((200, 384), (131, 250)):
+        k = splits * 512
+        x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=splits, scale_lo=120, scale_hi=134)
+        ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
+        for v in (_lib.VARIANT_T128x128_W2x2, _lib.VARIANT_T128x256_W2x2):
+            got = run_gemm(x, xs, w_t, ws, out_dtype, variant=v, split_k=splits)
+            assert not np.isnan(got).any()
+            assert_close(got, ref, out_dtype, f"{m}x{n} variant {v} split {splits}")
+
+
 def test_split_k_auto_and_caller_workspace():
     m, n, k = 256, 256, 8192
     x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=3)

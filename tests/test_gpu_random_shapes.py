@@ -8,6 +8,8 @@ import numpy as np
 import pytest
 import torch
 
+import wave_amd
+
 from oracle import c_oracle
 from oracle import mxfp4_oracle as orc
 from wave_amd import _lib
@@ -162,3 +164,27 @@ def test_half_empty_last_column_tile_against_oracle(m, n, k):
         got = run_gemm(x, xs, w_t, ws, dt)
         assert_close(got[rows], ref, dt, f"{m}x{n}x{k} {dt}")
         assert np.array_equal(got, run_gemm(x, xs, w_t, ws, dt, variant=_lib.VARIANT_T128x128_W2x2))
+
+
+@pytest.mark.parametrize("m,n,k", [(176, 3200, 8960), (97, 8832, 15616), (76, 4480, 13312), (384, 3584, 8192),
+                                   (134, 6272, 12032), (768, 3584, 11008), (1280, 3584, 4096), (256, 11008, 4096)])
+def test_estimated_tile_shape_and_split_against_oracle(m, n, k):
+    """Problems of at most two rounds of 256x256 tiles, where the library's own choice of tile shape and split comes
+    from its duration estimates: splits into 3, 5 and 7 uneven parts on the 128x128 and 128x256 tiles, a problem of
+    280 tiles of 128x128 with a short K (scales re-laid, not staged by the kernel), and one for the mid-M kernel.
+    Sampled rows against the exact oracle with row-major scales and with scales in MFMA32 order, both output types,
+    and without scratch (no split then)."""
+    x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + k, scale_lo=120, scale_hi=134)
+    rows = np.unique(np.concatenate([np.arange(0, m, max(1, m // 24)), np.arange(m - 4, m)]))
+    ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws, rows=rows)
+    xs32 = wave_amd.scale_convert(torch.from_numpy(xs).cuda(), m, k // 32, 0, _lib.SCALE_MFMA32).cpu().numpy()
+    ws32 = wave_amd.scale_convert(torch.from_numpy(ws).cuda(), n, k // 32, 0, _lib.SCALE_MFMA32).cpu().numpy()
+    for dt in (torch.float32, torch.bfloat16):
+        got = run_gemm(x, xs, w_t, ws, dt)
+        assert not np.isnan(got).any()
+        assert_close(got[rows], ref, dt, f"{m}x{n}x{k} {dt} row-major scales")
+        got = run_gemm(x, xs32, w_t, ws32, dt, a_scale_layout=_lib.SCALE_MFMA32, b_scale_layout=_lib.SCALE_MFMA32)
+        assert not np.isnan(got).any()
+        assert_close(got[rows], ref, dt, f"{m}x{n}x{k} {dt} MFMA32 scales")
+    got = run_gemm(x, xs, w_t, ws, torch.float32, workspace=False)
+    assert_close(got[rows], ref, torch.float32, f"{m}x{n}x{k} without scratch")

@@ -101,6 +101,104 @@ int device_cus() {
   return cached[dev];
 }
 
+// ---- Estimated duration of a dense problem on the tile kernels and the mid-M kernel ----
+// For problems of up to two rounds of 256x256 tiles the kernels are bound by how fast one workgroup streams its
+// operands from HBM, not by the matrix pipes, and which tile shape and split along K is fastest follows from a few
+// measured quantities (MI355X, B from HBM, called back to back from one host thread; us):
+//   a workgroup's time per K tile as a function of the workgroups in flight (flat up to one per CU - 0.72 on
+//   128x128 tiles, 1.03 on 128x256, 1.30 on 256x256 -, then rising: the tables below, for 256 CUs);
+//   a fixed part per call (launch, first fill, last C tile, and the scale re-layout launch in front when the scales
+//   come row-major: 13.5 / 11.5 / 14.0, with scales in MFMA32 order 5.0 / 6.5 / 9.5; the 128x128 kernel on up to
+//   8 K tiles of row-major scales stages them itself: 4.4, and 1.19 per K tile);
+//   a split's reduction: a launch (2, or 3.5 where no re-layout launch hides it), 0.4 per part for its fill, and 1.3
+//   per million f32 partials;
+//   the mid-M kernel: 4.5 + K tiles x (0.27 + 0.0025 M) per round of 128-column strips, + N / 14336.
+// Fitted to 768 shapes (M = 96..4096, N = 2048..14336, K = 4096..14336, both scale layouts, every tile shape with 1-8
+// parts by name): the choice by these estimates is within 5 % of the best measured kernel on 95 % of them and
+// within 10 % on 98 % (the borders it replaces: 80 % and 87 %).
+struct TileChoice {
+  int variant, split;
+  double us;
+};
+
+static double table_step(const double (*tab)[2], int rows, double wgs) {
+  if (wgs <= tab[0][0]) return tab[0][1];
+  for (int i = 1; i < rows; ++i)
+    if (wgs <= tab[i][0]) {
+      const double f = (wgs - tab[i - 1][0]) / (tab[i][0] - tab[i - 1][0]);
+      return tab[i - 1][1] + f * (tab[i][1] - tab[i - 1][1]);
+    }
+  return tab[rows - 1][1] * wgs / tab[rows - 1][0];  // (throughput-bound from there on)
+}
+
+// us of variant `v` (128x128, 128x256 or 256x256 tiles) with `s` parts along K; negative where `s` is no valid split
+static double tile_cost_us(int v, int s, int64_t m, int64_t n, int64_t k, bool native_scales) {
+  static const double t128[][2] = {{0, 0.70},    {256, 0.72},  {257, 0.82},  {320, 0.92},  {384, 0.97},
+                                   {448, 1.07},  {512, 1.10},  {513, 1.58},  {640, 1.86},  {768, 1.93},
+                                   {1024, 2.33}, {1025, 2.71}, {1344, 3.23}, {1792, 4.24}};
+  static const double t128x256[][2] = {{0, 1.02},   {192, 1.03}, {256, 1.12}, {257, 1.88}, {320, 2.15},
+                                       {384, 2.23}, {512, 2.37}, {513, 3.11}, {688, 3.43}, {896, 4.58}};
+  static const double t256[][2] = {{0, 1.30},   {140, 1.30}, {192, 1.49}, {256, 1.80},
+                                   {257, 2.18}, {336, 2.98}, {448, 3.39}, {512, 3.60}};
+  int bm, bn;
+  tile_variant_shape(v, &bm, &bn);
+  const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+  const int64_t k_tiles = (k + kTileK - 1) / kTileK, per = (k_tiles + s - 1) / s;
+  if (s > 1 && (k_tiles / s < 2 || (s - 1) * per >= k_tiles)) return -1.0;
+  const double wgs = (double)(tiles * s) * 256.0 / (double)device_cus();
+  double fixed, step;
+  if (bm == 128 && bn == 128) {
+    fixed = native_scales ? 5.0 : 13.5;
+    step = table_step(t128, sizeof(t128) / sizeof(t128[0]), wgs);
+    if (native_scales && wgs <= 256) step += 0.08;
+    if (!native_scales && wgs <= 256 && per <= 8 && k % kTileK == 0) fixed = 4.4, step = 1.19;
+  } else if (bm == 128) {
+    fixed = native_scales ? 6.5 : 11.5;
+    step = table_step(t128x256, sizeof(t128x256) / sizeof(t128x256[0]), wgs);
+  } else {
+    fixed = native_scales ? 9.5 : 14.0;
+    step = table_step(t256, sizeof(t256) / sizeof(t256[0]), wgs);
+  }
+  const double reduce = s > 1 ? (native_scales ? 3.5 : 2.0) + 0.4 * s + 1.3e-6 * (double)s * (double)m * (double)n : 0.0;
+  return fixed + (double)per * step + reduce;
+}
+
+static double mid_cost_us(int64_t m, int64_t n, int64_t k) {
+  const double rounds = (double)((n + 127) / 128) / (double)device_cus();
+  return 4.5 + (double)(k / kTileK) * (0.27 + 0.0025 * (double)(m < 64 ? 64 : m)) * (rounds < 1.0 ? 1.0 : rounds) +
+         (double)n / 14336.0;
+}
+
+// Where the estimates hold: whole K tiles, at most two rounds of 256x256 tiles, the measured range of N.
+static bool tile_model_applies(int64_t m, int64_t n, int64_t k) {
+  return m > 64 && n >= 2048 && n <= 16384 && k >= 3584 && k % kTileK == 0 && ((m + 255) / 256) * ((n + 255) / 256) <= 512;
+}
+
+// The cheapest tile shape and split by the estimates (`only`: 0, or the one variant to find the split for).
+static TileChoice best_tile_choice(int64_t m, int64_t n, int64_t k, bool native_scales, int only) {
+  static const int variants[] = {WAVE_MXFP4_VARIANT_T128x128_W2x2, WAVE_MXFP4_VARIANT_T128x256_W2x2,
+                                 WAVE_MXFP4_VARIANT_T256x256_W4x2};
+  TileChoice best = {only ? only : WAVE_MXFP4_VARIANT_T128x128_W2x2, 1, 1e30};
+  for (int v : variants) {
+    if (only && !(v == only || (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && only == WAVE_MXFP4_VARIANT_T256x256_W2x2))) continue;
+    int bm, bn;
+    tile_variant_shape(v, &bm, &bn);
+    const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+    for (int s = 1; s <= 8; ++s) {
+      if (s > 1 && tiles * s > 640) break;  // (beyond what was measured with a split, and never close)
+      const double us = tile_cost_us(v, s, m, n, k, native_scales);
+      if (us >= 0.0 && us < best.us) best = {only ? only : v, s, us};
+    }
+  }
+  return best;
+}
+
+// The tile shape for a dense problem: by the estimates where they hold, by the borders of pick_tile_variant beyond.
+int pick_tile_variant_k(int64_t m, int64_t n, int64_t k, bool native_scales) {
+  if (tile_model_applies(m, n, k)) return best_tile_choice(m, n, k, native_scales, 0).variant;
+  return pick_tile_variant_k(m, n, k, native_scales);
+}
+
 constexpr int64_t kGroupedMidMaxAvgRows = 160;  // (one pass of the 192-row block over every expert, as good as always)
 // Whether the mid-M kernel is the faster home of a grouped problem (one workgroup per expert and 128-column strip,
 // every expert's B streamed once per block of rows).  Up to 160 rows per expert on average it was, on every shape
@@ -167,7 +265,7 @@ bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
   return m >= 1 && m <= mid_max_m() && k % kTileK == 0 && k >= 4 * kTileK && n % 4 == 0;
 }
 
-int auto_split(int64_t m, int64_t n, int64_t k, int variant);
+int auto_split(int64_t m, int64_t n, int64_t k, int variant, bool native_scales = false);
 
 // Whether the streaming kernel would run this K in its counted-wait mode: the library's split leaves every
 // workgroup the same number of whole K tiles, and one, two or four waves share them evenly, at most eight each
@@ -205,6 +303,14 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     //     43.0 -> 44.5)
     //   M <= 16: the same range of N; up to 192 columns per CU only at K <= 4096 (16 x 28672 x 4096: 13.6 -> 13.0;
     //     a tie or 2 % lost at K = 8192: 16 x 40960 29.8 -> 30.3), beyond at any K (16 x 57344 x 8192: 41.4 -> 38.3)
+    // More than 64 rows, N up to 16384, at most two rounds of 256x256 tiles: by the estimates above, the mid-M
+    // kernel among the candidates up to 256 rows (the borders below were measured at K = 2048 .. 8192 and stay for
+    // what lies outside: wider B, fewer rows).
+    if (tile_model_applies(m, n, k)) {
+      const TileChoice t = best_tile_choice(m, n, k, native_scales, 0);
+      if (n >= 3584 && mid_shape_ok(m, n, k) && mid_cost_us(m, n, k) < t.us) return WAVE_MXFP4_VARIANT_MID_M;
+      return t.variant;
+    }
     if (mid_shape_ok(m, n, k)) {
       const int64_t cus = device_cus();
       const bool mid = m > 192  ? n >= 20480 && n <= 128 * cus
@@ -237,7 +343,7 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
              ((k_whole || m <= 16) && m <= 64 && second_round && 4 * strips <= 5 * cus)))
           return WAVE_MXFP4_VARIANT_SKINNY;
         if (k <= 4096 && ((m >= 48 && m <= 128 && second_round && !b_preshuffled) || (m > 128 && m <= 192 && strips <= 128)))
-          return pick_tile_variant(m, n, true);
+          return pick_tile_variant_k(m, n, k, true);
       }
       if (mid) return WAVE_MXFP4_VARIANT_MID_M;
     }
@@ -246,7 +352,7 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     // more CUs to work (us, streaming -> tiles; 64 x 1024 x 8192: 20.8 -> 12.2, 48 x 4096 x 8192: 17.9 -> 13.0,
     // 40 x 2048 x 14336: 19.7 -> 18.1, 64 x 3072 x 14336: 25.1 -> 19.8; at N = 4096, K = 14336 the streaming kernel
     // leads again, 16.1 against 19.5, and at K <= 4096 the two are within a microsecond)
-    if (m > 32 && m <= skinny_max_m() && k > 4096 && n <= (k <= 8192 ? 4096 : 3072)) return pick_tile_variant(m, n, native_scales);
+    if (m > 32 && m <= skinny_max_m() && k > 4096 && n <= (k <= 8192 ? 4096 : 3072)) return pick_tile_variant_k(m, n, k, native_scales);
     // A K that the streaming kernel cannot deal evenly over its waves (see stream_runs_counted): the mid-M kernel
     // against a wide B, the 128x128 tiles with the library's split against a narrow one (us, streaming -> taken:
     // 16 x 28672 x 12032 69.1 -> 30.9, 1 x 12288 x 9216 22.2 -> 16.7, 16 x 28672 x 6400 35.6 -> 19.2;
@@ -254,10 +360,10 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     if (m <= skinny_max_m() && k % kTileK == 0 && !stream_runs_counted(n, k)) {
       if (n >= 8192 && mid_shape_ok(m, n, k)) return WAVE_MXFP4_VARIANT_MID_M;
       // (up to 32 K tiles one workgroup still streams a narrow B faster than the tiles: 16 x 4096 x 6400 9.1 against 11.7)
-      if (k > 8192) return pick_tile_variant(m, n, native_scales);
+      if (k > 8192) return pick_tile_variant_k(m, n, k, native_scales);
     }
     if (m <= skinny_max_m()) return WAVE_MXFP4_VARIANT_SKINNY;
-    v = pick_tile_variant(m, n, native_scales);
+    v = pick_tile_variant_k(m, n, k, native_scales);
   }
   return v;
 }
@@ -287,7 +393,7 @@ bool needs_generic_k(const GemmParams &p) {
 
 // Split the library takes by itself for a tile kernel: only when the tile
 // grid leaves most of the 256 CUs idle and K is long.
-int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
+int auto_split(int64_t m, int64_t n, int64_t k, int variant, bool native_scales) {
   if (variant == WAVE_MXFP4_VARIANT_SKINNY) {
     // split K so that each workgroup's range fits the streaming kernel's resident A
     const int64_t k_tiles = (k + kTileK - 1) / kTileK, cap = stream_max_k_tiles();
@@ -301,6 +407,12 @@ int auto_split(int64_t m, int64_t n, int64_t k, int variant) {
   if (bm == 0 || variant == WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT) return 1;  // (that kernel takes whole K ranges)
   const int64_t tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
   const int64_t k_tiles = (k + kTileK - 1) / kTileK;  // a partial last K tile belongs to the last split
+  // (up to one workgroup per CU without a split: the parts by the estimates; the asymmetric 256x256 kernels of
+  // variant 1 share the 8-wave kernel's tables)
+  if (tile_model_applies(m, n, k) && tiles <= 256 &&
+      (variant == WAVE_MXFP4_VARIANT_T128x128_W2x2 || variant == WAVE_MXFP4_VARIANT_T128x256_W2x2 ||
+       variant == WAVE_MXFP4_VARIANT_T256x256_W4x2 || variant == WAVE_MXFP4_VARIANT_T256x256_W2x2))
+    return best_tile_choice(m, n, k, native_scales, variant).split;
   if (tiles > 128 || k_tiles < 8) return 1;
   if (bm == 128 && bn == 128) {
     // Estimate in us, fixed launch time left out: a workgroup's K tiles at the measured 0.52 us each while every
@@ -392,11 +504,11 @@ static size_t scale_buffer_bytes(int64_t rows, int64_t k) {
 }
 static size_t round_up_256(size_t v) { return (v + 255) / 256 * 256; }
 
-static size_t workspace_bytes_of(int64_t m, int64_t n, int64_t k, int split_k, int v) {
+static size_t workspace_bytes_of(int64_t m, int64_t n, int64_t k, int split_k, int v, bool native_scales) {
   size_t bytes = round_up_256((size_t)m * (size_t)(k / 32));  // per-row A scales spread out to [M, K/32]
   if (v == WAVE_MXFP4_VARIANT_NAIVE) return bytes;
   int splits = split_k;
-  if (splits == 0) splits = auto_split(m, n, k, v);
+  if (splits == 0) splits = auto_split(m, n, k, v, native_scales);
   if (splits > 1) bytes += round_up_256((size_t)splits * (size_t)m * (size_t)n * sizeof(float));
   if (wants_mfma32_scales(v)) bytes += round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
   if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && n % 256 == 0 && splits <= 1) {
@@ -416,8 +528,8 @@ static size_t workspace_bytes_of(int64_t m, int64_t n, int64_t k, int split_k, i
 size_t wave_mxfp4_workspace_bytes(int64_t m, int64_t n, int64_t k, int split_k, int variant) {
   if (m <= 0 || n <= 0 || k <= 0 || split_k < 0 || bad_enum(variant, WAVE_MXFP4_VARIANT_COUNT_)) return 0;
   // the library's own choice of kernel depends on the scale layouts of the call: the larger of the two
-  const size_t plain = workspace_bytes_of(m, n, k, split_k, pick_variant(m, n, k, variant, false, false));
-  const size_t native = workspace_bytes_of(m, n, k, split_k, pick_variant(m, n, k, variant, true, false));
+  const size_t plain = workspace_bytes_of(m, n, k, split_k, pick_variant(m, n, k, variant, false, false), false);
+  const size_t native = workspace_bytes_of(m, n, k, split_k, pick_variant(m, n, k, variant, true, false), true);
   return plain > native ? plain : native;
 }
 
@@ -436,7 +548,7 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   const bool native_scales = a_scale_layout == WAVE_MXFP4_SCALE_MFMA32 && b_scale_layout == WAVE_MXFP4_SCALE_MFMA32;
   int v = pick_variant(m, n, k, variant, native_scales, b_layout == WAVE_MXFP4_B_PRESHUFFLE);
   if (variant == WAVE_MXFP4_VARIANT_AUTO && v == WAVE_MXFP4_VARIANT_MID_M && split_k > 1)  // (it takes whole K ranges)
-    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n, native_scales);
+    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant_k(m, n, k, native_scales);
   if (v == WAVE_MXFP4_VARIANT_SKINNY && m > skinny_max_m()) return WAVE_MXFP4_ERR_UNSUPPORTED;
   // the fallback of the library's own choice of the B-direct mid-M kernel, should the scales not reach MFMA32 order
   const int v_plain = v;
@@ -492,9 +604,17 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
       splits = split_k;
       p.tiles_per_split = tps;
     } else if (split_k == 0) {
-      splits = auto_split(m, n, k, v);
-      const size_t need = (size_t)splits * m * n * sizeof(float);
-      if (splits > 1 && (!workspace || workspace_bytes < need)) splits = 1;  // no scratch: no split
+      splits = auto_split(m, n, k, v, native_scales);
+      // Scratch too small for the parts (and the re-laid scales behind them): fewer parts, down to none.
+      const size_t scale_room = wants_mfma32_scales(v) && !native_scales
+                                    ? round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k))
+                                    : 0;
+      while (splits > 1) {
+        const int64_t per = (p.k_tiles + splits - 1) / splits;
+        const bool valid = p.k_tiles / splits >= 2 && (int64_t)(splits - 1) * per < p.k_tiles;
+        if (valid && workspace && round_up_256((size_t)splits * m * n * sizeof(float)) + scale_room <= workspace_bytes) break;
+        --splits;
+      }
       if (splits > 1) p.tiles_per_split = (p.k_tiles + splits - 1) / splits;
     }
   }
@@ -526,11 +646,13 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   // instruction.  With scratch available, re-lay both operands out first
   // (a few MB, microseconds) and run the native-scale kernel.
   // (Not worth a second launch for a short K range on the 128x128 tiles: there the kernel stages the row-major
-  // scale rows of its tile through LDS itself, 0.1-0.2 us per K tile slower than with re-laid scales: with a split,
-  // whose parts are summed by a launch of their own anyway, the break-even was measured near 13 K tiles; without,
-  // 16 K tiles - all the kernel stages - still win: 1024 x 1024 x 4096 12.3 against 16.3 us.)
-  const bool small_short = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 && p.tiles_per_split <= (splits > 1 ? 12 : 16) &&
-                           k % kTileK == 0 &&
+  // scale rows of its tile through LDS itself.  With the operands from HBM that wins up to 8 K tiles per workgroup,
+  // split or not (128 x 4096 x 4096 in 4 parts: 15.6 against 19.4 us; 1024 x 1024 x 2048: 11.3 against 13.6), is
+  // level at 12 and loses beyond (16 K tiles: 25.3 against 22.6; 384 x 3584 x 8192 in 3 parts of 11: 34.5 against
+  // 25.6).  Nor beyond one workgroup per CU, where it lost to the re-layout on every shape measured: 1280 x 3584 x
+  // 4096, 280 tiles, 38.5 us.)
+  const bool small_short = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 && p.tiles_per_split <= 8 &&
+                           k % kTileK == 0 && ((m + 127) / 128) * ((n + 127) / 128) * splits <= device_cus() &&
                            p.a_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout == WAVE_MXFP4_SCALE_ROW_MAJOR;
   // Both tensors in e8m0_shuffle order, the reference's preshuffled format (tagged_mxfp4_gemm.py:334-403,485-536):
   // the 8-wave persistent kernels can read it in place (two dwords and a byte permute per lane instead of one
@@ -600,12 +722,12 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
     // (the library's own choice without scratch for the scales, or offsets beyond 32 bits: the kernels that
     // served these shapes before)
     if (variant == WAVE_MXFP4_VARIANT_MID_M) return WAVE_MXFP4_ERR_UNSUPPORTED;
-    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n, native_scales);
+    v = m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant_k(m, n, k, native_scales);
   }
   if (v == WAVE_MXFP4_VARIANT_MID_M_BDIRECT && !midb_gemm_applies(p)) {
     if (variant == WAVE_MXFP4_VARIANT_MID_M_BDIRECT) return WAVE_MXFP4_ERR_UNSUPPORTED;
     v = v_plain == WAVE_MXFP4_VARIANT_MID_M && !mid_gemm_applies(p)
-            ? (m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant(m, n, native_scales))
+            ? (m <= skinny_max_m() ? WAVE_MXFP4_VARIANT_SKINNY : pick_tile_variant_k(m, n, k, native_scales))
             : v_plain;
   }
   const int vv = v;
@@ -698,7 +820,10 @@ int wave_mxfp4_gemm_static(const void *a, const void *a_scale, const void *b, co
                               variant);
   if (rc <= 0) return rc;
   if (split_k < 0) return WAVE_MXFP4_ERR_BAD_SPLIT;
-  const size_t need = call_scratch_bytes(m, n, k, split_k, variant, a_scale_layout, b_scale_layout);
+  // (the library's own split takes fewer parts where the scratch is short: what has to fit is the call without one)
+  size_t need = call_scratch_bytes(m, n, k, split_k, variant, a_scale_layout, b_scale_layout);
+  if (split_k == 0 && need > kStaticScratchBytes)
+    need = call_scratch_bytes(m, n, k, 1, variant, a_scale_layout, b_scale_layout);
   if (need > kStaticScratchBytes) {
     snprintf(g_hip_error, sizeof(g_hip_error),
              "wave_mxfp4_gemm_static: %lld x %lld x %lld with split_k %d needs %zu bytes of scratch, the static "

@@ -456,7 +456,9 @@ hipError_t launch_splitk_reduce(const float *partial, void *c, int64_t mn, int s
       case 2: WAVE_REDUCE4(2); break;
       case 3: WAVE_REDUCE4(3); break;
       case 4: WAVE_REDUCE4(4); break;
+      case 5: WAVE_REDUCE4(5); break;
       case 6: WAVE_REDUCE4(6); break;
+      case 7: WAVE_REDUCE4(7); break;
       case 8: WAVE_REDUCE4(8); break;
       default: WAVE_REDUCE4(0); break;
     }

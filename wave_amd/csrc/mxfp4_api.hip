@@ -112,7 +112,8 @@ int device_cus() {
 //   8 K tiles of row-major scales stages them itself: 4.4, and 1.19 per K tile);
 //   a split's reduction: a launch (2, or 3.5 where no re-layout launch hides it), 0.4 per part for its fill, and 1.3
 //   per million f32 partials;
-//   the mid-M kernel: 4.5 + K tiles x (0.27 + 0.0025 M) per round of 128-column strips, + N / 14336.
+//   the mid-M kernel: 4.5 + K tiles x (0.27 + 0.0025 M) per round of 128-column strips, + N / 14336 (0.335 per K
+//   tile up to 32 rows, rising to 0.415 at 64).
 // Fitted to 768 shapes (M = 96..4096, N = 2048..14336, K = 4096..14336, both scale layouts, every tile shape with 1-8
 // parts by name): the choice by these estimates is within 5 % of the best measured kernel on 95 % of them and
 // within 10 % on 98 % (the borders it replaces: 80 % and 87 %).
@@ -165,8 +166,9 @@ static double tile_cost_us(int v, int s, int64_t m, int64_t n, int64_t k, bool n
 
 static double mid_cost_us(int64_t m, int64_t n, int64_t k) {
   const double rounds = (double)((n + 127) / 128) / (double)device_cus();
-  return 4.5 + (double)(k / kTileK) * (0.27 + 0.0025 * (double)(m < 64 ? 64 : m)) * (rounds < 1.0 ? 1.0 : rounds) +
-         (double)n / 14336.0;
+  // (up to 64 rows on its 32- and 64-row blocks: 0.335 per K tile up to 32 rows, 0.415 at 64)
+  const double step = m > 64 ? 0.27 + 0.0025 * (double)m : 0.335 + 0.0025 * (double)(m > 32 ? m - 32 : 0);
+  return 4.5 + (double)(k / kTileK) * step * (rounds < 1.0 ? 1.0 : rounds) + (double)n / 14336.0;
 }
 
 // Where the estimates hold: whole K tiles, at most two rounds of 256x256 tiles, the measured range of N.
@@ -297,7 +299,9 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     //     still does, 15.0 -> 20.7, and so does 256 x 40960, 71.5 -> 88.0: two rounds of 256-row blocks against 160
     //     tiles of 256 x 256)
     //   32 < M <= 64 against the streaming kernel: from N = 12288 on (48 x 28672 x 8192: 28.0 -> 22.5), and from
-    //     N = 4096 on at K <= 4096 (64 x 8192 x 4096: 14.5 -> 10.7; 48 x 8192 x 8192 loses, 14.4 -> 17.3)
+    //     N = 4096 on at K <= 4096 (64 x 8192 x 4096: 14.5 -> 10.7; 48 x 8192 x 8192 loses, 14.4 -> 17.3); with
+    //     row-major scales and operand sets that do not fit the memory-side cache also from N = 6144 on up to
+    //     K = 8192 (64 x 6144 x 8192: 25.6 -> 17.3, 64 x 6144 x 6400: 21.3 -> 14.4, 64 x 10240 x 8192: 19.9 -> 17.6)
     //   16 < M <= 32: N from 12288 up to 320 columns per CU (32 x 28672 x 8192: 24.8 -> 22.2; past one round of
     //     128-column strips two workgroups share a CU, 32 x 57344 x 8192: 44.6 -> 38.6; 32 x 114688 x 4096 loses,
     //     43.0 -> 44.5)
@@ -315,7 +319,7 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
       const int64_t cus = device_cus();
       const bool mid = m > 192  ? n >= 20480 && n <= 128 * cus
                        : m > 64 ? n >= 12288 || (k <= 4096 && n >= 8192 && m > 96)
-                       : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096)
+                       : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096) || (!native_scales && k <= 8192 && n >= 6144)
                        : m > 16 ? n >= 12288 && n <= 320 * cus
                                 : n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus);
       // Both scale tensors already in MFMA32 order (static weights, activations from the quantiser): no kernel
@@ -358,7 +362,23 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     // 16 x 28672 x 12032 69.1 -> 30.9, 1 x 12288 x 9216 22.2 -> 16.7, 16 x 28672 x 6400 35.6 -> 19.2;
     // 16 x 4096 x 14080 30.0 -> 16.2, 64 x 4096 x 12032 28.3 -> 15.7)
     if (m <= skinny_max_m() && k % kTileK == 0 && !stream_runs_counted(n, k)) {
-      if (n >= 8192 && mid_shape_ok(m, n, k)) return WAVE_MXFP4_VARIANT_MID_M;
+      // (A count of K tiles beyond the streaming kernel's 32 that the library cannot split evenly - 43 is prime -
+      // goes to the direct kernel over the whole K, which is ahead of both up to 8 rows against N <= 8192 and up to
+      // 16 rows against N <= 4096, weights from HBM: 1 x 4096 x 11008 with scales in MFMA32 order 11.8 us against
+      // 16.9 on the tiles, 1 x 8192: 15.3 against 20.2 on the mid-M kernel, 16 x 4096: 13.4 against 17.2; row-major
+      // scales 1 x 6144: 17.8 against 23.3; 16 x 10240 loses, 26.4 against 19.6 on the mid-M kernel)
+      const bool whole_k_kernel = k / kTileK > stream_max_k_tiles() && auto_split(1, n, k, WAVE_MXFP4_VARIANT_SKINNY) == 1;
+      if (whole_k_kernel && (m <= 8 ? n <= 8192 : m <= 16 && n <= 4096)) return WAVE_MXFP4_VARIANT_SKINNY;
+      // (between N = 6144 and 12288 by the estimates: with row-major scales the mid-M kernel, 32 x 6144 x 11008 24.6
+      // on the tiles against 19.3; with scales in MFMA32 order the tiles, which then need no launch in front,
+      // 64 x 8192 x 14080 22.9 against 30.2)
+      // (and up to 16 rows with scales in MFMA32 order a K of at most 32 tiles stays with the streaming kernel below
+      // N = 12288: one part, 1 x 8192 x 6400 9.9 us against 13.1 on the mid-M kernel; with row-major scales the
+      // mid-M kernel leads, 1 x 10240 x 6400 14.5 against 17.8)
+      const bool one_part_few_rows = native_scales && k / kTileK <= stream_max_k_tiles() && m <= 16 && n < 12288;
+      if (mid_shape_ok(m, n, k) && !one_part_few_rows &&
+          (n >= 12288 || (n >= 6144 && mid_cost_us(m, n, k) < best_tile_choice(m, n, k, native_scales, 0).us)))
+        return WAVE_MXFP4_VARIANT_MID_M;
       // (up to 32 K tiles one workgroup still streams a narrow B faster than the tiles: 16 x 4096 x 6400 9.1 against 11.7)
       if (k > 8192) return pick_tile_variant_k(m, n, k, native_scales);
     }

@@ -137,12 +137,14 @@ def test_narrow_b_long_k_against_oracle(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 8192, 9216), (16, 8448, 11008), (16, 4096, 14080), (64, 2048, 12032),
-                                   (8, 12288, 6400), (16, 4096, 6400), (5, 8192, 13824), (33, 8192, 14080)])
+                                   (8, 12288, 6400), (16, 4096, 6400), (5, 8192, 13824), (33, 8192, 14080),
+                                   (1, 4096, 11008), (8, 8192, 11008), (32, 6144, 11008), (64, 6144, 8192)])
 def test_decode_rows_with_uneven_k_tiles_against_oracle(m, n, k):
     """Up to 64 rows with a count of K tiles that the streaming kernel cannot deal evenly over its waves (25, 36, 43,
     47, 54 and 55 tiles: the K of Llama-2 down projections among them): the library's own choice is the mid-M
-    kernel against a wide B and the 128x128 tiles with a split along K against a narrow one.  Every row against the
-    exact oracle, both output types, with and without scratch."""
+    kernel against a wide B and the 128x128 tiles with a split along K against a narrow one (the last four: the
+    direct whole-K kernel for a prime count of K tiles at few rows, and the mid-M kernel from N = 6144 on).  Every
+    row against the exact oracle, both output types, with and without scratch."""
     x, xs, w_t, ws = orc.make_inputs(m, n, k, seed=m + k, scale_lo=120, scale_hi=134)
     ref = c_oracle.scaled_gemm_exact(x, w_t, xs, ws)
     for dt in (torch.float32, torch.bfloat16):

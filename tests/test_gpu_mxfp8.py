@@ -247,3 +247,30 @@ def test_mxfp8_argument_errors():
         wave_amd.mxfp8_gemm(torch.zeros(4, 96, dtype=torch.uint8, device=DEV), torch.zeros(4, 3, dtype=torch.uint8, device=DEV),
                             torch.zeros(4, 96, dtype=torch.uint8, device=DEV), torch.zeros(4, 3, dtype=torch.uint8, device=DEV),
                             torch.zeros(4, 4, device=DEV))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fmt", [o8.E5M2, (o8.E4M3, o8.E5M2), (o8.E5M2, o8.E2M1)], ids=["e5m2", "e4m3_x_e5m2", "e5m2_x_e2m1"])
+@pytest.mark.parametrize("m,n,k", [(128, 256, 4096), (300, 500, 8192), (1024, 1024, 6400), (64, 1536, 11008)])
+def test_mxfp8_few_tiles_long_k_split_by_the_library(m, n, k, fmt, out_dtype):
+    """At most 128 tiles of 128x128 and a long K: with scratch the library cuts K into parts (f32 partial tiles in
+    the scratch, one more launch to sum them; uneven parts for 50 and 86 K tiles), without scratch one workgroup
+    walks the whole K.  Both against the oracle, and close to each other."""
+    x, xs, w_t, ws = o8.make_inputs_mxfp8(m, n, k, seed=m + n + k, fmt=fmt, scale_lo=120, scale_hi=134)
+    ref = o8.scaled_gemm_mxfp8(x, w_t, xs, ws, fmt)
+    gx, gxs, gw, gws = to_gpu(x, xs, w_t, ws)
+    lib = _lib.load()
+    assert lib.wave_mxfp8_workspace_bytes(m, n, k) > 2 * m * n * 4      # room for at least two parts
+    out = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    wave_amd.mxfp8_gemm(gx, gxs, gw, gws, out, elem_format=fmt)
+    whole = torch.full_like(out, float("nan"))
+    wave_amd.mxfp8_gemm(gx, gxs, gw, gws, whole, elem_format=fmt, workspace=False)
+    torch.cuda.synchronize()
+    for got, what in ((out, "split"), (whole, "whole K")):
+        c = got.float().cpu().numpy()
+        if out_dtype == torch.float32:
+            assert_f32_close(c, ref, f"{what} {m}x{n}x{k}")
+        else:
+            # one bf16 ulp on top of what the f32 sums are allowed (1e-4 * max|Cref| with scales spread this wide)
+            tol = 2.0 ** -7 * np.abs(ref) + 1e-4 * np.abs(ref).max()
+            assert (np.abs(c - ref) <= tol).all(), f"{what} {m}x{n}x{k}: beyond one bf16 ulp + 1e-4 * max"

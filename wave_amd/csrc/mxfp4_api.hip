@@ -859,9 +859,28 @@ int wave_mxfp4_gemm_static(const void *a, const void *a_scale, const void *b, co
                          split_k, scratch, kStaticScratchBytes, variant, hip_stream);
 }
 
+// Parts along K the library takes for an MXFP8 problem on the 128x128 tiles: few tiles and a long K leave most CUs
+// idle, as for MXFP4.  Priced like there (a workgroup's 128-byte K tile 0.7 us while every CU holds at most one
+// workgroup, the sum over the parts 3.5 + 0.4 per part + 1.3 per million f32 partials); parts of at least 8 K tiles.
+static int mxfp8_auto_split(int64_t m, int64_t n, int64_t k) {
+  const int64_t tiles = ((m + 127) / 128) * ((n + 127) / 128), k_tiles = k / 128;
+  if (k % 256 != 0 || tiles > 128 || k_tiles < 16) return 1;
+  int best = 1;
+  double best_us = 0.7 * (double)k_tiles;
+  for (int s = 2; s <= 8; ++s) {
+    const int64_t per = (k_tiles + s - 1) / s;
+    if (per < 8 || (s - 1) * per >= k_tiles || tiles * s > device_cus()) continue;
+    const double us = 0.7 * (double)per + 3.5 + 0.4 * s + 1.3e-6 * (double)s * (double)m * (double)n;
+    if (us < 0.9 * best_us) best = s, best_us = us;
+  }
+  return best;
+}
+
 size_t wave_mxfp8_workspace_bytes(int64_t m, int64_t n, int64_t k) {
   if (m <= 0 || n <= 0 || k <= 0 || k % 256 != 0) return 0;
-  return round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k));
+  const int s = mxfp8_auto_split(m, n, k);
+  return round_up_256(scale_buffer_bytes(m, k)) + round_up_256(scale_buffer_bytes(n, k)) +
+         (s > 1 ? round_up_256((size_t)s * (size_t)m * (size_t)n * sizeof(float)) : 0);
 }
 
 int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const void *b_scale, void *c,
@@ -916,12 +935,23 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   p.tiles_n = (int)((n + bn - 1) / bn);
   // with scratch, re-lay both scale tensors out in MFMA32 order first (one launch), as the MXFP4 path does
   const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k));
-  if (workspace && k % 256 == 0 && workspace_bytes >= wave_mxfp8_workspace_bytes(m, n, k) &&
+  const size_t scale_bytes = a_bytes + round_up_256(scale_buffer_bytes(n, k));
+  if (workspace && k % 256 == 0 && workspace_bytes >= scale_bytes &&
       launch_scale_pair_to_mfma32(p.a_scale, (uint8_t *)workspace, m, p.b_scale, (uint8_t *)workspace + a_bytes, n,
                                   p.ks, stream) == hipSuccess) {
     p.a_scale = (const uint8_t *)workspace;
     p.b_scale = (const uint8_t *)workspace + a_bytes;
     p.a_scale_layout = p.b_scale_layout = WAVE_MXFP4_SCALE_MFMA32;
+    // the library's own split along K (128x128 tiles only): f32 parts behind the scales, summed by one more launch
+    const int s = v == WAVE_MXFP4_VARIANT_T128x128_W2x2 ? mxfp8_auto_split(m, n, k) : 1;
+    if (s > 1 && workspace_bytes >= scale_bytes + round_up_256((size_t)s * m * n * sizeof(float))) {
+      p.splits = s;
+      p.tiles_per_split = (p.k_tiles + s - 1) / s;
+      p.partial = (float *)((uint8_t *)workspace + scale_bytes);
+      const hipError_t e = launch_tile_gemm_fp8(p, v, a_format, b_format, stream);
+      if (e != hipSuccess) return record_hip(e);
+      return record_hip(launch_splitk_reduce(p.partial, c, m * n, s, p.out_bf16, stream));
+    }
   }
   // large dense problems on the 8-wave tiles with re-laid scales: the persistent kernel
   if (v == WAVE_MXFP4_VARIANT_T256x256_W4x2 && persist_gemm_fp8_applies(p, device_cus()))
@@ -979,7 +1009,7 @@ int wave_mxfp8_gemm_b_preshuffled(const void *a, const void *a_scale, const void
   if (!a_native || !b_native) {
     // the row-major ones into MFMA32 order first (one launch)
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k));
-    if (!workspace || workspace_bytes < wave_mxfp8_workspace_bytes(m, n, k)) return WAVE_MXFP4_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < a_bytes + round_up_256(scale_buffer_bytes(n, k))) return WAVE_MXFP4_ERR_UNSUPPORTED;
     const hipError_t e = launch_scale_pair_to_mfma32(p.a_scale, (uint8_t *)workspace, a_native ? 0 : m, p.b_scale,
                                                      (uint8_t *)workspace + a_bytes, b_native ? 0 : n, p.ks, stream);
     if (e != hipSuccess) return e == hipErrorInvalidValue ? WAVE_MXFP4_ERR_UNSUPPORTED : record_hip(e);

@@ -647,7 +647,7 @@ def main():
                     "time-based settle load every leg runs anyway)")
     ap.add_argument("--workload", default="cfg2",
                     choices=sorted(WORKLOADS) + ["cfg4", "quant_bf16", "mxfp8", "moe_glue", "ref_shapes", "mfma_ceiling",
-                                                 "decode_sweep", "moe_serving", "moe_layer"],
+                                                 "decode_sweep", "moe_serving", "moe_layer", "tile_choice"],
                     help="cfg*: the GEMM configurations; quant_bf16: the activation quantiser alone on the "
                          "8192 x 8192 bf16 activation of cfg2; mxfp8: the MXFP8 (e5m2) GEMM at 8192^3, f32 out; "
                          "cfg4: the grouped (MoE) GEMM, 8 experts, 8192 rows, N=14336, K=4096; moe_glue: the steps around "
@@ -657,7 +657,9 @@ def main():
                          "M = 1 .. 256 against wide weights from HBM, every kernel that serves the shape beside the "
                          "library's own choice; moe_serving: the grouped GEMM at serving batches, experts x rows per "
                          "expert, the mid-M kernel beside the tile kernels; moe_layer: one mixture-of-experts MLP end to end "
-                         "(alignment, gathered quantiser, grouped GEMM, gated quantiser, grouped GEMM), step by step and whole")
+                         "(alignment, gathered quantiser, grouped GEMM, gated quantiser, grouped GEMM), step by step and whole; "
+                         "tile_choice: the library's own choice against every tile shape, split and the mid-M kernel by name "
+                         "on random mid-size shapes with the weights from HBM (--steps: number of shapes, default 60)")
     ap.add_argument("--variant", type=int, default=0, help="kernel variant of include/wave_mxfp4.h (0 = auto)")
     ap.add_argument("--resident-scales", action="store_true",
                     help="decode_sweep: both scale tensors handed over in MFMA32 order (no re-layout launch for any kernel)")
@@ -757,6 +759,74 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                          "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": read_traffic("quant_bf16"),
                          "kernel": "quantize_kernel", "launch_us": round(qper * 1e6, 2)}})))
+        return
+
+    if args.workload == "tile_choice":
+        # The library's own choice of tile shape, split along K and kernel against every candidate asked for by
+        # name, on shapes drawn at random from the range where it chooses by duration estimates (more than 64 rows,
+        # N = 2048..16384, K >= 3584 in whole K tiles, at most two rounds of 256x256 tiles).  Operand sets are
+        # rotated past the 256 MB memory-side cache, so B comes from HBM as a model's weights do; bf16 out; either
+        # scale layout.  Every timing is the best of two; the library's choice is timed last.
+        import math
+        import numpy as np
+        from wave_amd import _lib as L
+
+        SETTLE["ms"] = 5.0
+        rng = np.random.default_rng(5)
+        names = [("mid", L.VARIANT_MID_M), ("t128", L.VARIANT_T128x128_W2x2), ("t128x256", L.VARIANT_T128x256_W2x2),
+                 ("t256w8", L.VARIANT_T256x256_W4x2)]
+        rows = []
+        count = 60 if args.steps == 300 else args.steps
+        while len(rows) < count:
+            m = int(2 ** rng.uniform(6.1, 11.6))
+            n = 128 * int(rng.integers(16, 121))
+            k = 256 * int(rng.integers(14, 65))
+            native = bool(rng.integers(0, 2))
+            if ((m + 255) // 256) * ((n + 255) // 256) > 512:
+                continue
+            copies = max(2, min(80, math.ceil(400e6 / (n * k / 2))))
+            sets = []
+            for _ in range(copies):
+                x = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=dev)
+                xs = torch.randint(120, 135, (m, k // 32), dtype=torch.uint8, device=dev)
+                w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev)
+                ws = torch.randint(120, 135, (n, k // 32), dtype=torch.uint8, device=dev)
+                if native:
+                    xs = wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
+                    ws = wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
+                sets.append((x, xs, w, ws))
+            kw = dict(a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32) if native else {}
+            out = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+            iters = max(16, copies)
+
+            def best_of_two(**opts):
+                return min(time_gemm(torch, wave_amd, sets, out, iters, 4, **opts, **kw)[1] for _ in range(2)) * 1e6
+
+            by_name = {}
+            for name, v in names:
+                for split in (0, 1, 2, 4, 8):
+                    if name == "mid" and (split or m > 256):
+                        continue
+                    try:
+                        by_name[f"{name}/{split}"] = round(best_of_two(variant=v, split_k=split), 1)
+                    except (RuntimeError, ValueError):
+                        pass   # (a split this K does not divide into, or a kernel that does not take the shape)
+            auto = round(best_of_two(variant=L.VARIANT_AUTO, split_k=0), 1)
+            best = min(by_name, key=by_name.get)
+            rows.append({"m": m, "n": n, "k": k, "mfma32_scales": native, "auto_us": auto, "best": best,
+                         "best_us": by_name[best], "ratio": round(auto / by_name[best], 3)})
+            del sets, out
+        ratios = [r["ratio"] for r in rows]
+        print(json.dumps(dict(common, **{
+            "metric": "library's choice / best kernel by name, geometric mean over random mid-size shapes",
+            "value": round(math.exp(sum(math.log(r) for r in ratios) / len(ratios)), 4), "unit": "ratio",
+            "higher_is_better": False,
+            "ms_per_step": round(sum(r["auto_us"] for r in rows) * 1e-3, 3),
+            "dtype": "mxfp4 (e2m1 x e8m0) in, f32 accumulate, bf16 out",
+            "data": "synthetic (uniform nibbles, scales 120..134), operand sets rotated past the memory-side cache",
+            "config": {"workload": f"tile_choice: {len(rows)} shapes, M 68..3100, N 2048..15360, K 3584..16384, seed 5"},
+            "within_5_percent": sum(r <= 1.05 for r in ratios), "within_10_percent": sum(r <= 1.10 for r in ratios),
+            "worst": max(ratios), "shapes": rows})))
         return
 
     if args.workload == "decode_sweep":

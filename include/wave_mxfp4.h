@@ -97,8 +97,10 @@ typedef enum {
    * applies and the problem has more tiles than the GPU has CUs. */
   WAVE_MXFP4_VARIANT_T256x256_W1x4_BDIRECT = 7,
   /* M <= 256 against a wide B from HBM: one workgroup per strip of 64 to 128 columns, B through deep
-   * wave-private LDS rings, A fed by a producer wave.  Needs K % 256 == 0, K >= 1024, N % 4 == 0, no split, and
+   * wave-private LDS rings, A fed by a producer wave.  Needs K > 768, N % 4 == 0, no split, and
    * each scale tensor row-major, MFMA32 or in e8m0_shuffle order (all three read as they are, no pass per call);
+   * a K that is not a multiple of 256 with both scale tensors in MFMA32 order, padding groups 0 as
+   * wave_mxfp4_scale_convert and the quantiser write them (row-major ones are re-laid in the workspace first);
    * WAVE_MXFP4_ERR_UNSUPPORTED otherwise.  AUTO takes it for 16 < M <= 256 and a wide N (M <= 16 too at K <= 4096), and for a grouped problem of few rows per expert
    * (see wave_mxfp4_gemm_grouped).  The reference runs such shapes through its generic tile kernel
    * (tests/kernel/wave_gemm_mxfp_test.py:291-339). */

@@ -142,3 +142,26 @@ def test_mid_rejects_what_it_does_not_take():
     x, xs, w, ws = orc.make_inputs(64, 256, 2048, seed=1)
     with pytest.raises((RuntimeError, ValueError)):
         run(x, xs, w, ws, torch.float32, variant=V, split_k=2)          # it takes whole K ranges
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(16, 5760, 2880), (64, 2880, 2880), (1, 4096, 1056), (200, 4100, 2848),
+                                   (256, 640, 1312), (33, 8192, 4000), (130, 1008, 2080)])
+def test_mid_partial_last_k_tile(m, n, k, dt):
+    """K in whole scale groups of 32 but not in whole K tiles of 256 (2880: the hidden size of gpt-oss): the kernel
+    walks ceil(K / 256) K tiles, and what the last one brings in from past the end of K is multiplied with the zero
+    padding of MFMA32-ordered scales (2^-127 each), which vanishes in f32.  By name with the scales handed over in
+    MFMA32 order, with row-major ones re-laid in scratch, with B preshuffled, and the library's own choice; without
+    scratch and row-major scales the kernel is refused by name and the library's choice takes another one.  Every
+    element against the exact oracle, last rows and columns included."""
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=m + k, scale_lo=112, scale_hi=140)
+    ref = c_oracle.scaled_gemm_exact(x, w, xs, ws)
+    assert_close(run(x, xs, w, ws, dt, la=M32, lb=M32, variant=V, split_k=1), ref, dt, f"{m}x{n}x{k} MFMA32 scales")
+    assert_close(run(x, xs, w, ws, dt, variant=V, split_k=1), ref, dt, f"{m}x{n}x{k} row-major scales, scratch")
+    if n % 16 == 0 and k % 64 == 0:
+        assert_close(run(x, xs, w, ws, dt, la=M32, lb=M32, pre=True, variant=V, split_k=1), ref, dt, f"{m}x{n}x{k} preshuffled B")
+    assert_close(run(x, xs, w, ws, dt), ref, dt, f"{m}x{n}x{k} library's choice")
+    assert_close(run(x, xs, w, ws, dt, la=M32, lb=M32), ref, dt, f"{m}x{n}x{k} library's choice, MFMA32 scales")
+    assert_close(run(x, xs, w, ws, dt, workspace=False), ref, dt, f"{m}x{n}x{k} library's choice without scratch")
+    with pytest.raises((RuntimeError, ValueError)):
+        run(x, xs, w, ws, dt, variant=V, split_k=1, workspace=False)

@@ -263,8 +263,10 @@ bool is_tile_variant(int v) {
 constexpr int kGroupedShortRows = 64;
 
 // What the mid-M kernel takes (the part of it that the shape alone decides).
+// (A partial last K tile is taken with both scale tensors in MFMA32 order, whose padding groups hold 0 = 2^-127:
+// what the kernel multiplies past the end of K vanishes in f32.)
 bool mid_shape_ok(int64_t m, int64_t n, int64_t k) {
-  return m >= 1 && m <= mid_max_m() && k % kTileK == 0 && k >= 4 * kTileK && n % 4 == 0;
+  return m >= 1 && m <= mid_max_m() && k % 32 == 0 && k > 3 * kTileK && n % 4 == 0;
 }
 
 int auto_split(int64_t m, int64_t n, int64_t k, int variant, bool native_scales = false);
@@ -315,13 +317,20 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
       if (n >= 3584 && mid_shape_ok(m, n, k) && mid_cost_us(m, n, k) < t.us) return WAVE_MXFP4_VARIANT_MID_M;
       return t.variant;
     }
-    if (mid_shape_ok(m, n, k)) {
+    // (a partial last K tile on the mid-M kernel wants both scale tensors in MFMA32 order: handed over that way, or
+    // re-laid by the one fast launch, which takes K in multiples of 128; the two launches of the general conversion
+    // cost more than the kernel saves, 16 x 5760 x 2880 12.3 -> 16.7 us)
+    if (mid_shape_ok(m, n, k) && (k % kTileK == 0 || native_scales || k % 128 == 0)) {
       const int64_t cus = device_cus();
+      // (a partial last K tile: the streaming kernel does not take it, and the direct kernel that would serve up to
+      // 64 rows loses from N = 4096 on; scales in MFMA32 order, us: 16 x 23040 x 2880 27.5 -> 13.0, 64 x 23040
+      // 32.9 -> 13.8, 64 x 5760 15.9 -> 12.2, and 256 x 23040 on the tiles 33.0 -> 20.4)
+      const bool k_tail = k % kTileK != 0;
       const bool mid = m > 192  ? n >= 20480 && n <= 128 * cus
                        : m > 64 ? n >= 12288 || (k <= 4096 && n >= 8192 && m > 96)
                        : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096) || (!native_scales && k <= 8192 && n >= 6144)
-                       : m > 16 ? n >= 12288 && n <= 320 * cus
-                                : n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus);
+                       : m > 16 ? (n >= 12288 && n <= 320 * cus) || (k_tail && n >= 4096)
+                                : (n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus)) || (k_tail && n >= 4096);
       // Both scale tensors already in MFMA32 order (static weights, activations from the quantiser): no kernel
       // needs a re-layout launch in front, and the mid-M kernel cannot narrow its strips (a wave's strip is a
       // 32-row scale block), which moves some borders.  Measured with the weights from HBM on a grid of M = 16 ..
@@ -437,7 +446,7 @@ int auto_split(int64_t m, int64_t n, int64_t k, int variant, bool native_scales)
   if (bm == 128 && bn == 128) {
     // Estimate in us, fixed launch time left out: a workgroup's K tiles at the measured 0.52 us each while every
     // CU holds at most one workgroup (1.28 us for the two of a CU beyond that), plus, for a split, the launch that
-    // sums the parts and their f32 traffic.  (1024 x 1024: K = 2048 stays whole, K = 8192 and 16384 take 4 parts.)
+    // sums the parts and their f32 traffic.  (1024 x 1024: K = 2048 stays whole, K = 8192 takes 3 parts, K = 16384 takes 4.)
     int best = 1;
     double best_us = 0.52 * (double)k_tiles;
     for (int s = 2; s <= 8; ++s) {
@@ -700,8 +709,10 @@ int wave_mxfp4_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (wants_mfma32_scales(v) && workspace && !small_short && !shuffled_in_place) {
     const size_t a_bytes = round_up_256(scale_buffer_bytes(m, k)), b_bytes = round_up_256(scale_buffer_bytes(n, k));
     const bool mid = v == WAVE_MXFP4_VARIANT_MID_M;
-    const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads(p.a_scale_layout)) ? a_bytes : 0;
-    const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid && mid_reads(p.b_scale_layout)) ? b_bytes : 0;
+    // (the mid-M kernel reads row-major and e8m0_shuffle scales in place, but only with whole K tiles)
+    const bool mid_in_place = mid && k % kTileK == 0;
+    const size_t a_need = p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid_in_place && mid_reads(p.a_scale_layout)) ? a_bytes : 0;
+    const size_t b_need = p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 && !(mid_in_place && mid_reads(p.b_scale_layout)) ? b_bytes : 0;
     if (ws_used + a_need + b_need <= workspace_bytes) {
       uint8_t *ws = (uint8_t *)workspace + ws_used;
       ws_scales_end = ws_used + a_need + b_need;

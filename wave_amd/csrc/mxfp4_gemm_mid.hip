@@ -665,7 +665,14 @@ bool mid_gemm_applies(const GemmParams &p) {
     return l == WAVE_MXFP4_SCALE_ROW_MAJOR || l == WAVE_MXFP4_SCALE_MFMA32 || l == WAVE_MXFP4_SCALE_E8M0_SHUFFLE;
   };
   if (!layout_ok(p.a_scale_layout) || !layout_ok(p.b_scale_layout)) return false;
-  if ((p.k & (kTileK - 1)) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
+  // A partial last K tile: both scale tensors in MFMA32 order.  Their padding groups hold 0 (2^-127 each), so the
+  // products of whatever the last K tile's requests bring in from past the end of K - the start of the next row, or
+  // the zeros the buffer descriptor returns past the last one - vanish in the f32 accumulators; the kernel walks
+  // ceil(K / 256) K tiles and knows nothing of it.
+  if ((p.k & (kTileK - 1)) != 0 &&
+      (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32))
+    return false;
+  if ((p.k & 31) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
   // 32-bit offsets: inside A, inside a wave's 48 rows of B, inside C, inside the scales of A and of a wave's rows
   if ((int64_t)p.m * p.kp >= ((int64_t)1 << 31) || (int64_t)48 * p.kp >= ((int64_t)1 << 31) ||
       (int64_t)p.m * p.n * 4 >= ((int64_t)1 << 31) || (int64_t)8 * p.k_tiles * 256 >= ((int64_t)1 << 31))

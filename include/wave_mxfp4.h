@@ -205,8 +205,9 @@ size_t wave_mxfp4_static_scratch_bytes(void);
  * and a long K - and enough experts x 128-column strips to occupy half the CUs)
  * runs on the mid-M kernel,
  * one workgroup per (expert, strip), with no table and no scale re-layout: the
- * call is then bound by reading every expert's B once.  It needs K % 256 == 0,
- * K >= 1024, N % 4 == 0, A's scales row-major and B's in any of the three orders;
+ * call is then bound by reading every expert's B once.  It needs K > 768,
+ * N % 4 == 0, A's scales row-major or MFMA32 and B's in any of the three orders
+ * (a K that is not a multiple of 256: both in MFMA32 order, padding groups 0);
  * WAVE_MXFP4_VARIANT_MID_M asks for it by name (WAVE_MXFP4_ERR_UNSUPPORTED
  * where it does not apply).  The other variants accepted here are AUTO, NAIVE
  * and the square tile shapes.

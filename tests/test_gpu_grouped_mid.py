@@ -170,3 +170,21 @@ def test_library_choice_beyond_160_rows_per_expert(e, n, k, rows, la):
         check(c[:, cols], ref, dt, f"E={e} {rows}x{n}x{k} library's choice")
         by_name = run(x, xs, w, ws, off, dt, lb=M32, la=la, variant=V)
         assert np.array_equal(c, by_name)
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("e,n,k,rows", [(8, 2880, 2880, 64), (4, 5760, 2880, 100), (6, 640, 1056, 333), (32, 256, 2848, 40)])
+def test_grouped_mid_partial_last_k_tile(e, n, k, rows, dt):
+    """K in whole scale groups but not in whole K tiles (2880: gpt-oss) with both scale tensors in MFMA32 order,
+    whose zero padding cancels what the last K tile reads past the end of K (the next row, the next expert's first
+    row, or nothing): by name and by the library's own choice, row-major and preshuffled expert weights; with
+    row-major scales the kernel is refused by name and the library's choice runs the tile kernels."""
+    x, xs, w, ws, off = inputs(e, n, k, rows, seed=e + rows + k)
+    ref = reference(x, xs, w, ws, off)
+    check(run(x, xs, w, ws, off, dt, lb=M32, la=M32, variant=V), ref, dt, f"E={e} {rows}x{n}x{k} by name")
+    check(run(x, xs, w, ws, off, dt, lb=M32, la=M32), ref, dt, f"E={e} {rows}x{n}x{k} library's choice")
+    if k % 64 == 0:
+        check(run(x, xs, w, ws, off, dt, lb=M32, la=M32, pre=True, variant=V), ref, dt, f"E={e} {rows}x{n}x{k} preshuffled")
+    check(run(x, xs, w, ws, off, dt), ref, dt, f"E={e} {rows}x{n}x{k} row-major scales")
+    with pytest.raises((RuntimeError, ValueError)):
+        run(x, xs, w, ws, off, dt, variant=V)

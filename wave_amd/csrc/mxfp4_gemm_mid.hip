@@ -689,7 +689,11 @@ bool mid_grouped_applies(const GemmParams &p) {
   if (p.b_scale_layout != WAVE_MXFP4_SCALE_ROW_MAJOR && p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32 &&
       p.b_scale_layout != WAVE_MXFP4_SCALE_E8M0_SHUFFLE)
     return false;
-  if ((p.k & (kTileK - 1)) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
+  // (a partial last K tile: both scale tensors in MFMA32 order, as for the dense problem)
+  if ((p.k & (kTileK - 1)) != 0 &&
+      (p.a_scale_layout != WAVE_MXFP4_SCALE_MFMA32 || p.b_scale_layout != WAVE_MXFP4_SCALE_MFMA32))
+    return false;
+  if ((p.k & 31) != 0 || p.k_tiles < 4 || (p.n & 3) != 0) return false;
   if ((int64_t)256 * p.kp >= ((int64_t)1 << 31) || (int64_t)48 * p.kp >= ((int64_t)1 << 31) ||
       (int64_t)256 * p.n * 4 >= ((int64_t)1 << 31) || (int64_t)8 * p.k_tiles * 256 >= ((int64_t)1 << 31))
     return false;

@@ -936,9 +936,21 @@ int wave_mxfp8_gemm(const void *a, const void *a_scale, const void *b, const voi
   if (v == WAVE_MXFP4_VARIANT_AUTO) {
     // (up to 512 tiles of 128x128 are one round of two workgroups per CU, where up to 170 tiles of 256x256 leave
     // CUs idle: 2048 x 4096 x 4096 57.2 -> 38.6 us, 1100 x 7168 x 4096 57.0 -> 39.7; from 576 on the two are level)
-    const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128);
-    v = t128 > 512 && ((m + 255) / 256) * ((n + 255) / 256) >= 128 ? WAVE_MXFP4_VARIANT_T256x256_W4x2  // 8 waves: 498 -> 476 us at 8192^3
-                                                                   : WAVE_MXFP4_VARIANT_T128x128_W2x2;
+    // Beyond that, by rounds over the CUs, fitted to 100 random shapes with the weights from HBM (us per 128-byte K
+    // tile: 1.05 per round of two 128x128 workgroups per CU, 1.565 per round of 256x256 tiles, 8 waves: 498 -> 476 us
+    // at 8192^3): the 256x256 tiles run in whole rounds unless the persistent kernel takes them (N in whole
+    // tiles, more tiles than CUs: a last round filled to a fraction f costs 0.4 + 0.6 f), the small ones fill the
+    // chip evenly (1387 x 12160 x 3584, 288 tiles of 256x256 in two rounds: 105.7 -> 88.5 us; 3103 x 4992 x 1536:
+    // 57.7 -> 38.2; 1532 x 13696 x 6912: 210.7 -> 175.4).
+    const int64_t t128 = ((m + 127) / 128) * ((n + 127) / 128), t256 = ((m + 255) / 256) * ((n + 255) / 256);
+    const int64_t cus = device_cus();
+    v = WAVE_MXFP4_VARIANT_T128x128_W2x2;
+    if (t128 > 2 * cus) {
+      double rounds256 = (double)((t256 + cus - 1) / cus);
+      if (n % 256 == 0 && t256 > cus && t256 % cus != 0) rounds256 = (double)(t256 / cus) + 0.4 + 0.6 * (double)(t256 % cus) / (double)cus;
+      const double kt = (double)(k / 128);
+      if (24.5 + 1.565 * kt * rounds256 < 29.2 + 1.05 * kt * (double)t128 / (double)(2 * cus)) v = WAVE_MXFP4_VARIANT_T256x256_W4x2;
+    }
   }
   int bm, bn;
   tile_variant_shape(v, &bm, &bn);

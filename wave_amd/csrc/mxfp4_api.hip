@@ -159,6 +159,9 @@ static double tile_cost_us(int v, int s, int64_t m, int64_t n, int64_t k, bool n
   } else {
     fixed = native_scales ? 9.5 : 14.0;
     step = table_step(t256, sizeof(t256) / sizeof(t256[0]), wgs);
+    // (beyond one workgroup per CU the table is the persistent kernel's; an N that is not in whole 256-column tiles
+    // runs one tile per workgroup in whole rounds: 3072 x 5504 x 8192, 264 tiles, 111 us = 2 x 1.52 per K tile)
+    if (n % 256 != 0 && wgs > 256) step = 1.55 * (double)(((int64_t)wgs + 255) / 256);
   }
   const double reduce = s > 1 ? (native_scales ? 3.5 : 2.0) + 0.4 * s + 1.3e-6 * (double)s * (double)m * (double)n : 0.0;
   return fixed + (double)per * step + reduce;

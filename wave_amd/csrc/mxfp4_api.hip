@@ -170,7 +170,9 @@ static double tile_cost_us(int v, int s, int64_t m, int64_t n, int64_t k, bool n
 static double mid_cost_us(int64_t m, int64_t n, int64_t k) {
   const double rounds = (double)((n + 127) / 128) / (double)device_cus();
   // (up to 64 rows on its 32- and 64-row blocks: 0.335 per K tile up to 32 rows, 0.415 at 64)
-  const double step = m > 64 ? 0.27 + 0.0025 * (double)m : 0.335 + 0.0025 * (double)(m > 32 ? m - 32 : 0);
+  // (the kernel's row blocks are 32 rows high: 68 rows cost what 96 do)
+  const int64_t mb = (m + 31) / 32 * 32;
+  const double step = mb > 64 ? 0.27 + 0.0025 * (double)mb : mb > 32 ? 0.415 : 0.335;
   return 4.5 + (double)(k / kTileK) * step * (rounds < 1.0 ? 1.0 : rounds) + (double)n / 14336.0;
 }
 

@@ -203,7 +203,7 @@ static TileChoice best_tile_choice(int64_t m, int64_t n, int64_t k, bool native_
 // The tile shape for a dense problem: by the estimates where they hold, by the borders of pick_tile_variant beyond.
 int pick_tile_variant_k(int64_t m, int64_t n, int64_t k, bool native_scales) {
   if (tile_model_applies(m, n, k)) return best_tile_choice(m, n, k, native_scales, 0).variant;
-  return pick_tile_variant_k(m, n, k, native_scales);
+  return pick_tile_variant(m, n, native_scales);
 }
 
 constexpr int64_t kGroupedMidMaxAvgRows = 160;  // (one pass of the 192-row block over every expert, as good as always)
@@ -323,17 +323,19 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
       return t.variant;
     }
     // (a partial last K tile on the mid-M kernel wants both scale tensors in MFMA32 order: handed over that way, or
-    // re-laid by the one fast launch, which takes K in multiples of 128; the two launches of the general conversion
-    // cost more than the kernel saves, 16 x 5760 x 2880 12.3 -> 16.7 us)
-    if (mid_shape_ok(m, n, k) && (k % kTileK == 0 || native_scales || k % 128 == 0)) {
+    // re-laid in scratch by the launch in front)
+    if (mid_shape_ok(m, n, k)) {
       const int64_t cus = device_cus();
       // (a partial last K tile: the streaming kernel does not take it, and the direct kernel that would serve up to
       // 64 rows loses from N = 4096 on; scales in MFMA32 order, us: 16 x 23040 x 2880 27.5 -> 13.0, 64 x 23040
       // 32.9 -> 13.8, 64 x 5760 15.9 -> 12.2, and 256 x 23040 on the tiles 33.0 -> 20.4)
-      const bool k_tail = k % kTileK != 0;
+      // (with row-major scales the launch that re-lays them costs a narrow B more than the kernel saves: 16 x 5760 x
+      // 2880 12.2 -> 16.0 us, against 27.5 -> 19.5 at N = 23040; there the borders of whole K tiles hold from N = 12288 on)
+      const bool k_tail = k % kTileK != 0 && native_scales;
+      const bool rm_tail = k % kTileK != 0 && !native_scales;
       const bool mid = m > 192  ? n >= 20480 && n <= 128 * cus
                        : m > 64 ? n >= 12288 || (k <= 4096 && n >= 8192 && m > 96)
-                       : m > 32 ? n >= 12288 || (k <= 4096 && n >= 4096) || (!native_scales && k <= 8192 && n >= 6144)
+                       : m > 32 ? n >= 12288 || (!rm_tail && ((k <= 4096 && n >= 4096) || (!native_scales && k <= 8192 && n >= 6144)))
                        : m > 16 ? (n >= 12288 && n <= 320 * cus) || (k_tail && n >= 4096)
                                 : (n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus)) || (k_tail && n >= 4096);
       // Both scale tensors already in MFMA32 order (static weights, activations from the quantiser): no kernel

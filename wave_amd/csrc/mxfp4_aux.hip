@@ -104,8 +104,8 @@ __global__ void scale_convert_kernel(const uint8_t *__restrict__ src, int src_la
   }
 }
 
-// Row-major -> MFMA32 for ks % 4 == 0, the conversion in front of every tile
-// GEMM with row-major scales.  A workgroup takes 32 blocks of (32 rows x one K
+// Row-major -> MFMA32, the conversion in front of every tile GEMM with row-major scales (8-byte reads as two
+// dwords where the rows start on dwords, ks % 4 == 0; byte reads otherwise).  A workgroup takes 32 blocks of (32 rows x one K
 // tile): 32 rows x 32 K tiles, or for short rows 64 x 16 or 128 x 8, so that all
 // of its threads have a piece whatever K is (with 16 K tiles a row, K = 4096, half
 // of them had none).  8-byte reads that walk each row contiguously, the even and
@@ -133,7 +133,7 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
   const uint8_t *src = blockIdx.z ? src1 : src0;
   uint8_t *dst = blockIdx.z ? dst1 : dst0;
   const int rows = blockIdx.z ? rows1 : rows0;
-  const int k_tiles = (ks + 7) >> 3;  // ks % 4 == 0: the last K tile may hold 4 groups only (the rest is written as 0)
+  const int k_tiles = (ks + 7) >> 3;  // the last K tile may hold fewer than 8 groups (the rest is written as 0)
   const int kt_log = scale_wg_kt_log(k_tiles), kt_mask = (1 << kt_log) - 1;
   const int rt0 = blockIdx.x << (5 - kt_log), kt0 = blockIdx.y << kt_log;  // row tiles along x: up to 2^31 - 1 workgroups
   const int row_base = rt0 * 32;
@@ -146,8 +146,17 @@ __global__ void __launch_bounds__(256) scale_to_mfma32_kernel(const uint8_t *__r
     uint2 v = make_uint2(0u, 0u);
     if (row < rows && kt < k_tiles) {
       const uint8_t *at = src + (int64_t)row * ks + (int64_t)kt * 8;
-      v.x = *(const uint32_t *)at;
-      if (kt * 8 + 4 < ks) v.y = *(const uint32_t *)(at + 4);
+      if ((ks & 3) == 0) {
+        v.x = *(const uint32_t *)at;
+        if (kt * 8 + 4 < ks) v.y = *(const uint32_t *)(at + 4);
+      } else {
+        // rows that do not start on dwords (K % 128 != 0): byte by byte, groups past the end of the row stay 0
+        const int valid = min(8, ks - kt * 8);
+        for (int b = 0; b < valid; ++b) {
+          const uint32_t byte = at[b];
+          if (b < 4) v.x |= byte << (8 * b); else v.y |= byte << (8 * (b - 4));
+        }
+      }
     }
     const int blk = ((r >> 5) << kt_log) + ktl;
     stage[blk * 65 + (r & 31)] = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u);       // groups 0, 2, 4, 6
@@ -399,7 +408,9 @@ hipError_t launch_scale_pair_to_mfma32(const uint8_t *a_src, uint8_t *a_dst, int
     b_rows = 0;
   }
   const int64_t rows_max = a_rows > b_rows ? a_rows : b_rows;
-  if ((ks & 3) != 0 || ks == 0 || ((uintptr_t)a_src & 3) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 3) != 0) ||
+  // (dword reads where the rows start on dwords, byte reads otherwise)
+  const bool dwords = (ks & 3) == 0;
+  if (ks == 0 || (dwords && (((uintptr_t)a_src & 3) != 0 || (b_rows > 0 && ((uintptr_t)b_src & 3) != 0))) ||
       rows_max >= ((int64_t)1 << 31) || ((ks + 7) / 8 + 31) / 32 > 65535 || a_rows <= 0 || b_rows < 0)
     return hipErrorInvalidValue;
   const int kt_log = scale_wg_kt_log((int)((ks + 7) / 8));

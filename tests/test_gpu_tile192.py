@@ -80,3 +80,26 @@ def test_tile192_auto_choice_where_n_is_not_in_whole_256_column_tiles():
     auto = run(x, xs, w, ws, torch.float32)
     rows = np.arange(0, m, 53)
     assert_close(auto[rows], c_oracle.scaled_gemm_exact(x, w, xs, ws, rows=rows), torch.float32, "one round")
+
+
+@pytest.mark.parametrize("native", [False, True], ids=["row_major_scales", "mfma32_scales"])
+def test_tile192_auto_choice_outside_the_range_of_the_duration_estimates(native):
+    """K below the range where the library chooses by duration estimates, N = 30 x 192 = 22.5 x 256, 16 tile rows: the
+    borders pick the 256x256 tiles, which would run in two whole rounds, and from there the persistent kernel on
+    480 tiles of 256x192 - with either scale layout the same bits as that kernel by name."""
+    m, n, k = 4096, 5760, 1024
+    x, xs, w, ws = orc.make_inputs(m, n, k, seed=12, scale_lo=110, scale_hi=142)
+    gx, gxs, gw, gws = to_gpu(x, xs, w, ws)
+    kw = {}
+    if native:
+        gxs = wave_amd.scale_convert(gxs, m, k // 32, _lib.SCALE_ROW_MAJOR, _lib.SCALE_MFMA32)
+        gws = wave_amd.scale_convert(gws, n, k // 32, _lib.SCALE_ROW_MAJOR, _lib.SCALE_MFMA32)
+        kw = dict(a_scale_layout=_lib.SCALE_MFMA32, b_scale_layout=_lib.SCALE_MFMA32)
+    auto = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
+    named = torch.full_like(auto, float("nan"))
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, auto, **kw)
+    wave_amd.mxfp4_gemm(gx, gxs, gw, gws, named, variant=V, split_k=1, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(auto, named)
+    rows = np.unique(np.concatenate([np.arange(0, m, 173), [255, 256, m - 1]]))
+    assert_close(auto.cpu().numpy()[rows], c_oracle.scaled_gemm_exact(x, w, xs, ws, rows=rows), torch.float32, "rows vs oracle")

@@ -764,7 +764,7 @@ def main():
     if args.workload == "tile_choice":
         # The library's own choice of tile shape, split along K and kernel against every candidate asked for by
         # name, on shapes drawn at random from the range where it chooses by duration estimates (more than 64 rows,
-        # N = 2048..16384, K >= 3584 in whole K tiles, at most two rounds of 256x256 tiles).  Operand sets are
+        # N = 2048..32768, K >= 3584 in whole K tiles, at most two rounds of 256x256 tiles; drawn here up to 15360).  Operand sets are
         # rotated past the 256 MB memory-side cache, so B comes from HBM as a model's weights do; bf16 out; either
         # scale layout.  Every timing is the best of two; the library's choice is timed last.
         import math

@@ -176,9 +176,11 @@ static double mid_cost_us(int64_t m, int64_t n, int64_t k) {
   return 4.5 + (double)(k / kTileK) * step * (rounds < 1.0 ? 1.0 : rounds) + (double)n / 14336.0;
 }
 
-// Where the estimates hold: whole K tiles, at most two rounds of 256x256 tiles, the measured range of N.
+// Where the estimates hold: whole K tiles, at most two rounds of 256x256 tiles, N up to one round of the mid-M
+// kernel's strips (fitted on N <= 14336; on 60 random shapes of N = 16512 .. 32768 the choice by them was at 1.012 of
+// the best kernel by name in the geometric mean, the borders at 1.026 with a worst case of 1.38).
 static bool tile_model_applies(int64_t m, int64_t n, int64_t k) {
-  return m > 64 && n >= 2048 && n <= 16384 && k >= 3584 && k % kTileK == 0 && ((m + 255) / 256) * ((n + 255) / 256) <= 512;
+  return m > 64 && n >= 2048 && n <= 32768 && k >= 3584 && k % kTileK == 0 && ((m + 255) / 256) * ((n + 255) / 256) <= 512;
 }
 
 // The cheapest tile shape and split by the estimates (`only`: 0, or the one variant to find the split for).
@@ -314,7 +316,7 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     //     43.0 -> 44.5)
     //   M <= 16: the same range of N; up to 192 columns per CU only at K <= 4096 (16 x 28672 x 4096: 13.6 -> 13.0;
     //     a tie or 2 % lost at K = 8192: 16 x 40960 29.8 -> 30.3), beyond at any K (16 x 57344 x 8192: 41.4 -> 38.3)
-    // More than 64 rows, N up to 16384, at most two rounds of 256x256 tiles: by the estimates above, the mid-M
+    // More than 64 rows, N up to 32768, at most two rounds of 256x256 tiles: by the estimates above, the mid-M
     // kernel among the candidates up to 256 rows (the borders below were measured at K = 2048 .. 8192 and stay for
     // what lies outside: wider B, fewer rows).
     if (tile_model_applies(m, n, k)) {

@@ -89,6 +89,19 @@ def make_gpu_inputs(torch, m, n, k, seed, scale_range, device, copies=1):
     return sets
 
 
+def make_gpu_inputs_on_device(torch, m, n, k, scale_range, device, copies):
+    """`copies` operand sets drawn on the GPU (uniform nibbles, scales in `scale_range`): for sweeps that rotate
+    enough sets to keep B out of the 256 MB memory-side cache, where drawing on the host would dominate the run."""
+    lo, hi = scale_range
+    sets = []
+    for _ in range(copies):
+        sets.append((torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=device),
+                     torch.randint(lo, hi + 1, (m, k // 32), dtype=torch.uint8, device=device),
+                     torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=device),
+                     torch.randint(lo, hi + 1, (n, k // 32), dtype=torch.uint8, device=device)))
+    return sets
+
+
 def settle(torch, run, min_ms=None):
     """Untimed clock-settle load: `run(n)` launches n of the leg's kernels; repeated until `min_ms` of GPU time have
     passed.  Returns the GPU milliseconds spent."""
@@ -785,16 +798,10 @@ def main():
             if ((m + 255) // 256) * ((n + 255) // 256) > 512:
                 continue
             copies = max(2, min(80, math.ceil(400e6 / (n * k / 2))))
-            sets = []
-            for _ in range(copies):
-                x = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=dev)
-                xs = torch.randint(120, 135, (m, k // 32), dtype=torch.uint8, device=dev)
-                w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev)
-                ws = torch.randint(120, 135, (n, k // 32), dtype=torch.uint8, device=dev)
-                if native:
-                    xs = wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
-                    ws = wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)
-                sets.append((x, xs, w, ws))
+            sets = make_gpu_inputs_on_device(torch, m, n, k, (120, 134), dev, copies)
+            if native:
+                sets = [(x, wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32), w,
+                         wave_amd.scale_convert(ws, n, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32)) for x, xs, w, ws in sets]
             kw = dict(a_scale_layout=L.SCALE_MFMA32, b_scale_layout=L.SCALE_MFMA32) if native else {}
             out = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
             iters = max(16, copies)
@@ -850,8 +857,9 @@ def main():
         for k in (8192, 4096):
             for n in grid_n:
                 for m in grid_m:
-                    copies = max(2, min(6, int(600e6 / (n * k / 2))))
-                    sets = make_gpu_inputs(torch, m, n, k, 2, (120, 134), dev, copies=copies)
+                    # (at least 400 MB of B in rotation: beyond the 256 MB memory-side cache at every shape)
+                    copies = max(2, -(-400_000_000 // (n * k // 2)))
+                    sets = make_gpu_inputs_on_device(torch, m, n, k, (120, 134), dev, copies)
                     if resident or pre:
                         sets = [(x, wave_amd.scale_convert(xs, m, k // 32, L.SCALE_ROW_MAJOR, L.SCALE_MFMA32) if resident else xs,
                                  wave_amd.b_preshuffle(w) if pre else w,

@@ -321,6 +321,9 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
     // what lies outside: wider B, fewer rows).
     if (tile_model_applies(m, n, k)) {
       const TileChoice t = best_tile_choice(m, n, k, native_scales, 0);
+      // (two tile rows against a B this wide stream it slower per workgroup than the tables say: 256 x 20480 x 8192
+      // with scales in MFMA32 order 44.3 us on the 128x128 tiles, estimated 34, against 36.5 on the mid-M kernel)
+      if (m > 192 && n >= 20480 && mid_shape_ok(m, n, k)) return WAVE_MXFP4_VARIANT_MID_M;
       if (n >= 3584 && mid_shape_ok(m, n, k) && mid_cost_us(m, n, k) < t.us) return WAVE_MXFP4_VARIANT_MID_M;
       return t.variant;
     }
@@ -339,7 +342,11 @@ int pick_variant(int64_t m, int64_t n, int64_t k, int variant, bool native_scale
                        : m > 64 ? n >= 12288 || (k <= 4096 && n >= 8192 && m > 96)
                        : m > 32 ? n >= 12288 || (!rm_tail && ((k <= 4096 && n >= 4096) || (!native_scales && k <= 8192 && n >= 6144)))
                        : m > 16 ? (n >= 12288 && n <= 320 * cus) || (k_tail && n >= 4096)
-                                : (n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus)) || (k_tail && n >= 4096);
+                                : (n >= 12288 && n <= 320 * cus && (k <= 4096 || n > 192 * cus)) || (k_tail && n >= 4096) ||
+                                      // (scales in MFMA32 order, a nearly full single round of strips: 16 x 28672 x
+                                      // 8192 23.2 us on the streaming kernel, 21.1 here; level with row-major scales
+                                      // and at N = 20480, behind at 40960)
+                                      (native_scales && n >= 24576 && n <= 128 * cus);
       // Both scale tensors already in MFMA32 order (static weights, activations from the quantiser): no kernel
       // needs a re-layout launch in front, and the mid-M kernel cannot narrow its strips (a wave's strip is a
       // 32-row scale block), which moves some borders.  Measured with the weights from HBM on a grid of M = 16 ..
